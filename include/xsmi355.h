@@ -1,0 +1,143 @@
+/*
+ * xsmi355.h -- C ABI of libxsmi355.so: the MI355X (gfx950) conv / max-pool
+ * backend behind xshinnosuke's functional API.
+ *
+ * Conventions
+ *   - Every function returns 0 on success and a non-zero code on failure; the
+ *     message for the calling thread's last failure is xsmi_last_error().
+ *     No C++ exception crosses this boundary.
+ *   - Tensors are dense NCHW float32 in device memory.  Device pointers are the
+ *     opaque values returned by xsmi_malloc.
+ *   - Ops never allocate: scratch memory (packed filters, split-reduction
+ *     partials) is a caller-provided workspace sized by the matching
+ *     *_workspace_bytes query.  The workspace contents are dead after the call
+ *     has completed on the stream.
+ *   - All work is enqueued on one library-owned stream; results are visible to
+ *     the host after xsmi_sync() or a (blocking) xsmi_memcpy_d2h.
+ *   - Window geometry follows the reference: symmetric integer zero padding
+ *     `pad`, stride (sh, sw), OH = (H + 2*pad - R)/sh + 1 (floor), no dilation,
+ *     no groups.
+ *
+ * The reference is pure Python and has no FFI of its own; each entry point
+ * below names the reference function whose arithmetic it replaces.
+ */
+#ifndef XSMI355_H
+#define XSMI355_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define XSMI_OK 0
+#define XSMI_ERR_INVALID 1   /* bad argument (shape, pointer, workspace too small) */
+#define XSMI_ERR_RUNTIME 2   /* HIP runtime failure */
+#define XSMI_ERR_STATE 3     /* library not initialised */
+
+/* flags for the conv entry points */
+#define XSMI_CONV_RELU 0x1u      /* y = max(0, conv + bias)  (fused epilogue)            */
+#define XSMI_CONV_BF16 0x2u      /* opt-in: bf16 MFMA operands, fp32 accumulate          */
+
+typedef struct xsmi_device_info {
+    int device;
+    int cu_count;
+    int clock_khz;
+    int lds_bytes_per_cu;
+    int wavefront;
+    int l2_bytes;
+    uint64_t hbm_bytes;
+    char name[128];
+    char arch[64];
+} xsmi_device_info_t;
+
+/* ---- runtime ------------------------------------------------------------
+ * Replaces the reference's array-module switch to CuPy
+ * (xs/core/__global.py:9, xs/core/base.py:143-146, 167-170) and the implicit
+ * host<->device copies of Tensor.to()/numpy() (xs/core/base.py:136-184, 211-217).
+ */
+int xsmi_init(int device);
+int xsmi_is_initialized(void);
+const char *xsmi_last_error(void);
+int xsmi_device_info(xsmi_device_info_t *info);
+int xsmi_malloc(void **ptr, size_t bytes);
+int xsmi_free(void *ptr);
+int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes);   /* blocking */
+int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes);   /* blocking */
+int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes);   /* async on the stream */
+int xsmi_memset(void *dst, int byte_value, size_t bytes);        /* async on the stream */
+int xsmi_sync(void);
+int xsmi_event_create(void **event);
+int xsmi_event_record(void *event);                               /* on the library stream */
+int xsmi_event_elapsed_ms(void *start, void *stop, float *ms);    /* waits for `stop` */
+int xsmi_event_destroy(void *event);
+/* plain float4 copy kernel of `bytes` bytes (multiple of 16); used to
+ * calibrate HBM counters and to quote the achievable copy bandwidth. */
+int xsmi_copy_kernel(void *dst, const void *src, size_t bytes);
+
+/* ---- convolution ---------------------------------------------------------
+ * x (N,C,H,W), w (K,C,R,S), bias (K) or NULL, y (N,K,OH,OW).
+ */
+
+/* Workspace needed by the three conv entry points for this geometry (the
+ * maximum over fwd / bwd_data / bwd_weight and over flags). */
+size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S,
+                                   int sh, int sw, int pad);
+
+/* Forward: replaces conv2d (xs/nn/functional.py:405-442) incl. im2col
+ * (xs/utils/common.py:35-46); with XSMI_CONV_RELU also the ReLU that
+ * Conv2D.call applies (xs/layers/convolutional.py:76-77, xs/nn/td_functional.py:59-60).
+ * neg_mask (N*K*OH*OW bytes) may be NULL; when given together with
+ * XSMI_CONV_RELU it receives 1 where the pre-activation is < 0 and 0 elsewhere
+ * (the strict mask of ReLUBackward, xs/nn/grad_fn.py:155-157). */
+int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
+                    uint8_t *neg_mask,
+                    int N, int C, int H, int W, int K, int R, int S,
+                    int sh, int sw, int pad, unsigned flags,
+                    void *workspace, size_t workspace_bytes);
+
+/* Backward w.r.t. the input: dx = beta*dx + fold(dy^T . w).  Replaces the dcol
+ * GEMM + col2im of Conv2DBackward (xs/nn/grad_fn.py:199-203, xs/utils/common.py:49-65).
+ * beta must be 0 (overwrite) or 1 (accumulate, what the reference always does). */
+int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx,
+                         int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int pad, float beta, unsigned flags,
+                         void *workspace, size_t workspace_bytes);
+
+/* Backward w.r.t. filter and bias: dw = beta*dw + dy . unfold(x), db = beta*db + sum(dy).
+ * Replaces xs/nn/grad_fn.py:191-197.  db may be NULL.  The reduction order is
+ * fixed (no float atomics): partial sums per pixel range, then one pass that adds
+ * the partials in float64 in ascending range order. */
+int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db,
+                           int N, int C, int H, int W, int K, int R, int S,
+                           int sh, int sw, int pad, float beta, unsigned flags,
+                           void *workspace, size_t workspace_bytes);
+
+/* ---- max pooling ---------------------------------------------------------
+ * x (N,C,H,W) -> y (N,C,OH,OW), square window k, zero-valued padding that takes
+ * part in the max, first maximum in row-major (ky,kx) order wins.
+ * idx holds ky*k+kx as uint8, stored in NCHW order (the reference keeps the same
+ * values as int64 in (n,oh,ow,c) order).
+ */
+
+/* Replaces max_pool2d (xs/nn/functional.py:445-491). idx may be NULL. */
+int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx,
+                       int N, int C, int H, int W, int k, int sh, int sw, int pad);
+
+/* Replaces Maxpool2DBackward (xs/nn/grad_fn.py:224-235): gather formulation,
+ * float64 sum over the covering windows in ascending (ky,kx) order, one rounding:
+ * dx = round32(beta*dx + sum). beta is 0 or 1. */
+int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx,
+                       int N, int C, int H, int W, int k, int sh, int sw, int pad,
+                       float beta);
+
+/* ---- ReLU mask backward ----------------------------------------------------
+ * dx = beta*dx + (neg_mask ? 0 : dy) over n elements.  Replaces ReLUBackward
+ * (xs/nn/grad_fn.py:146-157) for the fused conv epilogue. dx may alias dy. */
+int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size_t n, float beta);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* XSMI355_H */

@@ -1,0 +1,169 @@
+"""Conv parity on the GPU through the C ABI.
+
+Tolerance (fp32 MFMA path): relative L2 error <= 1e-5 against the oracle, which
+computes in float64 and rounds once to float32 like the reference.
+"""
+import os
+
+import numpy as np
+import pytest
+
+import oracle
+from util import rel_l2, he_normal
+
+pytestmark = pytest.mark.gpu
+TOL = 1e-5
+
+CASES = [  # n c h w k r s sh sw pad
+    (1, 1, 4, 4, 3, 3, 3, 1, 1, 0),        # tests/gradient_check/xs_pytorch/cnn.py shapes
+    (2, 3, 7, 6, 4, 3, 3, 1, 1, 1),
+    (1, 3, 5, 5, 1, 3, 3, 1, 1, 0),        # tests/gradient_check/check_cnn.py shapes
+    (4, 1, 28, 28, 8, 2, 2, 1, 1, 0),      # README net conv
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),    # BASELINE conv geometry, fewer images
+    (2, 3, 32, 32, 64, 7, 7, 2, 2, 3),     # ResNet stem geometry (small image)
+    (2, 64, 28, 28, 128, 3, 3, 2, 2, 1),   # layer2.0 conv_a
+    (2, 64, 28, 28, 128, 1, 1, 2, 2, 0),   # 1x1 / 2 shortcut
+    (3, 128, 14, 14, 128, 3, 3, 1, 1, 1),
+    (2, 256, 7, 7, 512, 3, 3, 2, 2, 1),    # small-M layer
+    (1, 5, 9, 11, 70, 3, 2, 1, 2, 2),      # ragged: rows not a multiple of 64, asymmetric filter/stride
+    (2, 7, 13, 12, 9, 5, 5, 3, 2, 2),      # stride 3x2, leftover input rows get zero gradient
+    (1, 2, 6, 6, 3, 3, 3, 1, 1, 2),        # pad > (R-1)/2
+    (5, 33, 10, 10, 65, 1, 1, 1, 1, 0),    # 1x1 == GEMM, odd sizes
+    (1, 1, 3, 3, 1, 3, 3, 1, 1, 0),        # single output pixel
+]
+
+
+def _oracle(x, w, b, stride, pad, dy):
+    y, col = oracle.conv2d_fwd(x, w, b, stride, pad)
+    dx, dw, db = oracle.conv2d_bwd(dy, x.shape, w, col, stride, pad,
+                                   np.zeros_like(x), np.zeros_like(w), np.zeros((w.shape[0],), dtype=np.float32))
+    return y, dx, dw, db
+
+
+@pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", CASES)
+def test_conv_fwd_bwd_parity(gpu, n, c, h, w, k, r, s, sh, sw, pad):
+    K = gpu.kernels
+    rng = np.random.default_rng(1000 + c * k + h)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = he_normal(rng, (k, c, r, s))
+    b = rng.standard_normal((k,)).astype(np.float32)
+    oh, ow = K.conv_out_hw(h, w, r, s, (sh, sw), pad)
+    dy = rng.standard_normal((n, k, oh, ow)).astype(np.float32)
+    y_ref, dx_ref, dw_ref, db_ref = _oracle(x, wt, b, (sh, sw), pad, dy)
+
+    dx_, dw_, db_, ddy = gpu.to_device(x), gpu.to_device(wt), gpu.to_device(b), gpu.to_device(dy)
+    y = K.conv2d_fwd(dx_, dw_, db_, (sh, sw), pad).numpy()
+    assert y.shape == y_ref.shape
+    assert rel_l2(y, y_ref) <= TOL
+    gx = K.conv2d_bwd_data(ddy, dw_, x.shape, (sh, sw), pad).numpy()
+    assert rel_l2(gx, dx_ref) <= TOL
+    gw, gb = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (sh, sw), pad, want_db=True)
+    assert rel_l2(gw.numpy(), dw_ref) <= TOL
+    assert rel_l2(gb.numpy(), db_ref) <= TOL
+
+
+def test_conv_accumulates_into_existing_gradients(gpu):
+    K = gpu.kernels
+    rng = np.random.default_rng(7)
+    x = rng.standard_normal((2, 6, 9, 9)).astype(np.float32); wt = he_normal(rng, (10, 6, 3, 3))
+    dy = rng.standard_normal((2, 10, 5, 5)).astype(np.float32)
+    _, col = oracle.conv2d_fwd(x, wt, None, (2, 2), 1)
+    dx0 = rng.standard_normal(x.shape).astype(np.float32); dw0 = rng.standard_normal(wt.shape).astype(np.float32)
+    db0 = rng.standard_normal((10,)).astype(np.float32)
+    dx_ref, dw_ref, db_ref = oracle.conv2d_bwd(dy, x.shape, wt, col, (2, 2), 1, dx0.copy(), dw0.copy(), db0.copy())
+    gx, gw, gb = gpu.to_device(dx0), gpu.to_device(dw0), gpu.to_device(db0)
+    ddy = gpu.to_device(dy)
+    K.conv2d_bwd_data(ddy, gpu.to_device(wt), x.shape, (2, 2), 1, dx=gx, accumulate=True)
+    K.conv2d_bwd_weight(ddy, gpu.to_device(x), wt.shape, (2, 2), 1, dw=gw, db=gb, accumulate=True)
+    assert rel_l2(gx.numpy(), dx_ref) <= TOL
+    assert rel_l2(gw.numpy(), dw_ref) <= TOL
+    assert rel_l2(gb.numpy(), db_ref) <= TOL
+
+
+def test_conv_fused_bias_relu_and_mask(gpu):
+    K = gpu.kernels
+    rng = np.random.default_rng(8)
+    x = rng.standard_normal((3, 4, 12, 12)).astype(np.float32); wt = he_normal(rng, (6, 4, 3, 3))
+    b = rng.standard_normal((6,)).astype(np.float32)
+    pre_ref, _ = oracle.conv2d_fwd(x, wt, b, (1, 1), 1)
+    dx_, dw_, db_ = gpu.to_device(x), gpu.to_device(wt), gpu.to_device(b)
+    pre = K.conv2d_fwd(dx_, dw_, db_, (1, 1), 1).numpy()
+    mask = gpu.empty(pre.shape, np.uint8)
+    act = K.conv2d_fwd(dx_, dw_, db_, (1, 1), 1, relu=True, neg_mask=mask).numpy()
+    np.testing.assert_array_equal(act, oracle.relu_fwd(pre))           # same kernel arithmetic, then max(0, .)
+    np.testing.assert_array_equal(mask.numpy(), (pre < 0).astype(np.uint8))
+    assert rel_l2(act, oracle.relu_fwd(pre_ref)) <= TOL
+    dy = rng.standard_normal(pre.shape).astype(np.float32)
+    g = K.relu_mask_bwd(gpu.to_device(dy), mask).numpy()
+    np.testing.assert_array_equal(g, oracle.relu_bwd(dy, pre))
+
+
+def test_conv_special_kernels_exact(gpu):
+    """Closed forms that need no rounding: delta filter == shift, ones filter on small integers == box sum."""
+    K = gpu.kernels
+    rng = np.random.default_rng(9)
+    x = rng.integers(-8, 9, size=(2, 1, 10, 12)).astype(np.float32)
+    wd = np.zeros((1, 1, 3, 3), dtype=np.float32); wd[0, 0, 0, 2] = 1.0
+    y = K.conv2d_fwd(gpu.to_device(x), gpu.to_device(wd), None, (1, 1), 1).numpy()
+    ref = np.zeros_like(x); ref[:, :, 1:, :-1] = x[:, :, :-1, 1:]
+    np.testing.assert_array_equal(y, ref)
+    wo = np.ones((1, 1, 2, 2), dtype=np.float32)
+    y = K.conv2d_fwd(gpu.to_device(x), gpu.to_device(wo), None, (1, 1), 0).numpy()
+    np.testing.assert_array_equal(y, x[:, :, :-1, :-1] + x[:, :, 1:, :-1] + x[:, :, :-1, 1:] + x[:, :, 1:, 1:])
+
+
+def test_conv_golden_fixture(gpu):
+    K = gpu.kernels
+    g = np.load(os.path.join(os.path.dirname(__file__), "golden", "conv_pool_small.npz"))
+    stride = tuple(int(v) for v in g["conv_stride"]); pad = int(g["conv_pad"])
+    x, w, b, dy = (gpu.to_device(g[k]) for k in ("conv_x", "conv_w", "conv_b", "conv_dy"))
+    # dyadic inputs: every partial sum is exactly representable, so the match is exact
+    np.testing.assert_array_equal(K.conv2d_fwd(x, w, b.reshape(-1), stride, pad).numpy(), g["conv_y"])
+    np.testing.assert_array_equal(K.conv2d_bwd_data(dy, w, x.shape, stride, pad).numpy(), g["conv_dx"])
+    gw, gb = K.conv2d_bwd_weight(dy, x, w.shape, stride, pad, want_db=True)
+    np.testing.assert_array_equal(gw.numpy(), g["conv_dw"])
+    np.testing.assert_array_equal(gb.numpy().reshape(1, -1), g["conv_db"])
+
+
+def test_conv_full_size_adjoint_and_slice(gpu):
+    """BASELINE conv config at full size (N=32, 64->64, 56x56, 3x3/1/1): bilinear identities in float64 on
+    the device results plus oracle parity on a slice of images."""
+    K = gpu.kernels
+    x = np.random.default_rng(1).standard_normal((32, 64, 56, 56), dtype=np.float32)
+    wt = he_normal(np.random.default_rng(2), (64, 64, 3, 3))
+    dy = np.random.default_rng(3).standard_normal((32, 64, 56, 56), dtype=np.float32)
+    dx_, dw_, ddy = gpu.to_device(x), gpu.to_device(wt), gpu.to_device(dy)
+    y = K.conv2d_fwd(dx_, dw_, None, (1, 1), 1).numpy()
+    gx = K.conv2d_bwd_data(ddy, dw_, x.shape, (1, 1), 1).numpy()
+    gw, gb = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (1, 1), 1, want_db=True)
+    gw, gb = gw.numpy(), gb.numpy()
+    f = np.float64
+    lhs = np.sum(dy.astype(f) * y.astype(f))
+    assert abs(lhs - np.sum(gx.astype(f) * x.astype(f))) <= 2e-5 * abs(lhs) + 1e-2 * np.sqrt(x.size) * 1e-5
+    assert abs(lhs - np.sum(gw.astype(f) * wt.astype(f))) <= 2e-5 * abs(lhs) + 1e-2 * np.sqrt(x.size) * 1e-5
+    assert rel_l2(gb, dy.astype(f).sum(axis=(0, 2, 3))) <= TOL
+    y_ref, col = oracle.conv2d_fwd(x[:2], wt, None, (1, 1), 1)
+    assert rel_l2(y[:2], y_ref) <= TOL
+    dx_ref, _, _ = oracle.conv2d_bwd(dy[:2], x[:2].shape, wt, col, (1, 1), 1, np.zeros_like(x[:2]), None, None)
+    assert rel_l2(gx[:2], dx_ref) <= TOL
+    # dW over the full batch in float64 (einsum over taps), the reference's dot(grad, col) without the 462 MB matrix
+    xp = np.pad(x, ((0, 0), (0, 0), (1, 1), (1, 1))).astype(f)
+    dw_ref = np.empty((64, 64, 3, 3))
+    dyf = dy.astype(f).transpose(1, 0, 2, 3).reshape(64, -1)
+    for r in range(3):
+        for s in range(3):
+            win = xp[:, :, r:r + 56, s:s + 56].transpose(1, 0, 2, 3).reshape(64, -1)
+            dw_ref[:, :, r, s] = dyf @ win.T
+    assert rel_l2(gw, dw_ref) <= TOL
+
+
+def test_conv_rejects_bad_arguments(gpu):
+    K = gpu.kernels
+    x = gpu.zeros((1, 3, 4, 4)); w = gpu.zeros((2, 4, 3, 3))
+    with pytest.raises(ValueError):
+        K.conv2d_fwd(x, w)                       # channel mismatch
+    w = gpu.zeros((2, 3, 5, 5))
+    with pytest.raises(ValueError):
+        K.conv2d_fwd(x, w)                       # filter larger than the input
+    with pytest.raises(ValueError):
+        K.conv2d_fwd(x, gpu.zeros((2, 3, 3, 3)), stride=(0, 1))

@@ -1,0 +1,168 @@
+"""Device-resident arrays owned by Python, allocated through the C ABI."""
+import ctypes
+
+import numpy as np
+
+from .capi import lib, ensure_init
+
+
+class _Block:
+    """One xsmi_malloc allocation, freed when the last view goes away."""
+
+    __slots__ = ("ptr", "nbytes")
+
+    def __init__(self, nbytes):
+        ensure_init()
+        p = ctypes.c_void_p()
+        lib.call("xsmi_malloc", ctypes.byref(p), int(nbytes))
+        self.ptr = p.value
+        self.nbytes = int(nbytes)
+
+    def __del__(self):
+        try:
+            if self.ptr:
+                lib.call("xsmi_free", ctypes.c_void_p(self.ptr))
+                self.ptr = None
+        except Exception:
+            pass
+
+
+class DeviceArray:
+    """Dense C-contiguous array in device memory (float32, uint8, int32 or int64).
+
+    Only what the conv / pool path needs: shape/dtype bookkeeping, host copies,
+    reshape, and slicing of the leading axis (the static graph re-slices its
+    preallocated buffers to a shorter last batch).
+    """
+
+    def __init__(self, shape, dtype=np.float32, _block=None, _offset=0):
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.nbytes = self.size * self.dtype.itemsize
+        self._block = _block if _block is not None else _Block(max(self.nbytes, 16))
+        self._offset = int(_offset)
+
+    @property
+    def ptr(self):
+        return self._block.ptr + self._offset
+
+    @property
+    def cptr(self):
+        return ctypes.c_void_p(self.ptr)
+
+    @property
+    def ndim(self):
+        return len(self.shape)
+
+    def numpy(self):
+        out = np.empty(self.shape, dtype=self.dtype)
+        if self.nbytes:
+            lib.call("xsmi_memcpy_d2h", out.ctypes.data_as(ctypes.c_void_p), self.cptr, self.nbytes)
+        return out
+
+    def __array__(self, dtype=None, copy=None):
+        a = self.numpy()
+        return a if dtype is None else a.astype(dtype, copy=False)
+
+    def set(self, host):
+        host = np.ascontiguousarray(host, dtype=self.dtype)
+        if host.shape != self.shape:
+            host = np.ascontiguousarray(np.broadcast_to(host, self.shape))
+        if self.nbytes:
+            lib.call("xsmi_memcpy_h2d", self.cptr, host.ctypes.data_as(ctypes.c_void_p), self.nbytes)
+        return self
+
+    def copy_from(self, other):
+        if other.nbytes != self.nbytes:
+            raise ValueError("size mismatch in device copy: %s vs %s" % (other.shape, self.shape))
+        if self.nbytes:
+            lib.call("xsmi_memcpy_d2d", self.cptr, other.cptr, self.nbytes)
+        return self
+
+    def copy(self):
+        return DeviceArray(self.shape, self.dtype).copy_from(self)
+
+    def fill_zero(self):
+        if self.nbytes:
+            lib.call("xsmi_memset", self.cptr, 0, self.nbytes)
+        return self
+
+    def reshape(self, *shape):
+        if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+            shape = tuple(shape[0])
+        shape = list(shape)
+        if -1 in shape:
+            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            shape[shape.index(-1)] = self.size // max(known, 1)
+        if int(np.prod(shape, dtype=np.int64)) != self.size:
+            raise ValueError("cannot reshape %s into %s" % (self.shape, tuple(shape)))
+        return DeviceArray(shape, self.dtype, _block=self._block, _offset=self._offset)
+
+    def leading(self, start, stop):
+        """View of rows [start, stop) of the leading axis."""
+        n = self.shape[0]
+        start = 0 if start is None else start
+        stop = n if stop is None else min(stop, n)
+        row = (self.size // n) * self.dtype.itemsize if n else 0
+        return DeviceArray((stop - start,) + self.shape[1:], self.dtype, _block=self._block,
+                           _offset=self._offset + start * row)
+
+    def __getitem__(self, item):
+        if isinstance(item, slice) and item.step in (None, 1):
+            return self.leading(item.start, item.stop)
+        raise TypeError("device arrays only support contiguous slices of the leading axis")
+
+    def __repr__(self):
+        return "DeviceArray(shape=%s, dtype=%s)" % (self.shape, self.dtype)
+
+
+def empty(shape, dtype=np.float32):
+    return DeviceArray(shape, dtype)
+
+
+def zeros(shape, dtype=np.float32):
+    return DeviceArray(shape, dtype).fill_zero()
+
+
+def to_device(host, dtype=None):
+    host = np.asarray(host)
+    if dtype is None:
+        dtype = np.float32 if host.dtype.kind == "f" else host.dtype
+    return DeviceArray(host.shape, dtype).set(host)
+
+
+class Workspace:
+    """Grow-only scratch buffer handed to the conv entry points."""
+
+    def __init__(self):
+        self._block = None
+
+    def get(self, nbytes):
+        if self._block is None or self._block.nbytes < nbytes:
+            self._block = None
+            self._block = _Block(max(int(nbytes), 256))
+        return ctypes.c_void_p(self._block.ptr), self._block.nbytes
+
+
+class Event:
+    def __init__(self):
+        ensure_init()
+        e = ctypes.c_void_p()
+        lib.call("xsmi_event_create", ctypes.byref(e))
+        self._e = e
+
+    def record(self):
+        lib.call("xsmi_event_record", self._e)
+        return self
+
+    def elapsed_ms(self, stop):
+        ms = ctypes.c_float()
+        lib.call("xsmi_event_elapsed_ms", self._e, stop._e, ctypes.byref(ms))
+        return ms.value
+
+    def __del__(self):
+        try:
+            lib.call("xsmi_event_destroy", self._e)
+        except Exception:
+            pass

@@ -1,0 +1,134 @@
+"""ctypes binding of ``libxsmi355.so`` (declared in ``include/xsmi355.h``).
+
+The library is the only compute path for conv / max-pool: if it is missing or
+cannot initialise a gfx950 device, the ops raise -- there is no CPU fallback.
+"""
+import ctypes
+import os
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libxsmi355.so")
+
+
+class XsmiError(RuntimeError):
+    """A call into libxsmi355.so failed."""
+
+
+class DeviceInfo(ctypes.Structure):
+    _fields_ = [
+        ("device", ctypes.c_int),
+        ("cu_count", ctypes.c_int),
+        ("clock_khz", ctypes.c_int),
+        ("lds_bytes_per_cu", ctypes.c_int),
+        ("wavefront", ctypes.c_int),
+        ("l2_bytes", ctypes.c_int),
+        ("hbm_bytes", ctypes.c_uint64),
+        ("name", ctypes.c_char * 128),
+        ("arch", ctypes.c_char * 64),
+    ]
+
+
+_c = ctypes
+_vp, _i, _sz, _f, _u = _c.c_void_p, _c.c_int, _c.c_size_t, _c.c_float, _c.c_uint
+_CONV_DIMS = [_i] * 10   # N C H W K R S sh sw pad
+
+# name -> (restype, argtypes); must list every symbol include/xsmi355.h declares
+SIGNATURES = {
+    "xsmi_init": (_i, [_i]),
+    "xsmi_is_initialized": (_i, []),
+    "xsmi_last_error": (_c.c_char_p, []),
+    "xsmi_device_info": (_i, [_c.POINTER(DeviceInfo)]),
+    "xsmi_malloc": (_i, [_c.POINTER(_vp), _sz]),
+    "xsmi_free": (_i, [_vp]),
+    "xsmi_memcpy_h2d": (_i, [_vp, _vp, _sz]),
+    "xsmi_memcpy_d2h": (_i, [_vp, _vp, _sz]),
+    "xsmi_memcpy_d2d": (_i, [_vp, _vp, _sz]),
+    "xsmi_memset": (_i, [_vp, _i, _sz]),
+    "xsmi_sync": (_i, []),
+    "xsmi_event_create": (_i, [_c.POINTER(_vp)]),
+    "xsmi_event_record": (_i, [_vp]),
+    "xsmi_event_elapsed_ms": (_i, [_vp, _vp, _c.POINTER(_f)]),
+    "xsmi_event_destroy": (_i, [_vp]),
+    "xsmi_copy_kernel": (_i, [_vp, _vp, _sz]),
+    "xsmi_conv2d_workspace_bytes": (_sz, _CONV_DIMS),
+    "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
+    "xsmi_conv2d_bwd_data": (_i, [_vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
+    "xsmi_conv2d_bwd_weight": (_i, [_vp, _vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
+    "xsmi_maxpool2d_fwd": (_i, [_vp, _vp, _vp] + [_i] * 8),
+    "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
+    "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),
+}
+
+CONV_RELU = 0x1
+CONV_BF16 = 0x2
+
+
+def library_path():
+    return _LIB_PATH
+
+
+class _Lib:
+    """Lazy handle: the shared object is opened on first use."""
+
+    def __init__(self):
+        self._dll = None
+
+    def _open(self):
+        if self._dll is not None:
+            return self._dll
+        if not os.path.exists(_LIB_PATH):
+            raise XsmiError(
+                "libxsmi355.so is not built (%s is missing); run "
+                "`make -C xshinnosuke_amd/csrc` or __graft_entry__.build()" % _LIB_PATH)
+        dll = ctypes.CDLL(_LIB_PATH)
+        for name, (res, args) in SIGNATURES.items():
+            fn = getattr(dll, name)          # AttributeError if the export is missing
+            fn.restype = res
+            fn.argtypes = args
+        self._dll = dll
+        return dll
+
+    def raw(self, name):
+        return getattr(self._open(), name)
+
+    def call(self, name, *args):
+        """Call an int-returning entry point; raise with the library's message on failure."""
+        dll = self._open()
+        rc = getattr(dll, name)(*args)
+        if rc != 0:
+            msg = dll.xsmi_last_error().decode("utf-8", "replace")
+            if rc == 1:
+                raise ValueError(msg)
+            raise XsmiError(msg)
+
+
+lib = _Lib()
+
+
+def init(device=0):
+    lib.call("xsmi_init", int(device))
+
+
+def is_initialized():
+    return bool(lib.raw("xsmi_is_initialized")())
+
+
+def ensure_init():
+    if not is_initialized():
+        init(0)
+
+
+def device_info():
+    ensure_init()
+    info = DeviceInfo()
+    lib.call("xsmi_device_info", ctypes.byref(info))
+    return {
+        "device": info.device, "cu_count": info.cu_count, "clock_khz": info.clock_khz,
+        "lds_bytes_per_cu": info.lds_bytes_per_cu, "wavefront": info.wavefront,
+        "l2_bytes": info.l2_bytes, "hbm_bytes": int(info.hbm_bytes),
+        "name": info.name.decode(), "arch": info.arch.decode(),
+    }
+
+
+def synchronize():
+    lib.call("xsmi_sync")

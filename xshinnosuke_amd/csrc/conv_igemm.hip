@@ -1,0 +1,433 @@
+// Implicit-GEMM convolution forward and backward-data on fp32 MFMA.
+//
+// Both directions are one "gather GEMM":
+//
+//     out[n, row, y, x] = sum_kk A[row][kk] * in[n, ch(kk), y*sy + dy(kk), x*sx + dx(kk)]
+//
+// where out-of-range (iy, ix) read as 0.  The unfolded matrix of the reference
+// (xs/utils/common.py:35-46) is never materialised: each thread owns one output
+// pixel for the whole reduction and forms its operand column from a per-kk
+// offset table while staging into LDS.
+//
+//   forward        rows = K filters, kk = (c, r, s), dy = r - pad, dx = s - pad,
+//                  sy = sh, sx = sw                  (xs/nn/functional.py:417-426)
+//   backward-data  one launch per residue class (ph, pw) of (h mod sh, w mod sw):
+//                  rows = C, kk = (k, t, u) over the taps r = r0 + sh*t, s = s0 + sw*u
+//                  that can reach that class, in = dy, sy = sx = 1, output written
+//                  with strides (sh*W, sw).  This equals the reference's
+//                  dcol GEMM + col2im (xs/nn/grad_fn.py:199-203,
+//                  xs/utils/common.py:49-65) without multiplying the zeros a
+//                  strided fold would meet.
+//
+// Tile: 64 rows x 128 pixels per 256-thread workgroup, reduction in chunks of 16;
+// wave w owns pixels [32w, 32w+32) x all 64 rows = two 32x32 accumulators fed by
+// v_mfma_f32_32x32x2_f32.  Within a chunk the lanes 0-31 of a wave take
+// kk = 0..7 and lanes 32-63 take kk = 8..15, so each lane reads its 8 operand
+// values for a row/pixel with two 128-bit LDS reads.
+#include "xsmi_internal.h"
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int TM = 64;    // rows per workgroup
+constexpr int BP = 128;   // pixels per workgroup
+constexpr int KC = 16;    // reduction chunk
+constexpr int LDP = 12;   // padded length of an 8-float LDS row
+
+struct IgemmParams {
+    const float *in;
+    const float *apk;      // packed A: [rowtile][chunk][half][64][8]
+    const int2 *ktab;      // per kk: {element offset, by | bx << 8}
+    const float *bias;
+    float *out;
+    uint8_t *mask;
+    uint32_t in_bytes;
+    int M;                 // pixels
+    int rows;              // valid rows
+    int nchunks;
+    int IH, IW, sy, sx, dymin, dxmin;
+    int in_n_stride;
+    int OY, OX;
+    xsmi::FastDiv dOX, dOY;
+    long long os_n, os_k, o_base;
+    int os_y, os_x;
+    int accumulate;
+    int relu;
+};
+
+__device__ __forceinline__ uint32_t range_mask(int lo_coord, int extent) {
+    // bit b (0..30) set iff 0 <= lo_coord + b < extent
+    int lo = lo_coord < 0 ? -lo_coord : 0;
+    int hi = extent - lo_coord;
+    if (hi > 31) hi = 31;
+    if (hi <= lo) return 0u;
+    return ((1u << (hi - lo)) - 1u) << lo;
+}
+
+__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t byte_off) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)byte_off, 0, 0));
+}
+
+__global__ void __launch_bounds__(256) igemm_f32_kernel(IgemmParams p) {
+    __shared__ __attribute__((aligned(16))) float As[2][2][TM][LDP];
+    __shared__ __attribute__((aligned(16))) float Bs[2][2][BP][LDP];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = t >> 6;
+    const int m0 = blockIdx.x * BP;
+    const int rowtile = blockIdx.y;
+
+    // ---- gather side: this thread stages pixel lj, reduction half lh ----
+    const int lj = t & (BP - 1);
+    const int lh = __builtin_amdgcn_readfirstlane(t >> 7);
+    uint32_t ymask = 0u, xmask = 0u;
+    uint32_t base_bytes = 0u;
+    {
+        int m = m0 + lj;
+        if (m < p.M) {
+            uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+            int x = m - (int)q * p.OX;
+            uint32_t n = xsmi::fdiv(q, p.dOY);
+            int y = (int)q - (int)n * p.OY;
+            int iy0 = y * p.sy + p.dymin;
+            int ix0 = x * p.sx + p.dxmin;
+            ymask = range_mask(iy0, p.IH);
+            xmask = range_mask(ix0, p.IW);
+            base_bytes = (uint32_t)(((int)n * p.in_n_stride + iy0 * p.IW + ix0) * 4);
+        }
+    }
+    // records beyond in_bytes read as 0: the invalid-lane offset is 0xffffffff
+    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.in, 0, p.in_bytes, 0x00020000);
+
+    const float4 *apk4 = reinterpret_cast<const float4 *>(p.apk) + (size_t)rowtile * p.nchunks * (TM * KC / 4) + t;
+    // LDS slot of the float4 this thread stages for A
+    const int a_h = (4 * t) >> 9, a_i = ((4 * t) & 511) >> 3, a_e = (4 * t) & 7;
+
+    float bnext[8];
+    float4 anext;
+
+    auto fetch = [&](int chunk) {
+        const int2 *kt = p.ktab + chunk * KC + lh * 8;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) {
+            int2 ent = kt[e];
+            uint32_t ok = (ymask >> (ent.y & 0xff)) & (xmask >> (ent.y >> 8)) & 1u;
+            uint32_t off = ok ? base_bytes + (uint32_t)ent.x * 4u : 0xffffffffu;
+            bnext[e] = buffer_load_f32(rsrc, off);
+        }
+        anext = apk4[(size_t)chunk * (TM * KC / 4)];
+    };
+    auto stage = [&](int buf) {
+        float4 *bd = reinterpret_cast<float4 *>(&Bs[buf][lh][lj][0]);
+        bd[0] = make_float4(bnext[0], bnext[1], bnext[2], bnext[3]);
+        bd[1] = make_float4(bnext[4], bnext[5], bnext[6], bnext[7]);
+        *reinterpret_cast<float4 *>(&As[buf][a_h][a_i][a_e]) = anext;
+    };
+
+    floatx16 acc0 = {0}, acc1 = {0};
+    const int h = lane >> 5, l31 = lane & 31;
+    const int jw = wave * 32;
+
+    if (p.nchunks > 0) {
+        fetch(0);
+        stage(0);
+    }
+    __syncthreads();
+    for (int c = 0; c < p.nchunks; ++c) {
+        const int cur = c & 1;
+        const bool more = c + 1 < p.nchunks;
+        if (more) fetch(c + 1);
+        const float4 *bp = reinterpret_cast<const float4 *>(&Bs[cur][h][jw + l31][0]);
+        const float4 *ap0 = reinterpret_cast<const float4 *>(&As[cur][h][l31][0]);
+        const float4 *ap1 = reinterpret_cast<const float4 *>(&As[cur][h][32 + l31][0]);
+        float4 b0 = bp[0], b1 = bp[1];
+        float4 a00 = ap0[0], a01 = ap0[1];
+        float4 a10 = ap1[0], a11 = ap1[1];
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a00.x, b0.x, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a10.x, b0.x, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a00.y, b0.y, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a10.y, b0.y, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a00.z, b0.z, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a10.z, b0.z, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a00.w, b0.w, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a10.w, b0.w, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.x, b1.x, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a11.x, b1.x, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.y, b1.y, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a11.y, b1.y, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.z, b1.z, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a11.z, b1.z, acc1, 0, 0, 0);
+        acc0 = __builtin_amdgcn_mfma_f32_32x32x2f32(a01.w, b1.w, acc0, 0, 0, 0);
+        acc1 = __builtin_amdgcn_mfma_f32_32x32x2f32(a11.w, b1.w, acc1, 0, 0, 0);
+        if (more) stage(cur ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: accumulator register v of lane l holds
+    //      row 8*(v/4) + 4*(l/32) + v%4, pixel l%32 of the 32x32 tile ----
+    const int m = m0 + jw + l31;
+    if (m >= p.M) return;
+    uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+    int x = m - (int)q * p.OX;
+    uint32_t n = xsmi::fdiv(q, p.dOY);
+    int y = (int)q - (int)n * p.OY;
+    const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
+    const int rbase = rowtile * TM + 4 * h;
+#pragma unroll
+    for (int it = 0; it < 2; ++it) {
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            int row = rbase + it * 32 + 8 * (v >> 2) + (v & 3);
+            if (row < p.rows) {
+                float val = it == 0 ? acc0[v] : acc1[v];
+                if (p.bias) val += p.bias[row];
+                long long o = pix_off + (long long)row * p.os_k;
+                if (p.relu) {
+                    if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
+                    val = val > 0.f ? val : 0.f;
+                }
+                if (p.accumulate) val += p.out[o];
+                p.out[o] = val;
+            }
+        }
+    }
+}
+
+// Packs the forward filter matrix and its offset table.
+//   A[row][kk] = w[row][kk]   (kk = (c*R + r)*S + s is the filter's own memory order)
+__global__ void __launch_bounds__(256) pack_fwd_kernel(const float *__restrict__ w, float *__restrict__ apk,
+                                                        int2 *__restrict__ ktab, int K, int C, int R, int S, int H,
+                                                        int W, int nchunks, int rowtiles) {
+    const int J = C * R * S;
+    const int total = rowtiles * nchunks * (TM * KC);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        int e = i & 7;
+        int r64 = (i >> 3) & 63;
+        int hh = (i >> 9) & 1;
+        int blk = i >> 10;                  // rowtile * nchunks + chunk
+        int chunk = blk % nchunks;
+        int rt = blk / nchunks;
+        int row = rt * TM + r64;
+        int kk = chunk * KC + hh * 8 + e;
+        apk[i] = (row < K && kk < J) ? w[(size_t)row * J + kk] : 0.f;
+    }
+    const int Kpad = nchunks * KC;
+    for (int kk = blockIdx.x * 256 + threadIdx.x; kk < Kpad; kk += gridDim.x * 256) {
+        int2 ent;
+        if (kk < J) {
+            int s = kk % S;
+            int r = (kk / S) % R;
+            int c = kk / (R * S);
+            ent.x = c * H * W + r * W + s;
+            ent.y = r | (s << 8);
+        } else {
+            ent.x = 0;
+            ent.y = 31 | (31 << 8);           // bit 31 of a range mask is never set
+        }
+        ktab[kk] = ent;
+    }
+}
+
+// Packs the backward-data matrix of one residue class.
+//   rows = c, kk = (k*T + t)*U + u, A[c][kk] = w[k][c][r0 + sh*t][s0 + sw*u],
+//   the gradient row read is y + cy - t  (cy = (ph + pad - r0)/sh), likewise columns.
+__global__ void __launch_bounds__(256) pack_bwd_kernel(const float *__restrict__ w, float *__restrict__ apk,
+                                                        int2 *__restrict__ ktab, int K, int C, int R, int S, int OH,
+                                                        int OW, int sh, int sw, int r0, int s0, int T, int U,
+                                                        int nchunks, int rowtiles) {
+    const int J = K * T * U;
+    const int total = rowtiles * nchunks * (TM * KC);
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        int e = i & 7;
+        int r64 = (i >> 3) & 63;
+        int hh = (i >> 9) & 1;
+        int blk = i >> 10;
+        int chunk = blk % nchunks;
+        int rt = blk / nchunks;
+        int c = rt * TM + r64;
+        int kk = chunk * KC + hh * 8 + e;
+        float v = 0.f;
+        if (c < C && kk < J) {
+            int u = kk % U;
+            int tt = (kk / U) % T;
+            int k = kk / (T * U);
+            v = w[(((size_t)k * C + c) * R + (r0 + sh * tt)) * S + (s0 + sw * u)];
+        }
+        apk[i] = v;
+    }
+    const int Kpad = nchunks * KC;
+    for (int kk = blockIdx.x * 256 + threadIdx.x; kk < Kpad; kk += gridDim.x * 256) {
+        int2 ent;
+        if (kk < J) {
+            int u = kk % U;
+            int tt = (kk / U) % T;
+            int k = kk / (T * U);
+            int by = T - 1 - tt, bx = U - 1 - u;
+            ent.x = k * OH * OW + by * OW + bx;
+            ent.y = by | (bx << 8);
+        } else {
+            ent.x = 0;
+            ent.y = 31 | (31 << 8);
+        }
+        ktab[kk] = ent;
+    }
+}
+
+struct ConvGeom {
+    int N, C, H, W, K, R, S, sh, sw, pad, OH, OW;
+};
+
+int check_conv(const char *fn, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, ConvGeom *g) {
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && K > 0, "%s: empty tensor (N=%d C=%d H=%d W=%d K=%d)", fn, N, C, H,
+                   W, K);
+    XSMI_CHECK_ARG(R >= 1 && S >= 1 && R <= 31 && S <= 31, "%s: filter %dx%d outside 1..31", fn, R, S);
+    XSMI_CHECK_ARG(sh >= 1 && sw >= 1, "%s: stride must be positive", fn);
+    XSMI_CHECK_ARG(pad >= 0, "%s: negative padding", fn);
+    XSMI_CHECK_ARG(H + 2 * pad >= R && W + 2 * pad >= S, "%s: filter %dx%d larger than the padded input %dx%d", fn, R, S,
+                   H + 2 * pad, W + 2 * pad);
+    g->N = N; g->C = C; g->H = H; g->W = W; g->K = K; g->R = R; g->S = S; g->sh = sh; g->sw = sw; g->pad = pad;
+    g->OH = (H + 2 * pad - R) / sh + 1;
+    g->OW = (W + 2 * pad - S) / sw + 1;
+    const double lim = 1073741824.0;   // 2^30 elements: byte offsets stay below 2^32
+    XSMI_CHECK_ARG((double)N * C * H * W < lim && (double)N * K * g->OH * g->OW < lim,
+                   "%s: tensors of 2^30 elements or more are not supported", fn);
+    XSMI_CHECK_ARG((double)C * R * S * K < lim, "%s: filter too large", fn);
+    return XSMI_OK;
+}
+
+size_t pack_bytes(int rows, int J) {
+    size_t rowtiles = (size_t)xsmi::ceil_div(rows, TM);
+    size_t nchunks = (size_t)xsmi::ceil_div(J, KC);
+    return xsmi::align_up(rowtiles * nchunks * TM * KC * sizeof(float), 256) +
+           xsmi::align_up(nchunks * KC * sizeof(int2), 256);
+}
+
+}  // namespace
+
+namespace xsmi {
+size_t conv_fwd_ws_bytes(int C, int K, int R, int S) { return pack_bytes(K, C * R * S); }
+size_t conv_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
+    size_t total = 0;
+    for (int ph = 0; ph < sh; ++ph)
+        for (int pw = 0; pw < sw; ++pw) {
+            // upper bound: every class gets at most ceil(R/sh) x ceil(S/sw) taps
+            total += pack_bytes(C, K * ceil_div(R, sh) * ceil_div(S, sw));
+        }
+    return total;
+}
+}  // namespace xsmi
+
+extern "C" {
+
+int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *neg_mask, int N, int C, int H,
+                    int W, int K, int R, int S, int sh, int sw, int pad, unsigned flags, void *workspace,
+                    size_t workspace_bytes) {
+    XSMI_REQUIRE_INIT();
+    ConvGeom g;
+    int rc = check_conv("xsmi_conv2d_fwd", N, C, H, W, K, R, S, sh, sw, pad, &g);
+    if (rc) return rc;
+    XSMI_CHECK_ARG(x && w && y, "xsmi_conv2d_fwd: null tensor pointer");
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16)) == 0, "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG(!(flags & XSMI_CONV_BF16), "xsmi_conv2d_fwd: the bf16 path is not available in this build");
+    const int J = C * R * S;
+    const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);
+    XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd: workspace of %zu bytes needed, %zu given", need,
+                   workspace_bytes);
+    const int rowtiles = xsmi::ceil_div(K, TM);
+    const int nchunks = xsmi::ceil_div(J, KC);
+    float *apk = (float *)workspace;
+    int2 *ktab = (int2 *)((char *)workspace + xsmi::align_up((size_t)rowtiles * nchunks * TM * KC * sizeof(float), 256));
+    hipStream_t st = xsmi::stream();
+    int pack_blocks = xsmi::ceil_div(rowtiles * nchunks * TM * KC, 256);
+    if (pack_blocks > 1024) pack_blocks = 1024;
+    hipLaunchKernelGGL(pack_fwd_kernel, dim3(pack_blocks), dim3(256), 0, st, w, apk, ktab, K, C, R, S, H, W, nchunks,
+                       rowtiles);
+    XSMI_LAUNCH_CHECK("pack_fwd_kernel");
+
+    IgemmParams p;
+    p.in = x; p.apk = apk; p.ktab = ktab; p.bias = bias; p.out = y;
+    p.mask = (flags & XSMI_CONV_RELU) ? neg_mask : nullptr;
+    p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
+    p.M = N * g.OH * g.OW;
+    p.rows = K;
+    p.nchunks = nchunks;
+    p.IH = H; p.IW = W; p.sy = sh; p.sx = sw; p.dymin = -pad; p.dxmin = -pad;
+    p.in_n_stride = C * H * W;
+    p.OY = g.OH; p.OX = g.OW;
+    p.dOX = xsmi::make_fastdiv(g.OW); p.dOY = xsmi::make_fastdiv(g.OH);
+    p.os_n = (long long)K * g.OH * g.OW; p.os_k = (long long)g.OH * g.OW; p.o_base = 0;
+    p.os_y = g.OW; p.os_x = 1;
+    p.accumulate = 0;
+    p.relu = (flags & XSMI_CONV_RELU) ? 1 : 0;
+    dim3 grid(xsmi::ceil_div(p.M, BP), rowtiles);
+    hipLaunchKernelGGL(igemm_f32_kernel, grid, dim3(256), 0, st, p);
+    XSMI_LAUNCH_CHECK("igemm_f32_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int pad, float beta, unsigned flags, void *workspace, size_t workspace_bytes) {
+    XSMI_REQUIRE_INIT();
+    ConvGeom g;
+    int rc = check_conv("xsmi_conv2d_bwd_data", N, C, H, W, K, R, S, sh, sw, pad, &g);
+    if (rc) return rc;
+    XSMI_CHECK_ARG(dy && w && dx, "xsmi_conv2d_bwd_data: null tensor pointer");
+    XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_conv2d_bwd_data: beta must be 0 or 1");
+    XSMI_CHECK_ARG((flags & ~XSMI_CONV_BF16) == 0, "xsmi_conv2d_bwd_data: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG(!(flags & XSMI_CONV_BF16), "xsmi_conv2d_bwd_data: the bf16 path is not available in this build");
+    const size_t need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
+    XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_bwd_data: workspace of %zu bytes needed, %zu given",
+                   need, workspace_bytes);
+    hipStream_t st = xsmi::stream();
+    char *ws = (char *)workspace;
+    const int rowtiles = xsmi::ceil_div(C, TM);
+    for (int ph = 0; ph < sh; ++ph) {
+        const int OYc = ph < H ? xsmi::ceil_div(H - ph, sh) : 0;
+        const int r0 = (ph + pad) % sh;
+        const int T = r0 < R ? xsmi::ceil_div(R - r0, sh) : 0;
+        const int cy = (ph + pad - r0) / sh;
+        for (int pw = 0; pw < sw; ++pw) {
+            const int OXc = pw < W ? xsmi::ceil_div(W - pw, sw) : 0;
+            if (OYc == 0 || OXc == 0) continue;
+            const int s0 = (pw + pad) % sw;
+            const int U = s0 < S ? xsmi::ceil_div(S - s0, sw) : 0;
+            const int cx = (pw + pad - s0) / sw;
+            const int J = K * T * U;
+            const int nchunks = xsmi::ceil_div(J, KC);
+            float *apk = (float *)ws;
+            size_t apk_bytes = xsmi::align_up((size_t)rowtiles * nchunks * TM * KC * sizeof(float), 256);
+            int2 *ktab = (int2 *)(ws + apk_bytes);
+            ws += apk_bytes + xsmi::align_up((size_t)nchunks * KC * sizeof(int2), 256);
+            if (nchunks > 0) {
+                int pack_blocks = xsmi::ceil_div(rowtiles * nchunks * TM * KC, 256);
+                if (pack_blocks > 1024) pack_blocks = 1024;
+                hipLaunchKernelGGL(pack_bwd_kernel, dim3(pack_blocks), dim3(256), 0, st, w, apk, ktab, K, C, R, S, g.OH,
+                                   g.OW, sh, sw, r0, s0, T, U, nchunks, rowtiles);
+                XSMI_LAUNCH_CHECK("pack_bwd_kernel");
+            }
+            IgemmParams p;
+            p.in = dy; p.apk = apk; p.ktab = ktab; p.bias = nullptr; p.out = dx; p.mask = nullptr;
+            p.in_bytes = (uint32_t)((size_t)N * K * g.OH * g.OW * 4);
+            p.M = N * OYc * OXc;
+            p.rows = C;
+            p.nchunks = nchunks;
+            p.IH = g.OH; p.IW = g.OW; p.sy = 1; p.sx = 1;
+            p.dymin = cy - (T - 1); p.dxmin = cx - (U - 1);
+            p.in_n_stride = K * g.OH * g.OW;
+            p.OY = OYc; p.OX = OXc;
+            p.dOX = xsmi::make_fastdiv(OXc); p.dOY = xsmi::make_fastdiv(OYc);
+            p.os_n = (long long)C * H * W; p.os_k = (long long)H * W; p.o_base = (long long)ph * W + pw;
+            p.os_y = sh * W; p.os_x = sw;
+            p.accumulate = beta == 1.f ? 1 : 0;
+            p.relu = 0;
+            dim3 grid(xsmi::ceil_div(p.M, BP), rowtiles);
+            hipLaunchKernelGGL(igemm_f32_kernel, grid, dim3(256), 0, st, p);
+            XSMI_LAUNCH_CHECK("igemm_f32_kernel");
+        }
+    }
+    return XSMI_OK;
+}
+
+}  // extern "C"

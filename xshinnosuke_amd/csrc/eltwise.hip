@@ -1,0 +1,62 @@
+// Element-wise helpers of the conv path and the workspace query.
+#include "xsmi_internal.h"
+
+namespace xsmi {
+size_t conv_fwd_ws_bytes(int C, int K, int R, int S);
+size_t conv_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw);
+size_t conv_bwd_weight_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW);
+}  // namespace xsmi
+
+namespace {
+
+// dx = (accumulate ? dx : 0) + (mask ? 0 : dy); four elements per thread when aligned.
+__global__ void __launch_bounds__(256) relu_mask_bwd_kernel(const float *__restrict__ dy, const uint8_t *__restrict__ mask,
+                                                             float *dx, size_t n, int accumulate) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {
+        float4 g = *reinterpret_cast<const float4 *>(dy + i);
+        uchar4 m = *reinterpret_cast<const uchar4 *>(mask + i);
+        float4 o = make_float4(m.x ? 0.f : g.x, m.y ? 0.f : g.y, m.z ? 0.f : g.z, m.w ? 0.f : g.w);
+        if (accumulate) {
+            float4 d = *reinterpret_cast<const float4 *>(dx + i);
+            o.x += d.x; o.y += d.y; o.z += d.z; o.w += d.w;
+        }
+        *reinterpret_cast<float4 *>(dx + i) = o;
+    } else {
+        for (; i < n; ++i) {
+            float o = mask[i] ? 0.f : dy[i];
+            if (accumulate) o += dx[i];
+            dx[i] = o;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad) {
+    if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || R <= 0 || S <= 0 || sh <= 0 || sw <= 0 || pad < 0) return 0;
+    if (H + 2 * pad < R || W + 2 * pad < S) return 0;
+    int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
+    size_t a = xsmi::conv_fwd_ws_bytes(C, K, R, S);
+    size_t b = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
+    size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
+    size_t m = a > b ? a : b;
+    return m > c ? m : c;
+}
+
+int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size_t n, float beta) {
+    XSMI_REQUIRE_INIT();
+    if (n == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dy && neg_mask && dx, "xsmi_relu_mask_bwd: null pointer");
+    XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_relu_mask_bwd: beta must be 0 or 1");
+    size_t threads = (n + 3) / 4;
+    hipLaunchKernelGGL(relu_mask_bwd_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, xsmi::stream(), dy,
+                       neg_mask, dx, n, beta == 1.f ? 1 : 0);
+    XSMI_LAUNCH_CHECK("relu_mask_bwd_kernel");
+    return XSMI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,263 @@
+// Max-pool forward (values + first-max index) and backward (gather) kernels.
+//
+// Semantics (reference xs/nn/functional.py:445-491, xs/nn/grad_fn.py:224-235):
+// the input is bordered with cells of value 0 that compete in the max; the
+// window is scanned in row-major (ky,kx) order and a later cell replaces the
+// current best only if it is strictly greater, which is np.argmax's "first
+// maximum".  Backward sums, per input cell, the upstream gradient of every
+// window whose recorded index points at that cell, in ascending (ky,kx) order in
+// float64, and rounds once.
+#include "xsmi_internal.h"
+
+namespace {
+
+struct PoolGeom {
+    int N, C, H, W, OH, OW, k, sh, sw, pad;
+    xsmi::FastDiv dOW, dOH;   // forward: decompose the flat output index
+    xsmi::FastDiv dW, dH;     // backward: decompose the flat input index
+    xsmi::FastDiv dsh, dsw;   // backward: window range
+};
+
+// One thread per output element; lanes run along ow so that loads of one
+// window row are contiguous across the wavefront.  KT > 0 unrolls the window.
+template <int KT>
+__global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restrict__ x, float *__restrict__ y,
+                                                            uint8_t *__restrict__ idx, PoolGeom g, uint32_t total) {
+    uint32_t o = blockIdx.x * 256u + threadIdx.x;
+    if (o >= total) return;
+    const int k = KT > 0 ? KT : g.k;
+    uint32_t t = xsmi::fdiv(o, g.dOW);
+    int ow = (int)(o - t * g.OW);
+    uint32_t nc = xsmi::fdiv(t, g.dOH);
+    int oh = (int)(t - nc * g.OH);
+    const float *plane = x + (size_t)nc * g.H * g.W;
+    int ih0 = oh * g.sh - g.pad;
+    int iw0 = ow * g.sw - g.pad;
+    float best = 0.f;
+    int where = 0;
+    bool first = true;
+#pragma unroll
+    for (int r = 0; r < k; ++r) {
+        int ih = ih0 + r;
+        bool rowok = (unsigned)ih < (unsigned)g.H;
+#pragma unroll
+        for (int s = 0; s < k; ++s) {
+            int iw = iw0 + s;
+            float v = 0.f;                                   // border cell
+            if (rowok && (unsigned)iw < (unsigned)g.W) v = plane[ih * g.W + iw];
+            if (first || v > best) {
+                best = v;
+                where = r * k + s;
+                first = false;
+            }
+        }
+    }
+    y[o] = best;
+    if (idx) idx[o] = (uint8_t)where;
+}
+
+// 3x3 window, stride 2, pad 1, W % 4 == 0 (so OW = W/2): one thread produces two
+// adjacent outputs of one row from float4 loads of columns [4j, 4j+3] of the
+// three input rows; column 4j-1 comes from the previous lane (or one scalar load
+// at a wavefront edge, or the zero border at j == 0).  x is fetched once per
+// window row; the row shared by vertically adjacent windows is re-read from
+// cache.
+__global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restrict__ x, float *__restrict__ y,
+                                                            uint8_t *__restrict__ idx, PoolGeom g,
+                                                            xsmi::FastDiv dQ, uint32_t total_pairs) {
+    uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    bool live = t < total_pairs;
+    if (!live) t = total_pairs - 1;
+    const int Q = g.OW >> 1;                 // output pairs per row == float4 per input row / 1
+    uint32_t row = xsmi::fdiv(t, dQ);        // (nc, oh)
+    int j = (int)(t - row * Q);
+    uint32_t nc = xsmi::fdiv(row, g.dOH);
+    int oh = (int)(row - nc * g.OH);
+    const float *plane = x + (size_t)nc * g.H * g.W;
+    const int lane = threadIdx.x & 63;
+
+    float b0 = 0.f, b1 = 0.f;
+    int w0 = 0, w1 = 0;
+    bool first = true;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        int ih = 2 * oh - 1 + r;
+        bool rowok = (unsigned)ih < (unsigned)g.H;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (rowok) v = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
+        float left = __shfl_up(v.w, 1);
+        if (j == 0) left = 0.f;                                       // zero border
+        else if (lane == 0) left = rowok ? plane[(size_t)ih * g.W + 4 * j - 1] : 0.f;
+        // output 2j: columns 4j-1, 4j, 4j+1 ; output 2j+1: columns 4j+1, 4j+2, 4j+3
+        if (first || left > b0) { b0 = left; w0 = r * 3 + 0; }
+        if (v.x > b0) { b0 = v.x; w0 = r * 3 + 1; }
+        if (v.y > b0) { b0 = v.y; w0 = r * 3 + 2; }
+        if (first || v.y > b1) { b1 = v.y; w1 = r * 3 + 0; }
+        if (v.z > b1) { b1 = v.z; w1 = r * 3 + 1; }
+        if (v.w > b1) { b1 = v.w; w1 = r * 3 + 2; }
+        first = false;
+    }
+    if (!live) return;
+    size_t o = (size_t)row * g.OW + 2 * j;
+    *reinterpret_cast<float2 *>(y + o) = make_float2(b0, b1);
+    if (idx) *reinterpret_cast<uchar2 *>(idx + o) = make_uchar2((unsigned char)w0, (unsigned char)w1);
+}
+
+// One thread per input-gradient element.
+__global__ void __launch_bounds__(256) maxpool_bwd_gather(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
+                                                           float *__restrict__ dx, PoolGeom g, uint32_t total, int accumulate) {
+    uint32_t e = blockIdx.x * 256u + threadIdx.x;
+    if (e >= total) return;
+    uint32_t t = xsmi::fdiv(e, g.dW);
+    int w = (int)(e - t * g.W);
+    uint32_t nc = xsmi::fdiv(t, g.dH);
+    int h = (int)(t - nc * g.H);
+    int qh = h + g.pad, qw = w + g.pad;
+    // windows oh with 0 <= qh - oh*sh < k, descending oh == ascending ky
+    int oh_hi = (int)xsmi::fdiv((uint32_t)qh, g.dsh);
+    int ow_hi = (int)xsmi::fdiv((uint32_t)qw, g.dsw);
+    if (oh_hi > g.OH - 1) oh_hi = g.OH - 1;
+    if (ow_hi > g.OW - 1) ow_hi = g.OW - 1;
+    const size_t obase = (size_t)nc * g.OH * g.OW;
+    double acc = 0.0;
+    for (int oh = oh_hi; oh >= 0; --oh) {
+        int r = qh - oh * g.sh;
+        if (r >= g.k) break;
+        for (int ow = ow_hi; ow >= 0; --ow) {
+            int s = qw - ow * g.sw;
+            if (s >= g.k) break;
+            size_t o = obase + (size_t)oh * g.OW + ow;
+            if ((int)idx[o] == r * g.k + s) acc += (double)dy[o];
+        }
+    }
+    if (accumulate) acc += (double)dx[e];
+    dx[e] = (float)acc;
+}
+
+// 3x3 / stride 2 / pad 1 with W % 4 == 0: one thread per four consecutive dx
+// columns 4j..4j+3 of one row.  Covering windows: ow in {2j-1+1.. } i.e. columns
+// qw = w+1 in [4j+1, 4j+4] are covered by ow = 2j (s = qw-4j in {1,2}),
+// ow = 2j+1 (s in {0,1,2} for qw = 4j+2..4j+4) and ow = 2j+2 (s = 0 for qw = 4j+4).
+__global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
+                                                            float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ4,
+                                                            uint32_t total_quads, int accumulate) {
+    uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= total_quads) return;
+    const int Q4 = g.W >> 2;
+    uint32_t row = xsmi::fdiv(t, dQ4);       // (nc, h)
+    int j = (int)(t - row * Q4);
+    uint32_t nc = xsmi::fdiv(row, g.dH);
+    int h = (int)(row - nc * g.H);
+    const size_t obase = (size_t)nc * g.OH * g.OW;
+    const int qh = h + 1;
+    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
+    // ascending ky == descending oh; for one oh ascending kx == descending ow
+    int oh_hi = qh >> 1;
+    for (int oh = oh_hi; oh >= 0 && oh >= oh_hi - 1; --oh) {
+        int r = qh - 2 * oh;
+        if (r > 2 || oh >= g.OH) continue;
+        const size_t ro = obase + (size_t)oh * g.OW;
+        const int r3 = r * 3;
+        // ow = 2j+2 (may be out of range), 2j+1, 2j
+        int owc = 2 * j + 2;
+        float gC = 0.f; int iC = -1;
+        if (owc < g.OW) { gC = dy[ro + owc]; iC = idx[ro + owc]; }
+        float2 gAB = *reinterpret_cast<const float2 *>(dy + ro + 2 * j);
+        uchar2 iAB = *reinterpret_cast<const uchar2 *>(idx + ro + 2 * j);
+        int iA = iAB.x, iB = iAB.y;
+        // column 4j   (qw=4j+1): ow=2j s=1
+        if (iA == r3 + 1) a0 += (double)gAB.x;
+        // column 4j+1 (qw=4j+2): ow=2j+1 s=0 first (higher ow == lower kx), then ow=2j s=2
+        if (iB == r3 + 0) a1 += (double)gAB.y;
+        if (iA == r3 + 2) a1 += (double)gAB.x;
+        // column 4j+2 (qw=4j+3): ow=2j+1 s=1
+        if (iB == r3 + 1) a2 += (double)gAB.y;
+        // column 4j+3 (qw=4j+4): ow=2j+2 s=0, then ow=2j+1 s=2
+        if (iC == r3 + 0) a3 += (double)gC;
+        if (iB == r3 + 2) a3 += (double)gAB.y;
+    }
+    float4 *out = reinterpret_cast<float4 *>(dx + (size_t)row * g.W + 4 * j);
+    if (accumulate) {
+        float4 old = *out;
+        a0 += (double)old.x; a1 += (double)old.y; a2 += (double)old.z; a3 += (double)old.w;
+    }
+    *out = make_float4((float)a0, (float)a1, (float)a2, (float)a3);
+}
+
+int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw, int pad, PoolGeom *g) {
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0, "%s: empty tensor (N=%d C=%d H=%d W=%d)", fn, N, C, H, W);
+    XSMI_CHECK_ARG(k >= 1 && k <= 15, "%s: window %d outside 1..15 (index is stored in one byte)", fn, k);
+    XSMI_CHECK_ARG(sh >= 1 && sw >= 1, "%s: stride must be positive", fn);
+    XSMI_CHECK_ARG(pad >= 0, "%s: negative padding", fn);
+    XSMI_CHECK_ARG(H + 2 * pad >= k && W + 2 * pad >= k, "%s: window %d larger than the padded input %dx%d", fn, k,
+                   H + 2 * pad, W + 2 * pad);
+    g->N = N; g->C = C; g->H = H; g->W = W; g->k = k; g->sh = sh; g->sw = sw; g->pad = pad;
+    g->OH = (H + 2 * pad - k) / sh + 1;
+    g->OW = (W + 2 * pad - k) / sw + 1;
+    XSMI_CHECK_ARG((double)N * C * H * W < 2147483648.0 && (double)N * C * g->OH * g->OW < 2147483648.0,
+                   "%s: tensors above 2^31 elements are not supported", fn);
+    g->dOW = xsmi::make_fastdiv(g->OW); g->dOH = xsmi::make_fastdiv(g->OH);
+    g->dW = xsmi::make_fastdiv(W); g->dH = xsmi::make_fastdiv(H);
+    g->dsh = xsmi::make_fastdiv(sh); g->dsw = xsmi::make_fastdiv(sw);
+    return XSMI_OK;
+}
+
+bool fast_3x3s2p1(const PoolGeom &g) {
+    return g.k == 3 && g.sh == 2 && g.sw == 2 && g.pad == 1 && (g.W % 4) == 0 && (g.H % 2) == 0;
+}
+
+}  // namespace
+
+extern "C" {
+
+int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int H, int W, int k, int sh, int sw,
+                       int pad) {
+    XSMI_REQUIRE_INIT();
+    PoolGeom g;
+    int rc = check_geom("xsmi_maxpool2d_fwd", N, C, H, W, k, sh, sw, pad, &g);
+    if (rc) return rc;
+    XSMI_CHECK_ARG(x && y, "xsmi_maxpool2d_fwd: null tensor pointer");
+    uint32_t total = (uint32_t)N * C * g.OH * g.OW;
+    hipStream_t st = xsmi::stream();
+    if (fast_3x3s2p1(g)) {
+        uint32_t pairs = total / 2;
+        xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 2);
+        hipLaunchKernelGGL(maxpool_fwd_3x3s2p1, dim3((pairs + 255) / 256), dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        XSMI_LAUNCH_CHECK("maxpool_fwd_3x3s2p1");
+        return XSMI_OK;
+    }
+    dim3 grid((total + 255) / 256);
+    if (k == 2)
+        hipLaunchKernelGGL(maxpool_fwd_generic<2>, grid, dim3(256), 0, st, x, y, idx, g, total);
+    else if (k == 3)
+        hipLaunchKernelGGL(maxpool_fwd_generic<3>, grid, dim3(256), 0, st, x, y, idx, g, total);
+    else
+        hipLaunchKernelGGL(maxpool_fwd_generic<0>, grid, dim3(256), 0, st, x, y, idx, g, total);
+    XSMI_LAUNCH_CHECK("maxpool_fwd_generic");
+    return XSMI_OK;
+}
+
+int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, int C, int H, int W, int k, int sh,
+                       int sw, int pad, float beta) {
+    XSMI_REQUIRE_INIT();
+    PoolGeom g;
+    int rc = check_geom("xsmi_maxpool2d_bwd", N, C, H, W, k, sh, sw, pad, &g);
+    if (rc) return rc;
+    XSMI_CHECK_ARG(dy && idx && dx, "xsmi_maxpool2d_bwd: null tensor pointer");
+    XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_maxpool2d_bwd: beta must be 0 or 1");
+    uint32_t total = (uint32_t)N * C * H * W;
+    hipStream_t st = xsmi::stream();
+    int acc = beta == 1.f ? 1 : 0;
+    if (fast_3x3s2p1(g)) {
+        uint32_t quads = total / 4;
+        xsmi::FastDiv dQ4 = xsmi::make_fastdiv(W / 4);
+        hipLaunchKernelGGL(maxpool_bwd_3x3s2p1, dim3((quads + 255) / 256), dim3(256), 0, st, dy, idx, dx, g, dQ4, quads, acc);
+        XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1");
+        return XSMI_OK;
+    }
+    hipLaunchKernelGGL(maxpool_bwd_gather, dim3((total + 255) / 256), dim3(256), 0, st, dy, idx, dx, g, total, acc);
+    XSMI_LAUNCH_CHECK("maxpool_bwd_gather");
+    return XSMI_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,185 @@
+// Runtime part of the C ABI: device selection, memory, stream, events.
+#include "xsmi_internal.h"
+#include <stdarg.h>
+#include <string.h>
+
+namespace {
+thread_local char g_err[512] = "";
+hipStream_t g_stream = nullptr;
+int g_device = -1;
+int g_cus = 0;
+bool g_ready = false;
+}  // namespace
+
+namespace xsmi {
+void set_error(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+}
+hipStream_t stream() { return g_stream; }
+bool ready() { return g_ready; }
+int cu_count() { return g_cus; }
+}  // namespace xsmi
+
+__global__ void __launch_bounds__(256) xsmi_copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    size_t stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n4; i += stride) dst[i] = src[i];
+}
+
+extern "C" {
+
+const char *xsmi_last_error(void) { return g_err; }
+
+int xsmi_is_initialized(void) { return g_ready ? 1 : 0; }
+
+int xsmi_init(int device) {
+    if (g_ready) {
+        if (device != g_device) {
+            xsmi::set_error("xsmi_init: already initialised on device %d", g_device);
+            return XSMI_ERR_STATE;
+        }
+        return XSMI_OK;
+    }
+    int count = 0;
+    XSMI_HIP(hipGetDeviceCount(&count));
+    XSMI_CHECK_ARG(device >= 0 && device < count, "xsmi_init: device %d out of range (%d visible)", device, count);
+    XSMI_HIP(hipSetDevice(device));
+    hipDeviceProp_t prop;
+    XSMI_HIP(hipGetDeviceProperties(&prop, device));
+    if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) {
+        xsmi::set_error("xsmi_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
+        return XSMI_ERR_RUNTIME;
+    }
+    XSMI_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    g_device = device;
+    g_cus = prop.multiProcessorCount;
+    g_ready = true;
+    return XSMI_OK;
+}
+
+int xsmi_device_info(xsmi_device_info_t *info) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(info != nullptr, "xsmi_device_info: null argument");
+    hipDeviceProp_t prop;
+    XSMI_HIP(hipGetDeviceProperties(&prop, g_device));
+    memset(info, 0, sizeof(*info));
+    info->device = g_device;
+    info->cu_count = prop.multiProcessorCount;
+    info->clock_khz = prop.clockRate;
+    info->lds_bytes_per_cu = (int)prop.maxSharedMemoryPerMultiProcessor;
+    info->wavefront = prop.warpSize;
+    info->l2_bytes = prop.l2CacheSize;
+    info->hbm_bytes = prop.totalGlobalMem;
+    strncpy(info->name, prop.name, sizeof(info->name) - 1);
+    strncpy(info->arch, prop.gcnArchName, sizeof(info->arch) - 1);
+    return XSMI_OK;
+}
+
+int xsmi_malloc(void **ptr, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(ptr != nullptr, "xsmi_malloc: null result pointer");
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 16;
+    XSMI_HIP(hipMalloc(ptr, bytes));
+    return XSMI_OK;
+}
+
+int xsmi_free(void *ptr) {
+    XSMI_REQUIRE_INIT();
+    if (ptr == nullptr) return XSMI_OK;
+    // hipFree waits for the device; work queued on the stream that still uses
+    // `ptr` has completed when it returns.
+    XSMI_HIP(hipFree(ptr));
+    return XSMI_OK;
+}
+
+int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    if (bytes == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_h2d: null pointer");
+    XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
+    XSMI_HIP(hipStreamSynchronize(g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    if (bytes == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_d2h: null pointer");
+    XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
+    XSMI_HIP(hipStreamSynchronize(g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    if (bytes == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_d2d: null pointer");
+    XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToDevice, g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_memset(void *dst, int byte_value, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    if (bytes == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dst != nullptr, "xsmi_memset: null pointer");
+    XSMI_HIP(hipMemsetAsync(dst, byte_value, bytes, g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_sync(void) {
+    XSMI_REQUIRE_INIT();
+    XSMI_HIP(hipStreamSynchronize(g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_event_create(void **event) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(event != nullptr, "xsmi_event_create: null result pointer");
+    hipEvent_t e;
+    XSMI_HIP(hipEventCreate(&e));
+    *event = (void *)e;
+    return XSMI_OK;
+}
+
+int xsmi_event_record(void *event) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(event != nullptr, "xsmi_event_record: null event");
+    XSMI_HIP(hipEventRecord((hipEvent_t)event, g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_event_elapsed_ms(void *start, void *stop, float *ms) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(start && stop && ms, "xsmi_event_elapsed_ms: null argument");
+    XSMI_HIP(hipEventSynchronize((hipEvent_t)stop));
+    XSMI_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
+    return XSMI_OK;
+}
+
+int xsmi_event_destroy(void *event) {
+    XSMI_REQUIRE_INIT();
+    if (event == nullptr) return XSMI_OK;
+    XSMI_HIP(hipEventDestroy((hipEvent_t)event));
+    return XSMI_OK;
+}
+
+int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(dst && src, "xsmi_copy_kernel: null pointer");
+    XSMI_CHECK_ARG(bytes % 16 == 0, "xsmi_copy_kernel: size must be a multiple of 16 bytes");
+    size_t n4 = bytes / 16;
+    if (n4 == 0) return XSMI_OK;
+    size_t blocks = (n4 + 255) / 256;
+    size_t cap = (size_t)g_cus * 32;
+    if (blocks > cap) blocks = cap;
+    hipLaunchKernelGGL(xsmi_copy_f4, dim3((unsigned)blocks), dim3(256), 0, g_stream,
+                       (const float4 *)src, (float4 *)dst, n4);
+    XSMI_LAUNCH_CHECK("xsmi_copy_f4");
+    return XSMI_OK;
+}
+
+}  // extern "C"
