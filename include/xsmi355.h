@@ -72,6 +72,12 @@ int xsmi_event_create(void **event);
 int xsmi_event_record(void *event);                               /* on the library stream */
 int xsmi_event_elapsed_ms(void *start, void *stop, float *ms);    /* waits for `stop` */
 int xsmi_event_destroy(void *event);
+/* Per-op device timing: after xsmi_profiling(1) every op records one event
+ * before and one after its main kernel (for conv: the MFMA kernel(s), not the
+ * filter packing or the split reduction); xsmi_last_kernel_ms waits for the last
+ * op and returns the time between the two. */
+int xsmi_profiling(int on);
+int xsmi_last_kernel_ms(float *ms);
 /* plain float4 copy kernel of `bytes` bytes (multiple of 16); used to
  * calibrate HBM counters and to quote the achievable copy bandwidth. */
 int xsmi_copy_kernel(void *dst, const void *src, size_t bytes);

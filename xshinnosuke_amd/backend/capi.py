@@ -49,6 +49,8 @@ SIGNATURES = {
     "xsmi_event_record": (_i, [_vp]),
     "xsmi_event_elapsed_ms": (_i, [_vp, _vp, _c.POINTER(_f)]),
     "xsmi_event_destroy": (_i, [_vp]),
+    "xsmi_profiling": (_i, [_i]),
+    "xsmi_last_kernel_ms": (_i, [_c.POINTER(_f)]),
     "xsmi_copy_kernel": (_i, [_vp, _vp, _sz]),
     "xsmi_conv2d_workspace_bytes": (_sz, _CONV_DIMS),
     "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
@@ -128,6 +130,17 @@ def device_info():
         "l2_bytes": info.l2_bytes, "hbm_bytes": int(info.hbm_bytes),
         "name": info.name.decode(), "arch": info.arch.decode(),
     }
+
+
+def profiling(on):
+    ensure_init()
+    lib.call("xsmi_profiling", 1 if on else 0)
+
+
+def last_kernel_ms():
+    ms = ctypes.c_float()
+    lib.call("xsmi_last_kernel_ms", ctypes.byref(ms))
+    return ms.value
 
 
 def synchronize():

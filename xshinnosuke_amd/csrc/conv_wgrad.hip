@@ -258,7 +258,9 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
 
     hipStream_t st = xsmi::stream();
     dim3 grid(p.Jp / TJ, p.Kp / TK, splits);
+    xsmi::prof_begin();
     hipLaunchKernelGGL(wgrad_f32_kernel, grid, dim3(256), 0, st, p);
+    xsmi::prof_end();
     XSMI_LAUNCH_CHECK("wgrad_f32_kernel");
     const int acc = beta == 1.f ? 1 : 0;
     hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(xsmi::ceil_div(K * p.J, 256)), dim3(256), 0, st, p.part, dw, K, p.J,

@@ -219,10 +219,12 @@ int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int
     XSMI_CHECK_ARG(x && y, "xsmi_maxpool2d_fwd: null tensor pointer");
     uint32_t total = (uint32_t)N * C * g.OH * g.OW;
     hipStream_t st = xsmi::stream();
+    xsmi::prof_begin();
     if (fast_3x3s2p1(g)) {
         uint32_t pairs = total / 2;
         xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 2);
         hipLaunchKernelGGL(maxpool_fwd_3x3s2p1, dim3((pairs + 255) / 256), dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_fwd_3x3s2p1");
         return XSMI_OK;
     }
@@ -233,6 +235,7 @@ int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int
         hipLaunchKernelGGL(maxpool_fwd_generic<3>, grid, dim3(256), 0, st, x, y, idx, g, total);
     else
         hipLaunchKernelGGL(maxpool_fwd_generic<0>, grid, dim3(256), 0, st, x, y, idx, g, total);
+    xsmi::prof_end();
     XSMI_LAUNCH_CHECK("maxpool_fwd_generic");
     return XSMI_OK;
 }
@@ -248,14 +251,17 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
     uint32_t total = (uint32_t)N * C * H * W;
     hipStream_t st = xsmi::stream();
     int acc = beta == 1.f ? 1 : 0;
+    xsmi::prof_begin();
     if (fast_3x3s2p1(g)) {
         uint32_t quads = total / 4;
         xsmi::FastDiv dQ4 = xsmi::make_fastdiv(W / 4);
         hipLaunchKernelGGL(maxpool_bwd_3x3s2p1, dim3((quads + 255) / 256), dim3(256), 0, st, dy, idx, dx, g, dQ4, quads, acc);
+        xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1");
         return XSMI_OK;
     }
     hipLaunchKernelGGL(maxpool_bwd_gather, dim3((total + 255) / 256), dim3(256), 0, st, dy, idx, dx, g, total, acc);
+    xsmi::prof_end();
     XSMI_LAUNCH_CHECK("maxpool_bwd_gather");
     return XSMI_OK;
 }

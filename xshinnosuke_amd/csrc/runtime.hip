@@ -9,6 +9,9 @@ hipStream_t g_stream = nullptr;
 int g_device = -1;
 int g_cus = 0;
 bool g_ready = false;
+bool g_profiling = false;
+hipEvent_t g_prof0 = nullptr, g_prof1 = nullptr;
+bool g_prof_valid = false;
 }  // namespace
 
 namespace xsmi {
@@ -21,6 +24,15 @@ void set_error(const char *fmt, ...) {
 hipStream_t stream() { return g_stream; }
 bool ready() { return g_ready; }
 int cu_count() { return g_cus; }
+void prof_begin() {
+    if (g_profiling) (void)hipEventRecord(g_prof0, g_stream);
+}
+void prof_end() {
+    if (g_profiling) {
+        (void)hipEventRecord(g_prof1, g_stream);
+        g_prof_valid = true;
+    }
+}
 }  // namespace xsmi
 
 __global__ void __launch_bounds__(256) xsmi_copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4) {
@@ -167,6 +179,26 @@ int xsmi_event_destroy(void *event) {
     return XSMI_OK;
 }
 
+int xsmi_profiling(int on) {
+    XSMI_REQUIRE_INIT();
+    if (on && !g_prof0) {
+        XSMI_HIP(hipEventCreate(&g_prof0));
+        XSMI_HIP(hipEventCreate(&g_prof1));
+    }
+    g_profiling = on != 0;
+    g_prof_valid = false;
+    return XSMI_OK;
+}
+
+int xsmi_last_kernel_ms(float *ms) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(ms != nullptr, "xsmi_last_kernel_ms: null argument");
+    XSMI_CHECK_ARG(g_prof_valid, "xsmi_last_kernel_ms: no op has run since xsmi_profiling(1)");
+    XSMI_HIP(hipEventSynchronize(g_prof1));
+    XSMI_HIP(hipEventElapsedTime(ms, g_prof0, g_prof1));
+    return XSMI_OK;
+}
+
 int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(dst && src, "xsmi_copy_kernel: null pointer");
@@ -176,8 +208,10 @@ int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
     size_t blocks = (n4 + 255) / 256;
     size_t cap = (size_t)g_cus * 32;
     if (blocks > cap) blocks = cap;
+    xsmi::prof_begin();
     hipLaunchKernelGGL(xsmi_copy_f4, dim3((unsigned)blocks), dim3(256), 0, g_stream,
                        (const float4 *)src, (float4 *)dst, n4);
+    xsmi::prof_end();
     XSMI_LAUNCH_CHECK("xsmi_copy_f4");
     return XSMI_OK;
 }

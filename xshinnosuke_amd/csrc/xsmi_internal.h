@@ -13,6 +13,10 @@ void set_error(const char *fmt, ...);
 hipStream_t stream();
 bool ready();
 int cu_count();
+// With xsmi_profiling(1) every op brackets its main kernel(s) with two events on
+// the library stream; xsmi_last_kernel_ms reads them back.
+void prof_begin();
+void prof_end();
 
 #define XSMI_REQUIRE_INIT()                                              \
     do {                                                                 \
