@@ -290,9 +290,9 @@ int check_conv(const char *fn, int N, int C, int H, int W, int K, int R, int S, 
     g->N = N; g->C = C; g->H = H; g->W = W; g->K = K; g->R = R; g->S = S; g->sh = sh; g->sw = sw; g->pad = pad;
     g->OH = (H + 2 * pad - R) / sh + 1;
     g->OW = (W + 2 * pad - S) / sw + 1;
-    const double lim = 1073741824.0;   // 2^30 elements: byte offsets stay below 2^32
+    const double lim = 536870912.0;   // 2^29 elements: byte offsets stay below 2^31
     XSMI_CHECK_ARG((double)N * C * H * W < lim && (double)N * K * g->OH * g->OW < lim,
-                   "%s: tensors of 2^30 elements or more are not supported", fn);
+                   "%s: tensors of 2^29 elements or more are not supported", fn);
     XSMI_CHECK_ARG((double)C * R * S * K < lim, "%s: filter too large", fn);
     return XSMI_OK;
 }
@@ -307,8 +307,11 @@ size_t pack_bytes(int rows, int J) {
 }  // namespace
 
 namespace xsmi {
-size_t conv_fwd_ws_bytes(int C, int K, int R, int S) { return pack_bytes(K, C * R * S); }
+size_t conv_fwd_ws_bytes(int C, int K, int R, int S) {
+    return tap_path_ok(C) ? tap_fwd_ws_bytes(C, K, R, S) : pack_bytes(K, C * R * S);
+}
 size_t conv_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
+    if (tap_path_ok(K)) return tap_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     size_t total = 0;
     for (int ph = 0; ph < sh; ++ph)
         for (int pw = 0; pw < sw; ++pw) {
@@ -335,6 +338,9 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd: workspace of %zu bytes needed, %zu given", need,
                    workspace_bytes);
+    if (xsmi::tap_path_ok(C))
+        return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
+                                  (flags & XSMI_CONV_RELU) ? 1 : 0, workspace);
     const int rowtiles = xsmi::ceil_div(K, TM);
     const int nchunks = xsmi::ceil_div(J, KC);
     float *apk = (float *)workspace;
@@ -382,6 +388,9 @@ int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int 
     const size_t need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_bwd_data: workspace of %zu bytes needed, %zu given",
                    need, workspace_bytes);
+    if (xsmi::tap_path_ok(K))
+        return xsmi::tap_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
+                                       workspace);
     hipStream_t st = xsmi::stream();
     char *ws = (char *)workspace;
     const int rowtiles = xsmi::ceil_div(C, TM);

@@ -232,9 +232,9 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
     XSMI_CHECK_ARG((flags & ~XSMI_CONV_BF16) == 0, "xsmi_conv2d_bwd_weight: unknown flags 0x%x", flags);
     XSMI_CHECK_ARG(!(flags & XSMI_CONV_BF16), "xsmi_conv2d_bwd_weight: the bf16 path is not available in this build");
     const int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
-    const double lim = 1073741824.0;
+    const double lim = 536870912.0;
     XSMI_CHECK_ARG((double)N * C * H * W < lim && (double)N * K * OH * OW < lim && (double)K * C * R * S < lim,
-                   "xsmi_conv2d_bwd_weight: tensors of 2^30 elements or more are not supported");
+                   "xsmi_conv2d_bwd_weight: tensors of 2^29 elements or more are not supported");
     const size_t need = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need,
                    "xsmi_conv2d_bwd_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);

@@ -74,6 +74,15 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f) {
     return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
+// tap-major fast path (conv_tap.hip): reduction channels must be a multiple of 32
+bool tap_path_ok(int reduce_channels);
+size_t tap_fwd_ws_bytes(int C, int K, int R, int S);
+size_t tap_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw);
+int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, void *workspace);
+int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
+                      int sw, int pad, int OH, int OW, int accumulate, void *workspace);
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
