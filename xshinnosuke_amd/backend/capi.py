@@ -7,7 +7,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-_LIB_PATH = os.path.join(os.path.dirname(_HERE), "lib", "libxsmi355.so")
+# XSMI355_LIBRARY lets a developer load another build of the same ABI; the default is the in-tree one
+_LIB_PATH = os.environ.get("XSMI355_LIBRARY") or os.path.join(os.path.dirname(_HERE), "lib", "libxsmi355.so")
 
 
 class XsmiError(RuntimeError):

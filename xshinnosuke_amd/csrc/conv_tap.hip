@@ -11,15 +11,22 @@
 // hardware range check turns into 0.0 (the scalar offset is not part of that
 // check, so valid lanes must and do stay inside the tensor).
 //
-// Tile: 64 rows x 64 pixels per 256-thread workgroup (2 x 2 waves of 32x32),
-// chunks of 32 channels, two LDS stages.  Wave w stages channels 8w..8w+7 of the
-// chunk for all 64 pixels (lane == pixel, so one load instruction covers 64
-// consecutive pixels of one channel plane).  For the MFMA, lanes 0-31 consume
-// channel groups 0 and 2, lanes 32-63 groups 1 and 3; each group of 8 values is
-// two 128-bit LDS reads.  LDS rows are 8 floats with the two halves swapped on
-// rows whose index has bit 2 set, which spreads any 8 consecutive lanes' 128-bit
-// accesses over all 32 banks without padding.
+// Data path: global -> LDS directly (buffer_load ... lds), no staging registers.
+// A stage holds
+//     A  [8 quads][64 rows][4 floats]   (one 128-bit LDS-direct load per lane = row)
+//     B  [32 channels][64 pixels]       (one dword LDS-direct load per lane = pixel)
+// so each wave-level load lands as one contiguous LDS block.  STAGES stages are
+// kept in flight (prefetch distance STAGES-1) and the loop waits with a vmcnt that
+// leaves the younger chunks outstanding; one barrier per chunk both publishes the
+// chunk that just landed and retires the stage that is about to be refilled.
+//
+// Tile: 64 rows x 64 pixels per 256-thread workgroup (2 x 2 waves of 32x32).  For
+// the MFMA (v_mfma_f32_32x32x2_f32), lanes 0-31 take channels 0..15 of the chunk
+// and lanes 32-63 channels 16..31: A comes as four 128-bit reads of consecutive
+// 16-byte slots (conflict-free), B as sixteen dword reads of 32 consecutive floats.
 #include "xsmi_internal.h"
+#include <stdlib.h>
+#include <type_traits>
 
 namespace {
 
@@ -28,15 +35,18 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 constexpr int TM = 64;
 constexpr int BP = 64;
 constexpr int KC = 32;
-constexpr int STAGE_FLOATS = 4 * 64 * 8;   // one operand, one stage
+constexpr int STAGE_FLOATS = 4096;         // A 2048 + B 2048
+constexpr int LOADS_PER_CHUNK = 10;        // per wave: 8 dword (B) + 2 dwordx4 (A)
+constexpr int TAP_STAGES = 3;
 
 struct TapParams {
     const float *in;
-    const float *apk;     // [rowtile][tap*nch + cc][group 4][row 64][8]
+    const float *apk;     // [rowtile][tap*nch + cc][quad 8][row 64][4]
     const float *bias;
     float *out;
     uint8_t *mask;
     uint32_t in_bytes;
+    uint32_t apk_bytes;
     int M, rows;
     int nch;              // channel chunks per tap
     int TR, TS;           // taps
@@ -51,16 +61,10 @@ struct TapParams {
     int accumulate, relu;
 };
 
-__device__ __forceinline__ float buffer_load_f32(__amdgpu_buffer_rsrc_t rsrc, uint32_t voff, uint32_t soff) {
-    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rsrc, (int)voff, (int)soff, 0));
-}
-
-// float offset of 128-bit half f (0/1) of LDS row `row` in group q
-__device__ __forceinline__ int lds_off(int q, int row, int f) { return ((q * 64 + row) * 2 + (f ^ ((row >> 2) & 1))) * 4; }
-
+template <int STAGES>
 __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
-    __shared__ __attribute__((aligned(16))) float As[2][STAGE_FLOATS];
-    __shared__ __attribute__((aligned(16))) float Bs[2][STAGE_FLOATS];
+    __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
+    constexpr int D = STAGES - 1;
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -68,7 +72,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
     const int m0 = blockIdx.x * BP;
     const int rowtile = blockIdx.y;
 
-    // ---- gather role: pixel m0 + lane, channel group `wave` ----
+    // ---- gather role: pixel m0 + lane, channels 8*wave .. 8*wave+7 of each chunk ----
     int iyb = 0, ixb = 0, nbase = 0;
     const bool live = m0 + lane < p.M;
     if (live) {
@@ -81,83 +85,157 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
         ixb = x * p.sx + p.dx0;
         nbase = (int)n * p.in_n_stride;
     }
-    __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc((void *)p.in, 0, p.in_bytes, 0x00020000);
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(p.in, p.in_bytes);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(p.apk, p.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];   // LDS byte address (low half of the flat address)
     const int iters = p.TR * p.TS * p.nch;
-    const float4 *apk4 = reinterpret_cast<const float4 *>(p.apk) + (size_t)rowtile * iters * (TM * KC / 4) + t;
+    const uint32_t a_voff = (uint32_t)((2 * wave * 64 + lane) * 16);
 
-    // LDS slots this thread writes
-    const int bw0 = lds_off(wave, lane, 0), bw1 = lds_off(wave, lane, 1);
-    const int aw0 = lds_off(t >> 7, (t & 127) >> 1, t & 1);           // float4 #t
-    const int aw1 = lds_off((t >> 7) + 2, (t & 127) >> 1, t & 1);     // float4 #t+256
-
-    float bnext[8];
-    float4 an0, an1;
-    int r = 0, s = 0, cc = 0;   // position of the NEXT chunk to fetch
-
-    auto fetch = [&](int it) {
+    // ---- issue state: position of the next chunk to load, kept in scalars ----
+    int r = 0, s = 0, cc = 0;
+    uint32_t ld_stage = lds0;                         // LDS byte address of the stage the next chunk goes to
+    uint32_t ld_asoff = (uint32_t)rowtile * (uint32_t)iters * (uint32_t)(TM * KC * 4);
+    uint32_t ld_voff = 0, ld_soff = 0;
+    // per-tap part of a chunk's addresses (vector) and per-chunk part (scalar)
+    auto issue_prep = [&]() {
         int iy = iyb + r * p.dstep, ix = ixb + s * p.dstep;
         bool ok = live && (unsigned)iy < (unsigned)p.IH && (unsigned)ix < (unsigned)p.IW;
-        uint32_t voff = ok ? (uint32_t)((nbase + iy * p.IW + ix) * 4) : 0x80000000u;
-        uint32_t soff = (uint32_t)(cc * KC + wave * 8) * p.plane_bytes;
-#pragma unroll
-        for (int e = 0; e < 8; ++e) bnext[e] = buffer_load_f32(rsrc, voff, soff + (uint32_t)e * p.plane_bytes);
-        const float4 *ap = apk4 + (size_t)it * (TM * KC / 4);
-        an0 = ap[0];
-        an1 = ap[256];
+        ld_voff = ok ? (uint32_t)((nbase + iy * p.IW + ix) * 4) : 0x80000000u;
+        ld_soff = (uint32_t)(cc * KC + wave * 8) * p.plane_bytes;
+    };
+    auto issue_b = [&](int e) {                       // channel 8*wave + e of the chunk, all 64 pixels
+        xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((2048 + (wave * 8 + e) * 64) * 4), ld_voff,
+                           ld_soff + (uint32_t)e * p.plane_bytes);
+    };
+    auto issue_a = [&](int qa) {                      // quad 2*wave + qa of the chunk, all 64 rows
+        xsmi::load_lds_b128(rap, ld_stage + (uint32_t)((2 * wave + qa) * 1024), a_voff + (uint32_t)qa * 1024u, ld_asoff);
+    };
+    auto issue_advance = [&]() {
+        ld_asoff += (uint32_t)(TM * KC * 4);
+        ld_stage += (uint32_t)(STAGE_FLOATS * 4);
+        if (ld_stage == lds0 + (uint32_t)(STAGES * STAGE_FLOATS * 4)) ld_stage = lds0;
         if (++cc == p.nch) {
             cc = 0;
             if (++s == p.TS) { s = 0; ++r; }
         }
     };
-    auto stage = [&](int buf) {
-        *reinterpret_cast<float4 *>(&Bs[buf][bw0]) = make_float4(bnext[0], bnext[1], bnext[2], bnext[3]);
-        *reinterpret_cast<float4 *>(&Bs[buf][bw1]) = make_float4(bnext[4], bnext[5], bnext[6], bnext[7]);
-        *reinterpret_cast<float4 *>(&As[buf][aw0]) = an0;
-        *reinterpret_cast<float4 *>(&As[buf][aw1]) = an1;
+    auto issue_all = [&]() {
+        issue_prep();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) issue_b(e);
+        issue_a(0);
+        issue_a(1);
+        issue_advance();
     };
 
-    floatx16 acc = {0};
+    // Two accumulators take alternate reduction steps; they are added once at the end.
+    floatx16 acc = {0}, acc2 = {0};
     const int h = lane >> 5, l31 = lane & 31;
     const int wr = wave >> 1, wc = wave & 1;
-    const int arow = wr * 32 + l31, bcol = wc * 32 + l31;
-    const int ar00 = lds_off(h, arow, 0), ar01 = lds_off(h, arow, 1);
-    const int ar10 = lds_off(h + 2, arow, 0), ar11 = lds_off(h + 2, arow, 1);
-    const int br00 = lds_off(h, bcol, 0), br01 = lds_off(h, bcol, 1);
-    const int br10 = lds_off(h + 2, bcol, 0), br11 = lds_off(h + 2, bcol, 1);
+    const int a_rd = (4 * h * 64 + wr * 32 + l31) * 4;           // float index of quad 4h, this lane's row
+    const int b_rd = 2048 + 16 * h * 64 + wc * 32 + l31;         // float index of channel 16h, this lane's pixel
 
+    // Operand fragments of two consecutive chunks live in registers.  An iteration
+    // is 16 MFMAs on the current fragments; after the first four it waits for the
+    // next chunk and crosses the barrier, and every later MFMA is followed in
+    // program order by one slice of the remaining work (one LDS fragment read of
+    // the next chunk, one LDS-direct load of the chunk STAGES-1 ahead), so that work
+    // issues while the matrix pipe is busy.  sched_barrier pins this order.
+    float4 fa[2][4];
+    float fb[2][16];
+    const float *rd_stage = smem[0];                  // stage the next fragments are read from
+    auto rd_advance = [&]() {
+        rd_stage += STAGE_FLOATS;
+        if (rd_stage == smem[0] + STAGES * STAGE_FLOATS) rd_stage = smem[0];
+    };
+#define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
+#define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto body = [&](auto buf_tag, auto static_tag, int it) {
+        constexpr int cur = decltype(buf_tag)::value;
+        constexpr int nxt = cur ^ 1;
+        constexpr bool all = decltype(static_tag)::value;         // steady state: next chunk and next load both exist
+        const bool has_next = all || it + 1 < iters;
+        const bool has_load = all || it + 1 + D < iters;
+        XSMI_MFMA(acc, fa[cur][0].x, fb[cur][0]);
+        XSMI_MFMA(acc2, fa[cur][0].y, fb[cur][1]);
+        XSMI_MFMA(acc, fa[cur][0].z, fb[cur][2]);
+        XSMI_MFMA(acc2, fa[cur][0].w, fb[cur][3]);
+        XSMI_PIN();
+        if (has_next) {
+            if (all || it + 1 + D <= iters) xsmi::wait_vmcnt<(D - 1) * LOADS_PER_CHUNK>();
+            else xsmi::wait_vmcnt<0>();
+            xsmi::block_barrier();
+        }
+        XSMI_PIN();
+        XSMI_MFMA(acc, fa[cur][1].x, fb[cur][4]);
+        if (has_next) fa[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + a_rd);
+        if (has_load) issue_prep();
+        XSMI_PIN();
+        XSMI_MFMA(acc2, fa[cur][1].y, fb[cur][5]);
+        if (has_next) fa[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 256);
+        if (has_load) issue_b(0);
+        XSMI_PIN();
+        XSMI_MFMA(acc, fa[cur][1].z, fb[cur][6]);
+        if (has_next) fa[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 512);
+        if (has_load) issue_b(1);
+        XSMI_PIN();
+        XSMI_MFMA(acc2, fa[cur][1].w, fb[cur][7]);
+        if (has_next) fa[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 768);
+        if (has_load) issue_b(2);
+        XSMI_PIN();
+#define XSMI_SLOT(ACC, AV, J, LOADSTMT)                                      \
+        XSMI_MFMA(ACC, AV, fb[cur][J]);                                      \
+        if (has_next) {                                                      \
+            fb[nxt][2 * (J - 8)] = rd_stage[b_rd + 64 * (2 * (J - 8))];        \
+            fb[nxt][2 * (J - 8) + 1] = rd_stage[b_rd + 64 * (2 * (J - 8) + 1)]; \
+        }                                                                    \
+        if (has_load) { LOADSTMT; }                                          \
+        XSMI_PIN();
+        XSMI_SLOT(acc, fa[cur][2].x, 8, issue_b(3))
+        XSMI_SLOT(acc2, fa[cur][2].y, 9, issue_b(4))
+        XSMI_SLOT(acc, fa[cur][2].z, 10, issue_b(5))
+        XSMI_SLOT(acc2, fa[cur][2].w, 11, issue_b(6))
+        XSMI_SLOT(acc, fa[cur][3].x, 12, issue_b(7))
+        XSMI_SLOT(acc2, fa[cur][3].y, 13, issue_a(0))
+        XSMI_SLOT(acc, fa[cur][3].z, 14, issue_a(1))
+        XSMI_SLOT(acc2, fa[cur][3].w, 15, issue_advance())
+#undef XSMI_SLOT
+        if (has_next) rd_advance();
+    };
+
+    // prologue: chunks 0..D-1 in flight, fragments of chunk 0 in registers, then chunk D
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (d < iters) issue_all();
     if (iters > 0) {
-        fetch(0);
-        stage(0);
+        if (D <= iters) xsmi::wait_vmcnt<(D - 1) * LOADS_PER_CHUNK>();
+        else xsmi::wait_vmcnt<0>();
+        xsmi::block_barrier();
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) fa[0][q4] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 256 * q4);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) fb[0][j] = rd_stage[b_rd + 64 * j];
+        rd_advance();
+        if (D < iters) issue_all();
     }
-    __syncthreads();
-    for (int it = 0; it < iters; ++it) {
-        const int cur = it & 1;
-        const bool more = it + 1 < iters;
-        if (more) fetch(it + 1);
-        const float *A = As[cur], *B = Bs[cur];
-        float4 a0 = *reinterpret_cast<const float4 *>(A + ar00), b0 = *reinterpret_cast<const float4 *>(B + br00);
-        float4 a1 = *reinterpret_cast<const float4 *>(A + ar01), b1 = *reinterpret_cast<const float4 *>(B + br01);
-        float4 a2 = *reinterpret_cast<const float4 *>(A + ar10), b2 = *reinterpret_cast<const float4 *>(B + br10);
-        float4 a3 = *reinterpret_cast<const float4 *>(A + ar11), b3 = *reinterpret_cast<const float4 *>(B + br11);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.x, b0.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.y, b0.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.z, b0.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a0.w, b0.w, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.x, b1.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.y, b1.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.z, b1.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a1.w, b1.w, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a2.x, b2.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a2.y, b2.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a2.z, b2.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a2.w, b2.w, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a3.x, b3.x, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a3.y, b3.y, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a3.z, b3.z, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_32x32x2f32(a3.w, b3.w, acc, 0, 0, 0);
-        if (more) stage(cur ^ 1);
-        __syncthreads();
+    {
+        using T0 = std::integral_constant<int, 0>;
+        using T1 = std::integral_constant<int, 1>;
+        int it = 0;
+        const int n_steady = iters - 1 - D;           // iterations whose next chunk and next load both exist
+        for (; it + 1 < n_steady; it += 2) {
+            body(T0{}, std::true_type{}, it);
+            body(T1{}, std::true_type{}, it + 1);
+        }
+        for (; it < iters; it += 2) {
+            body(T0{}, std::false_type{}, it);
+            if (it + 1 < iters) body(T1{}, std::false_type{}, it + 1);
+        }
     }
+#undef XSMI_MFMA
+#undef XSMI_PIN
+
+    acc += acc2;
 
     // ---- epilogue: register v of lane l = row 8*(v/4) + 4*(l/32) + v%4, pixel l%32 ----
     const int m = m0 + wc * 32 + l31;
@@ -194,15 +272,15 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     const int iters = TR * TS * nch;
     const size_t total = (size_t)rowtiles * iters * (TM * KC);
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
-        int e = (int)(i & 7);
-        int r64 = (int)((i >> 3) & 63);
-        int q = (int)((i >> 9) & 3);
+        int e = (int)(i & 3);
+        int r64 = (int)((i >> 2) & 63);
+        int q = (int)((i >> 8) & 7);
         size_t blk = i >> 11;
         int it = (int)(blk % iters);
         int rt = (int)(blk / iters);
         int cc = it % nch, tap = it / nch;
         int tr = tap / TS, ts = tap % TS;
-        int ch = cc * KC + q * 8 + e;
+        int ch = cc * KC + q * 4 + e;
         int row = rt * TM + r64;
         float v = 0.f;
         if (row < rows) {
@@ -212,6 +290,20 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
                 v = w[(((size_t)ch * rows + row) * R + (r0 + sh * tr)) * S + (s0 + sw * ts)];
         }
         apk[i] = v;
+    }
+}
+
+void launch_tap(dim3 grid, hipStream_t st, const TapParams &p) {
+    static int stages = -1;
+    if (stages < 0) {
+        const char *e = getenv("XSMI_TAP_STAGES");
+        stages = e ? atoi(e) : TAP_STAGES;
+    }
+    switch (stages) {
+        case 2: hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, grid, dim3(256), 0, st, p); break;
+        case 4: hipLaunchKernelGGL(tap_igemm_f32_kernel<4>, grid, dim3(256), 0, st, p); break;
+        case 5: hipLaunchKernelGGL(tap_igemm_f32_kernel<5>, grid, dim3(256), 0, st, p); break;
+        default: hipLaunchKernelGGL(tap_igemm_f32_kernel<3>, grid, dim3(256), 0, st, p); break;
     }
 }
 
@@ -265,7 +357,8 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     p.accumulate = 0; p.relu = relu;
     dim3 grid(ceil_div(p.M, BP), ceil_div(K, TM));
     prof_begin();
-    hipLaunchKernelGGL(tap_igemm_f32_kernel, grid, dim3(256), 0, st, p);
+    p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
+    launch_tap(grid, st, p);
     prof_end();
     XSMI_LAUNCH_CHECK("tap_igemm_f32_kernel");
     return XSMI_OK;
@@ -290,11 +383,13 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             const int U = s0 < S ? ceil_div(S - s0, sw) : 0;
             const int cx = (pw + pad - s0) / sw;
             float *apk = (float *)ws;
-            ws += tap_pack_bytes(C, K, T * U);
+            const size_t apk_bytes = tap_pack_bytes(C, K, T * U);
+            ws += apk_bytes;
             int rc = launch_pack(st, w, apk, 1, C, K, R, S, T, U, r0, s0, sh, sw);
             if (rc) return rc;
             TapParams p;
             p.in = dy; p.apk = apk; p.bias = nullptr; p.out = dx; p.mask = nullptr;
+            p.apk_bytes = (uint32_t)apk_bytes;
             p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
             p.M = N * OYc * OXc; p.rows = C; p.nch = K / KC; p.TR = T; p.TS = U;
             p.dy0 = cy; p.dx0 = cx; p.dstep = -1;
@@ -311,7 +406,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
     }
     prof_begin();
     for (int i = 0; i < nplans; ++i) {
-        hipLaunchKernelGGL(tap_igemm_f32_kernel, plans[i].grid, dim3(256), 0, st, plans[i].p);
+        launch_tap(plans[i].grid, st, plans[i].p);
         XSMI_LAUNCH_CHECK("tap_igemm_f32_kernel");
     }
     prof_end();

@@ -83,6 +83,59 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
                       int sw, int pad, int OH, int OW, int accumulate, void *workspace);
 
+// ---- global -> LDS direct loads ------------------------------------------
+// Written as inline asm on purpose: the compiler orders LDS reads after
+// LDS-direct loads it knows about with a full vmcnt(0) wait, which would undo
+// the multi-stage prefetch.  The kernels that use these helpers order the loads
+// themselves (vmcnt + workgroup barrier) and contain no other instruction that
+// depends on M0.
+typedef int xsmi_int32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ xsmi_int32x4 make_rsrc(const void *p, uint32_t bytes) {
+    uint64_t a = (uint64_t)p;
+    xsmi_int32x4 r;
+    r.x = (int)(uint32_t)a;
+    r.y = (int)(uint32_t)((a >> 32) & 0xffff);   // stride 0: raw buffer
+    r.z = (int)bytes;                           // offsets >= bytes read as 0
+    r.w = 0x00020000;
+    return r;
+}
+
+// One dword per lane: LDS[lds_addr + 4*lane] = buffer[voff + soff]; lds_addr and soff are wave-uniform.
+__device__ __forceinline__ void load_lds_b32(xsmi_int32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+#endif
+}
+
+// Four dwords per lane: LDS[lds_addr + 16*lane .. +15] = buffer[voff + soff .. +15].
+__device__ __forceinline__ void load_lds_b128(xsmi_int32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
+#endif
+}
+
+// s_waitcnt that constrains only the vector-memory counter (gfx9 encoding:
+// vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
+template <int N>
+__device__ __forceinline__ void wait_vmcnt() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_s_waitcnt((N & 15) | ((N >> 4) << 14) | (7 << 4) | (15 << 8));
+#endif
+}
+
+// Workgroup barrier the compiler may not move memory accesses across; it carries
+// no waits of its own.
+__device__ __forceinline__ void block_barrier() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    asm volatile("" ::: "memory");
+    __builtin_amdgcn_s_barrier();
+    asm volatile("" ::: "memory");
+#endif
+}
+
 inline size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 inline int ceil_div(int a, int b) { return (a + b - 1) / b; }
 
