@@ -37,7 +37,7 @@ constexpr int BP = 64;
 constexpr int KC = 32;
 constexpr int STAGE_FLOATS = 4096;         // A 2048 + B 2048
 constexpr int LOADS_PER_CHUNK = 10;        // per wave: 8 dword (B) + 2 dwordx4 (A)
-constexpr int TAP_STAGES = 3;
+constexpr int TAP_STAGES = 2;
 
 struct TapParams {
     const float *in;

@@ -213,7 +213,12 @@ size_t conv_bwd_weight_ws_bytes(int N, int C, int K, int R, int S, int OH, int O
     int splits, cps;
     plan_splits(N * OH * OW, K, C * R * S, &splits, &cps);
     size_t Kp = align_up(K, TK), Jp = align_up((size_t)C * R * S, TJ);
-    return align_up((size_t)splits * Kp * Jp * sizeof(float), 256) + align_up((size_t)splits * Kp * sizeof(float), 256);
+    size_t generic = align_up((size_t)splits * Kp * Jp * sizeof(float), 256) + align_up((size_t)splits * Kp * sizeof(float), 256);
+    if (C % 64 == 0 && K % 64 == 0 && (OH * OW) % 4 == 0) {
+        size_t tap = wgrad_tap_ws_bytes(N, C, K, R, S, OH, OW);
+        return tap > generic ? tap : generic;
+    }
+    return generic;
 }
 }  // namespace xsmi
 
@@ -238,6 +243,9 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
     const size_t need = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need,
                    "xsmi_conv2d_bwd_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+
+    if (xsmi::wgrad_tap_ok(dy, x, C, K, OH, OW))
+        return xsmi::wgrad_tap(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, OH, OW, beta == 1.f ? 1 : 0, workspace);
 
     WgradParams p;
     p.dy = dy; p.x = x;

@@ -1,0 +1,344 @@
+// Tap-major backward-weight on fp32 MFMA for layers with C % 64 == 0, K % 64 == 0
+// and OH*OW % 4 == 0.
+//
+// For one filter tap (r, s) the weight gradient is a plain GEMM over pixels,
+//
+//     dw[k][c][r][s] = sum_m dy[n, k, m] * x[n, c, (oh*sh + r - pad), (ow*sw + s - pad)]      m = (n, oh, ow)
+//
+// whose reduction index m is contiguous in memory for dy and (per output row) for
+// x.  A workgroup owns one (tap, 64 filters, 64 channels) tile and one contiguous
+// range of 32-pixel chunks; it writes its 64x64 partial to the workspace and a
+// second kernel adds the ranges in a fixed order in float64 (no float atomics).
+// Chunks never straddle two images.
+//
+// Data path: global -> LDS directly, two stages.
+//   A = dy  [64 filters][32 pixels]  128-bit loads, 8 filter rows per wave-load
+//   B = x   [64 channels][32 pixels] dword loads (the shifted, possibly strided
+//           and border-clipped pixel needs a per-lane address), 2 channels per
+//           wave-load; invalid lanes use an offset beyond the buffer, which the
+//           range check turns into 0.0
+// Both tiles keep the pixel axis innermost, which is what the MFMA operand layout
+// wants (lane = filter/channel, registers = consecutive pixels): each lane reads
+// its 16 pixels with four 128-bit LDS reads.  Rows are 128 bytes, so the 16-byte
+// groups of a row are stored XOR-swizzled by (row & 7) to spread a wavefront's
+// reads over all banks; since LDS-direct loads fix the LDS position of every
+// lane, the swizzle is applied to the global address each lane fetches instead.
+#include "xsmi_internal.h"
+#include <type_traits>
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int TK = 64, TC = 64, MC = 32;
+constexpr int STAGE_FLOATS = 4096;      // A 2048 + B 2048
+constexpr int STAGES = 2;
+constexpr int LOADS = 10;               // per wave and chunk: 2 dwordx4 (A) + 8 dword (B)
+constexpr int TARGET_BLOCKS = 1024;
+
+struct WgradTapParams {
+    const float *dy;
+    const float *x;
+    float *part;        // [split][tap][K][C]
+    float *dbpart;      // [split][K] or nullptr
+    uint32_t x_bytes, dy_bytes;
+    int N, C, K, H, W, OH, OW, OHW, R, S, sh, sw, pad;
+    int cpi;            // chunks per image
+    int total_chunks, cps, ctiles;
+    uint32_t xplane_bytes, yplane_bytes;
+    xsmi::FastDiv dOW, dCT, dS;
+};
+
+__global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
+    __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
+    constexpr int D = STAGES - 1;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave >> 1, wc = wave & 1;
+
+    const int tapidx = (int)xsmi::fdiv(blockIdx.x, p.dCT);
+    const int ctile = (int)blockIdx.x - tapidx * p.ctiles;
+    const int tr = (int)xsmi::fdiv((uint32_t)tapidx, p.dS);
+    const int ts = tapidx - tr * p.S;
+    const int c0 = ctile * TC, k0 = blockIdx.y * TK;
+    const int split = blockIdx.z;
+    const int chunk_begin = split * p.cps;
+    int nchunks = p.total_chunks - chunk_begin;
+    if (nchunks > p.cps) nchunks = p.cps;
+    if (nchunks < 0) nchunks = 0;
+
+    const xsmi::xsmi_int32x4 rx = xsmi::make_rsrc(p.x, p.x_bytes);
+    const xsmi::xsmi_int32x4 ry = xsmi::make_rsrc(p.dy, p.dy_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];
+
+    // ---- A load role: wave-load j (j = wave, wave + 4) fills rows 8j..8j+7; lane -> (row, swizzled group) ----
+    const int a_row0 = 8 * wave + (lane >> 3), a_row1 = a_row0 + 32;
+    const int a_q = (lane & 7) ^ (a_row0 & 7);                      // same for both rows (32 = 0 mod 8)
+    const uint32_t a_v0 = (uint32_t)a_row0 * p.yplane_bytes + (uint32_t)a_q * 16u;
+    const uint32_t a_v1 = (uint32_t)a_row1 * p.yplane_bytes + (uint32_t)a_q * 16u;
+    // ---- B load role: wave-load j = wave + 4e fills channels 2j, 2j+1; the pixel a lane fetches is the same for all e ----
+    const int b_chl = 2 * wave + (lane >> 5);                       // channel of wave-load e: b_chl + 8e
+    const int b_ms = lane & 31;
+    const int b_m = ((((b_ms >> 2) ^ (b_chl & 7)) << 2) | (b_ms & 3));   // pixel of the chunk this lane fetches
+
+    // ---- issue state ----
+    int in_img = 0, ci = 0;                                          // image and chunk-in-image of the next chunk to load
+    {
+        in_img = chunk_begin / p.cpi;
+        ci = chunk_begin - in_img * p.cpi;
+    }
+    uint32_t ld_stage = lds0;
+    uint32_t ld_va0 = 0, ld_va1 = 0, ld_vb = 0, ld_sa = 0, ld_sb = 0;
+    auto issue_prep = [&]() {
+        const int ml0 = ci * MC;
+        // A: groups of 4 pixels are inside the image or not as a whole (OHW % 4 == 0)
+        const bool a_ok = ml0 + 4 * a_q < p.OHW;
+        ld_va0 = a_ok ? a_v0 : 0x80000000u;
+        ld_va1 = a_ok ? a_v1 : 0x80000000u;
+        ld_sa = (uint32_t)((in_img * p.K + k0) * p.OHW + ml0) * 4u;
+        // B: the shifted input position of this lane's pixel
+        const int ml = ml0 + b_m;
+        const int oh = (int)xsmi::fdiv((uint32_t)ml, p.dOW);
+        const int ow = ml - oh * p.OW;
+        const int ih = oh * p.sh + tr - p.pad, iw = ow * p.sw + ts - p.pad;
+        const bool b_ok = ml < p.OHW && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+        ld_vb = b_ok ? (uint32_t)((ih * p.W + iw) * 4) + (uint32_t)b_chl * p.xplane_bytes : 0x80000000u;
+        ld_sb = (uint32_t)(in_img * p.C + c0) * p.xplane_bytes;
+    };
+    auto issue_a = [&](int j) {
+        xsmi::load_lds_b128(ry, ld_stage + (uint32_t)((wave + 4 * j) * 1024), j == 0 ? ld_va0 : ld_va1, ld_sa);
+    };
+    auto issue_b = [&](int e) {
+        xsmi::load_lds_b32(rx, ld_stage + (uint32_t)(8192 + (wave + 4 * e) * 256), ld_vb, ld_sb + (uint32_t)(8 * e) * p.xplane_bytes);
+    };
+    auto issue_advance = [&]() {
+        ld_stage += (uint32_t)(STAGE_FLOATS * 4);
+        if (ld_stage == lds0 + (uint32_t)(STAGES * STAGE_FLOATS * 4)) ld_stage = lds0;
+        if (++ci == p.cpi) { ci = 0; ++in_img; }
+    };
+    auto issue_all = [&]() {
+        issue_prep();
+        issue_a(0);
+        issue_a(1);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) issue_b(e);
+        issue_advance();
+    };
+
+    // ---- fragment role ----
+    const int f_arow = wr * 32 + l31, f_bch = wc * 32 + l31;
+    int a_rd[4], b_rd[4];                                            // float index of this lane's four 16-byte groups
+#pragma unroll
+    for (int g = 0; g < 4; ++g) {
+        a_rd[g] = (f_arow * 8 + ((4 * h + g) ^ (f_arow & 7))) * 4;
+        b_rd[g] = 2048 + (f_bch * 8 + ((4 * h + g) ^ (f_bch & 7))) * 4;
+    }
+    const bool want_db = p.dbpart != nullptr && blockIdx.x == 0 && wc == 0;
+    float dbacc = 0.f;
+
+    floatx16 acc = {0}, acc2 = {0};
+    float4 fa[2][4], fb[2][4];
+    const float *rd_stage = smem[0];
+    auto rd_advance = [&]() {
+        rd_stage += STAGE_FLOATS;
+        if (rd_stage == smem[0] + STAGES * STAGE_FLOATS) rd_stage = smem[0];
+    };
+#define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
+#define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto body = [&](auto buf_tag, auto static_tag, int it) {
+        constexpr int cur = decltype(buf_tag)::value;
+        constexpr int nxt = cur ^ 1;
+        constexpr bool all = decltype(static_tag)::value;
+        const bool has_next = all || it + 1 < nchunks;
+        const bool has_load = all || it + 1 + D < nchunks;
+        XSMI_MFMA(acc, fa[cur][0].x, fb[cur][0].x);
+        XSMI_MFMA(acc2, fa[cur][0].y, fb[cur][0].y);
+        XSMI_MFMA(acc, fa[cur][0].z, fb[cur][0].z);
+        XSMI_MFMA(acc2, fa[cur][0].w, fb[cur][0].w);
+        XSMI_PIN();
+        if (has_next) {
+            if (all || it + 1 + D <= nchunks) xsmi::wait_vmcnt<(D - 1) * LOADS>();
+            else xsmi::wait_vmcnt<0>();
+            xsmi::block_barrier();
+        }
+        XSMI_PIN();
+#define XSMI_SLOT(ACC, AV, BV, STMT1, STMT2)   \
+        XSMI_MFMA(ACC, AV, BV);                 \
+        if (has_next) { STMT1; }                \
+        if (has_load) { STMT2; }                \
+        XSMI_PIN();
+        XSMI_SLOT(acc, fa[cur][1].x, fb[cur][1].x, fa[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[0]), issue_prep())
+        XSMI_SLOT(acc2, fa[cur][1].y, fb[cur][1].y, fb[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[0]), issue_a(0))
+        XSMI_SLOT(acc, fa[cur][1].z, fb[cur][1].z, fa[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[1]), issue_a(1))
+        XSMI_SLOT(acc2, fa[cur][1].w, fb[cur][1].w, fb[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[1]), issue_b(0))
+        XSMI_SLOT(acc, fa[cur][2].x, fb[cur][2].x, fa[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[2]), issue_b(1))
+        XSMI_SLOT(acc2, fa[cur][2].y, fb[cur][2].y, fb[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[2]), issue_b(2))
+        XSMI_SLOT(acc, fa[cur][2].z, fb[cur][2].z, fa[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[3]), issue_b(3))
+        XSMI_SLOT(acc2, fa[cur][2].w, fb[cur][2].w, fb[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[3]), issue_b(4))
+        XSMI_SLOT(acc, fa[cur][3].x, fb[cur][3].x, (void)0, issue_b(5))
+        XSMI_SLOT(acc2, fa[cur][3].y, fb[cur][3].y, (void)0, issue_b(6))
+        XSMI_SLOT(acc, fa[cur][3].z, fb[cur][3].z, (void)0, issue_b(7))
+        XSMI_SLOT(acc2, fa[cur][3].w, fb[cur][3].w, (void)0, issue_advance())
+#undef XSMI_SLOT
+        if (want_db) {
+#pragma unroll
+            for (int g = 0; g < 4; ++g) dbacc += (fa[cur][g].x + fa[cur][g].y) + (fa[cur][g].z + fa[cur][g].w);
+        }
+        if (has_next) rd_advance();
+    };
+
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (d < nchunks) issue_all();
+    if (nchunks > 0) {
+        if (D <= nchunks) xsmi::wait_vmcnt<(D - 1) * LOADS>();
+        else xsmi::wait_vmcnt<0>();
+        xsmi::block_barrier();
+#pragma unroll
+        for (int g = 0; g < 4; ++g) {
+            fa[0][g] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[g]);
+            fb[0][g] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[g]);
+        }
+        rd_advance();
+        if (D < nchunks) issue_all();
+    }
+    {
+        using T0 = std::integral_constant<int, 0>;
+        using T1 = std::integral_constant<int, 1>;
+        int it = 0;
+        const int n_steady = nchunks - 1 - D;
+        for (; it + 1 < n_steady; it += 2) {
+            body(T0{}, std::true_type{}, it);
+            body(T1{}, std::true_type{}, it + 1);
+        }
+        for (; it < nchunks; it += 2) {
+            body(T0{}, std::false_type{}, it);
+            if (it + 1 < nchunks) body(T1{}, std::false_type{}, it + 1);
+        }
+    }
+#undef XSMI_MFMA
+#undef XSMI_PIN
+    acc += acc2;
+
+    // accumulator register v of lane l: filter row 8*(v/4) + 4*(l/32) + v%4, channel column l%32
+    const int taps = p.R * p.S;
+    float *dst = p.part + (((size_t)split * taps + tapidx) * p.K + k0 + wr * 32 + 4 * h) * p.C + c0 + wc * 32 + l31;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) dst[(size_t)(8 * (v >> 2) + (v & 3)) * p.C] = acc[v];
+
+    if (want_db) {
+        float other = __shfl_xor(dbacc, 32);
+        if (h == 0) p.dbpart[(size_t)split * p.K + k0 + wr * 32 + l31] = dbacc + other;
+    }
+}
+
+// dw[k][c][tap] = beta*dw + sum over splits (ascending, float64) of part[split][tap][k][c].
+// 256 threads = 64 consecutive c x 4 interleaved split groups, combined in group order.
+__global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                                int K, int C, int taps, int splits, int accumulate) {
+    __shared__ double sm[4][64];
+    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int ctiles = C / 64;
+    int b = blockIdx.x;
+    const int ct = b % ctiles; b /= ctiles;
+    const int k = b % K;
+    const int tap = b / K;
+    const int c = ct * 64 + cl;
+    const size_t stride = (size_t)taps * K * C;
+    const float *src = part + ((size_t)tap * K + k) * C + c;
+    double s0 = 0.0, s1 = 0.0;
+    int sp = g;
+    for (; sp + 4 < splits; sp += 8) {
+        s0 += (double)src[(size_t)sp * stride];
+        s1 += (double)src[(size_t)(sp + 4) * stride];
+    }
+    if (sp < splits) s0 += (double)src[(size_t)sp * stride];
+    sm[g][cl] = s0 + s1;
+    __syncthreads();
+    if (g == 0) {
+        double s = ((sm[0][cl] + sm[1][cl]) + sm[2][cl]) + sm[3][cl];
+        const size_t o = ((size_t)k * C + c) * taps + tap;
+        if (accumulate) s += (double)dw[o];
+        dw[o] = (float)s;
+    }
+}
+
+__global__ void __launch_bounds__(256) dbias_tap_reduce_kernel(const float *__restrict__ dbpart, float *__restrict__ db,
+                                                                int K, int splits, int accumulate) {
+    __shared__ double sm[4][64];
+    const int kl = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int k = blockIdx.x * 64 + kl;
+    double s0 = 0.0;
+    for (int sp = g; sp < splits; sp += 4) s0 += (double)dbpart[(size_t)sp * K + k];
+    sm[g][kl] = s0;
+    __syncthreads();
+    if (g == 0) {
+        double s = ((sm[0][kl] + sm[1][kl]) + sm[2][kl]) + sm[3][kl];
+        if (accumulate) s += (double)db[k];
+        db[k] = (float)s;
+    }
+}
+
+void plan(int N, int C, int K, int R, int S, int OHW, int *cpi, int *total, int *cps, int *splits) {
+    const int tiles = R * S * (C / TC) * (K / TK);
+    *cpi = xsmi::ceil_div(OHW, MC);
+    *total = N * *cpi;
+    int want = xsmi::ceil_div(TARGET_BLOCKS, tiles);
+    int c = xsmi::ceil_div(*total, want);
+    if (c < 8) c = 8;
+    if (c > *total) c = *total;
+    *cps = c;
+    *splits = xsmi::ceil_div(*total, c);
+}
+
+}  // namespace
+
+namespace xsmi {
+
+bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW) {
+    return C % TC == 0 && K % TK == 0 && (OH * OW) % 4 == 0 && ((uintptr_t)dy % 16) == 0 && ((uintptr_t)x % 4) == 0;
+}
+
+size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW) {
+    int cpi, total, cps, splits;
+    plan(N, C, K, R, S, OH * OW, &cpi, &total, &cps, &splits);
+    return align_up((size_t)splits * R * S * K * C * sizeof(float), 256) + align_up((size_t)splits * K * sizeof(float), 256);
+}
+
+int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int C, int H, int W, int K, int R, int S,
+              int sh, int sw, int pad, int OH, int OW, int accumulate, void *workspace) {
+    WgradTapParams p;
+    int splits;
+    plan(N, C, K, R, S, OH * OW, &p.cpi, &p.total_chunks, &p.cps, &splits);
+    p.dy = dy; p.x = x;
+    p.part = (float *)workspace;
+    float *dbpart = (float *)((char *)workspace + align_up((size_t)splits * R * S * K * C * sizeof(float), 256));
+    p.dbpart = db ? dbpart : nullptr;
+    p.x_bytes = (uint32_t)((size_t)N * C * H * W * 4);
+    p.dy_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
+    p.N = N; p.C = C; p.K = K; p.H = H; p.W = W; p.OH = OH; p.OW = OW; p.OHW = OH * OW; p.R = R; p.S = S;
+    p.sh = sh; p.sw = sw; p.pad = pad;
+    p.ctiles = C / TC;
+    p.xplane_bytes = (uint32_t)(H * W * 4); p.yplane_bytes = (uint32_t)(OH * OW * 4);
+    p.dOW = make_fastdiv(OW); p.dCT = make_fastdiv(p.ctiles); p.dS = make_fastdiv(S);
+
+    hipStream_t st = stream();
+    dim3 grid(R * S * p.ctiles, K / TK, splits);
+    prof_begin();
+    hipLaunchKernelGGL(wgrad_tap_f32_kernel, grid, dim3(256), 0, st, p);
+    prof_end();
+    XSMI_LAUNCH_CHECK("wgrad_tap_f32_kernel");
+    hipLaunchKernelGGL(wgrad_tap_reduce_kernel, dim3(R * S * K * p.ctiles), dim3(256), 0, st, p.part, dw, K, C, R * S,
+                       splits, accumulate);
+    XSMI_LAUNCH_CHECK("wgrad_tap_reduce_kernel");
+    if (db) {
+        hipLaunchKernelGGL(dbias_tap_reduce_kernel, dim3(K / 64), dim3(256), 0, st, dbpart, db, K, splits, accumulate);
+        XSMI_LAUNCH_CHECK("dbias_tap_reduce_kernel");
+    }
+    return XSMI_OK;
+}
+
+}  // namespace xsmi

@@ -83,6 +83,12 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
                       int sw, int pad, int OH, int OW, int accumulate, void *workspace);
 
+// tap-major backward-weight (conv_wgrad_tap.hip)
+bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW);
+size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW);
+int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int C, int H, int W, int K, int R, int S,
+              int sh, int sw, int pad, int OH, int OW, int accumulate, void *workspace);
+
 // ---- global -> LDS direct loads ------------------------------------------
 // Written as inline asm on purpose: the compiler orders LDS reads after
 // LDS-direct loads it knows about with a full vmcnt(0) wait, which would undo
@@ -104,6 +110,8 @@ __device__ __forceinline__ xsmi_int32x4 make_rsrc(const void *p, uint32_t bytes)
 // One dword per lane: LDS[lds_addr + 4*lane] = buffer[voff + soff]; lds_addr and soff are wave-uniform.
 __device__ __forceinline__ void load_lds_b32(xsmi_int32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
 #if defined(__HIP_DEVICE_COMPILE__)
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dword %1, %2, %3 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 #endif
@@ -112,6 +120,8 @@ __device__ __forceinline__ void load_lds_b32(xsmi_int32x4 rsrc, uint32_t lds_add
 // Four dwords per lane: LDS[lds_addr + 16*lane .. +15] = buffer[voff + soff .. +15].
 __device__ __forceinline__ void load_lds_b128(xsmi_int32x4 rsrc, uint32_t lds_addr, uint32_t voff, uint32_t soff) {
 #if defined(__HIP_DEVICE_COMPILE__)
+    lds_addr = __builtin_amdgcn_readfirstlane(lds_addr);
+    soff = __builtin_amdgcn_readfirstlane(soff);
     asm volatile("s_mov_b32 m0, %0\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
                  :: "s"(lds_addr), "v"(voff), "s"(rsrc), "s"(soff) : "memory");
 #endif
