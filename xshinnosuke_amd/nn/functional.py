@@ -1,0 +1,423 @@
+"""Functional API (counterpart of the reference's xs/nn/functional.py).
+
+``conv2d`` and ``max_pool2d`` keep the reference signatures, graph wiring,
+``cache`` keys and accumulate-into-grad convention, but their arithmetic is done
+by the HIP kernels of libxsmi355.so -- for device tensors in place, for host
+(NumPy-backed) tensors by staging through device memory.  There is no NumPy
+implementation of these two ops in this package: without the library or a
+gfx950 device they raise.
+
+The remaining functions are the small set of neighbours the README networks and
+ResNet-18 need; they run in NumPy for host tensors and through element-wise /
+reduction kernels for device tensors.
+"""
+import numpy as np
+
+from ..core import state as GLOBAL
+from ..core.base import Tensor, Parameter, is_device
+from ..backend import kernels as K, to_device
+from ..backend import array as dev
+from . import array_ops as A
+from .grad_fn import *  # noqa: F401,F403  (backward functions are part of this module's namespace, as in the reference)
+from .grad_fn import initialize_ops_grad, _f32_device
+
+
+def _mark_input(t):
+    if GLOBAL.INPUTS is None:
+        GLOBAL.INPUTS = t
+
+
+def _wire(out, *ins):
+    """Dynamic-graph bookkeeping: out.in_bounds = ins (None kept as a placeholder), ins[i].out_bounds += out."""
+    if out.is_dynamic:
+        out.add_in_bounds(*ins)
+        for t in ins:
+            if t is not None:
+                t.add_out_bounds(out)
+
+
+def _pair(v):
+    if isinstance(v, (tuple, list)):
+        return int(v[0]), int(v[1])
+    return int(v), int(v)
+
+
+# --------------------------------------------------------------------------- hot path
+def conv2d(inputs, weight, bias=None, stride=(1, 1), padding=0, out=None, activation=None):
+    """2-D cross-correlation, NCHW (reference xs/nn/functional.py:405-442).
+
+    ``stride`` is a pair, ``padding`` one symmetric int, no dilation or groups.  Output
+    ``(N, K, (H+2p-R)//sh+1, (W+2p-S)//sw+1)`` has the dtype of ``inputs``.  ``out`` may be a
+    preallocated (possibly batch-sliced) Tensor that is written in place.
+    ``activation='relu'`` is this package's extension: it fuses ``max(0, .)`` into the
+    kernel epilogue (what ``Conv2D(activation='relu')`` computes in the reference with a
+    second pass, xs/layers/convolutional.py:76-77) and keeps the strict ``pre < 0`` mask
+    for the backward.
+    """
+    _mark_input(inputs)
+    if activation not in (None, 'relu'):
+        raise ValueError("conv2d can only fuse activation='relu'")
+    x = inputs.eval
+    if len(x.shape) != 4 or len(weight.shape) != 4:
+        raise ValueError('conv2d expects NCHW input and KCRS weight, got %s and %s' % (x.shape, weight.shape))
+    stride = _pair(stride)
+    if isinstance(padding, (tuple, list)) or int(padding) != padding:
+        raise TypeError('padding must be a single integer')
+    padding = int(padding)
+    on_device = is_device(x)
+    x_dev = _f32_device(x)
+    w_dev = _f32_device(weight.eval)
+    b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
+    n, c, h, w = x.shape
+    k, _, r, s = weight.shape
+    oh, ow = K.conv_out_hw(h, w, r, s, stride, padding)
+    requires_grad = bool(inputs.requires_grad or weight.requires_grad or (bias is not None and bias.requires_grad))
+    track = GLOBAL.COMPUTE_GRAD and requires_grad
+    neg_mask = dev.empty((n, k, oh, ow), np.uint8) if (activation == 'relu' and track) else None
+
+    if out is None:
+        y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask)
+        out = Tensor(y_dev if on_device else y_dev.numpy().astype(x.dtype, copy=False))
+    else:
+        dst = out.eval
+        if is_device(dst):
+            K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask)
+        else:
+            y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask)
+            out.eval = y_dev.numpy()              # cast to the buffer's dtype on store
+    out.requires_grad = requires_grad
+    _wire(out, inputs, weight, bias)
+    if track:
+        out.cache['x'] = x_dev                    # the reference keeps the unfolded matrix 'col' here
+        out.cache['stride'] = stride
+        out.cache['padding'] = padding
+        if neg_mask is not None:
+            out.cache['neg_mask'] = neg_mask
+        out.grad_fn = Conv2DBackward
+        initialize_ops_grad(inputs, weight, bias)
+    return out
+
+
+def max_pool2d(inputs, kernel_size=2, stride=None, padding=0, out=None):
+    """Max pooling with zero-valued padding that takes part in the max and first-maximum
+    tie-breaking (reference xs/nn/functional.py:445-491).
+
+    ``kernel_size`` is an int (an equal pair is accepted, which the reference's README
+    shows but its code rejects); ``stride`` defaults to the kernel size.
+    """
+    _mark_input(inputs)
+    if isinstance(kernel_size, (tuple, list)):
+        if len(kernel_size) != 2 or kernel_size[0] != kernel_size[1]:
+            raise ValueError('max_pool2d supports square windows only')
+        kernel_size = kernel_size[0]
+    kernel_size = int(kernel_size)
+    stride = (kernel_size, kernel_size) if stride is None else _pair(stride)
+    padding = int(padding)
+    x = inputs.eval
+    if len(x.shape) != 4:
+        raise ValueError('max_pool2d expects an NCHW input, got shape %s' % (x.shape,))
+    on_device = is_device(x)
+    x_dev = _f32_device(x)
+    track = GLOBAL.COMPUTE_GRAD and inputs.requires_grad
+    if out is None:
+        y_dev, idx = K.maxpool2d_fwd(x_dev, kernel_size, stride, padding, want_idx=track)
+        out = Tensor(y_dev if on_device else y_dev.numpy().astype(x.dtype, copy=False))
+    else:
+        dst = out.eval
+        if is_device(dst):
+            _, idx = K.maxpool2d_fwd(x_dev, kernel_size, stride, padding, out=dst, want_idx=track)
+        else:
+            y_dev, idx = K.maxpool2d_fwd(x_dev, kernel_size, stride, padding, want_idx=track)
+            out.eval = y_dev.numpy()
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if track:
+        out.cache['pool_argmax'] = idx            # uint8, NCHW order, value ky*k + kx
+        out.cache['kernel_size'] = kernel_size
+        out.cache['mode'] = 'im2col'
+        out.cache['stride'] = stride
+        out.cache['padding'] = padding
+        out.grad_fn = Maxpool2DBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+# --------------------------------------------------------------------------- neighbours
+def _binary(lhs, rhs, fn, backward_fn, out):
+    _mark_input(lhs)
+    res = fn(lhs.eval, rhs.eval, None if out is None else out.eval)
+    if out is None:
+        out = Tensor(res)
+    out.requires_grad = bool(lhs.requires_grad or rhs.requires_grad)
+    _wire(out, lhs, rhs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        initialize_ops_grad(lhs, rhs)
+        out.grad_fn = backward_fn
+    return out
+
+
+def add(lhs, rhs, out=None):
+    return _binary(lhs, rhs, A.add, AddBackward, out)
+
+
+def sub(lhs, rhs, out=None):
+    def f(a, b, o):
+        if is_device(a):
+            return A.add(a, A.scale(A.same_place(a, b), -1.0), o)
+        r = np.subtract(a, A.same_place(a, b))
+        if o is not None:
+            o[...] = r
+            return o
+        return r
+    return _binary(lhs, rhs, f, SubBackward, out)
+
+
+def mul(lhs, rhs, out=None):
+    def f(a, b, o):
+        if is_device(a):
+            b = A.same_place(a, b)
+            if b.size == 1:
+                return A.scale(a, float(b.numpy().reshape(-1)[0]))
+            raise NotImplementedError('element-wise product of device tensors')
+        r = np.multiply(a, A.same_place(a, b))
+        if o is not None:
+            o[...] = r
+            return o
+        return r
+    return _binary(lhs, rhs, f, MultiplyBackward, out)
+
+
+def pow(inputs, exp, out=None):
+    """Element-wise power with a Python scalar exponent (host tensors)."""
+    _mark_input(inputs)
+    if is_device(inputs.eval):
+        raise NotImplementedError('pow on device tensors')
+    res = np.power(inputs.eval, exp)
+    out = Tensor(res)
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.cache['exp'] = exp
+        out.grad_fn = PowBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def mm(x1, x2, out=None):
+    _mark_input(x1)
+    res = A.addmm(x1.eval, x2.eval, None, None if out is None else out.eval)
+    if out is None:
+        out = Tensor(res)
+    out.requires_grad = bool(x1.requires_grad or x2.requires_grad)
+    _wire(out, x1, x2)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        initialize_ops_grad(x1, x2)
+        out.grad_fn = MMBackward
+    return out
+
+
+def addmm(b, x1, x2, out=None):
+    """x1 @ x2 + b (reference xs/nn/functional.py:99-120); in_bounds order is (x1, x2, b)."""
+    _mark_input(x1)
+    res = A.addmm(x1.eval, x2.eval, None if b is None else b.eval, None if out is None else out.eval)
+    if out is None:
+        out = Tensor(res)
+    out.requires_grad = bool(x1.requires_grad or x2.requires_grad or (b is not None and b.requires_grad))
+    _wire(out, x1, x2, b)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        initialize_ops_grad(b, x1, x2)
+        out.grad_fn = AddmmBackward
+    return out
+
+
+def relu(inputs, inplace=False, out=None):
+    """max(0, x) (reference xs/nn/functional.py:297-313).  The in-place form overwrites ``inputs``
+    and chains its backward in front of the tensor's existing grad_fn, as the reference's ReLU layer
+    does (xs/layers/activators.py:37-50)."""
+    _mark_input(inputs)
+    if inplace:
+        x = inputs.eval
+        if GLOBAL.COMPUTE_GRAD and inputs.requires_grad:
+            # the strict mask needs the sign of the pre-activation; y == 0 cannot tell x == 0 from x < 0
+            inputs.cache['pre_sign'] = x.copy() if not is_device(x) else x.copy()
+            inputs.cache.setdefault('grad_fn', []).append(inputs.grad_fn)
+            inputs.cache['inplace'] = True
+            inputs.grad_fn = ReLUBackward
+        A.relu(x, x)
+        return inputs
+    res = A.relu(inputs.eval, None if out is None else out.eval)
+    if out is None:
+        out = Tensor(res)
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.grad_fn = ReLUBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def flatten(inputs, start=1, out=None):
+    _mark_input(inputs)
+    x = inputs.eval
+    shape = tuple(x.shape[:start]) + (-1,)
+    res = x.reshape(shape)
+    if out is None:
+        out = Tensor(res)
+    else:
+        out.eval = res
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.grad_fn = FlattenBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def view(inputs, shape, out=None):
+    _mark_input(inputs)
+    if len(shape) == 1 and isinstance(shape[0], (tuple, list)):
+        shape = tuple(shape[0])
+    res = inputs.eval.reshape(tuple(shape))
+    out = Tensor(res)
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.grad_fn = ViewBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def _reduce(inputs, axis, keepdims, mean):
+    _mark_input(inputs)
+    x = inputs.eval
+    if axis is None:
+        res = A.total(x)
+        if mean:
+            res = A.scale(res, 1.0 / x.size)
+    else:
+        xh = x.numpy() if is_device(x) else x
+        res = (np.mean if mean else np.sum)(xh, axis=axis, keepdims=keepdims)
+        res = A.same_place(x, np.asarray(res, dtype=xh.dtype))
+    out = Tensor(res)
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.cache['axis'] = axis
+        out.cache['keepdims'] = keepdims
+        out.grad_fn = MeanBackward if mean else SumBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def sum(inputs, axis=None, keepdims=False):
+    return _reduce(inputs, axis, keepdims, mean=False)
+
+
+def mean(inputs, axis=None, keepdims=False):
+    return _reduce(inputs, axis, keepdims, mean=True)
+
+
+def avg_pool2d(inputs, kernel_size, stride=None, padding=0, out=None):
+    """Mean over non-overlapping k x k blocks.  The reference's overlapping and padded modes
+    (xs/nn/functional.py:539-583) are not reproduced: its padding arithmetic is wrong for
+    padding != 0 and every caller uses stride == kernel_size, padding == 0."""
+    _mark_input(inputs)
+    k = int(kernel_size[0] if isinstance(kernel_size, (tuple, list)) else kernel_size)
+    st = (k, k) if stride is None else _pair(stride)
+    if st != (k, k) or padding != 0:
+        raise NotImplementedError('avg_pool2d supports stride == kernel_size and padding == 0 only')
+    res = A.avg_pool_blocks(inputs.eval, k)
+    if out is None:
+        out = Tensor(res)
+    else:
+        out.eval = res
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.cache['kernel_size'] = k
+        out.cache['mode'] = 'reshape'
+        out.cache['stride'] = st
+        out.cache['padding'] = padding
+        out.grad_fn = Avgpool2DBackward
+        initialize_ops_grad(inputs)
+    return out
+
+
+def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, training=True, epsilon=1e-5,
+               momentum=0.9, out=None):
+    """Per-channel batch normalisation over axis 1 (reference xs/nn/functional.py:676-740)."""
+    _mark_input(inputs)
+    if axis != 1:
+        raise NotImplementedError('batch_norm normalises over axis 1 only')
+    x = inputs.eval
+    xhat = sqrtvar = None
+    if training:
+        y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon)
+        for mov, cur in ((moving_mean, mean_), (moving_variance, var_)):
+            m = mov.eval
+            cur = A.same_place(m, cur)
+            if is_device(m):
+                K.lerp_(m, cur, momentum)                       # m = momentum*m + (1-momentum)*cur
+            else:
+                m *= momentum
+                m += (1 - momentum) * np.asarray(cur).reshape(m.shape)
+    else:
+        y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon)
+    if out is None:
+        out = Tensor(y)
+    else:
+        out.eval = y
+    out.requires_grad = bool(inputs.requires_grad or gamma.requires_grad or beta.requires_grad)
+    _wire(out, inputs, gamma, beta)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad and training:
+        out.cache['sqrtvar'] = sqrtvar
+        out.cache['normalized_x'] = xhat
+        out.grad_fn = BatchNormBackward
+        initialize_ops_grad(inputs, gamma, beta)
+    return out
+
+
+def cross_entropy(x1, x2, reduction='mean', out=None):
+    """Softmax + negative log-likelihood on integer labels (reference xs/nn/functional.py:984-1010)."""
+    _mark_input(x1)
+    if reduction not in ('mean', 'sum'):
+        raise TypeError('unknown type for reduction')
+    loss, sm = A.softmax_cross_entropy(x1.eval, x2.eval, reduction)
+    x1.cache['softmax'] = Tensor(sm)
+    if out is None:
+        out = Tensor(loss)
+    else:
+        out.eval = loss
+    _wire(out, x1, x2)
+    if out.is_dynamic:
+        out.is_leaf = True
+    out.requires_grad = bool(x1.requires_grad or x2.requires_grad)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.cache['reduction'] = reduction
+        out.grad_fn = CrossEntropyLossBackward
+        initialize_ops_grad(x1)
+    return out
+
+
+def mse_loss(x1, x2, reduction='mean', out=None):
+    """0.5 * (x1 - x2)^2, mean or sum (the reference halves the squared error)."""
+    _mark_input(x1)
+    if is_device(x1.eval):
+        raise NotImplementedError('mse_loss on device tensors')
+    d = x1.eval - np.asarray(x2.eval).reshape(x1.shape)
+    val = 0.5 * (d * d)
+    val = val.mean() if reduction == 'mean' else val.sum()
+    res = np.asarray(val, dtype=x1.eval.dtype).reshape(1)
+    if out is None:
+        out = Tensor(res)
+    else:
+        out.eval = res
+    _wire(out, x1, x2)
+    if out.is_dynamic:
+        out.is_leaf = True
+    out.requires_grad = bool(x1.requires_grad or x2.requires_grad)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.cache['reduction'] = reduction
+        out.grad_fn = MSELossBackward
+        initialize_ops_grad(x1, x2)
+    return out

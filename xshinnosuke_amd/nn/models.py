@@ -1,0 +1,264 @@
+"""Sequential / Model (static graph) and Module (dynamic graph), counterparts of xs/nn/models.py.
+
+These are callers of the conv / pool path, not part of it; they reproduce the behaviours that
+path depends on: lazily created parameters, per-layer preallocated output tensors re-sliced for a
+shorter last batch (written through ``out=``), ``layer.backward()`` in reverse order for static
+graphs, and parameter discovery by graph walk for ``Module``.
+"""
+import time
+
+import numpy as np
+
+from ..core import state as GLOBAL
+from ..core import autograd
+from ..core.base import Tensor, Parameter
+from ..layers.base import Layer
+from ..optim import get_optimizer
+from ..utils.data import DataSet, DataLoader
+from .objectives import get_objective
+
+
+class _Base:
+    def __init__(self):
+        self._parameters = set()
+        self._device = 'cuda' if GLOBAL.USE_CUDA else 'cpu'
+
+    def train(self):
+        GLOBAL.TRAINING = True      # the reference sets an unused flag here (models.py:18-22); layers read TRAINING
+
+    def eval(self):
+        GLOBAL.TRAINING = False
+
+    def parameters(self, parameters=None):
+        if parameters is None:
+            return self._parameters
+        self._parameters = set(parameters)
+
+    def to(self, dst):
+        """'cuda' makes the device the default placement of parameters created from now on and moves the
+        existing ones (reference models.py:30-43 swaps the global array module instead)."""
+        if dst == 'cuda':
+            GLOBAL.USE_CUDA = True
+            self._device = 'cuda'
+            for p in self._parameters:
+                p.cuda_()
+        elif dst == 'cpu':
+            GLOBAL.USE_CUDA = False
+            self._device = 'cpu'
+            for p in self._parameters:
+                p.cpu_()
+        else:
+            raise ValueError('unknown destination %r' % (dst,))
+        return self
+
+
+class _Model(_Base):
+    def __init__(self):
+        super().__init__()
+        self.loss = None
+        self.optimizer = None
+        self._graph = None
+
+    def __call__(self, x, *args, **kwargs):
+        return self.forward(x)
+
+    def init_graph_out_tensor(self, x, y):
+        raise NotImplementedError
+
+    def _place(self, t):
+        return t.cuda() if self._device == 'cuda' and t.device != 'cuda' else t
+
+    def fit(self, x, y, batch_size=None, epochs=1, verbose=1, shuffle=True, validation_data=None,
+            validation_split=0., initial_epoch=0):
+        x, y = np.asarray(x), np.asarray(y)
+        if validation_data is None and 0. < validation_split < 1.:
+            split = int(x.shape[0] * validation_split)
+            validation_data = (x[-split:], y[-split:])
+            x, y = x[:-split], y[:-split]
+        loader = DataLoader(DataSet(x, y), batch_size, shuffle)
+        history = {'train_loss': [], 'train_acc': [], 'validation_loss': [], 'validation_acc': []}
+        self.train()
+        for epoch in range(initial_epoch, epochs):
+            t0 = time.time()
+            losses, accs = [], []
+            for idx, (bx, by) in enumerate(loader):
+                bx, by = self._place(bx), self._place(by)
+                if idx == 0 or idx == len(loader) - 1:
+                    self.init_graph_out_tensor(bx, by)
+                self.optimizer.zero_grad()
+                pred = self.forward(bx)
+                loss = self.loss.forward(pred, by)
+                self.backward(loss)
+                self.optimizer.step()
+                losses.append(loss.item())
+                accs.append(self.loss.calc_acc(pred, by))
+            history['train_loss'].append(float(np.mean(losses)))
+            history['train_acc'].append(float(np.mean(accs)))
+            msg = 'epoch %d/%d - %.2fs - loss %.4f - acc %.4f' % (epoch + 1, epochs, time.time() - t0,
+                                                                  history['train_loss'][-1], history['train_acc'][-1])
+            if validation_data is not None:
+                vacc, vloss = self.evaluate(validation_data[0], validation_data[1], batch_size)
+                history['validation_loss'].append(vloss)
+                history['validation_acc'].append(vacc)
+                msg += ' - val_loss %.4f - val_acc %.4f' % (vloss, vacc)
+                self.train()
+            if verbose:
+                print(msg)
+        return history
+
+    def backward(self, loss):
+        """Static-graph sweep: the loss's grad_fn, then every layer in reverse (reference models.py:138-144)."""
+        if loss.grad is None:
+            loss.zero_grad()
+            loss.grad.fill_(1.)
+        loss.grad_fn(loss)
+        for layer in reversed(self._graph):
+            layer.backward()
+        GLOBAL.INPUTS = None
+
+    def evaluate(self, x, y, batch_size=None):
+        self.eval()
+        x, y = np.asarray(x), np.asarray(y)
+        accs, losses = [], []
+        with GLOBAL.no_grad():
+            loader = DataLoader(DataSet(x, y), batch_size if batch_size is not None else x.shape[0])
+            for idx, (bx, by) in enumerate(loader):
+                bx, by = self._place(bx), self._place(by)
+                if idx == 0 or idx == len(loader) - 1:
+                    self.init_graph_out_tensor(bx, by)
+                pred = self.forward(bx)
+                acc, loss = self.loss.metric(pred, by)
+                accs.append(acc)
+                losses.append(loss)
+        GLOBAL.INPUTS = None
+        return float(np.mean(accs)), float(np.mean(losses))
+
+    def predict(self, x, batch_size=None):
+        self.eval()
+        x = np.asarray(x)
+        outs = []
+        with GLOBAL.no_grad():
+            loader = DataLoader(DataSet(x), batch_size if batch_size is not None else x.shape[0])
+            for idx, bx in enumerate(loader):
+                bx = self._place(bx)
+                if idx == 0 or idx == len(loader) - 1:
+                    self.init_graph_out_tensor(bx, None)
+                outs.append(self.forward(bx).numpy().copy())
+        GLOBAL.INPUTS = None
+        return Tensor(np.concatenate(outs, axis=0))
+
+    def __str__(self):
+        rows = ['%-24s %-20s %10s' % ('Layer', 'Output shape', 'Params')]
+        total = 0
+        for layer in self._graph or []:
+            n = layer.params_count() if isinstance(layer, Layer) else 0
+            total += n
+            rows.append('%-24s %-20s %10d' % (layer.__class__.__name__, (None,) + tuple(layer.shape or ()), n))
+        rows.append('Total params: %d' % total)
+        return '\n'.join(rows)
+
+
+class Sequential(_Model):
+    def __init__(self, *layers):
+        super().__init__()
+        self._graph = list(layers)
+        self._initialized = False
+
+    def add(self, layer):
+        self._graph.append(layer)
+
+    def pop(self, index=-1):
+        return self._graph.pop(index)
+
+    def init_graph_out_tensor(self, x, y):
+        for layer in self._graph:
+            layer.init_layer_out_tensor(x)
+            x = layer.data
+
+    def init_params(self, input_shape=None):
+        for layer in self._graph:
+            if isinstance(layer, _Model):
+                continue
+            if len(layer.parameters()) == 0:
+                layer.init_params(input_shape)
+            for v in layer.parameters():
+                if v is not None:
+                    self._parameters.add(v)
+            input_shape = layer.compute_output_shape(input_shape)
+        self._initialized = True
+
+    def compile(self, optimizer, loss, **kwargs):
+        assert self._graph
+        prev = None
+        for layer in self._graph:
+            layer.connect(prev)
+            prev = layer
+        self.init_params(self._graph[0]._input_shape)
+        self.loss = get_objective(loss)
+        self.optimizer = get_optimizer(optimizer, parameters=self._parameters, **kwargs)
+        if GLOBAL.USE_CUDA:
+            self.to('cuda')
+
+    def forward(self, x, *args, **kwargs):
+        for layer in self._graph:
+            x = layer(x) if isinstance(layer, _Base) else layer.forward(x)
+        return x
+
+
+class Model(_Model):
+    def __init__(self, inputs=None, outputs=None):
+        super().__init__()
+        self.inputs = inputs
+        self.outputs = outputs
+
+    def init_graph_out_tensor(self, x, y):
+        self.inputs._data = x
+        for layer in self._graph[1:]:
+            layer.init_layer_out_tensor()
+
+    def compile(self, optimizer, loss, **kwargs):
+        assert self.inputs is not None and self.outputs is not None
+        self._graph = autograd.topological_sort(self.inputs, self.outputs)
+        for g in self._graph:
+            if len(g.parameters()) == 0:
+                g.init_params(g._input_shape)
+            for v in g.parameters():
+                if v is not None:
+                    self._parameters.add(v)
+        self.loss = get_objective(loss)
+        self.optimizer = get_optimizer(optimizer, parameters=self._parameters, **kwargs)
+        if GLOBAL.USE_CUDA:
+            self.to('cuda')
+
+    def forward(self, x, *args, **kwargs):
+        self.inputs._data = x
+        out = None
+        for layer in self._graph[1:]:
+            out = layer.forward()
+        return out
+
+
+class Module(_Base):
+    """Dynamic graph: subclasses define ``forward``; parameters are collected after each call by walking
+    the graph from the input along ``out_bounds`` (reference models.py:341-360)."""
+
+    def __call__(self, x, *args, **kwargs):
+        out = self.forward(x)
+        self._collect(x)
+        out.is_leaf = True
+        return out
+
+    def _collect(self, x):
+        queue, seen = [x], {id(x)}
+        while queue:
+            v = queue.pop(0)
+            for n in v.out_bounds:
+                if id(n) not in seen:
+                    for p in n.in_bounds:
+                        if isinstance(p, Parameter):
+                            self._parameters.add(p)
+                    queue.append(n)
+                    seen.add(id(n))
+
+    def forward(self, x):
+        raise NotImplementedError
