@@ -143,6 +143,63 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx,
  * (xs/nn/grad_fn.py:146-157) for the fused conv epilogue. dx may alias dy. */
 int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size_t n, float beta);
 
+/* ---- neighbours of conv / pool in a network (device-resident tensors) --------
+ * Small element-wise, normalisation and reduction kernels so that activations need not
+ * leave the GPU between two convolutions.  They replace the NumPy expressions of the
+ * reference's xs/nn/td_functional.py and of the named functions; all are float32 and
+ * run on the library stream.  `ws` arguments are caller-provided scratch.
+ */
+
+/* y[i] += a * x[i]                       (gradient accumulation; SGD: xs/optim/sgd.py:4-9) */
+int xsmi_axpy(float *y, const float *x, float a, size_t n);
+/* out[i] = a[i] + b[i]                   (residual add, xs/nn/functional.py:6-21) */
+int xsmi_add(const float *a, const float *b, float *out, size_t n);
+/* out[i] = s * a[i] + t */
+int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n);
+/* y = max(0, x) (may be in place)        (xs/nn/td_functional.py:59-60) */
+int xsmi_relu_fwd(const float *x, float *y, size_t n);
+/* y = max(0, x) and neg_mask[i] = x[i] < 0 (for an in-place ReLU whose backward still needs the sign) */
+int xsmi_relu_fwd_mask(const float *x, float *y, uint8_t *neg_mask, size_t n);
+/* dx[i] = pre[i] < 0 ? 0 : dy[i]         (strict mask, xs/nn/grad_fn.py:146-157); dx may alias dy */
+int xsmi_relu_bwd(const float *dy, const float *pre, float *dx, size_t n);
+/* m[i] = momentum * m[i] + (1 - momentum) * cur[i]   (moving statistics, xs/nn/functional.py:700-707) */
+int xsmi_lerp(float *m, const float *cur, float momentum, size_t n);
+
+/* Batch normalisation over axis 1 of an (N, C, HW) tensor with batch statistics
+ * (xs/nn/functional.py:676-707): y = gamma * xhat + beta, xhat = (x - mean) / sqrt(var + eps),
+ * biased variance.  Outputs xhat (N*C*HW), sqrtvar/mean/var (C).  ws: xsmi_bn_workspace_bytes(C). */
+size_t xsmi_bn_workspace_bytes(int C);
+int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
+                float *mean, float *var, int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
+/* Inference form with given statistics (xs/nn/functional.py:708-725). */
+int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
+                  int N, int C, int HW, float eps);
+/* Backward (xs/nn/grad_fn.py:379-411): dgamma = sum(dy*xhat), dbeta = sum(dy),
+ * dx = gamma / (m*sqrtvar) * (m*dy - dbeta - xhat*dgamma), m = N*HW.  All three are overwritten. */
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, float *dx, float *dgamma,
+                float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes);
+
+/* Mean over non-overlapping k x k blocks of an NCHW tensor and its gradient
+ * (the live mode of avg_pool2d, xs/nn/functional.py:539-583, xs/nn/grad_fn.py:284-309). */
+int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k);
+int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k);
+
+/* C[M,N] = op(A) . op(B) (+ bias[N] broadcast over rows); row-major, float32.  op is a transpose when
+ * trans_a / trans_b is non-zero: A is stored (K,M) resp. B is stored (N,K).
+ * (Dense layer: xs/nn/functional.py:99-120, xs/nn/grad_fn.py:86-99.) */
+int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b);
+/* out[j] = sum_i a[i][j] over an (M, N) matrix */
+int xsmi_colsum(const float *a, float *out, int M, int N);
+/* out[0] = sum of all n elements (float64 accumulation, one workgroup) */
+int xsmi_sum_all(const float *a, float *out, size_t n);
+
+/* Softmax + negative log-likelihood over rows of an (M, N) matrix with int64 labels
+ * (xs/nn/functional.py:984-1010): sm = softmax(logits), loss[0] = mean or sum of -log sm[i, label[i]].
+ * `loss` must hold 1 + M floats (loss[1..M] receives the per-row terms). */
+int xsmi_softmax_ce_fwd(const float *logits, const int64_t *labels, float *sm, float *loss, int M, int N, int mean);
+/* dlogits = (sm - onehot(labels)) * scale      (xs/nn/grad_fn.py:604-620) */
+int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, float *dlogits, int M, int N, float scale);
+
 #ifdef __cplusplus
 }
 #endif

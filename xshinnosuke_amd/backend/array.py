@@ -6,22 +6,60 @@ import numpy as np
 from .capi import lib, ensure_init
 
 
+_POOL = {}            # rounded size -> list of free device pointers
+_POOL_BYTES = [0]
+_POOL_LIMIT = 64 << 30
+
+
+def _round_size(nbytes):
+    nbytes = max(int(nbytes), 256)
+    if nbytes <= (1 << 20):
+        return (nbytes + 255) & ~255
+    return (nbytes + (1 << 16) - 1) & ~((1 << 16) - 1)
+
+
+def release_cached_memory():
+    """Return every cached block to the driver."""
+    for ptrs in _POOL.values():
+        for ptr in ptrs:
+            lib.call("xsmi_free", ctypes.c_void_p(ptr))
+    _POOL.clear()
+    _POOL_BYTES[0] = 0
+
+
 class _Block:
-    """One xsmi_malloc allocation, freed when the last view goes away."""
+    """One device allocation shared by the views of an array.  Freed blocks are kept in a size-keyed
+    pool and handed out again: a training step allocates the same sizes every iteration, all work
+    runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
+    (which serialise with the device) in the steady state."""
 
     __slots__ = ("ptr", "nbytes")
 
     def __init__(self, nbytes):
         ensure_init()
-        p = ctypes.c_void_p()
-        lib.call("xsmi_malloc", ctypes.byref(p), int(nbytes))
-        self.ptr = p.value
-        self.nbytes = int(nbytes)
+        size = _round_size(nbytes)
+        free = _POOL.get(size)
+        if free:
+            self.ptr = free.pop()
+            _POOL_BYTES[0] -= size
+        else:
+            p = ctypes.c_void_p()
+            try:
+                lib.call("xsmi_malloc", ctypes.byref(p), size)
+            except Exception:
+                release_cached_memory()
+                lib.call("xsmi_malloc", ctypes.byref(p), size)
+            self.ptr = p.value
+        self.nbytes = size
 
     def __del__(self):
         try:
             if self.ptr:
-                lib.call("xsmi_free", ctypes.c_void_p(self.ptr))
+                if _POOL_BYTES[0] + self.nbytes <= _POOL_LIMIT:
+                    _POOL.setdefault(self.nbytes, []).append(self.ptr)
+                    _POOL_BYTES[0] += self.nbytes
+                else:
+                    lib.call("xsmi_free", ctypes.c_void_p(self.ptr))
                 self.ptr = None
         except Exception:
             pass

@@ -154,3 +154,177 @@ def relu_mask_bwd(dy, neg_mask, dx=None, accumulate=False):
 
 def copy_kernel(dst, src):
     lib.call("xsmi_copy_kernel", dst.cptr, src.cptr, src.nbytes)
+
+
+# ---- neighbours of conv / pool (device-resident element-wise, normalisation, reduction ops) ----
+def _like(a, out):
+    if out is None:
+        return empty(a.shape)
+    if out.size != a.size:
+        raise ValueError("output has %d elements, expected %d" % (out.size, a.size))
+    return out
+
+
+def axpy(y, x, a):
+    """y += a * x"""
+    _f32(y, "y"); _f32(x, "x")
+    if x.size != y.size:
+        raise ValueError("axpy: %s vs %s" % (x.shape, y.shape))
+    lib.call("xsmi_axpy", y.cptr, x.cptr, float(a), y.size)
+    return y
+
+
+def add(a, b, out=None):
+    _f32(a, "a"); _f32(b, "b")
+    out = _like(a, out)
+    lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
+    return out
+
+
+def scale(a, s, t=0.0, out=None):
+    _f32(a, "a")
+    out = _like(a, out)
+    lib.call("xsmi_scale_shift", a.cptr, out.cptr, float(s), float(t), a.size)
+    return out
+
+
+def add_scalar(a, t, out=None):
+    return scale(a, 1.0, t, out)
+
+
+def relu_fwd(x, out=None):
+    _f32(x, "x")
+    out = _like(x, out)
+    lib.call("xsmi_relu_fwd", x.cptr, out.cptr, x.size)
+    return out
+
+
+def relu_fwd_mask(x, out=None):
+    """Returns (max(0, x), uint8 mask of x < 0); ``out`` may be ``x`` itself."""
+    _f32(x, "x")
+    out = _like(x, out)
+    mask = empty(x.shape, np.uint8)
+    lib.call("xsmi_relu_fwd_mask", x.cptr, out.cptr, mask.cptr, x.size)
+    return out, mask
+
+
+def relu_bwd(dy, pre, dx=None):
+    _f32(dy, "dy"); _f32(pre, "pre")
+    dx = _like(dy, dx)
+    lib.call("xsmi_relu_bwd", dy.cptr, pre.cptr, dx.cptr, dy.size)
+    return dx
+
+
+def lerp_(m, cur, momentum):
+    """m = momentum*m + (1-momentum)*cur"""
+    lib.call("xsmi_lerp", m.cptr, cur.cptr, float(momentum), m.size)
+    return m
+
+
+def _nchw3(shape):
+    n, c = shape[0], shape[1]
+    hw = 1
+    for d in shape[2:]:
+        hw *= d
+    return int(n), int(c), int(hw)
+
+
+def bn_fwd(x, gamma, beta, eps):
+    _f32(x, "x")
+    n, c, hw = _nchw3(x.shape)
+    y = empty(x.shape); xhat = empty(x.shape)
+    sqrtvar = empty((c,)); mean = empty((c,)); var = empty((c,))
+    ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
+    lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr, sqrtvar.cptr, mean.cptr, var.cptr,
+             n, c, hw, float(eps), ws, ws_bytes)
+    return y, xhat, sqrtvar, mean, var
+
+
+def bn_infer(x, gamma, beta, mean, var, eps):
+    n, c, hw = _nchw3(x.shape)
+    y = empty(x.shape)
+    lib.call("xsmi_bn_infer", x.cptr, gamma.cptr, beta.cptr, mean.cptr, var.cptr, y.cptr, n, c, hw, float(eps))
+    return y
+
+
+def bn_bwd(dy, xhat, sqrtvar, gamma):
+    n, c, hw = _nchw3(dy.shape)
+    dx = empty(dy.shape); dgamma = empty((c,)); dbeta = empty((c,))
+    ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
+    lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, sqrtvar.cptr, gamma.cptr, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw,
+             ws, ws_bytes)
+    return dx, dgamma, dbeta
+
+
+def avgpool_fwd(x, k):
+    n, c, h, w = x.shape
+    y = empty((n, c, h // k, w // k))
+    lib.call("xsmi_avgpool_fwd", x.cptr, y.cptr, n, c, h, w, int(k))
+    return y
+
+
+def avgpool_bwd(dy, x_shape, k):
+    n, c, h, w = x_shape
+    dx = empty(x_shape)
+    lib.call("xsmi_avgpool_bwd", dy.cptr, dx.cptr, n, c, h, w, int(k))
+    return dx
+
+
+def gemm(a, b, bias=None, trans_a=False, trans_b=False, out=None):
+    """op(a) @ op(b) (+ bias over rows); a and b are 2-D row-major."""
+    _f32(a, "a"); _f32(b, "b")
+    m, k = (a.shape[1], a.shape[0]) if trans_a else a.shape
+    k2, n = (b.shape[1], b.shape[0]) if trans_b else b.shape
+    if k != k2:
+        raise ValueError("gemm: inner dimensions %d and %d differ" % (k, k2))
+    if out is None:
+        out = empty((m, n))
+    elif out.size != m * n:
+        raise ValueError("gemm: output has shape %s, expected %s" % (out.shape, (m, n)))
+    lib.call("xsmi_gemm", a.cptr, b.cptr, bias.cptr if bias is not None else None, out.cptr, int(m), int(n), int(k),
+             1 if trans_a else 0, 1 if trans_b else 0)
+    return out
+
+
+def dense_fwd(x, w, b=None, out=None):
+    return gemm(x, w, None if b is None else b.reshape(-1), out=out)
+
+
+def colsum(a):
+    m, n = a.shape
+    out = empty((n,))
+    lib.call("xsmi_colsum", a.cptr, out.cptr, int(m), int(n))
+    return out
+
+
+def sum_all(a):
+    out = empty((1,))
+    lib.call("xsmi_sum_all", a.cptr, out.cptr, a.size)
+    return out
+
+
+def _labels(labels):
+    if labels.dtype != np.int64:
+        from .array import to_device
+        labels = to_device(labels.numpy().astype(np.int64), np.int64)
+    return labels
+
+
+def softmax_ce_fwd(logits, labels, reduction):
+    m, n = logits.reshape(-1, logits.shape[-1]).shape
+    labels = _labels(labels)
+    sm = empty(logits.shape)
+    buf = empty((1 + m,))
+    lib.call("xsmi_softmax_ce_fwd", logits.cptr, labels.cptr, sm.cptr, buf.cptr, int(m), int(n),
+             1 if reduction == 'mean' else 0)
+    return buf.leading(0, 1), sm
+
+
+def softmax_ce_bwd(sm, labels, reduction, upstream):
+    m, n = sm.reshape(-1, sm.shape[-1]).shape
+    labels = _labels(labels)
+    up = float(np.asarray(upstream).reshape(-1)[0])
+    scale_ = up / m if reduction == 'mean' else up
+    dz = empty(sm.shape)
+    lib.call("xsmi_softmax_ce_bwd", sm.cptr, labels.cptr, dz.cptr, int(m), int(n), scale_)
+    return dz

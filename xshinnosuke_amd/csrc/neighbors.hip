@@ -1,0 +1,498 @@
+// Element-wise, normalisation and reduction kernels for the ops that sit between two
+// convolutions in a network (ReLU, residual add, batch norm, average pool, dense layer,
+// softmax cross-entropy, SGD).  All are HBM-bound float32 passes: 128-bit accesses where
+// the layout allows it, grid-stride loops, float64 for the long reductions.
+#include "xsmi_internal.h"
+
+namespace {
+
+constexpr int BN_SPLIT = 32;     // partial reductions per channel
+
+inline dim3 grid_for(size_t work_items, int per_block = 256, int cap_per_cu = 16) {
+    size_t blocks = (work_items + per_block - 1) / per_block;
+    size_t cap = (size_t)(xsmi::cu_count() > 0 ? xsmi::cu_count() : 256) * cap_per_cu;
+    if (blocks > cap) blocks = cap;
+    if (blocks < 1) blocks = 1;
+    return dim3((unsigned)blocks);
+}
+
+// Generic element-wise pass: vectorised by 4 when every pointer is 16-byte aligned.
+template <typename F>
+__global__ void __launch_bounds__(256) ew_kernel(size_t n, int vec, F f) {
+    size_t stride = (size_t)gridDim.x * 256;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (vec) {
+        size_t n4 = n >> 2;
+        for (size_t j = i; j < n4; j += stride) f.quad(j);
+        for (size_t j = (n4 << 2) + i; j < n; j += stride) f.one(j);
+    } else {
+        for (size_t j = i; j < n; j += stride) f.one(j);
+    }
+}
+
+inline int aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+struct AxpyF {
+    float *y; const float *x; float a;
+    __device__ void one(size_t i) const { y[i] += a * x[i]; }
+    __device__ void quad(size_t j) const {
+        float4 v = reinterpret_cast<const float4 *>(x)[j];
+        float4 o = reinterpret_cast<float4 *>(y)[j];
+        o.x += a * v.x; o.y += a * v.y; o.z += a * v.z; o.w += a * v.w;
+        reinterpret_cast<float4 *>(y)[j] = o;
+    }
+};
+struct AddF {
+    const float *a, *b; float *o;
+    __device__ void one(size_t i) const { o[i] = a[i] + b[i]; }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
+        reinterpret_cast<float4 *>(o)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+    }
+};
+struct ScaleF {
+    const float *a; float *o; float s, t;
+    __device__ void one(size_t i) const { o[i] = s * a[i] + t; }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(a)[j];
+        reinterpret_cast<float4 *>(o)[j] = make_float4(s * u.x + t, s * u.y + t, s * u.z + t, s * u.w + t);
+    }
+};
+struct ReluF {
+    const float *x; float *y;
+    __device__ void one(size_t i) const { float v = x[i]; y[i] = v > 0.f ? v : 0.f; }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(x)[j];
+        reinterpret_cast<float4 *>(y)[j] = make_float4(u.x > 0.f ? u.x : 0.f, u.y > 0.f ? u.y : 0.f, u.z > 0.f ? u.z : 0.f,
+                                                       u.w > 0.f ? u.w : 0.f);
+    }
+};
+struct ReluMaskF {
+    const float *x; float *y; uint8_t *m;
+    __device__ void one(size_t i) const { float v = x[i]; m[i] = v < 0.f ? 1 : 0; y[i] = v > 0.f ? v : 0.f; }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(x)[j];
+        reinterpret_cast<uchar4 *>(m)[j] = make_uchar4(u.x < 0.f, u.y < 0.f, u.z < 0.f, u.w < 0.f);
+        reinterpret_cast<float4 *>(y)[j] = make_float4(u.x > 0.f ? u.x : 0.f, u.y > 0.f ? u.y : 0.f, u.z > 0.f ? u.z : 0.f,
+                                                       u.w > 0.f ? u.w : 0.f);
+    }
+};
+struct ReluBwdF {
+    const float *dy, *pre; float *dx;
+    __device__ void one(size_t i) const { dx[i] = pre[i] < 0.f ? 0.f : dy[i]; }
+    __device__ void quad(size_t j) const {
+        float4 g = reinterpret_cast<const float4 *>(dy)[j], p = reinterpret_cast<const float4 *>(pre)[j];
+        reinterpret_cast<float4 *>(dx)[j] = make_float4(p.x < 0.f ? 0.f : g.x, p.y < 0.f ? 0.f : g.y, p.z < 0.f ? 0.f : g.z,
+                                                        p.w < 0.f ? 0.f : g.w);
+    }
+};
+struct LerpF {
+    float *m; const float *c; float mom;
+    __device__ void one(size_t i) const { m[i] = mom * m[i] + (1.f - mom) * c[i]; }
+    __device__ void quad(size_t j) const {
+        for (int e = 0; e < 4; ++e) one(4 * j + e);
+    }
+};
+
+template <typename F>
+int launch_ew(const char *name, size_t n, int vec, F f) {
+    if (n == 0) return XSMI_OK;
+    hipLaunchKernelGGL(ew_kernel<F>, grid_for(vec ? (n + 3) / 4 : n), dim3(256), 0, xsmi::stream(), n, vec, f);
+    XSMI_LAUNCH_CHECK(name);
+    return XSMI_OK;
+}
+
+// ---- block reductions ------------------------------------------------------
+__device__ __forceinline__ double wave_sum(double v) {
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+    return v;
+}
+__device__ __forceinline__ double block_sum(double v, double *sm) {   // 256 threads
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    return sm[0] + sm[1] + sm[2] + sm[3];
+}
+
+// channel of flat element i of an (N, C, HW) tensor (tensors stay below 2^29 elements)
+struct ChanIdx {
+    xsmi::FastDiv dHW, dC;
+    int C;
+    __device__ __forceinline__ int operator()(uint32_t i) const {
+        uint32_t q = xsmi::fdiv(i, dHW);
+        return (int)(q - xsmi::fdiv(q, dC) * (uint32_t)C);
+    }
+};
+inline ChanIdx make_chan(int C, int HW) {
+    ChanIdx ci;
+    ci.dHW = xsmi::make_fastdiv(HW);
+    ci.dC = xsmi::make_fastdiv(C);
+    ci.C = C;
+    return ci;
+}
+
+// ---- batch norm --------------------------------------------------------------
+// pass 1: per (channel, split) partial sums of a and a*b over the N*HW elements of the channel
+__global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict__ a, const float *__restrict__ b,
+                                                          double *__restrict__ part, int N, int C, int HW) {
+    __shared__ double sm[4];
+    const int c = blockIdx.x, sp = blockIdx.y;
+    const size_t per = (size_t)N * HW;
+    double s0 = 0.0, s1 = 0.0;
+    for (size_t i = (size_t)sp * 256 + threadIdx.x; i < per; i += (size_t)BN_SPLIT * 256) {
+        size_t n = i / HW, r = i - n * HW;
+        size_t off = (n * C + c) * (size_t)HW + r;
+        float u = a[off];
+        float v = b ? b[off] : u;
+        s0 += (double)u;
+        s1 += (double)u * (double)v;
+    }
+    s0 = block_sum(s0, sm);
+    s1 = block_sum(s1, sm);
+    if (threadIdx.x == 0) {
+        part[((size_t)c * BN_SPLIT + sp) * 2 + 0] = s0;
+        part[((size_t)c * BN_SPLIT + sp) * 2 + 1] = s1;
+    }
+}
+__global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar, float *mean, float *var, int C, double m,
+                                float eps) {
+    int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    double s0 = 0.0, s1 = 0.0;
+    for (int sp = 0; sp < BN_SPLIT; ++sp) {
+        s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
+        s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
+    }
+    double mu = s0 / m;
+    double v = s1 / m - mu * mu;
+    if (v < 0.0) v = 0.0;
+    mean[c] = (float)mu;
+    var[c] = (float)v;
+    sqrtvar[c] = (float)sqrt(v + (double)eps);
+}
+__global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, const float *__restrict__ mean,
+                                                        const float *__restrict__ sqrtvar, float *__restrict__ y,
+                                                        float *__restrict__ xhat, ChanIdx chan, uint32_t total) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        int c = chan(i);
+        float h = (x[i] - mean[c]) / sqrtvar[c];
+        if (xhat) xhat[i] = h;
+        y[i] = gamma[c] * h + beta[c];
+    }
+}
+__global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgamma, float *dbeta, int C) {
+    int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= C) return;
+    double s0 = 0.0, s1 = 0.0;
+    for (int sp = 0; sp < BN_SPLIT; ++sp) {
+        s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
+        s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
+    }
+    dbeta[c] = (float)s0;
+    dgamma[c] = (float)s1;
+}
+__global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
+                                                            const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
+                                                            const float *__restrict__ dgamma, const float *__restrict__ dbeta,
+                                                            float *__restrict__ dx, ChanIdx chan, uint32_t total, float m) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        int c = chan(i);
+        float g = gamma[c];
+        // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
+        dx[i] = g * (m * dy[i] - dbeta[c] - xhat[i] * dgamma[c]) / (m * sqrtvar[c]);
+    }
+}
+
+// ---- average pool over k x k blocks --------------------------------------------
+__global__ void __launch_bounds__(256) avgpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int H, int W,
+                                                           int OH, int OW, int k, size_t total) {
+    for (size_t o = (size_t)blockIdx.x * 256 + threadIdx.x; o < total; o += (size_t)gridDim.x * 256) {
+        int ow = (int)(o % OW);
+        size_t t = o / OW;
+        int oh = (int)(t % OH);
+        size_t nc = t / OH;
+        const float *p = x + (nc * H + (size_t)oh * k) * W + (size_t)ow * k;
+        double s = 0.0;
+        for (int r = 0; r < k; ++r)
+            for (int q = 0; q < k; ++q) s += (double)p[(size_t)r * W + q];
+        y[o] = (float)(s / (double)(k * k));
+    }
+}
+__global__ void __launch_bounds__(256) avgpool_bwd_kernel(const float *__restrict__ dy, float *__restrict__ dx, int H, int W,
+                                                           int OH, int OW, int k, size_t total) {
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+        int w = (int)(e % W);
+        size_t t = e / W;
+        int h = (int)(t % H);
+        size_t nc = t / H;
+        int oh = h / k, ow = w / k;
+        dx[e] = (oh < OH && ow < OW) ? dy[(nc * OH + oh) * OW + ow] / (float)(k * k) : 0.f;
+    }
+}
+
+// ---- small GEMM (dense layer) ----------------------------------------------------
+// 32x32 output tile per 256 threads (each thread 2x2), K in chunks of 32 through LDS.  The dense layer of the
+// networks here is a few tens of MFLOP, far below what would justify an MFMA kernel of its own.
+__global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, const float *__restrict__ B,
+                                                    const float *__restrict__ bias, float *__restrict__ C, int M, int N,
+                                                    int K, int ta, int tb) {
+    __shared__ float As[32][33], Bs[32][33];
+    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
+    float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+    for (int k0 = 0; k0 < K; k0 += 32) {
+        for (int i = threadIdx.x; i < 1024; i += 256) {
+            int r = i >> 5, c = i & 31;
+            int m = m0 + r, kk = k0 + c;
+            As[r][c] = (m < M && kk < K) ? (ta ? A[(size_t)kk * M + m] : A[(size_t)m * K + kk]) : 0.f;
+            int kb = k0 + r, n = n0 + c;
+            Bs[r][c] = (kb < K && n < N) ? (tb ? B[(size_t)n * K + kb] : B[(size_t)kb * N + n]) : 0.f;
+        }
+        __syncthreads();
+#pragma unroll 8
+        for (int kk = 0; kk < 32; ++kk) {
+            float a0 = As[ty * 2][kk], a1 = As[ty * 2 + 1][kk];
+            float b0 = Bs[kk][tx * 2], b1 = Bs[kk][tx * 2 + 1];
+            acc[0][0] += a0 * b0; acc[0][1] += a0 * b1; acc[1][0] += a1 * b0; acc[1][1] += a1 * b1;
+        }
+        __syncthreads();
+    }
+    for (int i = 0; i < 2; ++i)
+        for (int j = 0; j < 2; ++j) {
+            int m = m0 + ty * 2 + i, n = n0 + tx * 2 + j;
+            if (m < M && n < N) C[(size_t)m * N + n] = acc[i][j] + (bias ? bias[n] : 0.f);
+        }
+}
+
+__global__ void __launch_bounds__(256) colsum_kernel(const float *__restrict__ a, float *__restrict__ out, int M, int N) {
+    int j = blockIdx.x * 256 + threadIdx.x;
+    if (j >= N) return;
+    double s = 0.0;
+    for (int i = 0; i < M; ++i) s += (double)a[(size_t)i * N + j];
+    out[j] = (float)s;
+}
+
+__global__ void __launch_bounds__(256) sum_all_kernel(const float *__restrict__ a, float *__restrict__ out, size_t n) {
+    __shared__ double sm[4];
+    double s = 0.0;
+    for (size_t i = threadIdx.x; i < n; i += 256) s += (double)a[i];
+    s = block_sum(s, sm);
+    if (threadIdx.x == 0) out[0] = (float)s;
+}
+
+// ---- softmax cross-entropy: one wavefront per row ------------------------------------
+__global__ void __launch_bounds__(64) softmax_rows_kernel(const float *__restrict__ z, const int64_t *__restrict__ lab,
+                                                           float *__restrict__ sm, float *__restrict__ nll, int M, int N) {
+    const int row = blockIdx.x, lane = threadIdx.x;
+    const float *zr = z + (size_t)row * N;
+    float mx = -3.402823466e38f;
+    for (int j = lane; j < N; j += 64) mx = fmaxf(mx, zr[j]);
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    double s = 0.0;
+    for (int j = lane; j < N; j += 64) s += exp((double)(zr[j] - mx));
+    s = wave_sum(s);
+    for (int j = lane; j < N; j += 64) sm[(size_t)row * N + j] = (float)(exp((double)(zr[j] - mx)) / s);
+    if (lane == 0) {
+        int64_t l = lab[row];
+        double p = (l >= 0 && l < N) ? exp((double)(zr[l] - mx)) / s : 1.0;
+        nll[row] = (float)(-log(p));
+    }
+}
+__global__ void __launch_bounds__(256) nll_reduce_kernel(const float *__restrict__ nll, float *__restrict__ loss, int M,
+                                                          int mean) {
+    __shared__ double sm[4];
+    double s = 0.0;
+    for (int i = threadIdx.x; i < M; i += 256) s += (double)nll[i];
+    s = block_sum(s, sm);
+    if (threadIdx.x == 0) loss[0] = (float)(mean ? s / (double)M : s);
+}
+__global__ void __launch_bounds__(256) softmax_ce_bwd_kernel(const float *__restrict__ sm, const int64_t *__restrict__ lab,
+                                                              float *__restrict__ dz, int N, size_t total, float scale) {
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        size_t row = i / N;
+        int j = (int)(i - row * N);
+        float v = sm[i] - (lab[row] == (int64_t)j ? 1.f : 0.f);
+        dz[i] = v * scale;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+int xsmi_axpy(float *y, const float *x, float a, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (y && x), "xsmi_axpy: null pointer");
+    return launch_ew("axpy", n, aligned16(y) && aligned16(x), AxpyF{y, x, a});
+}
+int xsmi_add(const float *a, const float *b, float *out, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add: null pointer");
+    return launch_ew("add", n, aligned16(a) && aligned16(b) && aligned16(out), AddF{a, b, out});
+}
+int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (a && out), "xsmi_scale_shift: null pointer");
+    return launch_ew("scale_shift", n, aligned16(a) && aligned16(out), ScaleF{a, out, s, t});
+}
+int xsmi_relu_fwd(const float *x, float *y, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (x && y), "xsmi_relu_fwd: null pointer");
+    return launch_ew("relu_fwd", n, aligned16(x) && aligned16(y), ReluF{x, y});
+}
+int xsmi_relu_fwd_mask(const float *x, float *y, uint8_t *neg_mask, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (x && y && neg_mask), "xsmi_relu_fwd_mask: null pointer");
+    return launch_ew("relu_fwd_mask", n, aligned16(x) && aligned16(y) && (((uintptr_t)neg_mask & 3) == 0),
+                     ReluMaskF{x, y, neg_mask});
+}
+int xsmi_relu_bwd(const float *dy, const float *pre, float *dx, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (dy && pre && dx), "xsmi_relu_bwd: null pointer");
+    return launch_ew("relu_bwd", n, aligned16(dy) && aligned16(pre) && aligned16(dx), ReluBwdF{dy, pre, dx});
+}
+int xsmi_lerp(float *m, const float *cur, float momentum, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (m && cur), "xsmi_lerp: null pointer");
+    return launch_ew("lerp", n, 0, LerpF{m, cur, momentum});
+}
+
+size_t xsmi_bn_workspace_bytes(int C) { return C > 0 ? (size_t)C * BN_SPLIT * 2 * sizeof(double) : 0; }
+
+int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar, float *mean,
+                float *var, int N, int C, int HW, float eps, void *ws, size_t ws_bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_fwd: empty tensor");
+    XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_fwd: tensors of 2^29 elements or more are not supported");
+    XSMI_CHECK_ARG(x && gamma && beta && y && sqrtvar && mean && var, "xsmi_bn_fwd: null pointer");
+    XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
+    hipStream_t st = xsmi::stream();
+    double *part = (double *)ws;
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, BN_SPLIT), dim3(256), 0, st, x, (const float *)nullptr, part, N, C, HW);
+    XSMI_LAUNCH_CHECK("bn_partial_kernel");
+    hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
+                       (double)N * HW, eps);
+    XSMI_LAUNCH_CHECK("bn_stats_kernel");
+    size_t total = (size_t)N * C * HW;
+    hipLaunchKernelGGL(bn_apply_kernel, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y, xhat,
+                       make_chan(C, HW), (uint32_t)total);
+    XSMI_LAUNCH_CHECK("bn_apply_kernel");
+    return XSMI_OK;
+}
+
+__global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, const float *__restrict__ mean,
+                                                        const float *__restrict__ var, float *__restrict__ y, ChanIdx chan,
+                                                        uint32_t total, float eps) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        int c = chan(i);
+        y[i] = gamma[c] * ((x[i] - mean[c]) / sqrtf(var[c] + eps)) + beta[c];
+    }
+}
+
+int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
+                  int N, int C, int HW, float eps) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_infer: empty tensor");
+    XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_infer: tensors of 2^29 elements or more are not supported");
+    XSMI_CHECK_ARG(x && gamma && beta && mean && var && y, "xsmi_bn_infer: null pointer");
+    size_t total = (size_t)N * C * HW;
+    hipLaunchKernelGGL(bn_infer_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean, var, y,
+                       make_chan(C, HW), (uint32_t)total, eps);
+    XSMI_LAUNCH_CHECK("bn_infer_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, float *dx, float *dgamma,
+                float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_bwd: empty tensor");
+    XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_bwd: tensors of 2^29 elements or more are not supported");
+    XSMI_CHECK_ARG(dy && xhat && sqrtvar && gamma && dx && dgamma && dbeta, "xsmi_bn_bwd: null pointer");
+    XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd: workspace too small");
+    hipStream_t st = xsmi::stream();
+    double *part = (double *)ws;
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, BN_SPLIT), dim3(256), 0, st, dy, xhat, part, N, C, HW);
+    XSMI_LAUNCH_CHECK("bn_partial_kernel");
+    hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C);
+    XSMI_LAUNCH_CHECK("bn_bwd_stats_kernel");
+    size_t total = (size_t)N * C * HW;
+    hipLaunchKernelGGL(bn_bwd_apply_kernel, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, dx,
+                       make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
+    XSMI_LAUNCH_CHECK("bn_bwd_apply_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W, "xsmi_avgpool_fwd: bad geometry");
+    XSMI_CHECK_ARG(x && y, "xsmi_avgpool_fwd: null pointer");
+    int OH = H / k, OW = W / k;
+    size_t total = (size_t)N * C * OH * OW;
+    hipLaunchKernelGGL(avgpool_fwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, y, H, W, OH, OW, k, total);
+    XSMI_LAUNCH_CHECK("avgpool_fwd_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W, "xsmi_avgpool_bwd: bad geometry");
+    XSMI_CHECK_ARG(dy && dx, "xsmi_avgpool_bwd: null pointer");
+    int OH = H / k, OW = W / k;
+    size_t total = (size_t)N * C * H * W;
+    hipLaunchKernelGGL(avgpool_bwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), dy, dx, H, W, OH, OW, k, total);
+    XSMI_LAUNCH_CHECK("avgpool_bwd_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(M > 0 && N > 0 && K > 0, "xsmi_gemm: empty matrix");
+    XSMI_CHECK_ARG(A && B && C, "xsmi_gemm: null pointer");
+    hipLaunchKernelGGL(gemm_kernel, dim3((N + 31) / 32, (M + 31) / 32), dim3(256), 0, xsmi::stream(), A, B, bias, C, M, N,
+                       K, trans_a, trans_b);
+    XSMI_LAUNCH_CHECK("gemm_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_colsum(const float *a, float *out, int M, int N) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(M > 0 && N > 0 && a && out, "xsmi_colsum: bad argument");
+    hipLaunchKernelGGL(colsum_kernel, dim3((N + 255) / 256), dim3(256), 0, xsmi::stream(), a, out, M, N);
+    XSMI_LAUNCH_CHECK("colsum_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_sum_all(const float *a, float *out, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(a && out, "xsmi_sum_all: null pointer");
+    hipLaunchKernelGGL(sum_all_kernel, dim3(1), dim3(256), 0, xsmi::stream(), a, out, n);
+    XSMI_LAUNCH_CHECK("sum_all_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_softmax_ce_fwd(const float *logits, const int64_t *labels, float *sm, float *loss, int M, int N, int mean) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(M > 0 && N > 0 && logits && labels && sm && loss, "xsmi_softmax_ce_fwd: bad argument");
+    hipStream_t st = xsmi::stream();
+    // `loss` has room for 1 + M floats: loss[0] is the result, loss[1..M] the per-row terms
+    hipLaunchKernelGGL(softmax_rows_kernel, dim3(M), dim3(64), 0, st, logits, labels, sm, loss + 1, M, N);
+    XSMI_LAUNCH_CHECK("softmax_rows_kernel");
+    hipLaunchKernelGGL(nll_reduce_kernel, dim3(1), dim3(256), 0, st, loss + 1, loss, M, mean);
+    XSMI_LAUNCH_CHECK("nll_reduce_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, float *dlogits, int M, int N, float scale) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(M > 0 && N > 0 && sm && labels && dlogits, "xsmi_softmax_ce_bwd: bad argument");
+    size_t total = (size_t)M * N;
+    hipLaunchKernelGGL(softmax_ce_bwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), sm, labels, dlogits, N, total,
+                       scale);
+    XSMI_LAUNCH_CHECK("softmax_ce_bwd_kernel");
+    return XSMI_OK;
+}
+
+}  // extern "C"

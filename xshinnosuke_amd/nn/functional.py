@@ -30,6 +30,8 @@ def _mark_input(t):
 def _wire(out, *ins):
     """Dynamic-graph bookkeeping: out.in_bounds = ins (None kept as a placeholder), ins[i].out_bounds += out."""
     if out.is_dynamic:
+        if out.in_bounds:                # a reused output tensor (forward without backward): re-wire, do not append
+            del out.in_bounds[:]
         out.add_in_bounds(*ins)
         for t in ins:
             if t is not None:
@@ -239,11 +241,16 @@ def relu(inputs, inplace=False, out=None):
         x = inputs.eval
         if GLOBAL.COMPUTE_GRAD and inputs.requires_grad:
             # the strict mask needs the sign of the pre-activation; y == 0 cannot tell x == 0 from x < 0
-            inputs.cache['pre_sign'] = x.copy() if not is_device(x) else x.copy()
+            if is_device(x):
+                _, inputs.cache['neg_mask_inplace'] = K.relu_fwd_mask(x, x)
+            else:
+                inputs.cache['neg_mask_inplace'] = x < 0
+                A.relu(x, x)
             inputs.cache.setdefault('grad_fn', []).append(inputs.grad_fn)
             inputs.cache['inplace'] = True
             inputs.grad_fn = ReLUBackward
-        A.relu(x, x)
+        else:
+            A.relu(x, x)
         return inputs
     res = A.relu(inputs.eval, None if out is None else out.eval)
     if out is None:

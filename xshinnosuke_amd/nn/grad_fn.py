@@ -100,10 +100,16 @@ def Maxpool2DBackward(outputs):
 def ReLUBackward(outputs):
     """Reference xs/nn/grad_fn.py:146-157, both the in-place and the out-of-place form."""
     if outputs.cache.get('inplace'):
-        g = A.relu_grad(outputs.grad.eval, outputs.cache['pre_sign'])
-        outputs.grad.eval = g
-        outputs.grad_fn = outputs.cache['grad_fn'].pop()
-        outputs.grad_fn(outputs)
+        g, mask = outputs.grad.eval, outputs.cache['neg_mask_inplace']
+        if is_device(g):
+            K.relu_mask_bwd(g, mask, dx=g)                 # in place on the gradient
+        else:
+            g[mask] = 0
+        prev = outputs.cache['grad_fn'].pop()
+        outputs.cache['inplace'] = bool(outputs.cache['grad_fn'])
+        outputs.grad_fn = prev
+        if prev is not None:
+            prev(outputs)
     else:
         inputs, = outputs.in_bounds
         if inputs.requires_grad:

@@ -201,7 +201,7 @@ class Sequential(_Model):
 
     def forward(self, x, *args, **kwargs):
         for layer in self._graph:
-            x = layer(x) if isinstance(layer, _Base) else layer.forward(x)
+            x = layer.forward(x)
         return x
 
 
