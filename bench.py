@@ -138,6 +138,47 @@ def bench_pool(be, steps, warmup):
     }
 
 
+def bench_resnet18(be, steps, warmup):
+    """ResNet-18 (BasicBlock [2,2,2,2], 7x7/2 stem, 3x3/2 max-pool, global avg pool, FC 1000) fwd+bwd+SGD through the
+    layer API on device-resident tensors: N=32x3x224x224 fp32, He-normal weights, random labels."""
+    import xshinnosuke_amd as xs
+    from xshinnosuke_amd.utils.resnet import ResNet18
+    from xshinnosuke_amd.optim import SGD
+    np.random.seed(6)
+    x = xs.tensor(np.random.default_rng(6).standard_normal((32, 3, 224, 224), dtype=np.float32)).to('cuda')
+    y = xs.tensor(np.random.default_rng(7).integers(0, 1000, size=(32,))).to('cuda')
+    net = ResNet18(classes=1000, pool=7).to('cuda')
+    crit = xs.nn.CrossEntropyLoss()
+    with xs.no_grad():
+        net(x)                               # creates the parameters
+    xs.GLOBAL.INPUTS = None
+    opt = SGD(net.parameters(), lr=0.01)
+
+    def step():
+        opt.zero_grad()
+        loss = crit(net(x), y)
+        loss.backward()
+        opt.step()
+        return loss
+
+    for _ in range(warmup):
+        step()
+    be.synchronize()
+    t0 = time.perf_counter()
+    e0, e1 = be.Event(), be.Event()
+    e0.record()
+    for _ in range(steps):
+        loss = step()
+    e1.record()
+    ms = e0.elapsed_ms(e1)
+    be.synchronize()
+    wall = (time.perf_counter() - t0) * 1e3
+    xs.GLOBAL.USE_CUDA = False
+    return {"resnet18_train_images_per_sec": 32 * steps / (ms * 1e-3), "resnet18_ms_per_step": ms / steps,
+            "resnet18_wall_ms_per_step": wall / steps, "resnet18_last_loss": loss.item(),
+            "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
+
+
 def cpu_baseline():
     """Oracle (NumPy restatement of the reference algorithm) on the host cores, same workload."""
     import oracle
@@ -197,7 +238,7 @@ def main():
         "frac_fp32_mfma_peak": value / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
-                     "kernel": "igemm_f32_kernel", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
+                     "kernel": "tap_igemm_f32_kernel", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
         "kernels_ms": {"conv_fwd_igemm": per["fwd"], "conv_bwd_data_igemm": per["bwd_data"],
                        "conv_bwd_weight_wgrad": per["bwd_weight"]},
         "kernels_tflops": {k: flops_pass / (v * 1e-3) / 1e12 for k, v in per.items()},
@@ -206,6 +247,7 @@ def main():
     }
     if not args.no_extra:
         out["extra"] = bench_pool(be, max(args.steps, 20), args.warmup)
+        out["extra"].update(bench_resnet18(be, max(5, args.steps // 5), 3))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     else:
