@@ -55,6 +55,19 @@ def make_conv_inputs(c):
     return x, w, b, dy
 
 
+def batch_ms(be, launch, n):
+    """Average duration of n back-to-back launches, from two events on the library's stream."""
+    e0, e1 = be.Event(), be.Event()
+    be.synchronize()
+    e0.record()
+    for _ in range(n):
+        launch()
+    e1.record()
+    ms = e0.elapsed_ms(e1)
+    be.synchronize()
+    return ms / n
+
+
 def bench_conv(be, steps, warmup):
     K = be.kernels
     c = CONV
@@ -81,18 +94,14 @@ def bench_conv(be, steps, warmup):
     be.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
 
-    # second pass over the same K steps: per-kernel durations from the library's own event pairs
-    be.profiling(True)
-    per = {"fwd": [], "bwd_data": [], "bwd_weight": []}
-    for _ in range(steps):
-        K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y)
-        per["fwd"].append(be.last_kernel_ms())
-        K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx)
-        per["bwd_data"].append(be.last_kernel_ms())
-        K.conv2d_bwd_weight(ddy, dx_, w.shape, c["stride"], c["pad"], dw=gw, db=gb)
-        per["bwd_weight"].append(be.last_kernel_ms())
-    be.profiling(False)
-    return ms / steps, wall_ms / steps, {k: statistics.mean(v) for k, v in per.items()}
+    # second pass: each kernel launched K times back to back between one pair of events on the
+    # library's stream, so the average launch duration carries no per-launch event overhead
+    per = {
+        "fwd": batch_ms(be, lambda: K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y), steps),
+        "bwd_data": batch_ms(be, lambda: K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx), steps),
+        "bwd_weight": batch_ms(be, lambda: K.conv2d_bwd_weight(ddy, dx_, w.shape, c["stride"], c["pad"], dw=gw, db=gb), steps),
+    }
+    return ms / steps, wall_ms / steps, per
 
 
 def bench_pool(be, steps, warmup):
@@ -113,22 +122,14 @@ def bench_pool(be, steps, warmup):
         K.maxpool2d_fwd(dx_, p["k"], p["stride"], p["pad"], out=y, idx=idx)
         K.maxpool2d_bwd(ddy, idx, x.shape, p["k"], p["stride"], p["pad"], dx=gx)
     be.synchronize()
-    be.profiling(True)
-    f, b = [], []
-    for _ in range(steps):
-        K.maxpool2d_fwd(dx_, p["k"], p["stride"], p["pad"], out=y, idx=idx)
-        f.append(be.last_kernel_ms())
-        K.maxpool2d_bwd(ddy, idx, x.shape, p["k"], p["stride"], p["pad"], dx=gx)
-        b.append(be.last_kernel_ms())
+    fm = batch_ms(be, lambda: K.maxpool2d_fwd(dx_, p["k"], p["stride"], p["pad"], out=y, idx=idx), steps)
+    bm = batch_ms(be, lambda: K.maxpool2d_bwd(ddy, idx, x.shape, p["k"], p["stride"], p["pad"], dx=gx), steps)
     # plain copy of the same number of bytes, for the achievable-bandwidth reference
     src = be.empty((x.size + dy.size + dy.size // 4,)); dst = be.empty(src.shape)
-    cp = []
-    for _ in range(warmup + steps):
+    for _ in range(warmup):
         K.copy_kernel(dst, src)
-        cp.append(be.last_kernel_ms())
-    be.profiling(False)
+    cm = batch_ms(be, lambda: K.copy_kernel(dst, src), steps)
     bytes_alg = x.nbytes + dy.nbytes + dy.size          # x + y + 1-byte index  (fwd);  dy + idx + dx  (bwd)
-    fm, bm, cm = statistics.mean(f), statistics.mean(b), statistics.mean(cp[warmup:])
     return {
         "maxpool_workload": "N=32 C=64 112x112, 3x3 stride 2 pad 1, fp32, 5% ties",
         "maxpool_algorithmic_MB": bytes_alg / 1e6,

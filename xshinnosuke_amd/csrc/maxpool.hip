@@ -8,7 +8,6 @@
 // window whose recorded index points at that cell, in ascending (ky,kx) order in
 // float64, and rounds once.
 #include "xsmi_internal.h"
-#include <stdlib.h>
 
 namespace {
 
@@ -59,44 +58,55 @@ __global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restri
 
 // 3x3 window, stride 2, pad 1, W % 4 == 0 (so OW = W/2): one thread produces two
 // adjacent outputs of one row from float4 loads of columns [4j, 4j+3] of the
-// three input rows; column 4j-1 comes from the previous lane (or one scalar load
-// at a wavefront edge, or the zero border at j == 0).  x is fetched once per
-// window row; the row shared by vertically adjacent windows is re-read from
-// cache.
+// three input rows, so a wavefront's loads are contiguous.  Column 4j-1 comes
+// from the previous lane (or one scalar load at a wavefront edge, or the zero
+// border at j == 0).  All loads are issued before the first comparison so that
+// their latencies overlap.  x is fetched once per window row; the row shared by
+// vertically adjacent windows is re-read from cache.
 __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restrict__ x, float *__restrict__ y,
                                                             uint8_t *__restrict__ idx, PoolGeom g,
                                                             xsmi::FastDiv dQ, uint32_t total_pairs) {
     uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    bool live = t < total_pairs;
-    if (!live) t = total_pairs - 1;
-    const int Q = g.OW >> 1;                 // output pairs per row == float4 per input row / 1
+    const bool live = t < total_pairs;
+    if (!live) t = total_pairs - 1;          // keep the lane for the shuffles below
+    const int Q = g.OW >> 1;                 // output pairs per row == float4 per input row
     uint32_t row = xsmi::fdiv(t, dQ);        // (nc, oh)
-    int j = (int)(t - row * Q);
+    const int j = (int)(t - row * Q);
     uint32_t nc = xsmi::fdiv(row, g.dOH);
-    int oh = (int)(row - nc * g.OH);
+    const int oh = (int)(row - nc * g.OH);
     const float *plane = x + (size_t)nc * g.H * g.W;
     const int lane = threadIdx.x & 63;
 
-    float b0 = 0.f, b1 = 0.f;
-    int w0 = 0, w1 = 0;
-    bool first = true;
+    float4 v[3];
+    float lf[3];
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
-        int ih = 2 * oh - 1 + r;
-        bool rowok = (unsigned)ih < (unsigned)g.H;
-        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (rowok) v = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
-        float left = __shfl_up(v.w, 1);
+        const int ih = 2 * oh - 1 + r;
+        v[r] = make_float4(0.f, 0.f, 0.f, 0.f);   // border row
+        lf[r] = 0.f;
+        if ((unsigned)ih < (unsigned)g.H) v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
+    }
+    if (lane == 0 && j > 0) {
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int ih = 2 * oh - 1 + r;
+            if ((unsigned)ih < (unsigned)g.H) lf[r] = plane[(size_t)ih * g.W + 4 * j - 1];
+        }
+    }
+    float b0 = 0.f, b1 = 0.f;
+    int w0 = 0, w1 = 0;
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+        float left = __shfl_up(v[r].w, 1);
         if (j == 0) left = 0.f;                                       // zero border
-        else if (lane == 0) left = rowok ? plane[(size_t)ih * g.W + 4 * j - 1] : 0.f;
+        else if (lane == 0) left = lf[r];
         // output 2j: columns 4j-1, 4j, 4j+1 ; output 2j+1: columns 4j+1, 4j+2, 4j+3
-        if (first || left > b0) { b0 = left; w0 = r * 3 + 0; }
-        if (v.x > b0) { b0 = v.x; w0 = r * 3 + 1; }
-        if (v.y > b0) { b0 = v.y; w0 = r * 3 + 2; }
-        if (first || v.y > b1) { b1 = v.y; w1 = r * 3 + 0; }
-        if (v.z > b1) { b1 = v.z; w1 = r * 3 + 1; }
-        if (v.w > b1) { b1 = v.w; w1 = r * 3 + 2; }
-        first = false;
+        if (r == 0 || left > b0) { b0 = left; w0 = r * 3 + 0; }
+        if (v[r].x > b0) { b0 = v[r].x; w0 = r * 3 + 1; }
+        if (v[r].y > b0) { b0 = v[r].y; w0 = r * 3 + 2; }
+        if (r == 0 || v[r].y > b1) { b1 = v[r].y; w1 = r * 3 + 0; }
+        if (v[r].z > b1) { b1 = v[r].z; w1 = r * 3 + 1; }
+        if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
     }
     if (!live) return;
     size_t o = (size_t)row * g.OW + 2 * j;
@@ -135,199 +145,86 @@ __global__ void __launch_bounds__(256) maxpool_bwd_gather(const float *__restric
     dx[e] = (float)acc;
 }
 
-// 3x3 / stride 2 / pad 1 with W % 4 == 0: one thread per four consecutive dx
-// columns 4j..4j+3 of one row.  Covering windows: ow in {2j-1+1.. } i.e. columns
-// qw = w+1 in [4j+1, 4j+4] are covered by ow = 2j (s = qw-4j in {1,2}),
-// ow = 2j+1 (s in {0,1,2} for qw = 4j+2..4j+4) and ow = 2j+2 (s = 0 for qw = 4j+4).
+// 3x3 window, stride 2, pad 1, W % 4 == 0, H % 2 == 0: one thread produces dx
+// columns 4j .. 4j+3 of the two input rows 2a and 2a+1 with one float4 store per
+// row, contiguous across the wavefront.  It reads output columns 2j, 2j+1 of the
+// output rows a and a+1 (dy and index) and takes column 2j+2 from the next lane
+// (one scalar load at a wavefront edge, nothing at the row end).
+//   even row, even column: one contributor  (window row 1, kx 1)
+//   even row, odd column:  two              (kx 0 of the output column to the right, kx 2 of this one)
+//   odd row,  even column: two              (window row 0 of output row a+1, window row 2 of row a)
+//   odd row,  odd column:  four
+// The float32 sum of two float32 values equals their float64 sum rounded to
+// float32, so only the four-term cells, and every cell when the previous dx is
+// one more term (ACC), go through float64.
+template <bool ACC>
 __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
                                                             float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ4,
-                                                            uint32_t total_quads, int accumulate) {
-    uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    if (t >= total_quads) return;
-    const int Q4 = g.W >> 2;
-    uint32_t row = xsmi::fdiv(t, dQ4);       // (nc, h)
-    int j = (int)(t - row * Q4);
-    uint32_t nc = xsmi::fdiv(row, g.dH);
-    int h = (int)(row - nc * g.H);
-    const size_t obase = (size_t)nc * g.OH * g.OW;
-    const int qh = h + 1;
-    double a0 = 0.0, a1 = 0.0, a2 = 0.0, a3 = 0.0;
-    // ascending ky == descending oh; for one oh ascending kx == descending ow
-    int oh_hi = qh >> 1;
-    for (int oh = oh_hi; oh >= 0 && oh >= oh_hi - 1; --oh) {
-        int r = qh - 2 * oh;
-        if (r > 2 || oh >= g.OH) continue;
-        const size_t ro = obase + (size_t)oh * g.OW;
-        const int r3 = r * 3;
-        // ow = 2j+2 (may be out of range), 2j+1, 2j
-        int owc = 2 * j + 2;
-        float gC = 0.f; int iC = -1;
-        if (owc < g.OW) { gC = dy[ro + owc]; iC = idx[ro + owc]; }
-        float2 gAB = *reinterpret_cast<const float2 *>(dy + ro + 2 * j);
-        uchar2 iAB = *reinterpret_cast<const uchar2 *>(idx + ro + 2 * j);
-        int iA = iAB.x, iB = iAB.y;
-        // column 4j   (qw=4j+1): ow=2j s=1
-        if (iA == r3 + 1) a0 += (double)gAB.x;
-        // column 4j+1 (qw=4j+2): ow=2j+1 s=0 first (higher ow == lower kx), then ow=2j s=2
-        if (iB == r3 + 0) a1 += (double)gAB.y;
-        if (iA == r3 + 2) a1 += (double)gAB.x;
-        // column 4j+2 (qw=4j+3): ow=2j+1 s=1
-        if (iB == r3 + 1) a2 += (double)gAB.y;
-        // column 4j+3 (qw=4j+4): ow=2j+2 s=0, then ow=2j+1 s=2
-        if (iC == r3 + 0) a3 += (double)gC;
-        if (iB == r3 + 2) a3 += (double)gAB.y;
-    }
-    float4 *out = reinterpret_cast<float4 *>(dx + (size_t)row * g.W + 4 * j);
-    if (accumulate) {
-        float4 old = *out;
-        a0 += (double)old.x; a1 += (double)old.y; a2 += (double)old.z; a3 += (double)old.w;
-    }
-    *out = make_float4((float)a0, (float)a1, (float)a2, (float)a3);
-}
-
-// 3x3 / stride 2 / pad 1, W % 8 == 0, OH % RO == 0: one thread produces a 4-column x RO-row patch of outputs.
-// It streams the 2*RO+1 input rows that patch needs (two 128-bit loads per row, the left neighbour column from the
-// previous lane), so a row shared by vertically adjacent windows is loaded once per patch, and stores y as one
-// 128-bit and idx as one 32-bit access per output row.
-template <int RO>
-__global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1_patch(const float *__restrict__ x, float *__restrict__ y,
-                                                                  uint8_t *__restrict__ idx, PoolGeom g, xsmi::FastDiv dQ,
-                                                                  xsmi::FastDiv dG, uint32_t total) {
+                                                            xsmi::FastDiv dG, uint32_t total) {
     uint32_t t = blockIdx.x * 256u + threadIdx.x;
     const bool live = t < total;
-    if (!live) t = total - 1;
-    const int Q = g.OW >> 2, G = g.OH / RO;
-    uint32_t rowg = xsmi::fdiv(t, dQ);       // (nc, row group)
-    const int j = (int)(t - rowg * Q);
+    if (!live) t = total - 1;                // keep the lane for the shuffles below
+    const int Q4 = g.W >> 2, G = g.H >> 1;
+    uint32_t rowg = xsmi::fdiv(t, dQ4);      // (nc, a)
+    const int j = (int)(t - rowg * Q4);
     uint32_t nc = xsmi::fdiv(rowg, dG);
-    const int oh0 = ((int)(rowg - nc * G)) * RO;
-    const float *plane = x + (size_t)nc * g.H * g.W;
-    const int lane = threadIdx.x & 63;
-    float best[RO][4];
-    int where[RO][4];
-    // all loads first (independent of each other), then the compare chains
-    constexpr int NR = 2 * RO + 1;
-    float4 va[NR], vb[NR];
-    float lf[NR];
+    const int a = (int)(rowg - nc * G);
+    const size_t obase = (size_t)nc * g.OH * g.OW;
+    const bool edge = (threadIdx.x & 63) == 63;
+    float gv[2][3];
+    int iv[2][3];
 #pragma unroll
-    for (int i = 0; i < NR; ++i) {
-        const int ih = 2 * oh0 - 1 + i;
-        va[i] = make_float4(0.f, 0.f, 0.f, 0.f);
-        vb[i] = va[i];
-        lf[i] = 0.f;
-        if ((unsigned)ih < (unsigned)g.H) {
-            const float4 *src = reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 8 * j);
-            va[i] = src[0];
-            vb[i] = src[1];
+    for (int q = 0; q < 2; ++q) {
+        const int oh = a + q;                 // a + 1 == OH: below the last output row
+        float2 gg = make_float2(0.f, 0.f);
+        int i0 = -1, i1 = -1;
+        float gn = 0.f;
+        int in = -1;
+        const size_t ro = obase + (size_t)oh * g.OW + 2 * j;
+        if (oh < g.OH) {
+            gg = *reinterpret_cast<const float2 *>(dy + ro);
+            uchar2 ii = *reinterpret_cast<const uchar2 *>(idx + ro);
+            i0 = ii.x; i1 = ii.y;
         }
-    }
-    if (lane == 0 && j > 0) {                     // the column left of a wavefront's first patch is not in any lane
-#pragma unroll
-        for (int i = 0; i < NR; ++i) {
-            const int ih = 2 * oh0 - 1 + i;
-            if ((unsigned)ih < (unsigned)g.H) lf[i] = plane[(size_t)ih * g.W + 8 * j - 1];
+        float sg = __shfl_down(gg.x, 1);
+        int si = __shfl_down(i0, 1);
+        if (2 * j + 2 < g.OW && oh < g.OH) {
+            if (edge) { sg = dy[ro + 2]; si = idx[ro + 2]; }
+            gn = sg; in = si;
         }
-    }
-#pragma unroll
-    for (int i = 0; i <= 2 * RO; ++i) {
-        const float4 v0 = va[i], v1 = vb[i];
-        float left = __shfl_up(v1.w, 1);
-        if (j == 0) left = 0.f;                                           // zero border
-        else if (lane == 0) left = lf[i];
-        const float c[9] = {left, v0.x, v0.y, v0.z, v0.w, v1.x, v1.y, v1.z, v1.w};
-        // row i is window row 2 of output row i/2 - 1 (i even, i >= 2) and window row i%2 of output row i/2
-        if ((i & 1) == 0 && i >= 2) {
-            const int o = i / 2 - 1;
-#pragma unroll
-            for (int q = 0; q < 4; ++q)
-#pragma unroll
-                for (int e = 0; e < 3; ++e)
-                    if (c[2 * q + e] > best[o][q]) { best[o][q] = c[2 * q + e]; where[o][q] = 6 + e; }
-        }
-        if (i < 2 * RO) {
-            const int o = i / 2, r3 = (i & 1) * 3;
-#pragma unroll
-            for (int q = 0; q < 4; ++q) {
-                if ((i & 1) == 0) { best[o][q] = c[2 * q]; where[o][q] = 0; }   // first cell of the window
-                else if (c[2 * q] > best[o][q]) { best[o][q] = c[2 * q]; where[o][q] = r3; }
-                if (c[2 * q + 1] > best[o][q]) { best[o][q] = c[2 * q + 1]; where[o][q] = r3 + 1; }
-                if (c[2 * q + 2] > best[o][q]) { best[o][q] = c[2 * q + 2]; where[o][q] = r3 + 2; }
-            }
-        }
+        // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
+        gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gn + 0.f;
+        iv[q][0] = i0; iv[q][1] = i1; iv[q][2] = in;
     }
     if (!live) return;
+    const int h = 2 * a;
+    float4 *pe = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h) * g.W + 4 * j);
+    float4 *po = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h + 1) * g.W + 4 * j);
+    float e[4], o[4];
+    auto pick = [&](int q, int m, int tap) { return iv[q][m] == tap ? gv[q][m] : 0.f; };
+    if (ACC) {
+        const float4 ev = *pe, ov = *po;
+        const float pe4[4] = {ev.x, ev.y, ev.z, ev.w}, po4[4] = {ov.x, ov.y, ov.z, ov.w};
 #pragma unroll
-    for (int o = 0; o < RO; ++o) {
-        size_t off = ((size_t)nc * g.OH + oh0 + o) * g.OW + 4 * j;
-        *reinterpret_cast<float4 *>(y + off) = make_float4(best[o][0], best[o][1], best[o][2], best[o][3]);
-        if (idx)
-            *reinterpret_cast<uchar4 *>(idx + off) = make_uchar4((unsigned char)where[o][0], (unsigned char)where[o][1],
-                                                                 (unsigned char)where[o][2], (unsigned char)where[o][3]);
-    }
-}
-
-// Backward of the same geometry: one thread owns an 8-column x 2*RP-row patch of dx (rows 2a .. 2a+2RP-1) and reads
-// the RP+1 output rows a .. a+RP that can route gradient into it (columns 4j .. 4j+4), each once.
-// dx column 8j+2m   (even) is reached only through kx = 1 of output column 4j+m;
-// dx column 8j+2m+1 (odd) through kx = 0 of output column 4j+m+1, then kx = 2 of output column 4j+m.
-template <int RP>
-__global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_patch(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
-                                                                  float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ8,
-                                                                  xsmi::FastDiv dG, uint32_t total, int accumulate) {
-    uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    if (t >= total) return;
-    const int Q8 = g.W >> 3, G = g.H / (2 * RP);
-    uint32_t rowg = xsmi::fdiv(t, dQ8);
-    const int j = (int)(t - rowg * Q8);
-    uint32_t nc = xsmi::fdiv(rowg, dG);
-    const int a0 = ((int)(rowg - nc * G)) * RP;
-    const size_t obase = (size_t)nc * g.OH * g.OW;
-    float gv[RP + 1][5];
-    int iv[RP + 1][5];
+        for (int m = 0; m < 2; ++m) {
+            e[2 * m] = (float)((double)pick(0, m, 4) + (double)pe4[2 * m]);
+            e[2 * m + 1] = (float)(((double)pick(0, m + 1, 3) + (double)pick(0, m, 5)) + (double)pe4[2 * m + 1]);
+            o[2 * m] = (float)(((double)pick(1, m, 1) + (double)pick(0, m, 7)) + (double)po4[2 * m]);
+            o[2 * m + 1] = (float)(((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                    (double)pick(0, m, 8)) + (double)po4[2 * m + 1]);
+        }
+    } else {
 #pragma unroll
-    for (int q = 0; q <= RP; ++q) {
-        const int oh = a0 + q;
-#pragma unroll
-        for (int m = 0; m < 5; ++m) { gv[q][m] = 0.f; iv[q][m] = -1; }
-        if (oh < g.OH) {
-            const size_t ro = obase + (size_t)oh * g.OW + 4 * j;
-            float4 gg = *reinterpret_cast<const float4 *>(dy + ro);
-            uchar4 ii = *reinterpret_cast<const uchar4 *>(idx + ro);
-            gv[q][0] = gg.x; gv[q][1] = gg.y; gv[q][2] = gg.z; gv[q][3] = gg.w;
-            iv[q][0] = ii.x; iv[q][1] = ii.y; iv[q][2] = ii.z; iv[q][3] = ii.w;
-            if (4 * j + 4 < g.OW) { gv[q][4] = dy[ro + 4]; iv[q][4] = idx[ro + 4]; }
+        for (int m = 0; m < 2; ++m) {
+            e[2 * m] = pick(0, m, 4);
+            e[2 * m + 1] = pick(0, m + 1, 3) + pick(0, m, 5);
+            o[2 * m] = pick(1, m, 1) + pick(0, m, 7);
+            o[2 * m + 1] = (float)((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                   (double)pick(0, m, 8));
         }
     }
-    auto take = [&](int q, int r, double *c) {
-        const int r3 = 3 * r;
-#pragma unroll
-        for (int m = 0; m < 4; ++m) {
-            if (iv[q][m] == r3 + 1) c[2 * m] += (double)gv[q][m];
-            if (iv[q][m + 1] == r3 + 0) c[2 * m + 1] += (double)gv[q][m + 1];
-            if (iv[q][m] == r3 + 2) c[2 * m + 1] += (double)gv[q][m];
-        }
-    };
-#pragma unroll
-    for (int q = 0; q < RP; ++q) {
-        const int h = 2 * (a0 + q);
-        double ev[8] = {0, 0, 0, 0, 0, 0, 0, 0}, od[8] = {0, 0, 0, 0, 0, 0, 0, 0};
-        take(q, 1, ev);          // even row h: window row 1 of output row a0+q
-        take(q + 1, 0, od);      // odd row h+1: window row 0 of output row a0+q+1 first (ascending ky) ...
-        take(q, 2, od);          // ... then window row 2 of output row a0+q
-        float4 *pe = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h) * g.W + 8 * j);
-        float4 *po = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h + 1) * g.W + 8 * j);
-        if (accumulate) {
-            float4 a0v = pe[0], a1v = pe[1], b0v = po[0], b1v = po[1];
-            ev[0] += (double)a0v.x; ev[1] += (double)a0v.y; ev[2] += (double)a0v.z; ev[3] += (double)a0v.w;
-            ev[4] += (double)a1v.x; ev[5] += (double)a1v.y; ev[6] += (double)a1v.z; ev[7] += (double)a1v.w;
-            od[0] += (double)b0v.x; od[1] += (double)b0v.y; od[2] += (double)b0v.z; od[3] += (double)b0v.w;
-            od[4] += (double)b1v.x; od[5] += (double)b1v.y; od[6] += (double)b1v.z; od[7] += (double)b1v.w;
-        }
-        pe[0] = make_float4((float)ev[0], (float)ev[1], (float)ev[2], (float)ev[3]);
-        pe[1] = make_float4((float)ev[4], (float)ev[5], (float)ev[6], (float)ev[7]);
-        po[0] = make_float4((float)od[0], (float)od[1], (float)od[2], (float)od[3]);
-        po[1] = make_float4((float)od[4], (float)od[5], (float)od[6], (float)od[7]);
-    }
+    *pe = make_float4(e[0], e[1], e[2], e[3]);
+    *po = make_float4(o[0], o[1], o[2], o[3]);
 }
 
 int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw, int pad, PoolGeom *g) {
@@ -366,20 +263,6 @@ int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int
     uint32_t total = (uint32_t)N * C * g.OH * g.OW;
     hipStream_t st = xsmi::stream();
     xsmi::prof_begin();
-    static const int pool_rows = getenv("XSMI_POOL_ROWS") ? atoi(getenv("XSMI_POOL_ROWS")) : 1;
-    if (fast_3x3s2p1(g) && pool_rows >= 1 && g.W % 8 == 0 && g.OH % pool_rows == 0) {
-        const int RO = pool_rows;
-        uint32_t threads = total / 4 / RO;
-        xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 4), dG = xsmi::make_fastdiv(g.OH / RO);
-        dim3 grid((threads + 255) / 256);
-        if (RO == 1) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1_patch<1>, grid, dim3(256), 0, st, x, y, idx, g, dQ, dG, threads);
-        else if (RO == 2) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1_patch<2>, grid, dim3(256), 0, st, x, y, idx, g, dQ, dG, threads);
-        else if (RO == 4) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1_patch<4>, grid, dim3(256), 0, st, x, y, idx, g, dQ, dG, threads);
-        else return xsmi::set_error("XSMI_POOL_ROWS must be 0, 1, 2 or 4"), XSMI_ERR_INVALID;
-        xsmi::prof_end();
-        XSMI_LAUNCH_CHECK("maxpool_fwd_3x3s2p1_patch");
-        return XSMI_OK;
-    }
     if (fast_3x3s2p1(g)) {
         uint32_t pairs = total / 2;
         xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 2);
@@ -412,23 +295,12 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
     hipStream_t st = xsmi::stream();
     int acc = beta == 1.f ? 1 : 0;
     xsmi::prof_begin();
-    static const int pool_rp = getenv("XSMI_POOL_RP") ? atoi(getenv("XSMI_POOL_RP")) : 1;
-    if (fast_3x3s2p1(g) && pool_rp >= 1 && W % 8 == 0 && H % (2 * pool_rp) == 0) {
-        const int RP = pool_rp;
-        uint32_t threads = total / 8 / (2 * RP);
-        xsmi::FastDiv dQ8 = xsmi::make_fastdiv(W / 8), dG = xsmi::make_fastdiv(H / (2 * RP));
-        dim3 grid((threads + 255) / 256);
-        if (RP == 1) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_patch<1>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads, acc);
-        else if (RP == 2) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_patch<2>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads, acc);
-        else return xsmi::set_error("XSMI_POOL_RP must be 0, 1 or 2"), XSMI_ERR_INVALID;
-        xsmi::prof_end();
-        XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_patch");
-        return XSMI_OK;
-    }
     if (fast_3x3s2p1(g)) {
-        uint32_t quads = total / 4;
-        xsmi::FastDiv dQ4 = xsmi::make_fastdiv(W / 4);
-        hipLaunchKernelGGL(maxpool_bwd_3x3s2p1, dim3((quads + 255) / 256), dim3(256), 0, st, dy, idx, dx, g, dQ4, quads, acc);
+        uint32_t threads = total / 8;        // four columns of two rows each
+        xsmi::FastDiv dQ4 = xsmi::make_fastdiv(W / 4), dG = xsmi::make_fastdiv(H / 2);
+        dim3 grid((threads + 255) / 256);
+        if (acc) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1<true>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ4, dG, threads);
+        else hipLaunchKernelGGL(maxpool_bwd_3x3s2p1<false>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ4, dG, threads);
         xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1");
         return XSMI_OK;
