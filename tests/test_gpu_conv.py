@@ -9,7 +9,7 @@ import numpy as np
 import pytest
 
 import oracle
-from util import rel_l2, he_normal
+from util import rel_l2, he_normal, round_bf16
 
 pytestmark = pytest.mark.gpu
 TOL = 1e-5
@@ -96,6 +96,47 @@ def test_conv_fused_bias_relu_and_mask(gpu):
     dy = rng.standard_normal(pre.shape).astype(np.float32)
     g = K.relu_mask_bwd(gpu.to_device(dy), mask).numpy()
     np.testing.assert_array_equal(g, oracle.relu_bwd(dy, pre))
+
+
+BF16_CASES = [  # shapes whose reduction channels are a multiple of 32 take the bf16 MFMA kernel
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),
+    (2, 64, 28, 28, 128, 3, 3, 2, 2, 1),
+    (2, 64, 28, 28, 128, 1, 1, 2, 2, 0),
+    (3, 128, 14, 14, 130, 3, 3, 1, 1, 1),
+    (2, 3, 32, 32, 64, 7, 7, 2, 2, 3),     # stem: stays on the fp32 kernel, the flag only permits bf16
+]
+
+
+@pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", BF16_CASES)
+def test_conv_bf16_opt_in(gpu, n, c, h, w, k, r, s, sh, sw, pad):
+    """bf16 opt-in: tolerance rel-L2 <= 1e-2 against the fp32-rounded float64 oracle; against the oracle fed
+    with operands rounded to bf16 (round to nearest even) only the fp32 accumulation differs: <= 1e-5."""
+    K = gpu.kernels
+    rng = np.random.default_rng(77 + c + k)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = he_normal(rng, (k, c, r, s))
+    b = rng.standard_normal((k,)).astype(np.float32)
+    oh, ow = K.conv_out_hw(h, w, r, s, (sh, sw), pad)
+    dy = rng.standard_normal((n, k, oh, ow)).astype(np.float32)
+    y_ref, dx_ref, _, _ = _oracle(x, wt, b, (sh, sw), pad, dy)
+    dx_, dw_, db_, ddy = gpu.to_device(x), gpu.to_device(wt), gpu.to_device(b), gpu.to_device(dy)
+    y = K.conv2d_fwd(dx_, dw_, db_, (sh, sw), pad, bf16=True).numpy()
+    gx = K.conv2d_bwd_data(ddy, dw_, x.shape, (sh, sw), pad, bf16=True).numpy()
+    assert rel_l2(y, y_ref) <= 1e-2
+    assert rel_l2(gx, dx_ref) <= 1e-2
+    if c % 32 == 0:
+        y_r, _ = oracle.conv2d_fwd(round_bf16(x), round_bf16(wt), b, (sh, sw), pad)
+        assert rel_l2(y, y_r) <= TOL
+        assert rel_l2(y, y_ref) > 1e-4            # the bf16 kernel really ran
+    if k % 32 == 0:
+        _, col = oracle.conv2d_fwd(x, round_bf16(wt), None, (sh, sw), pad)
+        dx_r, _, _ = oracle.conv2d_bwd(round_bf16(dy), x.shape, round_bf16(wt), col, (sh, sw), pad, np.zeros_like(x),
+                                       np.zeros_like(wt), np.zeros((k,), dtype=np.float32))
+        assert rel_l2(gx, dx_r) <= TOL
+    # the weight gradient accepts the flag and stays on the fp32 path
+    gw, _ = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (sh, sw), pad, want_db=True, bf16=True)
+    gw32, _ = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (sh, sw), pad, want_db=True)
+    np.testing.assert_array_equal(gw.numpy(), gw32.numpy())
 
 
 def test_conv_special_kernels_exact(gpu):

@@ -33,3 +33,10 @@ def idx_nchw_to_ref(idx_nchw):
 
 def idx_ref_to_nchw(argmax, n, c, oh, ow):
     return np.ascontiguousarray(argmax.reshape(n, oh, ow, c).transpose(0, 3, 1, 2))
+
+
+def round_bf16(a):
+    """float32 array rounded to the nearest bf16 value (ties to even), returned as float32."""
+    u = np.ascontiguousarray(a, dtype=np.float32).view(np.uint32).astype(np.uint64)
+    u = (u + 0x7FFF + ((u >> 16) & 1)) & 0xFFFF0000
+    return u.astype(np.uint32).view(np.float32).reshape(np.shape(a))

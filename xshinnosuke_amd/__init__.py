@@ -12,7 +12,7 @@ import numpy as _np
 
 from . import backend  # noqa: F401
 from .core import state as GLOBAL
-from .core.state import no_grad
+from .core.state import no_grad, conv_precision
 from .core.base import Tensor, Parameter
 from . import nn, layers, optim, utils
 from .utils import gradient_check

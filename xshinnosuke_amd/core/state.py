@@ -10,6 +10,9 @@ GRAPH = None
 TRAINING = True
 COMPUTE_GRAD = True
 USE_CUDA = False
+# Opt-in: convolutions may round their MFMA operands to bf16 (fp32 accumulate).  Off by
+# default; the reference has no counterpart (its GEMMs run in float64).
+CONV_BF16 = False
 
 
 class no_grad:
@@ -23,3 +26,22 @@ class no_grad:
     def __exit__(self, *exc):
         global COMPUTE_GRAD
         COMPUTE_GRAD = self._saved
+
+
+class conv_precision:
+    """``with conv_precision('bf16'):`` lets conv2d forward / backward-data use bf16 MFMA operands
+    inside the block; ``'fp32'`` restores the default.  No counterpart in the reference."""
+
+    def __init__(self, mode):
+        if mode not in ('fp32', 'bf16'):
+            raise ValueError("conv_precision: mode must be 'fp32' or 'bf16', got %r" % (mode,))
+        self._mode = mode
+
+    def __enter__(self):
+        global CONV_BF16
+        self._saved = CONV_BF16
+        CONV_BF16 = self._mode == 'bf16'
+
+    def __exit__(self, *exc):
+        global CONV_BF16
+        CONV_BF16 = self._saved

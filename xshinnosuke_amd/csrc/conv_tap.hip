@@ -263,6 +263,141 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
     }
 }
 
+// bf16 variant (opt-in): the same fp32 tensors, loads and LDS layout, but the
+// fragments are rounded to bf16 (round to nearest even) in registers and a chunk
+// of 32 channels is two v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  A lane
+// keeps its 16 channels of the chunk (16*(lane/32) ..): MFMA u takes channels
+// 8u .. 8u+7 of them for both operands, which is a permutation of the reduction
+// index that A and B share.  With an eighth of the matrix instructions the loop is
+// bound by the global->LDS loads, so it is written plainly: convert, wait for
+// the next chunk, read its fragments, issue the loads of a later chunk, multiply.
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+template <int STAGES>
+__global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapParams p) {
+    __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
+    constexpr int D = STAGES - 1;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int m0 = blockIdx.x * BP;
+    const int rowtile = blockIdx.y;
+
+    int iyb = 0, ixb = 0, nbase = 0;
+    const bool live = m0 + lane < p.M;
+    if (live) {
+        uint32_t m = (uint32_t)(m0 + lane);
+        uint32_t q = xsmi::fdiv(m, p.dOX);
+        int x = (int)m - (int)q * p.OX;
+        uint32_t n = xsmi::fdiv(q, p.dOY);
+        int y = (int)q - (int)n * p.OY;
+        iyb = y * p.sy + p.dy0;
+        ixb = x * p.sx + p.dx0;
+        nbase = (int)n * p.in_n_stride;
+    }
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(p.in, p.in_bytes);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(p.apk, p.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];
+    const int iters = p.TR * p.TS * p.nch;
+    const uint32_t a_voff = (uint32_t)((2 * wave * 64 + lane) * 16);
+
+    int r = 0, s = 0, cc = 0;
+    uint32_t ld_stage = lds0;
+    uint32_t ld_asoff = (uint32_t)rowtile * (uint32_t)iters * (uint32_t)(TM * KC * 4);
+    auto issue_all = [&]() {
+        int iy = iyb + r * p.dstep, ix = ixb + s * p.dstep;
+        bool ok = live && (unsigned)iy < (unsigned)p.IH && (unsigned)ix < (unsigned)p.IW;
+        const uint32_t voff = ok ? (uint32_t)((nbase + iy * p.IW + ix) * 4) : 0x80000000u;
+        const uint32_t soff = (uint32_t)(cc * KC + wave * 8) * p.plane_bytes;
+#pragma unroll
+        for (int e = 0; e < 8; ++e)
+            xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((2048 + (wave * 8 + e) * 64) * 4), voff, soff + (uint32_t)e * p.plane_bytes);
+#pragma unroll
+        for (int qa = 0; qa < 2; ++qa)
+            xsmi::load_lds_b128(rap, ld_stage + (uint32_t)((2 * wave + qa) * 1024), a_voff + (uint32_t)qa * 1024u, ld_asoff);
+        ld_asoff += (uint32_t)(TM * KC * 4);
+        ld_stage += (uint32_t)(STAGE_FLOATS * 4);
+        if (ld_stage == lds0 + (uint32_t)(STAGES * STAGE_FLOATS * 4)) ld_stage = lds0;
+        if (++cc == p.nch) {
+            cc = 0;
+            if (++s == p.TS) { s = 0; ++r; }
+        }
+    };
+
+    floatx16 acc = {0};
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int a_rd = (4 * h * 64 + wr * 32 + l31) * 4;
+    const int b_rd = 2048 + 16 * h * 64 + wc * 32 + l31;
+    float4 fa[4];
+    float fb[16];
+    const float *rd_stage = smem[0];
+    auto read_frags = [&]() {
+#pragma unroll
+        for (int q4 = 0; q4 < 4; ++q4) fa[q4] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 256 * q4);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) fb[j] = rd_stage[b_rd + 64 * j];
+        rd_stage += STAGE_FLOATS;
+        if (rd_stage == smem[0] + STAGES * STAGE_FLOATS) rd_stage = smem[0];
+    };
+
+#pragma unroll
+    for (int d = 0; d < D; ++d)
+        if (d < iters) issue_all();
+    if (iters > 0) {
+        if (D <= iters) xsmi::wait_vmcnt<(D - 1) * LOADS_PER_CHUNK>();
+        else xsmi::wait_vmcnt<0>();
+        xsmi::block_barrier();
+        read_frags();
+        if (D < iters) issue_all();
+    }
+    for (int it = 0; it < iters; ++it) {
+        bf16x8 a0, a1, b0, b1;
+        a0[0] = (__bf16)fa[0].x; a0[1] = (__bf16)fa[0].y; a0[2] = (__bf16)fa[0].z; a0[3] = (__bf16)fa[0].w;
+        a0[4] = (__bf16)fa[1].x; a0[5] = (__bf16)fa[1].y; a0[6] = (__bf16)fa[1].z; a0[7] = (__bf16)fa[1].w;
+        a1[0] = (__bf16)fa[2].x; a1[1] = (__bf16)fa[2].y; a1[2] = (__bf16)fa[2].z; a1[3] = (__bf16)fa[2].w;
+        a1[4] = (__bf16)fa[3].x; a1[5] = (__bf16)fa[3].y; a1[6] = (__bf16)fa[3].z; a1[7] = (__bf16)fa[3].w;
+#pragma unroll
+        for (int e = 0; e < 8; ++e) { b0[e] = (__bf16)fb[e]; b1[e] = (__bf16)fb[8 + e]; }
+        // the conversions above consumed every fragment read, so no LDS read of the
+        // stage that the loads below refill is still outstanding past the barrier
+        if (it + 1 < iters) {
+            if (it + 1 + D <= iters) xsmi::wait_vmcnt<(D - 1) * LOADS_PER_CHUNK>();
+            else xsmi::wait_vmcnt<0>();
+            xsmi::block_barrier();
+            read_frags();
+            if (it + 1 + D < iters) issue_all();
+        }
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a0, b0, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a1, b1, acc, 0, 0, 0);
+    }
+
+    const int m = m0 + wc * 32 + l31;
+    if (m >= p.M) return;
+    uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+    int x = m - (int)q * p.OX;
+    uint32_t n = xsmi::fdiv(q, p.dOY);
+    int y = (int)q - (int)n * p.OY;
+    const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
+    const int rbase = rowtile * TM + wr * 32 + 4 * h;
+#pragma unroll
+    for (int v = 0; v < 16; ++v) {
+        int row = rbase + 8 * (v >> 2) + (v & 3);
+        if (row < p.rows) {
+            float val = acc[v];
+            if (p.bias) val += p.bias[row];
+            long long o = pix_off + (long long)row * p.os_k;
+            if (p.relu) {
+                if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
+                val = val > 0.f ? val : 0.f;
+            }
+            if (p.accumulate) val += p.out[o];
+            p.out[o] = val;
+        }
+    }
+}
+
 // Packs A for the tap-major kernel.  mode 0 (forward): A[row][tap=(r,s)][ch] = w[row][ch][r][s].
 // mode 1 (backward-data class): A[row=c][tap=(t,u)][ch=k] = w[k][c][r0 + sh*t][s0 + sw*u].
 __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__ w, float *__restrict__ apk, int mode,
@@ -293,7 +428,11 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
-void launch_tap(dim3 grid, hipStream_t st, const TapParams &p) {
+void launch_tap(dim3 grid, hipStream_t st, const TapParams &p, int bf16) {
+    if (bf16) {
+        hipLaunchKernelGGL(tap_igemm_bf16_kernel<3>, grid, dim3(256), 0, st, p);
+        return;
+    }
     static int stages = -1;
     if (stages < 0) {
         const char *e = getenv("XSMI_TAP_STAGES");
@@ -340,7 +479,7 @@ size_t tap_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
 }
 
 int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
-                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, void *workspace) {
+                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int bf16, void *workspace) {
     hipStream_t st = stream();
     float *apk = (float *)workspace;
     int rc = launch_pack(st, w, apk, 0, K, C, R, S, R, S, 0, 0, 1, 1);
@@ -358,14 +497,14 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     dim3 grid(ceil_div(p.M, BP), ceil_div(K, TM));
     prof_begin();
     p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
-    launch_tap(grid, st, p);
+    launch_tap(grid, st, p, bf16);
     prof_end();
-    XSMI_LAUNCH_CHECK("tap_igemm_f32_kernel");
+    XSMI_LAUNCH_CHECK("tap_igemm kernel");
     return XSMI_OK;
 }
 
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
-                      int sw, int pad, int OH, int OW, int accumulate, void *workspace) {
+                      int sw, int pad, int OH, int OW, int accumulate, int bf16, void *workspace) {
     hipStream_t st = stream();
     char *ws = (char *)workspace;
     struct Plan { TapParams p; dim3 grid; };
@@ -406,8 +545,8 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
     }
     prof_begin();
     for (int i = 0; i < nplans; ++i) {
-        launch_tap(plans[i].grid, st, plans[i].p);
-        XSMI_LAUNCH_CHECK("tap_igemm_f32_kernel");
+        launch_tap(plans[i].grid, st, plans[i].p, bf16);
+        XSMI_LAUNCH_CHECK("tap_igemm kernel");
     }
     prof_end();
     return XSMI_OK;

@@ -76,22 +76,24 @@ def conv2d(inputs, weight, bias=None, stride=(1, 1), padding=0, out=None, activa
     requires_grad = bool(inputs.requires_grad or weight.requires_grad or (bias is not None and bias.requires_grad))
     track = GLOBAL.COMPUTE_GRAD and requires_grad
     neg_mask = dev.empty((n, k, oh, ow), np.uint8) if (activation == 'relu' and track) else None
+    bf16 = bool(GLOBAL.CONV_BF16)
 
     if out is None:
-        y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask)
+        y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16)
         out = Tensor(y_dev if on_device else y_dev.numpy().astype(x.dtype, copy=False))
     else:
         dst = out.eval
         if is_device(dst):
-            K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask)
+            K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask, bf16=bf16)
         else:
-            y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask)
+            y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16)
             out.eval = y_dev.numpy()              # cast to the buffer's dtype on store
     out.requires_grad = requires_grad
     _wire(out, inputs, weight, bias)
     if track:
         out.cache['x'] = x_dev                    # the reference keeps the unfolded matrix 'col' here
         out.cache['stride'] = stride
+        out.cache['bf16'] = bf16
         out.cache['padding'] = padding
         if neg_mask is not None:
             out.cache['neg_mask'] = neg_mask

@@ -49,6 +49,7 @@ def Conv2DBackward(outputs):
     """
     inputs, weight, bias = outputs.in_bounds
     stride, pad = outputs.cache['stride'], outputs.cache['padding']
+    bf16 = bool(outputs.cache.get('bf16', False))
     x_dev = outputs.cache['x']                      # device copy of the forward input (stands in for 'col')
     dy = _f32_device(outputs.grad.eval)
     neg_mask = outputs.cache.get('neg_mask')
@@ -72,9 +73,9 @@ def Conv2DBackward(outputs):
     if inputs.requires_grad:
         dx_buf = inputs.grad.eval
         if is_device(dx_buf):
-            K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, dx=dx_buf, accumulate=True)
+            K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, dx=dx_buf, accumulate=True, bf16=bf16)
         else:
-            _accumulate(inputs, K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad))
+            _accumulate(inputs, K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, bf16=bf16))
 
 
 def Maxpool2DBackward(outputs):
