@@ -180,6 +180,47 @@ def bench_resnet18(be, steps, warmup):
             "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
 
 
+def bench_resnet18_infer(be, steps, warmup):
+    """ResNet-18 N=256 forward only, moving-statistics BN, convolutions allowed to use bf16 MFMA operands; the fp32
+    forward of the same weights and input runs beside it and gives the logits' relative L2 distance."""
+    import xshinnosuke_amd as xs
+    from xshinnosuke_amd.utils.resnet import ResNet18
+    xs.GLOBAL.INPUTS = None
+    X = np.random.default_rng(7).standard_normal((256, 3, 224, 224), dtype=np.float32)
+    x = xs.tensor(X).to('cuda')
+    net = ResNet18(classes=1000, pool=7).to('cuda')
+    out = {}
+    xs.GLOBAL.TRAINING = False
+    try:
+        with xs.no_grad():
+            logits = {}
+            for mode in ("fp32", "bf16"):
+                with xs.conv_precision(mode):
+                    for _ in range(warmup):
+                        y = net(x)
+                    be.synchronize()
+                    e0, e1 = be.Event(), be.Event()
+                    e0.record()
+                    for _ in range(steps):
+                        y = net(x)
+                    e1.record()
+                    ms = e0.elapsed_ms(e1)
+                    be.synchronize()
+                    logits[mode] = y.numpy().astype(np.float64)
+                    out["resnet18_infer_%s_images_per_sec" % mode] = 256 * steps / (ms * 1e-3)
+                    out["resnet18_infer_%s_ms_per_batch" % mode] = ms / steps
+    finally:
+        xs.GLOBAL.TRAINING = True
+        xs.GLOBAL.USE_CUDA = False
+        xs.GLOBAL.INPUTS = None
+    d = logits["bf16"] - logits["fp32"]
+    out["resnet18_infer_bf16_logits_rel_l2_vs_fp32"] = float(np.linalg.norm(d) / np.linalg.norm(logits["fp32"]))
+    out["resnet18_infer_workload"] = ("N=256x3x224x224, forward only, moving-statistics BN (fresh: mean 0, var 1), "
+                                      "fp32 tensors in HBM; bf16 = conv operands rounded to bf16 in registers, fp32 accumulate; "
+                                      "the 3-channel stem stays on the fp32 kernel")
+    return out
+
+
 def cpu_baseline():
     """Oracle (NumPy restatement of the reference algorithm) on the host cores, same workload."""
     import oracle
@@ -249,6 +290,9 @@ def main():
     if not args.no_extra:
         out["extra"] = bench_pool(be, max(args.steps, 20), args.warmup)
         out["extra"].update(bench_resnet18(be, max(5, args.steps // 5), 3))
+        be.release_cached_memory()
+        out["extra"].update(bench_resnet18_infer(be, 3, 1))
+        be.release_cached_memory()
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline()
     else:

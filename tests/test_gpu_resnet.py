@@ -98,3 +98,82 @@ def test_resnet18_trains_on_device():
         opt.step()
         losses.append(loss.item())
     assert np.isfinite(losses).all() and losses[-1] < losses[0]
+
+
+def _oracle_forward(net, x):
+    """ResNet-18 inference (moving-statistics batch norm) in NumPy: convolutions and the max-pool through the
+    oracle (float64 GEMM, one rounding), the rest in float64 rounded to float32 per op."""
+    import oracle
+
+    def bn(layer, a):
+        g, b = (p.numpy().astype(np.float64).reshape(1, -1, 1, 1) for p in layer.parameters())
+        mm = layer.moving_mean.numpy().astype(np.float64).reshape(1, -1, 1, 1)
+        mv = layer.moving_variance.numpy().astype(np.float64).reshape(1, -1, 1, 1)
+        return (g * (a - mm) / np.sqrt(mv + layer.epsilon) + b).astype(np.float32)
+
+    def run(layer, a):
+        name = type(layer).__name__
+        if name == 'Sequential':
+            for sub in layer._graph:
+                a = run(sub, a)
+            return a
+        if name == 'BasicBlock':
+            out = run(layer.conv1, a) + run(layer.shortcut, a)
+            return np.maximum(out, 0)
+        if name == 'Conv2D':
+            w, b = (p.numpy() for p in layer.parameters())
+            return oracle.conv2d_fwd(a, w.astype(np.float32), b.reshape(-1).astype(np.float32), layer.stride, layer.pad_size)[0]
+        if name == 'BatchNormalization':
+            return bn(layer, a)
+        if name == 'ReLU':
+            return np.maximum(a, 0)
+        raise AssertionError(name)
+
+    a = run(net.conv1, x)
+    a = oracle.max_pool2d_fwd(a, 3, (2, 2), 1)[0]
+    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
+        a = run(stage, a)
+    k = net.pool2.kernel_size
+    n, c, h, w = a.shape
+    a = a.astype(np.float64).reshape(n, c, h // k, k, w // k, k).mean(axis=(3, 5)).astype(np.float32)
+    wfc, bfc = (p.numpy().astype(np.float64) for p in net.fc.parameters())
+    return (a.reshape(n, -1).astype(np.float64) @ wfc + bfc).astype(np.float32)
+
+
+def test_resnet18_bf16_inference_against_oracle():
+    """Inference configuration: moving-statistics batch norm, forward only, convolutions allowed to use bf16
+    MFMA operands.  Logits against the NumPy/oracle forward: rel-L2 <= 1e-2 for bf16, <= 1e-4 for fp32."""
+    np.random.seed(7)
+    X = np.random.randn(4, 3, 64, 64).astype(np.float32)
+    net = ResNet18(classes=10, pool=2).to('cuda')
+    xd = xs.tensor(X).to('cuda')
+    net(xd)                                        # creates the parameters
+    xs.GLOBAL.INPUTS = None
+    # moving statistics that are not the identity, so the inference formula is exercised
+    rng = np.random.default_rng(3)
+
+    def walk(layer):
+        if type(layer).__name__ == 'BatchNormalization':
+            layer.moving_mean.eval = (0.1 * rng.standard_normal(layer.moving_mean.shape)).astype(np.float32)
+            layer.moving_variance.eval = rng.uniform(0.5, 1.5, layer.moving_variance.shape).astype(np.float32)
+        for sub in getattr(layer, '_graph', []):
+            walk(sub)
+        for attr in ('conv1', 'shortcut'):
+            if hasattr(layer, attr) and type(layer).__name__ == 'BasicBlock':
+                walk(getattr(layer, attr))
+    walk(net.conv1)
+    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
+        walk(stage)
+    ref = _oracle_forward(net, X)
+    xs.GLOBAL.TRAINING = False
+    try:
+        with xs.no_grad():
+            y32 = net(xs.tensor(X).to('cuda')).numpy()
+            xs.GLOBAL.INPUTS = None
+            with xs.conv_precision('bf16'):
+                y16 = net(xs.tensor(X).to('cuda')).numpy()
+    finally:
+        xs.GLOBAL.TRAINING = True
+    assert rel_l2(y32, ref) <= 1e-4
+    assert rel_l2(y16, ref) <= 1e-2
+    assert rel_l2(y16, y32) > 1e-5                 # the bf16 kernels really ran
