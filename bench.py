@@ -221,6 +221,29 @@ def bench_resnet18_infer(be, steps, warmup):
     return out
 
 
+def traffic_run(be, reps=3):
+    """A short fixed sequence for hardware-counter runs (one counter set per profiler run): the conv workload's three
+    kernels, the max-pool pair, and the plain copy kernel of known size that calibrates the byte counters."""
+    K = be.kernels
+    c, p = CONV, POOL
+    x, w, b, dy = make_conv_inputs(c)
+    dx_, dw_, db_, ddy = be.to_device(x), be.to_device(w), be.to_device(b), be.to_device(dy)
+    y = be.empty(dy.shape); gx = be.empty(x.shape); gw = be.empty(w.shape); gb = be.empty(b.shape)
+    px = be.to_device(np.random.default_rng(4).standard_normal((p["N"], p["C"], p["H"], p["W"]), dtype=np.float32))
+    pdy = be.to_device(np.random.default_rng(5).standard_normal((p["N"], p["C"], p["H"] // 2, p["W"] // 2), dtype=np.float32))
+    py = be.empty(pdy.shape); pidx = be.empty(pdy.shape, np.uint8); pgx = be.empty(px.shape)
+    src = be.empty((px.size + pdy.size + pdy.size // 4,)); dst = be.empty(src.shape)
+    for _ in range(reps):
+        K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y)
+        K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx)
+        K.conv2d_bwd_weight(ddy, dx_, w.shape, c["stride"], c["pad"], dw=gw, db=gb)
+        K.maxpool2d_fwd(px, p["k"], p["stride"], p["pad"], out=py, idx=pidx)
+        K.maxpool2d_bwd(pdy, pidx, px.shape, p["k"], p["stride"], p["pad"], dx=pgx)
+        K.copy_kernel(dst, src)
+        be.synchronize()
+    return {"traffic_run": reps, "copy_kernel_bytes_each_way": src.nbytes}
+
+
 def cpu_baseline():
     """Oracle (NumPy restatement of the reference algorithm) on the host cores, same workload."""
     import oracle
@@ -254,6 +277,8 @@ def main():
     ap.add_argument("--steps", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-side NumPy baseline")
+    ap.add_argument("--traffic-run", action="store_true",
+                    help="run a short fixed kernel sequence (conv, max-pool, calibration copy) for counter collection and exit")
     ap.add_argument("--no-extra", action="store_true", help="skip the max-pool / copy measurements")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -263,6 +288,9 @@ def main():
     from xshinnosuke_amd import backend as be
     be.init(0)
     info = be.device_info()
+    if args.traffic_run:
+        print(json.dumps(traffic_run(be)))
+        return
 
     ms_step, wall_ms_step, per = bench_conv(be, args.steps, args.warmup)
     flops_pass = conv_flops(CONV)

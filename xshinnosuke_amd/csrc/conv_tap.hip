@@ -69,8 +69,11 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int m0 = blockIdx.x * BP;
-    const int rowtile = blockIdx.y;
+    // logical block = (pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
+    // tiles of one pixel tile and neighbouring pixel tiles (shared halo) meet in one L2
+    const uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+    const int rowtile = gridDim.y == 1 ? 0 : (int)(logical % gridDim.y);
+    const int m0 = (int)(gridDim.y == 1 ? logical : logical / gridDim.y) * BP;
 
     // ---- gather role: pixel m0 + lane, channels 8*wave .. 8*wave+7 of each chunk ----
     int iyb = 0, ixb = 0, nbase = 0;
@@ -281,8 +284,11 @@ __global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapParams p) {
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    const int m0 = blockIdx.x * BP;
-    const int rowtile = blockIdx.y;
+    // logical block = (pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
+    // tiles of one pixel tile and neighbouring pixel tiles (shared halo) meet in one L2
+    const uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
+    const int rowtile = gridDim.y == 1 ? 0 : (int)(logical % gridDim.y);
+    const int m0 = (int)(gridDim.y == 1 ? logical : logical / gridDim.y) * BP;
 
     int iyb = 0, ixb = 0, nbase = 0;
     const bool live = m0 + lane < p.M;

@@ -59,12 +59,18 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
     const int h = lane >> 5, l31 = lane & 31;
     const int wr = wave >> 1, wc = wave & 1;
 
-    const int tapidx = (int)xsmi::fdiv(blockIdx.x, p.dCT);
-    const int ctile = (int)blockIdx.x - tapidx * p.ctiles;
+    // logical block = (split, k tile, tap, c tile) with the tap fastest: the R*S blocks that read the
+    // same dy and x pixels are neighbours in logical order and run on one XCD
+    const uint32_t nbx = gridDim.x, nby = gridDim.y;
+    const uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x + nbx * (blockIdx.y + nby * blockIdx.z), nbx * nby * gridDim.z);
+    const uint32_t lz = logical / (nbx * nby), lxy = logical - lz * (nbx * nby);
+    const uint32_t ly = lxy / nbx, lx = lxy - ly * nbx;
+    const int tapidx = (int)xsmi::fdiv(lx, p.dCT);
+    const int ctile = (int)lx - tapidx * p.ctiles;
     const int tr = (int)xsmi::fdiv((uint32_t)tapidx, p.dS);
     const int ts = tapidx - tr * p.S;
-    const int c0 = ctile * TC, k0 = blockIdx.y * TK;
-    const int split = blockIdx.z;
+    const int c0 = ctile * TC, k0 = (int)ly * TK;
+    const int split = (int)lz;
     const int chunk_begin = split * p.cps;
     int nchunks = p.total_chunks - chunk_begin;
     if (nchunks > p.cps) nchunks = p.cps;
@@ -136,7 +142,7 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
         a_rd[g] = (f_arow * 8 + ((4 * h + g) ^ (f_arow & 7))) * 4;
         b_rd[g] = 2048 + (f_bch * 8 + ((4 * h + g) ^ (f_bch & 7))) * 4;
     }
-    const bool want_db = p.dbpart != nullptr && blockIdx.x == 0 && wc == 0;
+    const bool want_db = p.dbpart != nullptr && lx == 0 && wc == 0;
     float dbacc = 0.f;
 
     floatx16 acc = {0}, acc2 = {0};

@@ -74,6 +74,15 @@ __device__ __forceinline__ uint32_t fdiv(uint32_t n, const FastDiv &f) {
     return (__umulhi(n, f.mul) + n) >> f.shift;
 }
 
+// Workgroups are handed to the 8 XCDs round-robin by linear workgroup id, and each XCD
+// has its own L2.  This maps the launch's linear id to a logical id such that every XCD
+// works on one contiguous range of logical ids: neighbours in logical order, which share
+// operand tiles, then share an L2.  Bijective on [0, total) for any total.
+__device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t lin, uint32_t total) {
+    const uint32_t q = total >> 3, rem = total & 7u, xcd = lin & 7u, slot = lin >> 3;
+    return xcd * q + (xcd < rem ? xcd : rem) + slot;
+}
+
 // tap-major fast path (conv_tap.hip): reduction channels must be a multiple of 32
 bool tap_path_ok(int reduce_channels);
 size_t tap_fwd_ws_bytes(int C, int K, int R, int S);
