@@ -244,3 +244,30 @@ def test_conv2d_rejects_what_the_reference_rejects():
         F.conv2d(x, xs.tensor(np.zeros((2, 3, 3, 3), dtype=np.float32)), padding=(1, 1))
     with pytest.raises(ValueError):
         F.max_pool2d(x, (2, 3))
+
+
+def test_pending_zero_gradient_buffers(gpu):
+    """Gradient buffers are cleared lazily: they read as zero, an op that overwrites all of one skips the
+    clear, and accumulation into a used buffer still adds."""
+    z = gpu.zeros((4, 8), lazy=True)
+    assert z.is_fresh()
+    np.testing.assert_array_equal(z.numpy(), np.zeros((4, 8), np.float32))      # reading clears it for real
+    assert not z.is_fresh()
+    z = gpu.zeros((4, 8), lazy=True)
+    view = z.leading(1, 3)                                                      # part of the allocation
+    assert not view.take_fresh()
+    np.testing.assert_array_equal(z.numpy(), np.zeros((4, 8), np.float32))
+    K = gpu.kernels
+    g = gpu.to_device(np.arange(32, dtype=np.float32).reshape(4, 8))
+    acc = gpu.zeros((4, 8), lazy=True)
+    K.axpy(acc, g, 1.0)                                                          # fresh: becomes a copy
+    K.axpy(acc, g, 0.5)                                                          # used: adds
+    np.testing.assert_array_equal(acc.numpy(), 1.5 * g.numpy())
+    # conv weight gradient: dw pending, db already used -> both must end up accumulated correctly
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((2, 3, 6, 6)).astype(np.float32); dy = rng.standard_normal((2, 4, 4, 4)).astype(np.float32)
+    dw = gpu.zeros((4, 3, 3, 3), lazy=True); db = gpu.to_device(np.ones(4, np.float32))
+    K.conv2d_bwd_weight(gpu.to_device(dy), gpu.to_device(x), (4, 3, 3, 3), (1, 1), 0, dw=dw, db=db, accumulate=True)
+    dw_ref, db_ref = K.conv2d_bwd_weight(gpu.to_device(dy), gpu.to_device(x), (4, 3, 3, 3), (1, 1), 0, want_db=True)
+    np.testing.assert_allclose(dw.numpy(), dw_ref.numpy(), rtol=1e-6, atol=1e-6)
+    np.testing.assert_allclose(db.numpy(), db_ref.numpy() + 1.0, rtol=1e-6, atol=1e-6)

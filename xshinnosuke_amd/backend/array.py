@@ -33,10 +33,12 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero")
 
     def __init__(self, nbytes):
         ensure_init()
+        self.logical = int(nbytes)
+        self.lazy_zero = False
         size = _round_size(nbytes)
         free = _POOL.get(size)
         if free:
@@ -78,12 +80,37 @@ class DeviceArray:
         self.dtype = np.dtype(dtype)
         self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
         self.nbytes = self.size * self.dtype.itemsize
-        self._block = _block if _block is not None else _Block(max(self.nbytes, 16))
+        if _block is None:
+            _block = _Block(max(self.nbytes, 16))
+            _block.logical = self.nbytes
+        self._block = _block
         self._offset = int(_offset)
 
     @property
     def ptr(self):
-        return self._block.ptr + self._offset
+        blk = self._block
+        if blk.lazy_zero:                    # logically zero, memory not cleared yet: clear it on first use
+            blk.lazy_zero = False
+            lib.call("xsmi_memset", ctypes.c_void_p(blk.ptr), 0, blk.nbytes)
+        return blk.ptr + self._offset
+
+    def is_fresh(self):
+        """True if the array is a whole allocation whose clear is still pending."""
+        blk = self._block
+        return blk.lazy_zero and self._offset == 0 and self.nbytes >= blk.logical
+
+    def take_fresh(self):
+        """True if this array is a pending all-zero buffer that the caller will now overwrite completely
+        (the pending clear is dropped).  An array that covers only part of its allocation is cleared
+        for real instead and reports False."""
+        blk = self._block
+        if not blk.lazy_zero:
+            return False
+        if self._offset == 0 and self.nbytes >= blk.logical:
+            blk.lazy_zero = False
+            return True
+        self.ptr                              # materialise the zeros
+        return False
 
     @property
     def cptr(self):
@@ -107,6 +134,7 @@ class DeviceArray:
         host = np.ascontiguousarray(host, dtype=self.dtype)
         if host.shape != self.shape:
             host = np.ascontiguousarray(np.broadcast_to(host, self.shape))
+        self.take_fresh()                     # everything is overwritten: a pending clear is moot
         if self.nbytes:
             lib.call("xsmi_memcpy_h2d", self.cptr, host.ctypes.data_as(ctypes.c_void_p), self.nbytes)
         return self
@@ -114,6 +142,7 @@ class DeviceArray:
     def copy_from(self, other):
         if other.nbytes != self.nbytes:
             raise ValueError("size mismatch in device copy: %s vs %s" % (other.shape, self.shape))
+        self.take_fresh()
         if self.nbytes:
             lib.call("xsmi_memcpy_d2d", self.cptr, other.cptr, self.nbytes)
         return self
@@ -121,7 +150,13 @@ class DeviceArray:
     def copy(self):
         return DeviceArray(self.shape, self.dtype).copy_from(self)
 
-    def fill_zero(self):
+    def fill_zero(self, lazy=False):
+        """Clear the array.  ``lazy=True`` only marks a whole allocation as zero: the memset happens on
+        the first ordinary use, and not at all if the first use overwrites everything (take_fresh)."""
+        blk = self._block
+        if lazy and self._offset == 0 and self.nbytes >= blk.logical:
+            blk.lazy_zero = True
+            return self
         if self.nbytes:
             lib.call("xsmi_memset", self.cptr, 0, self.nbytes)
         return self
@@ -159,8 +194,8 @@ def empty(shape, dtype=np.float32):
     return DeviceArray(shape, dtype)
 
 
-def zeros(shape, dtype=np.float32):
-    return DeviceArray(shape, dtype).fill_zero()
+def zeros(shape, dtype=np.float32, lazy=False):
+    return DeviceArray(shape, dtype).fill_zero(lazy)
 
 
 def to_device(host, dtype=None):

@@ -63,6 +63,18 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
     return out
 
 
+def _beta(accumulate, *outs):
+    """1.0 to add into the outputs, 0.0 to overwrite them.  Outputs that are all pending all-zero
+    buffers are overwritten instead of cleared and added to; in a mix the pending ones are cleared
+    for real when their pointer is taken."""
+    outs = [o for o in outs if o is not None]
+    if accumulate and not all(o.is_fresh() for o in outs):
+        return 1.0
+    for o in outs:
+        o.take_fresh()
+    return 0.0
+
+
 def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=False, bf16=False):
     _f32(dy, "dy"); _f32(w, "w")
     dims = _dims(x_shape, w.shape, stride, pad)
@@ -76,7 +88,8 @@ def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=Fa
     elif dx.shape != tuple(x_shape):
         raise ValueError("conv2d backward: dx has shape %s, expected %s" % (dx.shape, tuple(x_shape)))
     ws, ws_bytes = _workspace(dims)
-    lib.call("xsmi_conv2d_bwd_data", dy.cptr, w.cptr, dx.cptr, *dims, 1.0 if accumulate else 0.0,
+    beta = _beta(accumulate, dx)
+    lib.call("xsmi_conv2d_bwd_data", dy.cptr, w.cptr, dx.cptr, *dims, beta,
              CONV_BF16 if bf16 else 0, ws, ws_bytes)
     return dx
 
@@ -99,8 +112,9 @@ def conv2d_bwd_weight(dy, x, w_shape, stride=(1, 1), pad=0, dw=None, db=None, ac
     if db is not None and db.size != k:
         raise ValueError("conv2d backward: db has %d elements for %d filters" % (db.size, k))
     ws, ws_bytes = _workspace(dims)
+    beta = _beta(accumulate, dw, db)
     lib.call("xsmi_conv2d_bwd_weight", dy.cptr, x.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
-             1.0 if accumulate else 0.0, CONV_BF16 if bf16 else 0, ws, ws_bytes)
+             beta, CONV_BF16 if bf16 else 0, ws, ws_bytes)
     return dw, db
 
 
@@ -138,8 +152,9 @@ def maxpool2d_bwd(dy, idx, x_shape, k, stride, pad=0, dx=None, accumulate=False)
         accumulate = False
     elif dx.shape != tuple(x_shape):
         raise ValueError("max_pool2d backward: dx has shape %s, expected %s" % (dx.shape, tuple(x_shape)))
+    beta = _beta(accumulate, dx)
     lib.call("xsmi_maxpool2d_bwd", dy.cptr, idx.cptr, dx.cptr, n, c, h, w, int(k), int(stride[0]), int(stride[1]),
-             int(pad), 1.0 if accumulate else 0.0)
+             int(pad), beta)
     return dx
 
 
@@ -148,7 +163,8 @@ def relu_mask_bwd(dy, neg_mask, dx=None, accumulate=False):
     if dx is None:
         dx = empty(dy.shape)
         accumulate = False
-    lib.call("xsmi_relu_mask_bwd", dy.cptr, neg_mask.cptr, dx.cptr, dy.size, 1.0 if accumulate else 0.0)
+    beta = 0.0 if dx is dy else _beta(accumulate, dx)
+    lib.call("xsmi_relu_mask_bwd", dy.cptr, neg_mask.cptr, dx.cptr, dy.size, beta)
     return dx
 
 
@@ -170,6 +186,11 @@ def axpy(y, x, a):
     _f32(y, "y"); _f32(x, "x")
     if x.size != y.size:
         raise ValueError("axpy: %s vs %s" % (x.shape, y.shape))
+    if y.take_fresh():                        # y is a pending all-zero buffer: y = a * x, no clear, no read of y
+        if float(a) == 1.0:
+            return y.copy_from(x)
+        lib.call("xsmi_scale_shift", x.cptr, y.cptr, float(a), 0.0, y.size)
+        return y
     lib.call("xsmi_axpy", y.cptr, x.cptr, float(a), y.size)
     return y
 
@@ -247,9 +268,16 @@ def bn_infer(x, gamma, beta, mean, var, eps):
     return y
 
 
-def bn_bwd(dy, xhat, sqrtvar, gamma):
+def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None):
+    """dx, dgamma, dbeta; buffers passed in are overwritten completely."""
     n, c, hw = _nchw3(dy.shape)
-    dx = empty(dy.shape); dgamma = empty((c,)); dbeta = empty((c,))
+    dx = empty(dy.shape) if dx is None else dx
+    dgamma = empty((c,)) if dgamma is None else dgamma
+    dbeta = empty((c,)) if dbeta is None else dbeta
+    if dx.size != dy.size or dgamma.size != c or dbeta.size != c:
+        raise ValueError("bn_bwd: output buffers do not match %s" % (dy.shape,))
+    for o in (dx, dgamma, dbeta):
+        o.take_fresh()
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
     lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, sqrtvar.cptr, gamma.cptr, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw,
              ws, ws_bytes)

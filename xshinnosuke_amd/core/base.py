@@ -288,7 +288,7 @@ class Tensor(object):
 
     def zero_(self):
         if is_device(self._data):
-            self._data.fill_zero()
+            self._data.fill_zero(lazy=True)
         else:
             self._data = np.zeros_like(self._data)
 
@@ -303,7 +303,7 @@ class Tensor(object):
         (reference xs/core/base.py:312-316)."""
         if self._grad is None:
             if is_device(self._data):
-                self._grad = Tensor(_dev.zeros(self.shape, self._data.dtype))
+                self._grad = Tensor(_dev.zeros(self.shape, self._data.dtype, lazy=True))
             else:
                 self._grad = Tensor(np.zeros(self.shape, dtype=self._data.dtype))
         else:

@@ -138,15 +138,27 @@ __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict
                                                           double *__restrict__ part, int N, int C, int HW) {
     __shared__ double sm[4];
     const int c = blockIdx.x, sp = blockIdx.y;
-    const size_t per = (size_t)N * HW;
     double s0 = 0.0, s1 = 0.0;
-    for (size_t i = (size_t)sp * 256 + threadIdx.x; i < per; i += (size_t)BN_SPLIT * 256) {
-        size_t n = i / HW, r = i - n * HW;
-        size_t off = (n * C + c) * (size_t)HW + r;
-        float u = a[off];
-        float v = b ? b[off] : u;
-        s0 += (double)u;
-        s1 += (double)u * (double)v;
+    const int hw4 = (HW & 3) == 0 ? HW >> 2 : 0;       // planes are 16-byte aligned when HW % 4 == 0
+    for (int n = sp; n < N; n += BN_SPLIT) {           // fixed assignment of images to splits: deterministic sums
+        const size_t base = ((size_t)n * C + c) * (size_t)HW;
+        if (hw4) {
+            const float4 *pa = reinterpret_cast<const float4 *>(a + base);
+            const float4 *pb = b ? reinterpret_cast<const float4 *>(b + base) : pa;
+            for (int i = threadIdx.x; i < hw4; i += 256) {
+                const float4 u = pa[i], v = pb[i];
+                s0 += ((double)u.x + (double)u.y) + ((double)u.z + (double)u.w);
+                s1 += ((double)u.x * (double)v.x + (double)u.y * (double)v.y) +
+                      ((double)u.z * (double)v.z + (double)u.w * (double)v.w);
+            }
+        } else {
+            for (int i = threadIdx.x; i < HW; i += 256) {
+                const float u = a[base + i];
+                const float v = b ? b[base + i] : u;
+                s0 += (double)u;
+                s1 += (double)u * (double)v;
+            }
+        }
     }
     s0 = block_sum(s0, sm);
     s1 = block_sum(s1, sm);

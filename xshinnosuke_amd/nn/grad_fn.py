@@ -218,16 +218,33 @@ def Avgpool2DBackward(outputs):
         _accumulate(inputs, A.avg_pool_blocks_grad(outputs.grad.eval, inputs.shape, outputs.cache['kernel_size']))
 
 
+def _fresh_grad(t):
+    """The gradient buffer of ``t`` if it is a device array still pending its clear, so that a kernel may
+    write its result straight into it; None otherwise (the result then goes through _accumulate)."""
+    if t is None or not t.requires_grad or t.grad is None:
+        return None
+    g = t.grad.eval
+    return g if is_device(g) and g.take_fresh() else None
+
+
 def BatchNormBackward(outputs):
     """Reference xs/nn/grad_fn.py:379-411."""
     inputs, gamma, beta = outputs.in_bounds
-    dx, dgamma, dbeta = A.batch_norm_backward(outputs.grad.eval, outputs.cache['normalized_x'],
-                                              outputs.cache['sqrtvar'], gamma.eval)
-    if gamma.requires_grad:
+    dy = outputs.grad.eval
+    if is_device(dy):
+        out_dx, out_dg, out_db = _fresh_grad(inputs), _fresh_grad(gamma), _fresh_grad(beta)
+        gam = A.same_place(dy, gamma.eval)
+        dx, dgamma, dbeta = K.bn_bwd(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gam,
+                                     dx=out_dx, dgamma=None if out_dg is None else out_dg.reshape(-1),
+                                     dbeta=None if out_db is None else out_db.reshape(-1))
+    else:
+        out_dx = out_dg = out_db = None
+        dx, dgamma, dbeta = A.batch_norm_backward(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gamma.eval)
+    if gamma.requires_grad and out_dg is None:
         _accumulate(gamma, dgamma)
-    if beta.requires_grad:
+    if beta.requires_grad and out_db is None:
         _accumulate(beta, dbeta)
-    if inputs.requires_grad:
+    if inputs.requires_grad and out_dx is None:
         _accumulate(inputs, dx)
 
 
