@@ -243,18 +243,32 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
 
 // dw[k][c][tap] = beta*dw + sum over splits (ascending, float64) of part[split][tap][k][c].
 // 256 threads = 64 consecutive c x 4 interleaved split groups, combined in group order.
+// Blocks past the last dw block reduce the bias partials the same way (64 filters each), so
+// that db costs no launch of its own: db[k] = beta*db + sum over splits of dbpart[split][k].
 __global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__restrict__ part, float *__restrict__ dw,
-                                                                int K, int C, int taps, int splits, int accumulate) {
+                                                                const float *__restrict__ dbpart, float *__restrict__ db,
+                                                                int K, int C, int taps, int splits, int dw_blocks,
+                                                                int accumulate) {
     __shared__ double sm[4][64];
     const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int ctiles = C / 64;
     int b = blockIdx.x;
-    const int ct = b % ctiles; b /= ctiles;
-    const int k = b % K;
-    const int tap = b / K;
-    const int c = ct * 64 + cl;
-    const size_t stride = (size_t)taps * K * C;
-    const float *src = part + ((size_t)tap * K + k) * C + c;
+    const bool bias_block = b >= dw_blocks;               // uniform per block
+    const float *src;
+    size_t stride, o;
+    float *dst;
+    if (bias_block) {
+        const int k = (b - dw_blocks) * 64 + cl;
+        src = dbpart + k; stride = (size_t)K; dst = db; o = (size_t)k;
+    } else {
+        const int ctiles = C / 64;
+        const int ct = b % ctiles; b /= ctiles;
+        const int k = b % K;
+        const int tap = b / K;
+        const int c = ct * 64 + cl;
+        stride = (size_t)taps * K * C;
+        src = part + ((size_t)tap * K + k) * C + c;
+        dst = dw; o = ((size_t)k * C + c) * taps + tap;
+    }
     double s0 = 0.0, s1 = 0.0;
     int sp = g;
     for (; sp + 4 < splits; sp += 8) {
@@ -266,25 +280,8 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__re
     __syncthreads();
     if (g == 0) {
         double s = ((sm[0][cl] + sm[1][cl]) + sm[2][cl]) + sm[3][cl];
-        const size_t o = ((size_t)k * C + c) * taps + tap;
-        if (accumulate) s += (double)dw[o];
-        dw[o] = (float)s;
-    }
-}
-
-__global__ void __launch_bounds__(256) dbias_tap_reduce_kernel(const float *__restrict__ dbpart, float *__restrict__ db,
-                                                                int K, int splits, int accumulate) {
-    __shared__ double sm[4][64];
-    const int kl = threadIdx.x & 63, g = threadIdx.x >> 6;
-    const int k = blockIdx.x * 64 + kl;
-    double s0 = 0.0;
-    for (int sp = g; sp < splits; sp += 4) s0 += (double)dbpart[(size_t)sp * K + k];
-    sm[g][kl] = s0;
-    __syncthreads();
-    if (g == 0) {
-        double s = ((sm[0][kl] + sm[1][kl]) + sm[2][kl]) + sm[3][kl];
-        if (accumulate) s += (double)db[k];
-        db[k] = (float)s;
+        if (accumulate) s += (double)dst[o];
+        dst[o] = (float)s;
     }
 }
 
@@ -337,13 +334,10 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     hipLaunchKernelGGL(wgrad_tap_f32_kernel, grid, dim3(256), 0, st, p);
     prof_end();
     XSMI_LAUNCH_CHECK("wgrad_tap_f32_kernel");
-    hipLaunchKernelGGL(wgrad_tap_reduce_kernel, dim3(R * S * K * p.ctiles), dim3(256), 0, st, p.part, dw, K, C, R * S,
-                       splits, accumulate);
+    const int dw_blocks = R * S * K * p.ctiles;
+    hipLaunchKernelGGL(wgrad_tap_reduce_kernel, dim3(dw_blocks + (db ? K / 64 : 0)), dim3(256), 0, st, p.part, dw, dbpart, db,
+                       K, C, R * S, splits, dw_blocks, accumulate);
     XSMI_LAUNCH_CHECK("wgrad_tap_reduce_kernel");
-    if (db) {
-        hipLaunchKernelGGL(dbias_tap_reduce_kernel, dim3(K / 64), dim3(256), 0, st, dbpart, db, K, splits, accumulate);
-        XSMI_LAUNCH_CHECK("dbias_tap_reduce_kernel");
-    }
     return XSMI_OK;
 }
 
