@@ -135,29 +135,33 @@ inline ChanIdx make_chan(int C, int HW) {
 // ---- batch norm --------------------------------------------------------------
 // pass 1: per (channel, split) partial sums of a and a*b over the N*HW elements of the channel
 __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          double *__restrict__ part, int N, int C, int HW) {
+                                                          double *__restrict__ part, int N, int C, int HW, int nsplit) {
     __shared__ double sm[4];
     const int c = blockIdx.x, sp = blockIdx.y;
     double s0 = 0.0, s1 = 0.0;
-    const int hw4 = (HW & 3) == 0 ? HW >> 2 : 0;       // planes are 16-byte aligned when HW % 4 == 0
-    for (int n = sp; n < N; n += BN_SPLIT) {           // fixed assignment of images to splits: deterministic sums
-        const size_t base = ((size_t)n * C + c) * (size_t)HW;
-        if (hw4) {
-            const float4 *pa = reinterpret_cast<const float4 *>(a + base);
-            const float4 *pb = b ? reinterpret_cast<const float4 *>(b + base) : pa;
-            for (int i = threadIdx.x; i < hw4; i += 256) {
-                const float4 u = pa[i], v = pb[i];
-                s0 += ((double)u.x + (double)u.y) + ((double)u.z + (double)u.w);
-                s1 += ((double)u.x * (double)v.x + (double)u.y * (double)v.y) +
-                      ((double)u.z * (double)v.z + (double)u.w * (double)v.w);
-            }
-        } else {
-            for (int i = threadIdx.x; i < HW; i += 256) {
-                const float u = a[base + i];
-                const float v = b ? b[base + i] : u;
-                s0 += (double)u;
-                s1 += (double)u * (double)v;
-            }
+    // split sp takes images sp, sp + nsplit, ... (a fixed assignment: deterministic sums) and walks
+    // them as one flat range of float4 (planes are 16-byte aligned when HW % 4 == 0) or float units
+    const int nimg = sp < N ? (N - sp + nsplit - 1) / nsplit : 0;
+    if ((HW & 3) == 0) {
+        const uint32_t U = (uint32_t)HW >> 2, total = (uint32_t)nimg * U;
+        for (uint32_t e = threadIdx.x; e < total; e += 256) {
+            const uint32_t j = e / U, i = e - j * U;
+            const size_t base = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW;
+            const float4 u = reinterpret_cast<const float4 *>(a + base)[i];
+            const float4 v = b ? reinterpret_cast<const float4 *>(b + base)[i] : u;
+            s0 += ((double)u.x + (double)u.y) + ((double)u.z + (double)u.w);
+            s1 += ((double)u.x * (double)v.x + (double)u.y * (double)v.y) +
+                  ((double)u.z * (double)v.z + (double)u.w * (double)v.w);
+        }
+    } else {
+        const uint32_t U = (uint32_t)HW, total = (uint32_t)nimg * U;
+        for (uint32_t e = threadIdx.x; e < total; e += 256) {
+            const uint32_t j = e / U, i = e - j * U;
+            const size_t off = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW + i;
+            const float u = a[off];
+            const float v = b ? b[off] : u;
+            s0 += (double)u;
+            s1 += (double)u * (double)v;
         }
     }
     s0 = block_sum(s0, sm);
@@ -167,12 +171,21 @@ __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict
         part[((size_t)c * BN_SPLIT + sp) * 2 + 1] = s1;
     }
 }
+// number of partial reductions per channel: enough work per block (about 1024 load units) to hide latency
+static int bn_splits(int N, int HW) {
+    const long long units = (long long)N * ((HW & 3) == 0 ? HW >> 2 : HW);
+    long long s = units / 1024;
+    if (s < 1) s = 1;
+    if (s > BN_SPLIT) s = BN_SPLIT;
+    if (s > N) s = N;
+    return (int)s;
+}
 __global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar, float *mean, float *var, int C, double m,
-                                float eps) {
+                                float eps, int nsplit) {
     int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     double s0 = 0.0, s1 = 0.0;
-    for (int sp = 0; sp < BN_SPLIT; ++sp) {
+    for (int sp = 0; sp < nsplit; ++sp) {
         s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
         s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
     }
@@ -194,11 +207,11 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__
         y[i] = gamma[c] * h + beta[c];
     }
 }
-__global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgamma, float *dbeta, int C) {
+__global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgamma, float *dbeta, int C, int nsplit) {
     int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     double s0 = 0.0, s1 = 0.0;
-    for (int sp = 0; sp < BN_SPLIT; ++sp) {
+    for (int sp = 0; sp < nsplit; ++sp) {
         s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
         s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
     }
@@ -245,26 +258,40 @@ __global__ void __launch_bounds__(256) avgpool_bwd_kernel(const float *__restric
 }
 
 // ---- small GEMM (dense layer) ----------------------------------------------------
-// 32x32 output tile per 256 threads (each thread 2x2), K in chunks of 32 through LDS.  The dense layer of the
-// networks here is a few tens of MFLOP, far below what would justify an MFMA kernel of its own.
+// 32x32 output tile per 256 threads (each thread 2x2), K in chunks of 128 through LDS: the dense layer's
+// matrices are skinny (a batch of 32 rows), so few workgroups run and each must keep many loads in
+// flight; a chunk is 32 independent loads per thread.  Lanes always run along the contiguous axis of
+// the operand in memory, whichever way it is transposed.  The dense layer of the networks here is a
+// few tens of MFLOP, far below what would justify an MFMA kernel of its own.
+constexpr int GEMM_KC = 128;
 __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                     const float *__restrict__ bias, float *__restrict__ C, int M, int N,
                                                     int K, int ta, int tb) {
-    __shared__ float As[32][33], Bs[32][33];
+    __shared__ float As[32][GEMM_KC + 1], Bs[GEMM_KC][33];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
-    for (int k0 = 0; k0 < K; k0 += 32) {
-        for (int i = threadIdx.x; i < 1024; i += 256) {
-            int r = i >> 5, c = i & 31;
-            int m = m0 + r, kk = k0 + c;
-            As[r][c] = (m < M && kk < K) ? (ta ? A[(size_t)kk * M + m] : A[(size_t)m * K + kk]) : 0.f;
-            int kb = k0 + r, n = n0 + c;
-            Bs[r][c] = (kb < K && n < N) ? (tb ? B[(size_t)n * K + kb] : B[(size_t)kb * N + n]) : 0.f;
+    for (int k0 = 0; k0 < K; k0 += GEMM_KC) {
+#pragma unroll 4
+        for (int i = threadIdx.x; i < 32 * GEMM_KC; i += 256) {
+            if (ta) {                                   // A stored (K, M): lanes along m
+                const int kk = i >> 5, r = i & 31;
+                As[r][kk] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(k0 + kk) * M + m0 + r] : 0.f;
+            } else {                                    // A stored (M, K): lanes along k
+                const int r = i / GEMM_KC, kk = i % GEMM_KC;
+                As[r][kk] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(m0 + r) * K + k0 + kk] : 0.f;
+            }
+            if (tb) {                                   // B stored (N, K): lanes along k
+                const int c = i / GEMM_KC, kk = i % GEMM_KC;
+                Bs[kk][c] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(n0 + c) * K + k0 + kk] : 0.f;
+            } else {                                    // B stored (K, N): lanes along n
+                const int kk = i >> 5, c = i & 31;
+                Bs[kk][c] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(k0 + kk) * N + n0 + c] : 0.f;
+            }
         }
         __syncthreads();
 #pragma unroll 8
-        for (int kk = 0; kk < 32; ++kk) {
+        for (int kk = 0; kk < GEMM_KC; ++kk) {
             float a0 = As[ty * 2][kk], a1 = As[ty * 2 + 1][kk];
             float b0 = Bs[kk][tx * 2], b1 = Bs[kk][tx * 2 + 1];
             acc[0][0] += a0 * b0; acc[0][1] += a0 * b1; acc[1][0] += a1 * b0; acc[1][1] += a1 * b1;
@@ -382,10 +409,11 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, BN_SPLIT), dim3(256), 0, st, x, (const float *)nullptr, part, N, C, HW);
+    const int nsplit = bn_splits(N, HW);
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, x, (const float *)nullptr, part, N, C, HW, nsplit);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
-                       (double)N * HW, eps);
+                       (double)N * HW, eps, nsplit);
     XSMI_LAUNCH_CHECK("bn_stats_kernel");
     size_t total = (size_t)N * C * HW;
     hipLaunchKernelGGL(bn_apply_kernel, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y, xhat,
@@ -426,9 +454,10 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const 
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd: workspace too small");
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, BN_SPLIT), dim3(256), 0, st, dy, xhat, part, N, C, HW);
+    const int nsplit = bn_splits(N, HW);
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, dy, xhat, part, N, C, HW, nsplit);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
-    hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C);
+    hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C, nsplit);
     XSMI_LAUNCH_CHECK("bn_bwd_stats_kernel");
     size_t total = (size_t)N * C * HW;
     hipLaunchKernelGGL(bn_bwd_apply_kernel, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, dx,
