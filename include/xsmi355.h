@@ -65,11 +65,19 @@ int xsmi_malloc(void **ptr, size_t bytes);
 int xsmi_free(void *ptr);
 int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes);   /* blocking */
 int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes);   /* blocking */
+/* Page-locked host memory and an upload from it that only enqueues on the stream: the source must
+ * stay untouched until an event recorded after the call has completed.  They carry the batch
+ * upload of the reference's DataLoader (xs/utils/data/dataloader.py:30-43, one fixed tensor per
+ * loader refilled for every batch) without stalling the host on each copy. */
+int xsmi_host_alloc(void **ptr, size_t bytes);
+int xsmi_host_free(void *ptr);
+int xsmi_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes);   /* async on the stream */
 int xsmi_memset(void *dst, int byte_value, size_t bytes);        /* async on the stream */
 int xsmi_sync(void);
 int xsmi_event_create(void **event);
 int xsmi_event_record(void *event);                               /* on the library stream */
+int xsmi_event_synchronize(void *event);                          /* host waits for the event */
 int xsmi_event_elapsed_ms(void *start, void *stop, float *ms);    /* waits for `stop` */
 int xsmi_event_destroy(void *event);
 /* Per-op device timing: after xsmi_profiling(1) every op records one event

@@ -67,6 +67,15 @@ class _Block:
             pass
 
 
+def _rebuild_array(host):
+    """Unpickling side of DeviceArray.__reduce__: back onto the device when one can be used, else the
+    host array itself (tensors then simply live on the host)."""
+    try:
+        return to_device(host, host.dtype)
+    except Exception:
+        return host
+
+
 class DeviceArray:
     """Dense C-contiguous array in device memory (float32, uint8, int32 or int64).
 
@@ -112,6 +121,10 @@ class DeviceArray:
         self.ptr                              # materialise the zeros
         return False
 
+    def __reduce__(self):
+        # checkpoints hold host arrays (reference xs/nn/models.py:188-202 pickles NumPy arrays)
+        return _rebuild_array, (self.numpy(),)
+
     @property
     def cptr(self):
         return ctypes.c_void_p(self.ptr)
@@ -137,6 +150,19 @@ class DeviceArray:
         self.take_fresh()                     # everything is overwritten: a pending clear is moot
         if self.nbytes:
             lib.call("xsmi_memcpy_h2d", self.cptr, host.ctypes.data_as(ctypes.c_void_p), self.nbytes)
+        return self
+
+    def set_async(self, pinned, count=None):
+        """Enqueue an upload of the first ``count`` leading rows (all by default) of a PinnedArray.  The
+        caller keeps the pinned memory unchanged until an event recorded afterwards has completed."""
+        rows = self.shape[0] if count is None else int(count)
+        if pinned.dtype != self.dtype or pinned.shape[1:] != self.shape[1:] or rows > pinned.shape[0] or rows > self.shape[0]:
+            raise ValueError("set_async: pinned %s %s does not fit device %s %s" % (pinned.shape, pinned.dtype, self.shape, self.dtype))
+        nbytes = (self.nbytes // self.shape[0]) * rows if self.shape[0] else 0
+        if rows == self.shape[0]:
+            self.take_fresh()
+        if nbytes:
+            lib.call("xsmi_memcpy_h2d_async", self.cptr, ctypes.c_void_p(pinned._ptr), nbytes)
         return self
 
     def copy_from(self, other):
@@ -205,6 +231,31 @@ def to_device(host, dtype=None):
     return DeviceArray(host.shape, dtype).set(host)
 
 
+class PinnedArray:
+    """Page-locked host array (``.array`` is a NumPy view of it) for uploads that only enqueue on the
+    stream.  The memory is returned when the object dies."""
+
+    def __init__(self, shape, dtype=np.float32):
+        ensure_init()
+        self.shape = tuple(int(s) for s in shape)
+        self.dtype = np.dtype(dtype)
+        self.nbytes = int(np.prod(self.shape, dtype=np.int64)) * self.dtype.itemsize
+        p = ctypes.c_void_p()
+        lib.call("xsmi_host_alloc", ctypes.byref(p), max(self.nbytes, 16))
+        self._ptr = p.value
+        buf = (ctypes.c_char * max(self.nbytes, 1)).from_address(self._ptr)
+        self.array = np.frombuffer(buf, dtype=self.dtype, count=self.nbytes // self.dtype.itemsize).reshape(self.shape)
+
+    def __del__(self):
+        try:
+            if self._ptr:
+                self.array = None
+                lib.call("xsmi_host_free", ctypes.c_void_p(self._ptr))
+                self._ptr = None
+        except Exception:
+            pass
+
+
 class Workspace:
     """Grow-only scratch buffer handed to the conv entry points."""
 
@@ -227,6 +278,10 @@ class Event:
 
     def record(self):
         lib.call("xsmi_event_record", self._e)
+        return self
+
+    def synchronize(self):
+        lib.call("xsmi_event_synchronize", self._e)
         return self
 
     def elapsed_ms(self, stop):

@@ -43,11 +43,15 @@ SIGNATURES = {
     "xsmi_free": (_i, [_vp]),
     "xsmi_memcpy_h2d": (_i, [_vp, _vp, _sz]),
     "xsmi_memcpy_d2h": (_i, [_vp, _vp, _sz]),
+    "xsmi_host_alloc": (_i, [_c.POINTER(_vp), _sz]),
+    "xsmi_host_free": (_i, [_vp]),
+    "xsmi_memcpy_h2d_async": (_i, [_vp, _vp, _sz]),
     "xsmi_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "xsmi_memset": (_i, [_vp, _i, _sz]),
     "xsmi_sync": (_i, []),
     "xsmi_event_create": (_i, [_c.POINTER(_vp)]),
     "xsmi_event_record": (_i, [_vp]),
+    "xsmi_event_synchronize": (_i, [_vp]),
     "xsmi_event_elapsed_ms": (_i, [_vp, _vp, _c.POINTER(_f)]),
     "xsmi_event_destroy": (_i, [_vp]),
     "xsmi_profiling": (_i, [_i]),

@@ -117,6 +117,30 @@ int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes) {
     return XSMI_OK;
 }
 
+int xsmi_host_alloc(void **ptr, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(ptr != nullptr, "xsmi_host_alloc: null result pointer");
+    *ptr = nullptr;
+    if (bytes == 0) bytes = 16;
+    XSMI_HIP(hipHostMalloc(ptr, bytes, hipHostMallocDefault));
+    return XSMI_OK;
+}
+
+int xsmi_host_free(void *ptr) {
+    XSMI_REQUIRE_INIT();
+    if (ptr == nullptr) return XSMI_OK;
+    XSMI_HIP(hipHostFree(ptr));
+    return XSMI_OK;
+}
+
+int xsmi_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes) {
+    XSMI_REQUIRE_INIT();
+    if (bytes == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dst && pinned_src, "xsmi_memcpy_h2d_async: null pointer");
+    XSMI_HIP(hipMemcpyAsync(dst, pinned_src, bytes, hipMemcpyHostToDevice, g_stream));
+    return XSMI_OK;
+}
+
 int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     XSMI_REQUIRE_INIT();
     if (bytes == 0) return XSMI_OK;
@@ -145,6 +169,13 @@ int xsmi_memset(void *dst, int byte_value, size_t bytes) {
 int xsmi_sync(void) {
     XSMI_REQUIRE_INIT();
     XSMI_HIP(hipStreamSynchronize(g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_event_synchronize(void *event) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(event != nullptr, "xsmi_event_synchronize: null event");
+    XSMI_HIP(hipEventSynchronize((hipEvent_t)event));
     return XSMI_OK;
 }
 

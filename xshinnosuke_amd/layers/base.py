@@ -99,10 +99,16 @@ class Layer:
             self._data = self._new_out_tensor(x)
             self._data.add_in_bounds(x)
             self._data.add_in_bounds(*self.parameters())
-        elif x.shape[0] < self._data.shape_capacity[0]:
-            self._data.slices(slice(None, x.shape[0], None))
         else:
-            self._data.slices(slice(None, None, None))
+            if x.shape[0] < self._data.shape_capacity[0]:
+                self._data.slices(slice(None, x.shape[0], None))
+            else:
+                self._data.slices(slice(None, None, None))
+            # a reused output tensor must read from the tensor that feeds it now: the reference keeps the
+            # tensor it was created with (xs/layers/base.py:88-104), which goes stale as soon as a new
+            # loader hands in different batch tensors (fit after predict, a second fit)
+            if self._data.in_bounds and self._data.in_bounds[0] is not x:
+                self._data.in_bounds[0] = x
 
     def compute_output_shape(self, input_shape=None):
         self._shape = (input_shape,) if isinstance(input_shape, int) else tuple(input_shape)

@@ -5,6 +5,7 @@ path depends on: lazily created parameters, per-layer preallocated output tensor
 shorter last batch (written through ``out=``), ``layer.backward()`` in reverse order for static
 graphs, and parameter discovery by graph walk for ``Module``.
 """
+import pickle
 import time
 
 import numpy as np
@@ -75,7 +76,7 @@ class _Model(_Base):
             split = int(x.shape[0] * validation_split)
             validation_data = (x[-split:], y[-split:])
             x, y = x[:-split], y[:-split]
-        loader = DataLoader(DataSet(x, y), batch_size, shuffle)
+        loader = DataLoader(DataSet(x, y), batch_size, shuffle, device=self._device)
         history = {'train_loss': [], 'train_acc': [], 'validation_loss': [], 'validation_acc': []}
         self.train()
         for epoch in range(initial_epoch, epochs):
@@ -121,7 +122,7 @@ class _Model(_Base):
         x, y = np.asarray(x), np.asarray(y)
         accs, losses = [], []
         with GLOBAL.no_grad():
-            loader = DataLoader(DataSet(x, y), batch_size if batch_size is not None else x.shape[0])
+            loader = DataLoader(DataSet(x, y), batch_size if batch_size is not None else x.shape[0], device=self._device)
             for idx, (bx, by) in enumerate(loader):
                 bx, by = self._place(bx), self._place(by)
                 if idx == 0 or idx == len(loader) - 1:
@@ -138,7 +139,7 @@ class _Model(_Base):
         x = np.asarray(x)
         outs = []
         with GLOBAL.no_grad():
-            loader = DataLoader(DataSet(x), batch_size if batch_size is not None else x.shape[0])
+            loader = DataLoader(DataSet(x), batch_size if batch_size is not None else x.shape[0], device=self._device)
             for idx, bx in enumerate(loader):
                 bx = self._place(bx)
                 if idx == 0 or idx == len(loader) - 1:
@@ -146,6 +147,32 @@ class _Model(_Base):
                 outs.append(self.forward(bx).numpy().copy())
         GLOBAL.INPUTS = None
         return Tensor(np.concatenate(outs, axis=0))
+
+    def save(self, save_path):
+        """Pickle ``[graph, optimizer, loss]`` (reference xs/nn/models.py:188-192).  Device arrays are
+        written as host arrays, so a checkpoint made on the GPU loads anywhere."""
+        if not save_path.endswith('.pkl'):
+            save_path += '.pkl'
+        with open(save_path, 'wb') as f:
+            pickle.dump([self._graph, self.optimizer, self.loss], f)
+
+    def load(self, model_path):
+        """Counterpart of reference xs/nn/models.py:194-202; additionally re-collects the parameter set
+        from the loaded layers.  Only load files this package wrote: unpickling runs code."""
+        if not model_path.endswith('.pkl'):
+            model_path += '.pkl'
+        with open(model_path, 'rb') as f:
+            graph, optimizer, loss = pickle.load(f)
+        self._graph = graph
+        self.optimizer = optimizer
+        self.loss = loss
+        self._parameters = set()
+        for layer in self._graph:
+            for v in (layer.parameters() if hasattr(layer, 'parameters') else []):
+                if v is not None:
+                    self._parameters.add(v)
+        if any(p.device == 'cuda' for p in self._parameters):
+            self._device = 'cuda'
 
     def __str__(self):
         rows = ['%-24s %-20s %10s' % ('Layer', 'Output shape', 'Params')]
