@@ -40,6 +40,12 @@ CONV = dict(N=32, C=64, H=56, W=56, K=64, R=3, S=3, stride=(1, 1), pad=1)
 POOL = dict(N=32, C=64, H=112, W=112, k=3, stride=(2, 2), pad=1)
 
 
+# HBM bytes per launch of tap_igemm_f32_kernel on the CONV workload, from two hardware-counter runs
+# (FETCH_SIZE 13 454.3 KiB scaled by 1.9996, the factor that makes the plain copy kernel's known read size come
+# out right, plus WRITE_SIZE 25 088.0 KiB at factor 1.0): 27.55 MB read + 25.69 MB written.
+TAP_IGEMM_TRAFFIC_BYTES = 53.24e6
+
+
 def conv_flops(c):
     oh = (c["H"] + 2 * c["pad"] - c["R"]) // c["stride"][0] + 1
     ow = (c["W"] + 2 * c["pad"] - c["S"]) // c["stride"][1] + 1
@@ -307,7 +313,7 @@ def main():
                    "gflop_per_step": 3 * flops_pass / 1e9},
         "frac_fp32_mfma_peak": value / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": None,
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": TAP_IGEMM_TRAFFIC_BYTES,
                      "kernel": "tap_igemm_f32_kernel", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
         "kernels_ms": {"conv_fwd_igemm": per["fwd"], "conv_bwd_data_igemm": per["bwd_data"],
                        "conv_bwd_weight_wgrad": per["bwd_weight"]},

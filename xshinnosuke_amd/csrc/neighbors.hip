@@ -272,22 +272,31 @@ __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, 
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
     for (int k0 = 0; k0 < K; k0 += GEMM_KC) {
-#pragma unroll 4
-        for (int i = threadIdx.x; i < 32 * GEMM_KC; i += 256) {
+        // all loads of the chunk first (independent, so their latencies overlap), then the LDS stores
+        float ra[GEMM_KC / 8], rb[GEMM_KC / 8];
+#pragma unroll
+        for (int u = 0; u < GEMM_KC / 8; ++u) {
+            const int i = threadIdx.x + 256 * u;
             if (ta) {                                   // A stored (K, M): lanes along m
                 const int kk = i >> 5, r = i & 31;
-                As[r][kk] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(k0 + kk) * M + m0 + r] : 0.f;
+                ra[u] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(k0 + kk) * M + m0 + r] : 0.f;
             } else {                                    // A stored (M, K): lanes along k
                 const int r = i / GEMM_KC, kk = i % GEMM_KC;
-                As[r][kk] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(m0 + r) * K + k0 + kk] : 0.f;
+                ra[u] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(m0 + r) * K + k0 + kk] : 0.f;
             }
             if (tb) {                                   // B stored (N, K): lanes along k
                 const int c = i / GEMM_KC, kk = i % GEMM_KC;
-                Bs[kk][c] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(n0 + c) * K + k0 + kk] : 0.f;
+                rb[u] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(n0 + c) * K + k0 + kk] : 0.f;
             } else {                                    // B stored (K, N): lanes along n
                 const int kk = i >> 5, c = i & 31;
-                Bs[kk][c] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(k0 + kk) * N + n0 + c] : 0.f;
+                rb[u] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(k0 + kk) * N + n0 + c] : 0.f;
             }
+        }
+#pragma unroll
+        for (int u = 0; u < GEMM_KC / 8; ++u) {
+            const int i = threadIdx.x + 256 * u;
+            if (ta) As[i & 31][i >> 5] = ra[u]; else As[i / GEMM_KC][i % GEMM_KC] = ra[u];
+            if (tb) Bs[i % GEMM_KC][i / GEMM_KC] = rb[u]; else Bs[i >> 5][i & 31] = rb[u];
         }
         __syncthreads();
 #pragma unroll 8
