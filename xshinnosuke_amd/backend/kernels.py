@@ -250,10 +250,11 @@ def _nchw3(shape):
     return int(n), int(c), int(hw)
 
 
-def bn_fwd(x, gamma, beta, eps):
+def bn_fwd(x, gamma, beta, eps, y=None):
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
-    y = empty(x.shape); xhat = empty(x.shape)
+    y = _like(x, y); xhat = empty(x.shape)
+    y.take_fresh()
     sqrtvar = empty((c,)); mean = empty((c,)); var = empty((c,))
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
     lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr, sqrtvar.cptr, mean.cptr, var.cptr,
@@ -261,9 +262,10 @@ def bn_fwd(x, gamma, beta, eps):
     return y, xhat, sqrtvar, mean, var
 
 
-def bn_infer(x, gamma, beta, mean, var, eps):
+def bn_infer(x, gamma, beta, mean, var, eps, y=None):
     n, c, hw = _nchw3(x.shape)
-    y = empty(x.shape)
+    y = _like(x, y)
+    y.take_fresh()
     lib.call("xsmi_bn_infer", x.cptr, gamma.cptr, beta.cptr, mean.cptr, var.cptr, y.cptr, n, c, hw, float(eps))
     return y
 

@@ -360,8 +360,9 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
         raise NotImplementedError('batch_norm normalises over axis 1 only')
     x = inputs.eval
     xhat = sqrtvar = None
+    dst = None if out is None else out.eval
     if training:
-        y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon)
+        y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst)
         for mov, cur in ((moving_mean, mean_), (moving_variance, var_)):
             m = mov.eval
             cur = A.same_place(m, cur)
@@ -371,10 +372,10 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
                 m *= momentum
                 m += (1 - momentum) * np.asarray(cur).reshape(m.shape)
     else:
-        y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon)
+        y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon, dst)
     if out is None:
         out = Tensor(y)
-    else:
+    elif y is not dst:
         out.eval = y
     out.requires_grad = bool(inputs.requires_grad or gamma.requires_grad or beta.requires_grad)
     _wire(out, inputs, gamma, beta)
