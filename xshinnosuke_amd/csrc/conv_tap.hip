@@ -59,6 +59,10 @@ struct TapParams {
     long long os_n, os_k, o_base;
     int os_y, os_x;
     int accumulate, relu;
+    // persistent kernel only
+    uint32_t *counters;   // 8 tile counters (one per XCD), zeroed by the pack kernel
+    uint32_t tiles;       // pixel tiles x row tiles
+    int rowtiles;
 };
 
 template <int STAGES>
@@ -266,6 +270,256 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
     }
 }
 
+// Persistent form of the kernel above (same tile, same loop body, 2 stages).  A launch has at most
+// four workgroups per CU and every workgroup walks a sequence of tiles: the loads of a tile's first
+// chunks are issued while the previous tile's last chunks multiply, and a tile's output stores
+// drain while the next tile multiplies, so a CU's matrix pipes do not idle while a finished
+// workgroup is replaced.  Tiles are split into eight contiguous ranges, one per XCD (workgroup
+// b runs on XCD b % 8); a workgroup's first two tiles are fixed (slot, slot + P with P workgroups
+// per XCD) and the rest come from its XCD's counter, fetched one tile ahead of use.  Requires an
+// even chunk count >= 4 per tile and at least 8 tiles.
+__global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p) {
+    constexpr int STAGES = 2;
+    __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
+    __shared__ uint32_t s_next;
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, P = gridDim.x >> 3;
+    const uint32_t tq = p.tiles >> 3, trem = p.tiles & 7u;
+    const uint32_t t_start = xcd * tq + (xcd < trem ? xcd : trem), t_count = tq + (xcd < trem ? 1u : 0u);
+    const int iters = p.TR * p.TS * p.nch;
+
+    // tile -> (first pixel, row tile); row tiles of one pixel tile are neighbours
+    auto decode = [&](uint32_t local, int &m0, int &rowtile) {
+        const uint32_t L = t_start + local;
+        const uint32_t mt = p.rowtiles == 1 ? L : L / (uint32_t)p.rowtiles;
+        rowtile = p.rowtiles == 1 ? 0 : (int)(L - mt * (uint32_t)p.rowtiles);
+        m0 = (int)mt * BP;
+    };
+    // gather role of a lane in a tile: pixel m0 + lane
+    auto lane_geom = [&](int m0, int &iyb, int &ixb, int &nbase, bool &live) {
+        iyb = 0; ixb = 0; nbase = 0;
+        live = m0 + lane < p.M;
+        if (live) {
+            uint32_t m = (uint32_t)(m0 + lane);
+            uint32_t q = xsmi::fdiv(m, p.dOX);
+            int x = (int)m - (int)q * p.OX;
+            uint32_t n = xsmi::fdiv(q, p.dOY);
+            int y = (int)q - (int)n * p.OY;
+            iyb = y * p.sy + p.dy0;
+            ixb = x * p.sx + p.dx0;
+            nbase = (int)n * p.in_n_stride;
+        }
+    };
+
+    int cur_m0, cur_rowtile, nxt_m0 = 0, nxt_rowtile = 0;
+    uint32_t nxt_local = slot + P;
+    bool nxt_valid = nxt_local < t_count;
+    decode(slot, cur_m0, cur_rowtile);
+    int iyb, ixb, nbase, iyb_n = 0, ixb_n = 0, nbase_n = 0;
+    bool live, live_n = false;
+    lane_geom(cur_m0, iyb, ixb, nbase, live);
+    if (nxt_valid) {
+        decode(nxt_local, nxt_m0, nxt_rowtile);
+        lane_geom(nxt_m0, iyb_n, ixb_n, nbase_n, live_n);
+    }
+
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(p.in, p.in_bytes);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(p.apk, p.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];
+    const uint32_t a_voff = (uint32_t)((2 * wave * 64 + lane) * 16);
+    const uint32_t a_tile_bytes = (uint32_t)iters * (uint32_t)(TM * KC * 4);
+
+    int r = 0, s = 0, cc = 0;
+    uint32_t ld_stage = lds0;
+    uint32_t ld_asoff = (uint32_t)cur_rowtile * a_tile_bytes;
+    uint32_t ld_voff = 0, ld_soff = 0;
+    auto issue_prep = [&]() {
+        int iy = iyb + r * p.dstep, ix = ixb + s * p.dstep;
+        bool ok = live && (unsigned)iy < (unsigned)p.IH && (unsigned)ix < (unsigned)p.IW;
+        ld_voff = ok ? (uint32_t)((nbase + iy * p.IW + ix) * 4) : 0x80000000u;
+        ld_soff = (uint32_t)(cc * KC + wave * 8) * p.plane_bytes;
+    };
+    auto issue_b = [&](int e) {
+        xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((2048 + (wave * 8 + e) * 64) * 4), ld_voff,
+                           ld_soff + (uint32_t)e * p.plane_bytes);
+    };
+    auto issue_a = [&](int qa) {
+        xsmi::load_lds_b128(rap, ld_stage + (uint32_t)((2 * wave + qa) * 1024), a_voff + (uint32_t)qa * 1024u, ld_asoff);
+    };
+    auto issue_advance = [&]() {
+        ld_asoff += (uint32_t)(TM * KC * 4);
+        ld_stage += (uint32_t)(STAGE_FLOATS * 4);
+        if (ld_stage == lds0 + (uint32_t)(STAGES * STAGE_FLOATS * 4)) ld_stage = lds0;
+        if (++cc == p.nch) {
+            cc = 0;
+            if (++s == p.TS) {
+                s = 0;
+                if (++r == p.TR) {               // the issue side moves on to the next tile
+                    r = 0;
+                    iyb = iyb_n; ixb = ixb_n; nbase = nbase_n; live = live_n;
+                    ld_asoff = (uint32_t)nxt_rowtile * a_tile_bytes;
+                }
+            }
+        }
+    };
+    auto issue_all = [&]() {
+        issue_prep();
+#pragma unroll
+        for (int e = 0; e < 8; ++e) issue_b(e);
+        issue_a(0);
+        issue_a(1);
+        issue_advance();
+    };
+
+    floatx16 acc = {0}, acc2 = {0};
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave >> 1, wc = wave & 1;
+    const int a_rd = (4 * h * 64 + wr * 32 + l31) * 4;
+    const int b_rd = 2048 + 16 * h * 64 + wc * 32 + l31;
+
+    float4 fa[2][4];
+    float fb[2][16];
+    const float *rd_stage = smem[0];
+    auto rd_advance = [&]() {
+        rd_stage += STAGE_FLOATS;
+        if (rd_stage == smem[0] + STAGES * STAGE_FLOATS) rd_stage = smem[0];
+    };
+#define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
+#define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
+    auto body = [&](auto buf_tag, int) {
+        constexpr int cur = decltype(buf_tag)::value;
+        constexpr int nxt = cur ^ 1;
+        constexpr bool has_next = true, has_load = true;
+        XSMI_MFMA(acc, fa[cur][0].x, fb[cur][0]);
+        XSMI_MFMA(acc2, fa[cur][0].y, fb[cur][1]);
+        XSMI_MFMA(acc, fa[cur][0].z, fb[cur][2]);
+        XSMI_MFMA(acc2, fa[cur][0].w, fb[cur][3]);
+        XSMI_PIN();
+        if (has_next) {
+            xsmi::wait_vmcnt<0>();
+            xsmi::block_barrier();
+        }
+        XSMI_PIN();
+        XSMI_MFMA(acc, fa[cur][1].x, fb[cur][4]);
+        if (has_next) fa[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + a_rd);
+        if (has_load) issue_prep();
+        XSMI_PIN();
+        XSMI_MFMA(acc2, fa[cur][1].y, fb[cur][5]);
+        if (has_next) fa[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 256);
+        if (has_load) issue_b(0);
+        XSMI_PIN();
+        XSMI_MFMA(acc, fa[cur][1].z, fb[cur][6]);
+        if (has_next) fa[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 512);
+        if (has_load) issue_b(1);
+        XSMI_PIN();
+        XSMI_MFMA(acc2, fa[cur][1].w, fb[cur][7]);
+        if (has_next) fa[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 768);
+        if (has_load) issue_b(2);
+        XSMI_PIN();
+#define XSMI_SLOT(ACC, AV, J, LOADSTMT)                                      \
+        XSMI_MFMA(ACC, AV, fb[cur][J]);                                      \
+        if (has_next) {                                                      \
+            fb[nxt][2 * (J - 8)] = rd_stage[b_rd + 64 * (2 * (J - 8))];        \
+            fb[nxt][2 * (J - 8) + 1] = rd_stage[b_rd + 64 * (2 * (J - 8) + 1)]; \
+        }                                                                    \
+        if (has_load) { LOADSTMT; }                                          \
+        XSMI_PIN();
+        XSMI_SLOT(acc, fa[cur][2].x, 8, issue_b(3))
+        XSMI_SLOT(acc2, fa[cur][2].y, 9, issue_b(4))
+        XSMI_SLOT(acc, fa[cur][2].z, 10, issue_b(5))
+        XSMI_SLOT(acc2, fa[cur][2].w, 11, issue_b(6))
+        XSMI_SLOT(acc, fa[cur][3].x, 12, issue_b(7))
+        XSMI_SLOT(acc2, fa[cur][3].y, 13, issue_a(0))
+        XSMI_SLOT(acc, fa[cur][3].z, 14, issue_a(1))
+        XSMI_SLOT(acc2, fa[cur][3].w, 15, issue_advance())
+#undef XSMI_SLOT
+        if (has_next) rd_advance();
+    };
+
+    // prologue of the first tile: chunk 0 landed and in registers, chunk 1 in flight
+    issue_all();
+    xsmi::wait_vmcnt<0>();
+    xsmi::block_barrier();
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4) fa[0][q4] = *reinterpret_cast<const float4 *>(rd_stage + a_rd + 256 * q4);
+#pragma unroll
+    for (int j = 0; j < 16; ++j) fb[0][j] = rd_stage[b_rd + 64 * j];
+    rd_advance();
+    issue_all();
+
+    using T0 = std::integral_constant<int, 0>;
+    using T1 = std::integral_constant<int, 1>;
+    for (;;) {
+        const bool last_tile = !nxt_valid;                    // uniform over the workgroup
+        uint32_t fetched = 0;
+        if (!last_tile && t == 0) fetched = atomicAdd(p.counters + xcd, 1u);   // tile after the next one
+        // Every chunk runs the full body.  In a workgroup's last tile the two chunks "after the end" are
+        // loaded from a dummy tile (no live pixel: the activation loads are all out of range and touch
+        // no memory; the filter loads re-read row tile 0), and their fragments are never multiplied.
+        for (int it = 0; it < iters; it += 2) {
+            body(T0{}, it);
+            body(T1{}, it + 1);
+        }
+        acc += acc2;
+
+        // ---- epilogue: register v of lane l = row 8*(v/4) + 4*(l/32) + v%4, pixel l%32 ----
+        {
+            const int m = cur_m0 + wc * 32 + l31;
+            if (m < p.M) {
+                uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+                int x = m - (int)q * p.OX;
+                uint32_t n = xsmi::fdiv(q, p.dOY);
+                int y = (int)q - (int)n * p.OY;
+                const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
+                const int rbase = cur_rowtile * TM + wr * 32 + 4 * h;
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int row = rbase + 8 * (v >> 2) + (v & 3);
+                    if (row < p.rows) {
+                        float val = acc[v];
+                        if (p.bias) val += p.bias[row];
+                        long long o = pix_off + (long long)row * p.os_k;
+                        if (p.relu) {
+                            if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
+                            val = val > 0.f ? val : 0.f;
+                        }
+                        if (p.accumulate) val += p.out[o];
+                        p.out[o] = val;
+                    }
+                }
+            }
+        }
+        if (last_tile) {
+            xsmi::wait_vmcnt<0>();                            // the dummy chunk's loads target this workgroup's LDS
+            break;
+        }
+#pragma unroll
+        for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc2[v] = 0.f; }
+
+        // the tile fetched at the top of this iteration becomes the next one; the issue side has
+        // already moved into what was the next tile and now becomes the current one
+        if (t == 0) s_next = 2u * P + fetched;
+        asm volatile("" ::: "memory");                        // the LDS store stays ahead of the wait below
+        xsmi::wait_lgkmcnt0();
+        xsmi::block_barrier();
+        const uint32_t nn = __builtin_amdgcn_readfirstlane(s_next);
+        cur_m0 = nxt_m0; cur_rowtile = nxt_rowtile;
+        nxt_local = nn;
+        nxt_valid = nn < t_count;
+        if (nxt_valid) {
+            decode(nxt_local, nxt_m0, nxt_rowtile);
+            lane_geom(nxt_m0, iyb_n, ixb_n, nbase_n, live_n);
+        } else {
+            nxt_rowtile = 0; live_n = false;                  // dummy tile
+        }
+    }
+#undef XSMI_MFMA
+#undef XSMI_PIN
+}
+
 // bf16 variant (opt-in): the same fp32 tensors, loads and LDS layout, but the
 // fragments are rounded to bf16 (round to nearest even) in registers and a chunk
 // of 32 channels is two v_mfma_f32_32x32x16_bf16 with fp32 accumulation.  A lane
@@ -408,7 +662,8 @@ __global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapParams p) {
 // mode 1 (backward-data class): A[row=c][tap=(t,u)][ch=k] = w[k][c][r0 + sh*t][s0 + sw*u].
 __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__ w, float *__restrict__ apk, int mode,
                                                         int rows, int CH, int R, int S, int TR, int TS, int r0, int s0,
-                                                        int sh, int sw, int rowtiles) {
+                                                        int sh, int sw, int rowtiles, uint32_t *__restrict__ counters) {
+    if (blockIdx.x == 0 && threadIdx.x < 8) counters[threadIdx.x] = 0;   // tile counters of the persistent kernel
     const int nch = CH / KC;
     const int iters = TR * TS * nch;
     const size_t total = (size_t)rowtiles * iters * (TM * KC);
@@ -434,15 +689,31 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
-void launch_tap(dim3 grid, hipStream_t st, const TapParams &p, int bf16) {
+void launch_tap(dim3 grid, hipStream_t st, TapParams p, int bf16) {
     if (bf16) {
         hipLaunchKernelGGL(tap_igemm_bf16_kernel<3>, grid, dim3(256), 0, st, p);
         return;
     }
-    static int stages = -1;
+    static int stages = -1, persist = -1;
     if (stages < 0) {
         const char *e = getenv("XSMI_TAP_STAGES");
         stages = e ? atoi(e) : TAP_STAGES;
+        e = getenv("XSMI_TAP_PERSIST");
+        persist = e ? atoi(e) : 1;
+    }
+    const int iters = p.TR * p.TS * p.nch;
+    const uint32_t tiles = grid.x * grid.y;
+    // Measured at steady clocks: with no more tiles than resident workgroups (one tile each, no tail
+    // code) the persistent kernel wins by 1-4 %; with more tiles the hardware's own workgroup
+    // hand-over is as fast as the in-kernel one, and the plain kernel's dynamic dispatch balances better.
+    const uint32_t resident = (uint32_t)xsmi::cu_count() * 4u;          // four workgroups per CU fit (registers)
+    if (persist && stages == 2 && iters >= 4 && (iters & 1) == 0 && tiles >= 16 && (tiles <= resident || persist > 1)) {
+        uint32_t g = tiles < resident ? tiles : resident;
+        g &= ~7u;
+        p.tiles = tiles;
+        p.rowtiles = (int)grid.y;
+        hipLaunchKernelGGL(tap_igemm_f32_persist_kernel, dim3(g), dim3(256), 0, st, p);
+        return;
     }
     switch (stages) {
         case 2: hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, grid, dim3(256), 0, st, p); break;
@@ -452,19 +723,22 @@ void launch_tap(dim3 grid, hipStream_t st, const TapParams &p, int bf16) {
     }
 }
 
+// packed filter + 256 bytes that hold the persistent kernel's eight tile counters
 size_t tap_pack_bytes(int rows, int CH, int taps) {
-    return xsmi::align_up((size_t)xsmi::ceil_div(rows, TM) * taps * (CH / KC) * TM * KC * sizeof(float), 256);
+    return xsmi::align_up((size_t)xsmi::ceil_div(rows, TM) * taps * (CH / KC) * TM * KC * sizeof(float), 256) + 256;
 }
+uint32_t *tap_counters(float *apk, size_t pack_bytes) { return (uint32_t *)((char *)apk + pack_bytes - 256); }
 
 int launch_pack(hipStream_t st, const float *w, float *apk, int mode, int rows, int CH, int R, int S, int TR, int TS,
                 int r0, int s0, int sh, int sw) {
+    uint32_t *counters = tap_counters(apk, tap_pack_bytes(rows, CH, TR * TS));
     const int rowtiles = xsmi::ceil_div(rows, TM);
     size_t total = (size_t)rowtiles * TR * TS * (CH / KC) * TM * KC;
     if (total == 0) return XSMI_OK;
     int blocks = (int)((total + 255) / 256);
     if (blocks > 2048) blocks = 2048;
     hipLaunchKernelGGL(tap_pack_kernel, dim3(blocks), dim3(256), 0, st, w, apk, mode, rows, CH, R, S, TR, TS, r0, s0, sh,
-                       sw, rowtiles);
+                       sw, rowtiles, counters);
     XSMI_LAUNCH_CHECK("tap_pack_kernel");
     return XSMI_OK;
 }
@@ -503,6 +777,7 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     dim3 grid(ceil_div(p.M, BP), ceil_div(K, TM));
     prof_begin();
     p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
+    p.counters = tap_counters(apk, tap_pack_bytes(K, C, R * S));
     launch_tap(grid, st, p, bf16);
     prof_end();
     XSMI_LAUNCH_CHECK("tap_igemm kernel");
@@ -535,6 +810,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             TapParams p;
             p.in = dy; p.apk = apk; p.bias = nullptr; p.out = dx; p.mask = nullptr;
             p.apk_bytes = (uint32_t)apk_bytes;
+            p.counters = tap_counters(apk, apk_bytes);
             p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
             p.M = N * OYc * OXc; p.rows = C; p.nch = K / KC; p.TR = T; p.TS = U;
             p.dy0 = cy; p.dx0 = cx; p.dstep = -1;

@@ -145,6 +145,13 @@ __device__ __forceinline__ void wait_vmcnt() {
 #endif
 }
 
+// s_waitcnt on the LDS/scalar-memory counter only (vmcnt and expcnt left at their maxima).
+__device__ __forceinline__ void wait_lgkmcnt0() {
+#if defined(__HIP_DEVICE_COMPILE__)
+    __builtin_amdgcn_s_waitcnt(15 | (3 << 14) | (7 << 4) | (0 << 8));
+#endif
+}
+
 // Workgroup barrier the compiler may not move memory accesses across; it carries
 // no waits of its own.
 __device__ __forceinline__ void block_barrier() {
