@@ -116,13 +116,19 @@ def bench_conv(be, steps, warmup):
     be.synchronize()
     wall_ms = (time.perf_counter() - t0) * 1e3
 
-    # second pass: each kernel launched K times back to back between one pair of events on the
-    # library's stream, so the average launch duration carries no per-launch event overhead
+    # second pass: each op launched K times back to back between one pair of events on the library's
+    # stream, so the average launch duration carries no per-launch event overhead.  "fwd"/"bwd_data"/
+    # "bwd_weight" are whole ops (filter layout kernel or split reduction included); "*_kernel" repeat the
+    # forward / backward-data launch with XSMI_CONV_WS_PACKED, i.e. the tap-major MFMA kernel alone.
     per = {
         "fwd": batch_ms(be, lambda: K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y), steps),
         "bwd_data": batch_ms(be, lambda: K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx), steps),
         "bwd_weight": batch_ms(be, lambda: K.conv2d_bwd_weight(ddy, dx_, w.shape, c["stride"], c["pad"], dw=gw, db=gb), steps),
     }
+    K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y)
+    per["fwd_kernel"] = batch_ms(be, lambda: K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y, packed=True), steps)
+    K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx)
+    per["bwd_data_kernel"] = batch_ms(be, lambda: K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx, packed=True), steps)
     return ms / steps, wall_ms / steps, per
 
 
@@ -322,7 +328,7 @@ def main():
     ms_step, wall_ms_step, per = bench_conv(be, args.steps, args.warmup)
     flops_pass = conv_flops(CONV)
     value = 3 * flops_pass / (ms_step * 1e-3) / 1e12
-    igemm_ms = 0.5 * (per["fwd"] + per["bwd_data"])      # the same kernel, one launch each per step
+    igemm_ms = 0.5 * (per["fwd_kernel"] + per["bwd_data_kernel"])      # the same kernel, one launch each per step
     achieved = flops_pass / (igemm_ms * 1e-3) / 1e12
     out = {
         "metric": "conv fwd+bwd TFLOP/s", "value": value, "unit": "TFLOP/s",
@@ -336,9 +342,9 @@ def main():
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": TAP_IGEMM_TRAFFIC_BYTES,
                      "kernel": "tap_igemm_f32_kernel", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
-        "kernels_ms": {"conv_fwd_igemm": per["fwd"], "conv_bwd_data_igemm": per["bwd_data"],
-                       "conv_bwd_weight_wgrad": per["bwd_weight"]},
-        "kernels_tflops": {k: flops_pass / (v * 1e-3) / 1e12 for k, v in per.items()},
+        "ops_ms": {"conv_fwd": per["fwd"], "conv_bwd_data": per["bwd_data"], "conv_bwd_weight": per["bwd_weight"]},
+        "kernels_ms": {"tap_igemm_fwd": per["fwd_kernel"], "tap_igemm_bwd_data": per["bwd_data_kernel"]},
+        "ops_tflops": {k: flops_pass / (per[k] * 1e-3) / 1e12 for k in ("fwd", "bwd_data", "bwd_weight")},
         "wall_ms_per_step": wall_ms_step,
         "preheat_s": PREHEAT_S,
         "device": {"name": info["name"], "arch": info["arch"], "cus": info["cu_count"], "clock_mhz": info["clock_khz"] / 1000.0},

@@ -39,6 +39,10 @@ extern "C" {
 /* flags for the conv entry points */
 #define XSMI_CONV_RELU 0x1u      /* y = max(0, conv + bias)  (fused epilogue)            */
 #define XSMI_CONV_BF16 0x2u      /* opt-in: bf16 MFMA operands, fp32 accumulate          */
+#define XSMI_CONV_WS_PACKED 0x4u /* the workspace still holds what the previous call of the same
+                                    entry point with the same geometry and the same filter values
+                                    left there: the filter is not laid out again (inference loops).
+                                    Ignored where no reusable layout exists.                */
 
 typedef struct xsmi_device_info {
     int device;

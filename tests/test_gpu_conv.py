@@ -139,6 +139,23 @@ def test_conv_bf16_opt_in(gpu, n, c, h, w, k, r, s, sh, sw, pad):
     np.testing.assert_array_equal(gw.numpy(), gw32.numpy())
 
 
+def test_conv_packed_workspace_flag(gpu):
+    """XSMI_CONV_WS_PACKED: a repeated forward / backward-data call may skip laying the filter out again."""
+    K = gpu.kernels
+    rng = np.random.default_rng(21)
+    for (n, c, h, w, k, st) in ((2, 64, 20, 20, 64, 1), (2, 64, 20, 20, 128, 2), (1, 3, 9, 9, 5, 1)):
+        x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+        wt = he_normal(rng, (k, c, 3, 3))
+        dx_, dw_ = gpu.to_device(x), gpu.to_device(wt)
+        y0 = K.conv2d_fwd(dx_, dw_, None, (st, st), 1).numpy()
+        y1 = K.conv2d_fwd(dx_, dw_, None, (st, st), 1, packed=True).numpy()
+        np.testing.assert_array_equal(y0, y1)
+        dy = gpu.to_device(rng.standard_normal(y0.shape).astype(np.float32))
+        g0 = K.conv2d_bwd_data(dy, dw_, x.shape, (st, st), 1).numpy()
+        g1 = K.conv2d_bwd_data(dy, dw_, x.shape, (st, st), 1, packed=True).numpy()
+        np.testing.assert_array_equal(g0, g1)
+
+
 def test_conv_special_kernels_exact(gpu):
     """Closed forms that need no rounding: delta filter == shift, ones filter on small integers == box sum."""
     K = gpu.kernels

@@ -86,6 +86,7 @@ SIGNATURES = {
 
 CONV_RELU = 0x1
 CONV_BF16 = 0x2
+CONV_WS_PACKED = 0x4
 
 
 def library_path():

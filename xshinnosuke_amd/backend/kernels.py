@@ -8,7 +8,7 @@ import ctypes
 
 import numpy as np
 
-from .capi import lib, CONV_RELU, CONV_BF16
+from .capi import lib, CONV_RELU, CONV_BF16, CONV_WS_PACKED
 from .array import DeviceArray, Workspace, empty
 
 _ws = Workspace()
@@ -39,7 +39,9 @@ def _f32(a, what):
     return a
 
 
-def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False):
+def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False, packed=False):
+    """``packed=True`` promises that the previous conv call was this same forward with the same geometry and
+    filter values (the shared workspace still holds the filter's packed form), so it is not laid out again."""
     _f32(x, "x"); _f32(w, "w")
     dims = _dims(x.shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -56,7 +58,7 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
         raise ValueError("conv2d: out has shape %s, expected %s" % (out.shape, (n, k, oh, ow)))
     if neg_mask is not None and (neg_mask.dtype != np.uint8 or neg_mask.size != out.size):
         raise ValueError("conv2d: neg_mask must be uint8 with one byte per output element")
-    flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0)
+    flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0)
     ws, ws_bytes = _workspace(dims)
     lib.call("xsmi_conv2d_fwd", x.cptr, w.cptr, bias.cptr if bias is not None else None, out.cptr,
              neg_mask.cptr if neg_mask is not None else None, *dims, flags, ws, ws_bytes)
@@ -75,7 +77,7 @@ def _beta(accumulate, *outs):
     return 0.0
 
 
-def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=False, bf16=False):
+def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=False, bf16=False, packed=False):
     _f32(dy, "dy"); _f32(w, "w")
     dims = _dims(x_shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -90,7 +92,7 @@ def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=Fa
     ws, ws_bytes = _workspace(dims)
     beta = _beta(accumulate, dx)
     lib.call("xsmi_conv2d_bwd_data", dy.cptr, w.cptr, dx.cptr, *dims, beta,
-             CONV_BF16 if bf16 else 0, ws, ws_bytes)
+             (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0), ws, ws_bytes)
     return dx
 
 

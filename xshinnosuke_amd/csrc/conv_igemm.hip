@@ -332,14 +332,15 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     int rc = check_conv("xsmi_conv2d_fwd", N, C, H, W, K, R, S, sh, sw, pad, &g);
     if (rc) return rc;
     XSMI_CHECK_ARG(x && w && y, "xsmi_conv2d_fwd: null tensor pointer");
-    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16)) == 0, "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
     const int J = C * R * S;
     const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd: workspace of %zu bytes needed, %zu given", need,
                    workspace_bytes);
     if (xsmi::tap_path_ok(C))
         return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
-                                  (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_BF16) ? 1 : 0, workspace);
+                                  (flags & XSMI_CONV_RELU) ? 1 : 0,
+                                  ((flags & XSMI_CONV_BF16) ? 1 : 0) | ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0), workspace);
     const int rowtiles = xsmi::ceil_div(K, TM);
     const int nchunks = xsmi::ceil_div(J, KC);
     float *apk = (float *)workspace;
@@ -382,13 +383,13 @@ int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int 
     if (rc) return rc;
     XSMI_CHECK_ARG(dy && w && dx, "xsmi_conv2d_bwd_data: null tensor pointer");
     XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_conv2d_bwd_data: beta must be 0 or 1");
-    XSMI_CHECK_ARG((flags & ~XSMI_CONV_BF16) == 0, "xsmi_conv2d_bwd_data: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_bwd_data: unknown flags 0x%x", flags);
     const size_t need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_bwd_data: workspace of %zu bytes needed, %zu given",
                    need, workspace_bytes);
     if (xsmi::tap_path_ok(K))
         return xsmi::tap_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
-                                       (flags & XSMI_CONV_BF16) ? 1 : 0, workspace);
+                                       ((flags & XSMI_CONV_BF16) ? 1 : 0) | ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0), workspace);
     hipStream_t st = xsmi::stream();
     char *ws = (char *)workspace;
     const int rowtiles = xsmi::ceil_div(C, TM);

@@ -689,7 +689,8 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
-void launch_tap(dim3 grid, hipStream_t st, TapParams p, int bf16) {
+void launch_tap(dim3 grid, hipStream_t st, TapParams p, int opts) {
+    const int bf16 = opts & 1, counters_zeroed = !(opts & 2);   // the pack kernel zeroes the tile counters
     if (bf16) {
         hipLaunchKernelGGL(tap_igemm_bf16_kernel<3>, grid, dim3(256), 0, st, p);
         return;
@@ -707,7 +708,8 @@ void launch_tap(dim3 grid, hipStream_t st, TapParams p, int bf16) {
     // code) the persistent kernel wins by 1-4 %; with more tiles the hardware's own workgroup
     // hand-over is as fast as the in-kernel one, and the plain kernel's dynamic dispatch balances better.
     const uint32_t resident = (uint32_t)xsmi::cu_count() * 4u;          // four workgroups per CU fit (registers)
-    if (persist && stages == 2 && iters >= 4 && (iters & 1) == 0 && tiles >= 16 && (tiles <= resident || persist > 1)) {
+    if (persist && stages == 2 && iters >= 4 && (iters & 1) == 0 && tiles >= 16 &&
+        (tiles <= resident || (persist > 1 && counters_zeroed))) {
         uint32_t g = tiles < resident ? tiles : resident;
         g &= ~7u;
         p.tiles = tiles;
@@ -759,11 +761,13 @@ size_t tap_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
 }
 
 int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
-                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int bf16, void *workspace) {
+                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace) {
     hipStream_t st = stream();
     float *apk = (float *)workspace;
-    int rc = launch_pack(st, w, apk, 0, K, C, R, S, R, S, 0, 0, 1, 1);
-    if (rc) return rc;
+    if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
+        int rc = launch_pack(st, w, apk, 0, K, C, R, S, R, S, 0, 0, 1, 1);
+        if (rc) return rc;
+    }
     TapParams p;
     p.in = x; p.apk = apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
     p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
@@ -778,14 +782,14 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     prof_begin();
     p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
     p.counters = tap_counters(apk, tap_pack_bytes(K, C, R * S));
-    launch_tap(grid, st, p, bf16);
+    launch_tap(grid, st, p, opts);
     prof_end();
     XSMI_LAUNCH_CHECK("tap_igemm kernel");
     return XSMI_OK;
 }
 
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
-                      int sw, int pad, int OH, int OW, int accumulate, int bf16, void *workspace) {
+                      int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace) {
     hipStream_t st = stream();
     char *ws = (char *)workspace;
     struct Plan { TapParams p; dim3 grid; };
@@ -805,8 +809,10 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             float *apk = (float *)ws;
             const size_t apk_bytes = tap_pack_bytes(C, K, T * U);
             ws += apk_bytes;
-            int rc = launch_pack(st, w, apk, 1, C, K, R, S, T, U, r0, s0, sh, sw);
-            if (rc) return rc;
+            if (!(opts & 2)) {
+                int rc = launch_pack(st, w, apk, 1, C, K, R, S, T, U, r0, s0, sh, sw);
+                if (rc) return rc;
+            }
             TapParams p;
             p.in = dy; p.apk = apk; p.bias = nullptr; p.out = dx; p.mask = nullptr;
             p.apk_bytes = (uint32_t)apk_bytes;
@@ -827,7 +833,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
     }
     prof_begin();
     for (int i = 0; i < nplans; ++i) {
-        launch_tap(plans[i].grid, st, plans[i].p, bf16);
+        launch_tap(plans[i].grid, st, plans[i].p, opts);
         XSMI_LAUNCH_CHECK("tap_igemm kernel");
     }
     prof_end();

@@ -234,7 +234,7 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
     XSMI_CHECK_ARG(H + 2 * pad >= R && W + 2 * pad >= S, "xsmi_conv2d_bwd_weight: filter larger than the padded input");
     XSMI_CHECK_ARG(dy && x && dw, "xsmi_conv2d_bwd_weight: null tensor pointer");
     XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_conv2d_bwd_weight: beta must be 0 or 1");
-    XSMI_CHECK_ARG((flags & ~XSMI_CONV_BF16) == 0, "xsmi_conv2d_bwd_weight: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_bwd_weight: unknown flags 0x%x", flags);
     // XSMI_CONV_BF16 is a permission, not a request: the weight gradient always runs on fp32 MFMA
     const int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
     const double lim = 536870912.0;

@@ -83,14 +83,15 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t lin, uint32_t tot
     return xcd * q + (xcd < rem ? xcd : rem) + slot;
 }
 
-// tap-major fast path (conv_tap.hip): reduction channels must be a multiple of 32
+// tap-major fast path (conv_tap.hip): reduction channels must be a multiple of 32.
+// opts: bit 0 = bf16 MFMA operands, bit 1 = the workspace already holds the packed filter
 bool tap_path_ok(int reduce_channels);
 size_t tap_fwd_ws_bytes(int C, int K, int R, int S);
 size_t tap_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw);
 int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
-                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int bf16, void *workspace);
+                 int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace);
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
-                      int sw, int pad, int OH, int OW, int accumulate, int bf16, void *workspace);
+                      int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace);
 
 // tap-major backward-weight (conv_wgrad_tap.hip)
 bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW);
