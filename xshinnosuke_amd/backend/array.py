@@ -1,10 +1,13 @@
 """Device-resident arrays owned by Python, allocated through the C ABI."""
 import ctypes
+import math
 
 import numpy as np
 
 from .capi import lib, ensure_init
 
+
+_DTYPE_CLASS = np.dtype(np.float32).__class__
 
 _POOL = {}            # rounded size -> list of free device pointers
 _POOL_BYTES = [0]
@@ -85,9 +88,9 @@ class DeviceArray:
     """
 
     def __init__(self, shape, dtype=np.float32, _block=None, _offset=0):
-        self.shape = tuple(int(s) for s in shape)
-        self.dtype = np.dtype(dtype)
-        self.size = int(np.prod(self.shape, dtype=np.int64)) if self.shape else 1
+        self.shape = shape = tuple(map(int, shape))
+        self.dtype = dtype if dtype.__class__ is _DTYPE_CLASS else np.dtype(dtype)
+        self.size = math.prod(shape)
         self.nbytes = self.size * self.dtype.itemsize
         if _block is None:
             _block = _Block(max(self.nbytes, 16))
@@ -192,9 +195,9 @@ class DeviceArray:
             shape = tuple(shape[0])
         shape = list(shape)
         if -1 in shape:
-            known = int(np.prod([s for s in shape if s != -1], dtype=np.int64))
+            known = math.prod(s for s in shape if s != -1)
             shape[shape.index(-1)] = self.size // max(known, 1)
-        if int(np.prod(shape, dtype=np.int64)) != self.size:
+        if math.prod(shape) != self.size:
             raise ValueError("cannot reshape %s into %s" % (self.shape, tuple(shape)))
         return DeviceArray(shape, self.dtype, _block=self._block, _offset=self._offset)
 
