@@ -41,9 +41,9 @@ POOL = dict(N=32, C=64, H=112, W=112, k=3, stride=(2, 2), pad=1)
 
 
 # HBM bytes per launch of tap_igemm_f32_kernel on the CONV workload, from two hardware-counter runs
-# (FETCH_SIZE 13 454.3 KiB scaled by 1.9996, the factor that makes the plain copy kernel's known read size come
-# out right, plus WRITE_SIZE 25 088.0 KiB at factor 1.0): 27.55 MB read + 25.69 MB written.
-TAP_IGEMM_TRAFFIC_BYTES = 53.24e6
+# (FETCH_SIZE 13 480.7 KiB scaled by 1.9996, the factor that makes the plain copy kernel's known read size come
+# out right, plus WRITE_SIZE 25 088.0 KiB at factor 1.0): 27.60 MB read + 25.69 MB written.
+TAP_IGEMM_TRAFFIC_BYTES = 53.29e6
 
 
 def conv_flops(c):
