@@ -214,7 +214,7 @@ size_t conv_bwd_weight_ws_bytes(int N, int C, int K, int R, int S, int OH, int O
     plan_splits(N * OH * OW, K, C * R * S, &splits, &cps);
     size_t Kp = align_up(K, TK), Jp = align_up((size_t)C * R * S, TJ);
     size_t generic = align_up((size_t)splits * Kp * Jp * sizeof(float), 256) + align_up((size_t)splits * Kp * sizeof(float), 256);
-    if (C % 64 == 0 && K % 64 == 0 && (OH * OW) % 4 == 0) {
+    if (C % 64 == 0 && K % 64 == 0) {
         size_t tap = wgrad_tap_ws_bytes(N, C, K, R, S, OH, OW);
         return tap > generic ? tap : generic;
     }

@@ -1,5 +1,7 @@
-// Tap-major backward-weight on fp32 MFMA for layers with C % 64 == 0, K % 64 == 0
-// and OH*OW % 4 == 0.
+// Tap-major backward-weight on fp32 MFMA for layers with C % 64 == 0 and K % 64 == 0.
+// When OH*OW is not a multiple of 4 (7x7 images) dy is first copied into the workspace with
+// every plane padded by zeros to the next multiple of 4, which restores the 16-byte alignment
+// and the whole-group validity that the 128-bit dy loads rely on.
 //
 // For one filter tap (r, s) the weight gradient is a plain GEMM over pixels,
 //
@@ -43,6 +45,7 @@ struct WgradTapParams {
     float *dbpart;      // [split][K] or nullptr
     uint32_t x_bytes, dy_bytes;
     int N, C, K, H, W, OH, OW, OHW, R, S, sh, sw, pad;
+    int OHWa;           // plane length of the dy operand as stored (OHW rounded up to a multiple of 4)
     int cpi;            // chunks per image
     int total_chunks, cps, ctiles;
     uint32_t xplane_bytes, yplane_bytes;
@@ -100,11 +103,11 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
     uint32_t ld_va0 = 0, ld_va1 = 0, ld_vb = 0, ld_sa = 0, ld_sb = 0;
     auto issue_prep = [&]() {
         const int ml0 = ci * MC;
-        // A: groups of 4 pixels are inside the image or not as a whole (OHW % 4 == 0)
-        const bool a_ok = ml0 + 4 * a_q < p.OHW;
+        // A: groups of 4 pixels are inside the (padded) plane or not as a whole
+        const bool a_ok = ml0 + 4 * a_q < p.OHWa;
         ld_va0 = a_ok ? a_v0 : 0x80000000u;
         ld_va1 = a_ok ? a_v1 : 0x80000000u;
-        ld_sa = (uint32_t)((in_img * p.K + k0) * p.OHW + ml0) * 4u;
+        ld_sa = (uint32_t)((in_img * p.K + k0) * p.OHWa + ml0) * 4u;
         // B: the shifted input position of this lane's pixel
         const int ml = ml0 + b_m;
         const int oh = (int)xsmi::fdiv((uint32_t)ml, p.dOW);
@@ -285,6 +288,15 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__re
     }
 }
 
+// dst[plane][0 .. OHWa) = src[plane][0 .. OHW) followed by zeros
+__global__ void __launch_bounds__(256) pad_planes_kernel(const float *__restrict__ src, float *__restrict__ dst, int OHW,
+                                                          int OHWa, uint32_t total) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        const uint32_t pl = i / (uint32_t)OHWa, m = i - pl * (uint32_t)OHWa;
+        dst[i] = m < (uint32_t)OHW ? src[(size_t)pl * OHW + m] : 0.f;
+    }
+}
+
 void plan(int N, int C, int K, int R, int S, int OHW, int *cpi, int *total, int *cps, int *splits) {
     const int tiles = R * S * (C / TC) * (K / TK);
     *cpi = xsmi::ceil_div(OHW, MC);
@@ -302,13 +314,15 @@ void plan(int N, int C, int K, int R, int S, int OHW, int *cpi, int *total, int 
 namespace xsmi {
 
 bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW) {
-    return C % TC == 0 && K % TK == 0 && (OH * OW) % 4 == 0 && ((uintptr_t)dy % 16) == 0 && ((uintptr_t)x % 4) == 0;
+    return C % TC == 0 && K % TK == 0 && ((uintptr_t)dy % 16) == 0 && ((uintptr_t)x % 4) == 0;
 }
 
 size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW) {
     int cpi, total, cps, splits;
     plan(N, C, K, R, S, OH * OW, &cpi, &total, &cps, &splits);
-    return align_up((size_t)splits * R * S * K * C * sizeof(float), 256) + align_up((size_t)splits * K * sizeof(float), 256);
+    const int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
+    const size_t padded = OHWa != OHW ? align_up((size_t)N * K * OHWa * sizeof(float), 256) : 0;
+    return align_up((size_t)splits * R * S * K * C * sizeof(float), 256) + align_up((size_t)splits * K * sizeof(float), 256) + padded;
 }
 
 int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int C, int H, int W, int K, int R, int S,
@@ -319,16 +333,26 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     p.dy = dy; p.x = x;
     p.part = (float *)workspace;
     float *dbpart = (float *)((char *)workspace + align_up((size_t)splits * R * S * K * C * sizeof(float), 256));
+    hipStream_t st = stream();
+    const int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
+    if (OHWa != OHW) {
+        float *dyp = (float *)((char *)dbpart + align_up((size_t)splits * K * sizeof(float), 256));
+        const uint32_t total = (uint32_t)((size_t)N * K * OHWa);
+        uint32_t blocks = (total + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(pad_planes_kernel, dim3(blocks), dim3(256), 0, st, dy, dyp, OHW, OHWa, total);
+        XSMI_LAUNCH_CHECK("pad_planes_kernel");
+        p.dy = dyp;
+    }
     p.dbpart = db ? dbpart : nullptr;
     p.x_bytes = (uint32_t)((size_t)N * C * H * W * 4);
-    p.dy_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
-    p.N = N; p.C = C; p.K = K; p.H = H; p.W = W; p.OH = OH; p.OW = OW; p.OHW = OH * OW; p.R = R; p.S = S;
+    p.dy_bytes = (uint32_t)((size_t)N * K * OHWa * 4);
+    p.N = N; p.C = C; p.K = K; p.H = H; p.W = W; p.OH = OH; p.OW = OW; p.OHW = OHW; p.OHWa = OHWa; p.R = R; p.S = S;
     p.sh = sh; p.sw = sw; p.pad = pad;
     p.ctiles = C / TC;
-    p.xplane_bytes = (uint32_t)(H * W * 4); p.yplane_bytes = (uint32_t)(OH * OW * 4);
+    p.xplane_bytes = (uint32_t)(H * W * 4); p.yplane_bytes = (uint32_t)(OHWa * 4);
     p.dOW = make_fastdiv(OW); p.dCT = make_fastdiv(p.ctiles); p.dS = make_fastdiv(S);
 
-    hipStream_t st = stream();
     dim3 grid(R * S * p.ctiles, K / TK, splits);
     prof_begin();
     hipLaunchKernelGGL(wgrad_tap_f32_kernel, grid, dim3(256), 0, st, p);
