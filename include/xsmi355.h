@@ -164,6 +164,9 @@ int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size
 
 /* y[i] += a * x[i]                       (gradient accumulation; SGD: xs/optim/sgd.py:4-9) */
 int xsmi_axpy(float *y, const float *x, float a, size_t n);
+/* the same for `count` tensors in one or a few launches (one SGD step over all parameters);
+ * ys, xs, ns are host arrays of device pointers / element counts */
+int xsmi_axpy_multi(int count, float *const *ys, const float *const *xs, const size_t *ns, float a);
 /* out[i] = a[i] + b[i]                   (residual add, xs/nn/functional.py:6-21) */
 int xsmi_add(const float *a, const float *b, float *out, size_t n);
 /* out[i] = s * a[i] + t */
@@ -182,7 +185,10 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n);
  * biased variance.  Outputs xhat (N*C*HW), sqrtvar/mean/var (C).  ws: xsmi_bn_workspace_bytes(C). */
 size_t xsmi_bn_workspace_bytes(int C);
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
-                float *mean, float *var, int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
+                float *mean, float *var, float *moving_mean, float *moving_var, float momentum, int N, int C, int HW,
+                float eps, void *ws, size_t ws_bytes);
+/* moving_mean / moving_var (both or neither): m = momentum*m + (1-momentum)*batch statistic, the update the
+ * reference performs after the forward (xs/nn/functional.py:700-707), done by the statistics kernel. */
 /* Inference form with given statistics (xs/nn/functional.py:708-725). */
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
                   int N, int C, int HW, float eps);

@@ -1,0 +1,96 @@
+"""Device kernels next to the conv / pool path (batch norm, element-wise, reductions, dense GEMM, loss, SGD)
+against plain NumPy float64 formulas of the reference's expressions.  Tolerances are for float32 kernels."""
+import numpy as np
+import pytest
+
+from util import rel_l2
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.mark.parametrize("shape", [(4, 8, 6, 6), (32, 64, 14, 14), (5, 3, 7, 7), (2, 130, 9, 5), (64, 16)])
+def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
+    """xs/nn/functional.py:676-707 and xs/nn/grad_fn.py:379-411."""
+    K = gpu.kernels
+    rng = np.random.default_rng(sum(shape))
+    c = shape[1]
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, c).astype(np.float32); beta = rng.standard_normal(c).astype(np.float32)
+    mm0 = rng.standard_normal(c).astype(np.float32); mv0 = rng.uniform(0.5, 2.0, c).astype(np.float32)
+    dy = rng.standard_normal(shape).astype(np.float32)
+    axes = tuple(i for i in range(len(shape)) if i != 1)
+    b = [1, -1] + [1] * (len(shape) - 2)
+    x64 = x.astype(np.float64)
+    mean = x64.mean(axis=axes); var = x64.var(axis=axes); eps = 1e-5
+    sq = np.sqrt(var + eps)
+    xhat = (x64 - mean.reshape(b)) / sq.reshape(b)
+    y_ref = gamma.reshape(b) * xhat + beta.reshape(b)
+    mm, mv = gpu.to_device(mm0), gpu.to_device(mv0)
+    y, xh, sqv, mean_d, var_d = K.bn_fwd(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), eps,
+                                          moving=(mm, mv), momentum=0.9)
+    assert rel_l2(y.numpy(), y_ref) <= 1e-5 and rel_l2(xh.numpy(), xhat) <= 1e-5
+    np.testing.assert_allclose(mean_d.numpy(), mean, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(var_d.numpy(), var, rtol=1e-5)
+    np.testing.assert_allclose(mm.numpy(), 0.9 * mm0 + 0.1 * mean, rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(mv.numpy(), 0.9 * mv0 + 0.1 * var, rtol=1e-5)
+    m = x.size // c
+    dxh = dy.astype(np.float64) * gamma.reshape(b)
+    dx_ref = (dxh * m - dxh.sum(axis=axes).reshape(b) - xhat * (dxh * xhat).sum(axis=axes).reshape(b)) / (m * sq.reshape(b))
+    dx, dg, db = K.bn_bwd(gpu.to_device(dy), xh, sqv, gpu.to_device(gamma))
+    assert rel_l2(dx.numpy(), dx_ref) <= 2e-5
+    np.testing.assert_allclose(dg.numpy(), (dy * xhat).sum(axis=axes), rtol=2e-5, atol=1e-4)
+    np.testing.assert_allclose(db.numpy(), dy.astype(np.float64).sum(axis=axes), rtol=2e-5, atol=1e-4)
+    # inference form with the given statistics (xs/nn/functional.py:708-725)
+    yi = K.bn_infer(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), gpu.to_device(mm0), gpu.to_device(mv0), eps)
+    yi_ref = gamma.reshape(b) * (x64 - mm0.reshape(b)) / np.sqrt(mv0.reshape(b) + eps) + beta.reshape(b)
+    assert rel_l2(yi.numpy(), yi_ref) <= 1e-5
+
+
+def test_multi_tensor_axpy_is_one_sgd_step(gpu):
+    """xs/optim/sgd.py:4-9 over many parameters of ragged sizes, more than one launch group."""
+    K = gpu.kernels
+    rng = np.random.default_rng(2)
+    sizes = [1, 3, 1023, 1024, 1025, 4097, 64 * 64 * 9] + [int(v) for v in rng.integers(1, 5000, size=60)]
+    ps = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    gs = [rng.standard_normal(n).astype(np.float32) for n in sizes]
+    dp, dg = [gpu.to_device(p) for p in ps], [gpu.to_device(g) for g in gs]
+    K.axpy_multi(dp, dg, -0.05)
+    for p, g, d in zip(ps, gs, dp):
+        # the kernel may fuse the multiply-add (one rounding instead of two)
+        np.testing.assert_allclose(d.numpy(), p.astype(np.float64) - 0.05 * g.astype(np.float64), rtol=1e-6, atol=1e-7)
+    K.axpy_multi([], [], 1.0)                       # nothing to do is fine
+    with pytest.raises(ValueError):
+        K.axpy_multi([dp[0]], [dg[1]], 1.0)
+
+
+def test_dense_gemm_all_transposes(gpu):
+    """addmm forward and the two gradient products (xs/nn/functional.py:99-120, xs/nn/grad_fn.py:86-99)."""
+    K = gpu.kernels
+    rng = np.random.default_rng(3)
+    for (m, k, n) in ((32, 512, 1000), (7, 130, 33), (256, 64, 10), (1, 1, 1)):
+        a = rng.standard_normal((m, k)).astype(np.float32); b = rng.standard_normal((k, n)).astype(np.float32)
+        bias = rng.standard_normal(n).astype(np.float32); g = rng.standard_normal((m, n)).astype(np.float32)
+        da, db_, dg = gpu.to_device(a), gpu.to_device(b), gpu.to_device(g)
+        assert rel_l2(K.gemm(da, db_, bias=gpu.to_device(bias)).numpy(), a.astype(np.float64) @ b + bias) <= 1e-5
+        assert rel_l2(K.gemm(dg, db_, trans_b=True).numpy(), g.astype(np.float64) @ b.T) <= 1e-5
+        assert rel_l2(K.gemm(da, dg, trans_a=True).numpy(), a.T.astype(np.float64) @ g) <= 1e-5
+
+
+def test_softmax_cross_entropy(gpu):
+    """xs/nn/functional.py:984-1010 and xs/nn/grad_fn.py:604-620."""
+    K = gpu.kernels
+    rng = np.random.default_rng(4)
+    logits = (rng.standard_normal((37, 100)) * 3).astype(np.float32); labels = rng.integers(0, 100, size=37)
+    z = logits.astype(np.float64); z -= z.max(axis=1, keepdims=True)
+    sm = np.exp(z); sm /= sm.sum(axis=1, keepdims=True)
+    for reduction in ("mean", "sum"):
+        dl = gpu.to_device(labels.astype(np.int64), np.int64)
+        loss, smd = K.softmax_ce_fwd(gpu.to_device(logits), dl, reduction)
+        ref = -np.log(sm[np.arange(37), labels])
+        ref = ref.mean() if reduction == "mean" else ref.sum()
+        assert abs(float(np.asarray(loss.numpy()).reshape(-1)[0]) - ref) <= 1e-5 * abs(ref)
+        g = K.softmax_ce_bwd(smd, dl, reduction, 1.0).numpy()
+        gref = sm.copy(); gref[np.arange(37), labels] -= 1.0
+        if reduction == "mean":
+            gref /= 37
+        assert rel_l2(g, gref) <= 1e-5

@@ -65,6 +65,7 @@ SIGNATURES = {
     "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
     "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),
     "xsmi_axpy": (_i, [_vp, _vp, _f, _sz]),
+    "xsmi_axpy_multi": (_i, [_i, _c.POINTER(_vp), _c.POINTER(_vp), _c.POINTER(_sz), _f]),
     "xsmi_add": (_i, [_vp, _vp, _vp, _sz]),
     "xsmi_scale_shift": (_i, [_vp, _vp, _f, _f, _sz]),
     "xsmi_relu_fwd": (_i, [_vp, _vp, _sz]),
@@ -72,7 +73,7 @@ SIGNATURES = {
     "xsmi_relu_bwd": (_i, [_vp, _vp, _vp, _sz]),
     "xsmi_lerp": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_bn_workspace_bytes": (_sz, [_i]),
-    "xsmi_bn_fwd": (_i, [_vp] * 8 + [_i, _i, _i, _f, _vp, _sz]),
+    "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 7 + [_i, _i, _i, _vp, _sz]),
     "xsmi_avgpool_fwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),

@@ -197,6 +197,21 @@ def axpy(y, x, a):
     return y
 
 
+def axpy_multi(ys, xs, a):
+    """y += a * x for every pair, in one launch per 48 tensors (one optimizer step over all parameters)."""
+    n = len(ys)
+    if n == 0:
+        return
+    for y, x in zip(ys, xs):
+        _f32(y, "y"); _f32(x, "x")
+        if x.size != y.size:
+            raise ValueError("axpy_multi: %s vs %s" % (x.shape, y.shape))
+    yp = (ctypes.c_void_p * n)(*[y.ptr for y in ys])
+    xp = (ctypes.c_void_p * n)(*[x.ptr for x in xs])
+    ns = (ctypes.c_size_t * n)(*[y.size for y in ys])
+    lib.call("xsmi_axpy_multi", n, yp, xp, ns, float(a))
+
+
 def add(a, b, out=None):
     _f32(a, "a"); _f32(b, "b")
     out = _like(a, out)
@@ -252,14 +267,19 @@ def _nchw3(shape):
     return int(n), int(c), int(hw)
 
 
-def bn_fwd(x, gamma, beta, eps, y=None):
+def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0):
+    """``moving=(moving_mean, moving_var)`` device arrays are updated in place: m = momentum*m + (1-momentum)*stat."""
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
     y = _like(x, y); xhat = empty(x.shape)
     y.take_fresh()
     sqrtvar = empty((c,)); mean = empty((c,)); var = empty((c,))
+    mm, mv = moving if moving is not None else (None, None)
+    if mm is not None and (mm.size != c or mv.size != c):
+        raise ValueError("bn_fwd: moving statistics must have %d elements" % c)
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
     lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr, sqrtvar.cptr, mean.cptr, var.cptr,
+             mm.cptr if mm is not None else None, mv.cptr if mv is not None else None, float(momentum),
              n, c, hw, float(eps), ws, ws_bytes)
     return y, xhat, sqrtvar, mean, var
 

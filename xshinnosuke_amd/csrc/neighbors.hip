@@ -102,6 +102,35 @@ int launch_ew(const char *name, size_t n, int vec, F f) {
     return XSMI_OK;
 }
 
+// y_t[i] += a * x_t[i] for up to AXPY_GROUP tensors in one launch: the tensors are concatenated in units of
+// 1024 elements (one workgroup each); first[t] is the first workgroup of tensor t.  The table travels in the
+// kernel arguments, so no device-side pointer array has to be kept up to date.
+constexpr int AXPY_GROUP = 48;
+struct AxpyMulti {
+    float *y[AXPY_GROUP];
+    const float *x[AXPY_GROUP];
+    uint32_t n[AXPY_GROUP];
+    uint32_t first[AXPY_GROUP + 1];
+    int count;
+    float a;
+};
+__global__ void __launch_bounds__(256) axpy_multi_kernel(AxpyMulti m) {
+    int lo = 0, hi = m.count - 1;                    // last tensor whose first workgroup is <= blockIdx.x
+    while (lo < hi) {
+        const int mid = (lo + hi + 1) >> 1;
+        if (m.first[mid] <= blockIdx.x) lo = mid; else hi = mid - 1;
+    }
+    float *y = m.y[lo];
+    const float *x = m.x[lo];
+    const uint32_t n = m.n[lo];
+    const uint32_t base = (blockIdx.x - m.first[lo]) * 1024u;
+#pragma unroll
+    for (int u = 0; u < 4; ++u) {
+        const uint32_t i = base + u * 256u + threadIdx.x;
+        if (i < n) y[i] += m.a * x[i];
+    }
+}
+
 // ---- block reductions ------------------------------------------------------
 __device__ __forceinline__ double wave_sum(double v) {
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
@@ -181,7 +210,7 @@ static int bn_splits(int N, int HW) {
     return (int)s;
 }
 __global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar, float *mean, float *var, int C, double m,
-                                float eps, int nsplit) {
+                                float eps, int nsplit, float *moving_mean, float *moving_var, float momentum) {
     int c = blockIdx.x * 256 + threadIdx.x;
     if (c >= C) return;
     double s0 = 0.0, s1 = 0.0;
@@ -195,6 +224,10 @@ __global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar,
     mean[c] = (float)mu;
     var[c] = (float)v;
     sqrtvar[c] = (float)sqrt(v + (double)eps);
+    if (moving_mean) {                               // m = momentum*m + (1-momentum)*cur, as xsmi_lerp computes it
+        moving_mean[c] = momentum * moving_mean[c] + (1.f - momentum) * (float)mu;
+        moving_var[c] = momentum * moving_var[c] + (1.f - momentum) * (float)v;
+    }
 }
 __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                         const float *__restrict__ beta, const float *__restrict__ mean,
@@ -375,6 +408,30 @@ int xsmi_axpy(float *y, const float *x, float a, size_t n) {
     XSMI_CHECK_ARG(n == 0 || (y && x), "xsmi_axpy: null pointer");
     return launch_ew("axpy", n, aligned16(y) && aligned16(x), AxpyF{y, x, a});
 }
+int xsmi_axpy_multi(int count, float *const *ys, const float *const *xs, const size_t *ns, float a) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(count >= 0 && (count == 0 || (ys && xs && ns)), "xsmi_axpy_multi: bad argument");
+    for (int done = 0; done < count;) {
+        AxpyMulti m;
+        m.a = a;
+        m.count = 0;
+        uint32_t blocks = 0;
+        for (; done < count && m.count < AXPY_GROUP; ++done) {
+            if (ns[done] == 0) continue;
+            XSMI_CHECK_ARG(ys[done] && xs[done], "xsmi_axpy_multi: null pointer in tensor %d", done);
+            XSMI_CHECK_ARG(ns[done] < 4294967296.0, "xsmi_axpy_multi: tensor %d too large", done);
+            m.y[m.count] = ys[done]; m.x[m.count] = xs[done]; m.n[m.count] = (uint32_t)ns[done];
+            m.first[m.count] = blocks;
+            blocks += (uint32_t)((ns[done] + 1023) / 1024);
+            ++m.count;
+        }
+        if (m.count == 0) break;
+        m.first[m.count] = blocks;
+        hipLaunchKernelGGL(axpy_multi_kernel, dim3(blocks), dim3(256), 0, xsmi::stream(), m);
+        XSMI_LAUNCH_CHECK("axpy_multi_kernel");
+    }
+    return XSMI_OK;
+}
 int xsmi_add(const float *a, const float *b, float *out, size_t n) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add: null pointer");
@@ -410,11 +467,13 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n) {
 size_t xsmi_bn_workspace_bytes(int C) { return C > 0 ? (size_t)C * BN_SPLIT * 2 * sizeof(double) : 0; }
 
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar, float *mean,
-                float *var, int N, int C, int HW, float eps, void *ws, size_t ws_bytes) {
+                float *var, float *moving_mean, float *moving_var, float momentum, int N, int C, int HW, float eps,
+                void *ws, size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_fwd: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_fwd: tensors of 2^29 elements or more are not supported");
     XSMI_CHECK_ARG(x && gamma && beta && y && sqrtvar && mean && var, "xsmi_bn_fwd: null pointer");
+    XSMI_CHECK_ARG((moving_mean == nullptr) == (moving_var == nullptr), "xsmi_bn_fwd: give both moving statistics or neither");
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
@@ -422,7 +481,7 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, x, (const float *)nullptr, part, N, C, HW, nsplit);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
-                       (double)N * HW, eps, nsplit);
+                       (double)N * HW, eps, nsplit, moving_mean, moving_var, momentum);
     XSMI_LAUNCH_CHECK("bn_stats_kernel");
     size_t total = (size_t)N * C * HW;
     hipLaunchKernelGGL(bn_apply_kernel, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y, xhat,

@@ -130,12 +130,13 @@ def fill_like(a, value):
     return np.full(a.shape, value, dtype=a.dtype)
 
 
-def batch_norm_train(x, gamma, beta, eps, out=None):
+def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0):
     """Per-channel batch statistics over (N, H, W) or (N,).  Returns y, xhat, sqrtvar, mean, var.  A device
-    ``out`` of the right size receives y directly."""
+    ``out`` of the right size receives y directly; device ``moving`` statistics are updated by the same call
+    (host ones are left to the caller)."""
     if is_device(x):
         y = out if (out is not None and is_device(out) and out.size == x.size) else None
-        return K.bn_fwd(x, same_place(x, gamma), same_place(x, beta), eps, y=y)
+        return K.bn_fwd(x, same_place(x, gamma), same_place(x, beta), eps, y=y, moving=moving, momentum=momentum)
     axes = tuple(i for i in range(x.ndim) if i != 1)
     mean = x.mean(axis=axes, keepdims=True)
     var = x.var(axis=axes, keepdims=True)
@@ -215,6 +216,17 @@ def softmax_cross_entropy_grad(sm, labels, reduction, upstream):
         g /= sm.shape[0]
     g *= np.asarray(upstream).reshape(-1)[0]
     return g.reshape(sm.shape)
+
+
+def sgd_step_all(pairs, lr):
+    """param -= lr * grad for every (param, grad) pair; the device-resident pairs share one launch."""
+    dev_p, dev_g = [], []
+    for param, grad in pairs:
+        if is_device(param) and is_device(grad) and param.dtype == np.float32 and grad.dtype == np.float32:
+            dev_p.append(param); dev_g.append(grad)
+        else:
+            sgd_step(param, grad, lr)
+    K.axpy_multi(dev_p, dev_g, -float(lr))
 
 
 def sgd_step(param, grad, lr):

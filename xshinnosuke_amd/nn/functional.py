@@ -362,15 +362,19 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
     xhat = sqrtvar = None
     dst = None if out is None else out.eval
     if training:
-        y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst)
-        for mov, cur in ((moving_mean, mean_), (moving_variance, var_)):
-            m = mov.eval
-            cur = A.same_place(m, cur)
-            if is_device(m):
-                K.lerp_(m, cur, momentum)                       # m = momentum*m + (1-momentum)*cur
-            else:
-                m *= momentum
-                m += (1 - momentum) * np.asarray(cur).reshape(m.shape)
+        mm, mv = moving_mean.eval, moving_variance.eval
+        fused = is_device(x) and is_device(mm) and is_device(mv)      # the statistics kernel updates them
+        y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst,
+                                                           (mm.reshape(-1), mv.reshape(-1)) if fused else None, momentum)
+        if not fused:
+            for mov, cur in ((moving_mean, mean_), (moving_variance, var_)):
+                m = mov.eval
+                cur = A.same_place(m, cur)
+                if is_device(m):
+                    K.lerp_(m, cur, momentum)                   # m = momentum*m + (1-momentum)*cur
+                else:
+                    m *= momentum
+                    m += (1 - momentum) * np.asarray(cur).reshape(m.shape)
     else:
         y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon, dst)
     if out is None:

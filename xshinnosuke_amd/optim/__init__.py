@@ -21,9 +21,8 @@ class Optimizer:
 class SGD(Optimizer):
     def step(self):
         """v -= lr * v.grad for every trainable parameter (reference xs/optim/sgd.py:4-9)."""
-        for v in self._parameters:
-            if v.requires_grad and v.grad is not None:
-                A.sgd_step(v.eval, v.grad.eval, self.lr)
+        A.sgd_step_all([(v.eval, v.grad.eval) for v in self._parameters if v.requires_grad and v.grad is not None],
+                       self.lr)
         super().step()
 
 
