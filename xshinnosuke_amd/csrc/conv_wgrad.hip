@@ -173,25 +173,45 @@ __global__ void __launch_bounds__(256) wgrad_f32_kernel(WgradParams p) {
     }
 }
 
+// dw[k][j] = beta*dw + sum over splits of part[split][k][j]; blocks past the last dw block do the same for
+// db[k] from dbpart[split][k].  256 threads = 64 consecutive columns x 4 interleaved split groups with two
+// running sums each; the groups are combined in a fixed order, all in float64 (deterministic, no atomics).
 __global__ void __launch_bounds__(256) wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ dw,
-                                                            int K, int J, int Kp, int Jp, int splits, int accumulate) {
-    int i = blockIdx.x * 256 + threadIdx.x;
-    if (i >= K * J) return;
-    int k = i / J, j = i - k * J;
-    double s = 0.0;
-    for (int sp = 0; sp < splits; ++sp) s += (double)part[((size_t)sp * Kp + k) * Jp + j];
-    if (accumulate) s += (double)dw[i];
-    dw[i] = (float)s;
-}
-
-__global__ void __launch_bounds__(256) dbias_reduce_kernel(const float *__restrict__ dbpart, float *__restrict__ db,
-                                                            int K, int Kp, int splits, int accumulate) {
-    int k = blockIdx.x * 256 + threadIdx.x;
-    if (k >= K) return;
-    double s = 0.0;
-    for (int sp = 0; sp < splits; ++sp) s += (double)dbpart[(size_t)sp * Kp + k];
-    if (accumulate) s += (double)db[k];
-    db[k] = (float)s;
+                                                            const float *__restrict__ dbpart, float *__restrict__ db,
+                                                            int K, int J, int Kp, int Jp, int splits, int dw_blocks,
+                                                            int accumulate) {
+    __shared__ double sm[4][64];
+    const int cl = threadIdx.x & 63, g = threadIdx.x >> 6;
+    const int jt = (J + 63) / 64;
+    const bool bias_block = (int)blockIdx.x >= dw_blocks;      // uniform per block
+    const float *src = nullptr;
+    float *dst = nullptr;
+    size_t stride = 0;
+    if (bias_block) {
+        const int k = ((int)blockIdx.x - dw_blocks) * 64 + cl;
+        if (k < K) { src = dbpart + k; dst = db + k; }
+        stride = (size_t)Kp;
+    } else {
+        const int k = (int)blockIdx.x / jt, j = ((int)blockIdx.x - k * jt) * 64 + cl;
+        if (j < J) { src = part + (size_t)k * Jp + j; dst = dw + (size_t)k * J + j; }
+        stride = (size_t)Kp * Jp;
+    }
+    double s0 = 0.0, s1 = 0.0;
+    if (src) {
+        int sp = g;
+        for (; sp + 4 < splits; sp += 8) {
+            s0 += (double)src[(size_t)sp * stride];
+            s1 += (double)src[(size_t)(sp + 4) * stride];
+        }
+        if (sp < splits) s0 += (double)src[(size_t)sp * stride];
+    }
+    sm[g][cl] = s0 + s1;
+    __syncthreads();
+    if (g == 0 && dst) {
+        double s = ((sm[0][cl] + sm[1][cl]) + sm[2][cl]) + sm[3][cl];
+        if (accumulate) s += (double)*dst;
+        *dst = (float)s;
+    }
 }
 
 void plan_splits(int M, int K, int J, int *splits, int *chunks_per_split) {
@@ -271,14 +291,10 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
     xsmi::prof_end();
     XSMI_LAUNCH_CHECK("wgrad_f32_kernel");
     const int acc = beta == 1.f ? 1 : 0;
-    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(xsmi::ceil_div(K * p.J, 256)), dim3(256), 0, st, p.part, dw, K, p.J,
-                       p.Kp, p.Jp, splits, acc);
+    const int dw_blocks = K * xsmi::ceil_div(p.J, 64);
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(dw_blocks + (db ? xsmi::ceil_div(K, 64) : 0)), dim3(256), 0, st, p.part, dw,
+                       dbpart, db, K, p.J, p.Kp, p.Jp, splits, dw_blocks, acc);
     XSMI_LAUNCH_CHECK("wgrad_reduce_kernel");
-    if (db) {
-        hipLaunchKernelGGL(dbias_reduce_kernel, dim3(xsmi::ceil_div(K, 256)), dim3(256), 0, st, dbpart, db, K, p.Kp,
-                           splits, acc);
-        XSMI_LAUNCH_CHECK("dbias_reduce_kernel");
-    }
     return XSMI_OK;
 }
 
