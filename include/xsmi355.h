@@ -185,17 +185,21 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n);
  * biased variance.  Outputs xhat (N*C*HW), sqrtvar/mean/var (C).  ws: xsmi_bn_workspace_bytes(C). */
 size_t xsmi_bn_workspace_bytes(int C);
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
-                float *mean, float *var, float *moving_mean, float *moving_var, float momentum, int N, int C, int HW,
-                float eps, void *ws, size_t ws_bytes);
+                float *mean, float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask,
+                int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
 /* moving_mean / moving_var (both or neither): m = momentum*m + (1-momentum)*batch statistic, the update the
- * reference performs after the forward (xs/nn/functional.py:700-707), done by the statistics kernel. */
-/* Inference form with given statistics (xs/nn/functional.py:708-725). */
+ * reference performs after the forward (xs/nn/functional.py:700-707), done by the statistics kernel.
+ * neg_mask (or NULL) fuses the ReLU that follows the normalisation in a residual block
+ * (xs/layers/activators.py:37-50): neg_mask[i] = pre-activation < 0, y = max(pre-activation, 0). */
+/* Inference form with given statistics (xs/nn/functional.py:708-725); relu != 0 clips at zero. */
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
-                  int N, int C, int HW, float eps);
+                  int N, int C, int HW, float eps, int relu);
 /* Backward (xs/nn/grad_fn.py:379-411): dgamma = sum(dy*xhat), dbeta = sum(dy),
- * dx = gamma / (m*sqrtvar) * (m*dy - dbeta - xhat*dgamma), m = N*HW.  All three are overwritten. */
-int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, float *dx, float *dgamma,
-                float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes);
+ * dx = gamma / (m*sqrtvar) * (m*dy - dbeta - xhat*dgamma), m = N*HW.  All three are overwritten.
+ * With neg_mask (the byte mask of a fused ReLU) dy counts as 0 where the mask is set (strict mask,
+ * xs/nn/grad_fn.py:146-157). */
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, const uint8_t *neg_mask,
+                float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes);
 
 /* Mean over non-overlapping k x k blocks of an NCHW tensor and its gradient
  * (the live mode of avg_pool2d, xs/nn/functional.py:539-583, xs/nn/grad_fn.py:284-309). */

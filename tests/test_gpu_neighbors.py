@@ -40,10 +40,24 @@ def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     assert rel_l2(dx.numpy(), dx_ref) <= 2e-5
     np.testing.assert_allclose(dg.numpy(), (dy * xhat).sum(axis=axes), rtol=2e-5, atol=1e-4)
     np.testing.assert_allclose(db.numpy(), dy.astype(np.float64).sum(axis=axes), rtol=2e-5, atol=1e-4)
+    # fused ReLU: clipped output, strict mask, and a backward that ignores the clipped gradient entries
+    mask = gpu.empty(shape, np.uint8)
+    yr, xh2, sqv2, _, _ = K.bn_fwd(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), eps, neg_mask=mask)
+    np.testing.assert_array_equal(yr.numpy(), np.maximum(y.numpy(), 0))
+    np.testing.assert_array_equal(mask.numpy(), (y.numpy() < 0).astype(np.uint8))
+    dym = np.where(y.numpy() < 0, np.float32(0), dy)
+    dx2, dg2, db2 = K.bn_bwd(gpu.to_device(dy), xh2, sqv2, gpu.to_device(gamma), neg_mask=mask)
+    dx3, dg3, db3 = K.bn_bwd(gpu.to_device(dym), xh2, sqv2, gpu.to_device(gamma))
+    np.testing.assert_array_equal(dx2.numpy(), dx3.numpy())
+    np.testing.assert_array_equal(dg2.numpy(), dg3.numpy())
+    np.testing.assert_array_equal(db2.numpy(), db3.numpy())
     # inference form with the given statistics (xs/nn/functional.py:708-725)
     yi = K.bn_infer(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), gpu.to_device(mm0), gpu.to_device(mv0), eps)
     yi_ref = gamma.reshape(b) * (x64 - mm0.reshape(b)) / np.sqrt(mv0.reshape(b) + eps) + beta.reshape(b)
     assert rel_l2(yi.numpy(), yi_ref) <= 1e-5
+    yir = K.bn_infer(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), gpu.to_device(mm0), gpu.to_device(mv0), eps,
+                     relu=True)
+    np.testing.assert_array_equal(yir.numpy(), np.maximum(yi.numpy(), 0))
 
 
 def test_multi_tensor_axpy_is_one_sgd_step(gpu):

@@ -267,8 +267,9 @@ def _nchw3(shape):
     return int(n), int(c), int(hw)
 
 
-def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0):
-    """``moving=(moving_mean, moving_var)`` device arrays are updated in place: m = momentum*m + (1-momentum)*stat."""
+def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None):
+    """``moving=(moving_mean, moving_var)`` device arrays are updated in place: m = momentum*m + (1-momentum)*stat.
+    A uint8 ``neg_mask`` of x's size fuses a ReLU: it receives pre-activation < 0 and y is clipped at 0."""
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
     y = _like(x, y); xhat = empty(x.shape)
@@ -280,20 +281,22 @@ def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0):
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
     lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr, sqrtvar.cptr, mean.cptr, var.cptr,
              mm.cptr if mm is not None else None, mv.cptr if mv is not None else None, float(momentum),
-             n, c, hw, float(eps), ws, ws_bytes)
+             neg_mask.cptr if neg_mask is not None else None, n, c, hw, float(eps), ws, ws_bytes)
     return y, xhat, sqrtvar, mean, var
 
 
-def bn_infer(x, gamma, beta, mean, var, eps, y=None):
+def bn_infer(x, gamma, beta, mean, var, eps, y=None, relu=False):
     n, c, hw = _nchw3(x.shape)
     y = _like(x, y)
     y.take_fresh()
-    lib.call("xsmi_bn_infer", x.cptr, gamma.cptr, beta.cptr, mean.cptr, var.cptr, y.cptr, n, c, hw, float(eps))
+    lib.call("xsmi_bn_infer", x.cptr, gamma.cptr, beta.cptr, mean.cptr, var.cptr, y.cptr, n, c, hw, float(eps),
+             1 if relu else 0)
     return y
 
 
-def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None):
-    """dx, dgamma, dbeta; buffers passed in are overwritten completely."""
+def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=None):
+    """dx, dgamma, dbeta; buffers passed in are overwritten completely.  ``neg_mask`` is the byte mask of a fused
+    ReLU: the upstream gradient counts as 0 where it is set."""
     n, c, hw = _nchw3(dy.shape)
     dx = empty(dy.shape) if dx is None else dx
     dgamma = empty((c,)) if dgamma is None else dgamma
@@ -303,8 +306,8 @@ def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None):
     for o in (dx, dgamma, dbeta):
         o.take_fresh()
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
-    lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, sqrtvar.cptr, gamma.cptr, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw,
-             ws, ws_bytes)
+    lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, sqrtvar.cptr, gamma.cptr,
+             neg_mask.cptr if neg_mask is not None else None, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw, ws, ws_bytes)
     return dx, dgamma, dbeta
 
 

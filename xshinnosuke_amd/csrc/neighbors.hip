@@ -163,8 +163,11 @@ inline ChanIdx make_chan(int C, int HW) {
 
 // ---- batch norm --------------------------------------------------------------
 // pass 1: per (channel, split) partial sums of a and a*b over the N*HW elements of the channel
+// `zero` (optional, one byte per element): elements whose byte is set count as a == 0 (the gradient of a fused
+// ReLU that was clipped)
 __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict__ a, const float *__restrict__ b,
-                                                          double *__restrict__ part, int N, int C, int HW, int nsplit) {
+                                                          const uint8_t *__restrict__ zero, double *__restrict__ part,
+                                                          int N, int C, int HW, int nsplit) {
     __shared__ double sm[4];
     const int c = blockIdx.x, sp = blockIdx.y;
     double s0 = 0.0, s1 = 0.0;
@@ -176,7 +179,14 @@ __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict
         for (uint32_t e = threadIdx.x; e < total; e += 256) {
             const uint32_t j = e / U, i = e - j * U;
             const size_t base = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW;
-            const float4 u = reinterpret_cast<const float4 *>(a + base)[i];
+            float4 u = reinterpret_cast<const float4 *>(a + base)[i];
+            if (zero) {
+                const uchar4 z = reinterpret_cast<const uchar4 *>(zero + base)[i];
+                if (z.x) u.x = 0.f;
+                if (z.y) u.y = 0.f;
+                if (z.z) u.z = 0.f;
+                if (z.w) u.w = 0.f;
+            }
             const float4 v = b ? reinterpret_cast<const float4 *>(b + base)[i] : u;
             s0 += ((double)u.x + (double)u.y) + ((double)u.z + (double)u.w);
             s1 += ((double)u.x * (double)v.x + (double)u.y * (double)v.y) +
@@ -187,7 +197,7 @@ __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict
         for (uint32_t e = threadIdx.x; e < total; e += 256) {
             const uint32_t j = e / U, i = e - j * U;
             const size_t off = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW + i;
-            const float u = a[off];
+            const float u = (zero && zero[off]) ? 0.f : a[off];
             const float v = b ? b[off] : u;
             s0 += (double)u;
             s1 += (double)u * (double)v;
@@ -229,15 +239,37 @@ __global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar,
         moving_var[c] = momentum * moving_var[c] + (1.f - momentum) * (float)v;
     }
 }
+// VEC: four consecutive elements per thread (HW % 4 == 0, so they share a channel and planes are 16-byte
+// aligned).  neg_mask != nullptr fuses a ReLU: mask = pre-activation < 0, y = max(pre-activation, 0).
+template <bool VEC>
 __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                         const float *__restrict__ beta, const float *__restrict__ mean,
                                                         const float *__restrict__ sqrtvar, float *__restrict__ y,
-                                                        float *__restrict__ xhat, ChanIdx chan, uint32_t total) {
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-        int c = chan(i);
-        float h = (x[i] - mean[c]) / sqrtvar[c];
-        if (xhat) xhat[i] = h;
-        y[i] = gamma[c] * h + beta[c];
+                                                        float *__restrict__ xhat, uint8_t *__restrict__ neg_mask,
+                                                        ChanIdx chan, uint32_t total) {
+    constexpr int W = VEC ? 4 : 1;
+    for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
+        const int c = chan(i);
+        const float mu = mean[c], rs = sqrtvar[c], g = gamma[c], bt = beta[c];
+        float xv[W], hv[W], yv[W];
+        unsigned char mv[W];
+        if (VEC) *reinterpret_cast<float4 *>(xv) = *reinterpret_cast<const float4 *>(x + i); else xv[0] = x[i];
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            hv[e] = (xv[e] - mu) / rs;
+            const float pre = g * hv[e] + bt;
+            mv[e] = pre < 0.f ? 1 : 0;
+            yv[e] = (neg_mask && pre < 0.f) ? 0.f : pre;
+        }
+        if (VEC) {
+            if (xhat) *reinterpret_cast<float4 *>(xhat + i) = *reinterpret_cast<float4 *>(hv);
+            *reinterpret_cast<float4 *>(y + i) = *reinterpret_cast<float4 *>(yv);
+            if (neg_mask) *reinterpret_cast<uchar4 *>(neg_mask + i) = make_uchar4(mv[0], mv[1], mv[2], mv[3]);
+        } else {
+            if (xhat) xhat[i] = hv[0];
+            y[i] = yv[0];
+            if (neg_mask) neg_mask[i] = mv[0];
+        }
     }
 }
 __global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgamma, float *dbeta, int C, int nsplit) {
@@ -251,15 +283,33 @@ __global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgam
     dbeta[c] = (float)s0;
     dgamma[c] = (float)s1;
 }
+template <bool VEC>
 __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
                                                             const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
                                                             const float *__restrict__ dgamma, const float *__restrict__ dbeta,
-                                                            float *__restrict__ dx, ChanIdx chan, uint32_t total, float m) {
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-        int c = chan(i);
-        float g = gamma[c];
-        // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
-        dx[i] = g * (m * dy[i] - dbeta[c] - xhat[i] * dgamma[c]) / (m * sqrtvar[c]);
+                                                            const uint8_t *__restrict__ zero, float *__restrict__ dx,
+                                                            ChanIdx chan, uint32_t total, float m) {
+    constexpr int W = VEC ? 4 : 1;
+    for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
+        const int c = chan(i);
+        const float g = gamma[c], db = dbeta[c], dg = dgamma[c], den = m * sqrtvar[c];
+        float gv[W], hv[W], ov[W];
+        unsigned char zv[W];
+        if (VEC) {
+            *reinterpret_cast<float4 *>(gv) = *reinterpret_cast<const float4 *>(dy + i);
+            *reinterpret_cast<float4 *>(hv) = *reinterpret_cast<const float4 *>(xhat + i);
+            if (zero) *reinterpret_cast<uchar4 *>(zv) = *reinterpret_cast<const uchar4 *>(zero + i);
+        } else {
+            gv[0] = dy[i]; hv[0] = xhat[i];
+            if (zero) zv[0] = zero[i];
+        }
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            const float d = (zero && zv[e]) ? 0.f : gv[e];
+            // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
+            ov[e] = g * (m * d - db - hv[e] * dg) / den;
+        }
+        if (VEC) *reinterpret_cast<float4 *>(dx + i) = *reinterpret_cast<float4 *>(ov); else dx[i] = ov[0];
     }
 }
 
@@ -467,8 +517,8 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n) {
 size_t xsmi_bn_workspace_bytes(int C) { return C > 0 ? (size_t)C * BN_SPLIT * 2 * sizeof(double) : 0; }
 
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar, float *mean,
-                float *var, float *moving_mean, float *moving_var, float momentum, int N, int C, int HW, float eps,
-                void *ws, size_t ws_bytes) {
+                float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask, int N, int C, int HW,
+                float eps, void *ws, size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_fwd: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_fwd: tensors of 2^29 elements or more are not supported");
@@ -478,14 +528,21 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
     const int nsplit = bn_splits(N, HW);
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, x, (const float *)nullptr, part, N, C, HW, nsplit);
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, x, (const float *)nullptr,
+                       (const uint8_t *)nullptr, part, N, C, HW, nsplit);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
                        (double)N * HW, eps, nsplit, moving_mean, moving_var, momentum);
     XSMI_LAUNCH_CHECK("bn_stats_kernel");
     size_t total = (size_t)N * C * HW;
-    hipLaunchKernelGGL(bn_apply_kernel, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y, xhat,
-                       make_chan(C, HW), (uint32_t)total);
+    const bool vec = (HW & 3) == 0 && aligned16(x) && aligned16(y) && (!xhat || aligned16(xhat)) &&
+                     (!neg_mask || ((uintptr_t)neg_mask & 3) == 0);
+    if (vec)
+        hipLaunchKernelGGL(bn_apply_kernel<true>, grid_for(total / 4), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y,
+                           xhat, neg_mask, make_chan(C, HW), (uint32_t)total);
+    else
+        hipLaunchKernelGGL(bn_apply_kernel<false>, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y,
+                           xhat, neg_mask, make_chan(C, HW), (uint32_t)total);
     XSMI_LAUNCH_CHECK("bn_apply_kernel");
     return XSMI_OK;
 }
@@ -493,28 +550,29 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
 __global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                         const float *__restrict__ beta, const float *__restrict__ mean,
                                                         const float *__restrict__ var, float *__restrict__ y, ChanIdx chan,
-                                                        uint32_t total, float eps) {
+                                                        uint32_t total, float eps, int relu) {
     for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
         int c = chan(i);
-        y[i] = gamma[c] * ((x[i] - mean[c]) / sqrtf(var[c] + eps)) + beta[c];
+        float v = gamma[c] * ((x[i] - mean[c]) / sqrtf(var[c] + eps)) + beta[c];
+        y[i] = (relu && v < 0.f) ? 0.f : v;
     }
 }
 
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
-                  int N, int C, int HW, float eps) {
+                  int N, int C, int HW, float eps, int relu) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_infer: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_infer: tensors of 2^29 elements or more are not supported");
     XSMI_CHECK_ARG(x && gamma && beta && mean && var && y, "xsmi_bn_infer: null pointer");
     size_t total = (size_t)N * C * HW;
     hipLaunchKernelGGL(bn_infer_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean, var, y,
-                       make_chan(C, HW), (uint32_t)total, eps);
+                       make_chan(C, HW), (uint32_t)total, eps, relu);
     XSMI_LAUNCH_CHECK("bn_infer_kernel");
     return XSMI_OK;
 }
 
-int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, float *dx, float *dgamma,
-                float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes) {
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, const uint8_t *neg_mask,
+                float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_bwd: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_bwd: tensors of 2^29 elements or more are not supported");
@@ -523,13 +581,19 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const 
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
     const int nsplit = bn_splits(N, HW);
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, dy, xhat, part, N, C, HW, nsplit);
+    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, dy, xhat, neg_mask, part, N, C, HW, nsplit);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C, nsplit);
     XSMI_LAUNCH_CHECK("bn_bwd_stats_kernel");
     size_t total = (size_t)N * C * HW;
-    hipLaunchKernelGGL(bn_bwd_apply_kernel, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, dx,
-                       make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
+    const bool vec = (HW & 3) == 0 && aligned16(dy) && aligned16(xhat) && aligned16(dx) &&
+                     (!neg_mask || ((uintptr_t)neg_mask & 3) == 0);
+    if (vec)
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<true>, grid_for(total / 4), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
+                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
+    else
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<false>, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
+                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
     XSMI_LAUNCH_CHECK("bn_bwd_apply_kernel");
     return XSMI_OK;
 }

@@ -25,8 +25,10 @@ class BatchNormalization(Layer):
         self.moving_mean = self.moving_mean_initializer(n_in)
         self.moving_variance = self.moving_variance_initializer(n_in)
 
-    def call(self, x, *args, **kwargs):
+    def call(self, x, *args, fuse_relu=False, **kwargs):
+        """``fuse_relu`` is set by Sequential when an in-place ReLU layer follows on a device-resident dynamic
+        graph: the normalisation kernel then applies it."""
         gamma, beta = self._parameters
         self._data = F.batch_norm(x, gamma, beta, self.moving_mean, self.moving_variance, self.axis, GLOBAL.TRAINING,
-                                  self.epsilon, self.momentum, self._data)
+                                  self.epsilon, self.momentum, self._data, 'relu' if fuse_relu else None)
         return self._data

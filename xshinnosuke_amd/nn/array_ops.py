@@ -130,13 +130,14 @@ def fill_like(a, value):
     return np.full(a.shape, value, dtype=a.dtype)
 
 
-def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0):
+def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0, neg_mask=None):
     """Per-channel batch statistics over (N, H, W) or (N,).  Returns y, xhat, sqrtvar, mean, var.  A device
     ``out`` of the right size receives y directly; device ``moving`` statistics are updated by the same call
     (host ones are left to the caller)."""
     if is_device(x):
         y = out if (out is not None and is_device(out) and out.size == x.size) else None
-        return K.bn_fwd(x, same_place(x, gamma), same_place(x, beta), eps, y=y, moving=moving, momentum=momentum)
+        return K.bn_fwd(x, same_place(x, gamma), same_place(x, beta), eps, y=y, moving=moving, momentum=momentum,
+                        neg_mask=neg_mask)
     axes = tuple(i for i in range(x.ndim) if i != 1)
     mean = x.mean(axis=axes, keepdims=True)
     var = x.var(axis=axes, keepdims=True)
@@ -148,10 +149,11 @@ def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0):
     return y.astype(x.dtype, copy=False), xhat, sqrtvar, mean.ravel(), var.ravel()
 
 
-def batch_norm_infer(x, gamma, beta, mean, var, eps, out=None):
+def batch_norm_infer(x, gamma, beta, mean, var, eps, out=None, relu=False):
     if is_device(x):
         y = out if (out is not None and is_device(out) and out.size == x.size) else None
-        return K.bn_infer(x, same_place(x, gamma), same_place(x, beta), same_place(x, mean), same_place(x, var), eps, y=y)
+        return K.bn_infer(x, same_place(x, gamma), same_place(x, beta), same_place(x, mean), same_place(x, var), eps, y=y,
+                          relu=relu)
     bshape = [1] * x.ndim
     bshape[1] = -1
     y = (x - mean.reshape(bshape)) / np.sqrt(var.reshape(bshape) + eps)

@@ -353,19 +353,33 @@ def avg_pool2d(inputs, kernel_size, stride=None, padding=0, out=None):
 
 
 def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, training=True, epsilon=1e-5,
-               momentum=0.9, out=None):
-    """Per-channel batch normalisation over axis 1 (reference xs/nn/functional.py:676-740)."""
+               momentum=0.9, out=None, activation=None):
+    """Per-channel batch normalisation over axis 1 (reference xs/nn/functional.py:676-740).
+
+    ``activation='relu'`` (device tensors only) is this package's extension, the counterpart of conv2d's: the
+    ReLU that follows the normalisation is applied by the same kernel and its strict ``pre < 0`` mask is kept for
+    the backward, which then needs no pass of its own either."""
     _mark_input(inputs)
     if axis != 1:
         raise NotImplementedError('batch_norm normalises over axis 1 only')
     x = inputs.eval
+    if activation not in (None, 'relu'):
+        raise ValueError("batch_norm can only fuse activation='relu'")
+    if activation == 'relu' and not is_device(x):
+        raise NotImplementedError('the fused ReLU needs device tensors')
+    relu = activation == 'relu'
     xhat = sqrtvar = None
     dst = None if out is None else out.eval
     if training:
         mm, mv = moving_mean.eval, moving_variance.eval
         fused = is_device(x) and is_device(mm) and is_device(mv)      # the statistics kernel updates them
+        track = GLOBAL.COMPUTE_GRAD and bool(inputs.requires_grad or gamma.requires_grad or beta.requires_grad)
+        neg_mask = dev.empty(x.shape, np.uint8) if relu else None
         y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst,
-                                                           (mm.reshape(-1), mv.reshape(-1)) if fused else None, momentum)
+                                                           (mm.reshape(-1), mv.reshape(-1)) if fused else None, momentum,
+                                                           neg_mask)
+        if not track:
+            neg_mask = None
         if not fused:
             for mov, cur in ((moving_mean, mean_), (moving_variance, var_)):
                 m = mov.eval
@@ -376,7 +390,8 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
                     m *= momentum
                     m += (1 - momentum) * np.asarray(cur).reshape(m.shape)
     else:
-        y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon, dst)
+        neg_mask = None
+        y = A.batch_norm_infer(x, gamma.eval, beta.eval, moving_mean.eval, moving_variance.eval, epsilon, dst, relu)
     if out is None:
         out = Tensor(y)
     elif y is not dst:
@@ -386,6 +401,10 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
     if GLOBAL.COMPUTE_GRAD and out.requires_grad and training:
         out.cache['sqrtvar'] = sqrtvar
         out.cache['normalized_x'] = xhat
+        if neg_mask is not None:
+            out.cache['neg_mask'] = neg_mask
+        else:
+            out.cache.pop('neg_mask', None)
         out.grad_fn = BatchNormBackward
         initialize_ops_grad(inputs, gamma, beta)
     return out

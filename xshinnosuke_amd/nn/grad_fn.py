@@ -236,7 +236,8 @@ def BatchNormBackward(outputs):
         gam = A.same_place(dy, gamma.eval)
         dx, dgamma, dbeta = K.bn_bwd(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gam,
                                      dx=out_dx, dgamma=None if out_dg is None else out_dg.reshape(-1),
-                                     dbeta=None if out_db is None else out_db.reshape(-1))
+                                     dbeta=None if out_db is None else out_db.reshape(-1),
+                                     neg_mask=outputs.cache.get('neg_mask'))       # fused ReLU: strict mask on dy
     else:
         out_dx = out_dg = out_db = None
         dx, dgamma, dbeta = A.batch_norm_backward(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gamma.eval)

@@ -14,6 +14,8 @@ from ..core import state as GLOBAL
 from ..core import autograd
 from ..core.base import Tensor, Parameter
 from ..layers.base import Layer
+from ..layers.normalize import BatchNormalization
+from ..layers.activators import ReLU
 from ..optim import get_optimizer
 from ..utils.data import DataSet, DataLoader
 from .objectives import get_objective
@@ -227,8 +229,22 @@ class Sequential(_Model):
             self.to('cuda')
 
     def forward(self, x, *args, **kwargs):
-        for layer in self._graph:
-            x = layer.forward(x)
+        layers = self._graph
+        i, n = 0, len(layers)
+        while i < n:
+            layer = layers[i]
+            nxt = layers[i + 1] if i + 1 < n else None
+            # BatchNormalization followed by an in-place ReLU on a device-resident dynamic graph: one kernel does
+            # both (same values and gradients as the two layers; the ReLU layer's output is the same tensor, as
+            # an in-place activation's is).  Static graphs drive the layers' backward one by one and are left alone.
+            if (isinstance(layer, BatchNormalization) and isinstance(nxt, ReLU) and nxt.inplace and
+                    isinstance(x, Tensor) and x.is_dynamic and x.device == 'cuda'):
+                x = layer.forward(x, fuse_relu=True)
+                nxt.data = x
+                i += 2
+            else:
+                x = layer.forward(x)
+                i += 1
         return x
 
 
