@@ -65,19 +65,35 @@ struct TapParams {
     int rowtiles;
 };
 
+// One launch can cover several parameter sets that share the row (output channel) tiling: the residue classes
+// of a strided backward-data pass, each with its own pixel count, taps and packed filter.  Workgroup ids are
+// concatenated class after class; first[c] is the first logical workgroup of class c.
+constexpr int TAP_MAX_CLASSES = 4;
+struct TapMulti {
+    TapParams cls[TAP_MAX_CLASSES];
+    uint32_t first[TAP_MAX_CLASSES + 1];
+    int ncls;
+    int rowtiles;
+};
+
 template <int STAGES>
-__global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapParams p) {
+__global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     constexpr int D = STAGES - 1;
 
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    // logical block = (pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
+    // logical block = (class, pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
     // tiles of one pixel tile and neighbouring pixel tiles (shared halo) meet in one L2
-    const uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-    const int rowtile = gridDim.y == 1 ? 0 : (int)(logical % gridDim.y);
-    const int m0 = (int)(gridDim.y == 1 ? logical : logical / gridDim.y) * BP;
+    uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int ci = 0;
+    while (ci + 1 < mp.ncls && logical >= mp.first[ci + 1]) ++ci;
+    const TapParams &p = mp.cls[ci];
+    logical -= mp.first[ci];
+    const uint32_t nrt = (uint32_t)mp.rowtiles;
+    const int rowtile = nrt == 1 ? 0 : (int)(logical % nrt);
+    const int m0 = (int)(nrt == 1 ? logical : logical / nrt) * BP;
 
     // ---- gather role: pixel m0 + lane, channels 8*wave .. 8*wave+7 of each chunk ----
     int iyb = 0, ixb = 0, nbase = 0;
@@ -531,18 +547,23 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 
 template <int STAGES>
-__global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapParams p) {
+__global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapMulti mp) {
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     constexpr int D = STAGES - 1;
 
     const int t = threadIdx.x;
     const int lane = t & 63;
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
-    // logical block = (pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
+    // logical block = (class, pixel tile, row tile) with the row tile fastest, contiguous per XCD: the row
     // tiles of one pixel tile and neighbouring pixel tiles (shared halo) meet in one L2
-    const uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x + gridDim.x * blockIdx.y, gridDim.x * gridDim.y);
-    const int rowtile = gridDim.y == 1 ? 0 : (int)(logical % gridDim.y);
-    const int m0 = (int)(gridDim.y == 1 ? logical : logical / gridDim.y) * BP;
+    uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int ci = 0;
+    while (ci + 1 < mp.ncls && logical >= mp.first[ci + 1]) ++ci;
+    const TapParams &p = mp.cls[ci];
+    logical -= mp.first[ci];
+    const uint32_t nrt = (uint32_t)mp.rowtiles;
+    const int rowtile = nrt == 1 ? 0 : (int)(logical % nrt);
+    const int m0 = (int)(nrt == 1 ? logical : logical / nrt) * BP;
 
     int iyb = 0, ixb = 0, nbase = 0;
     const bool live = m0 + lane < p.M;
@@ -660,20 +681,36 @@ __global__ void __launch_bounds__(256) tap_igemm_bf16_kernel(TapParams p) {
 
 // Packs A for the tap-major kernel.  mode 0 (forward): A[row][tap=(r,s)][ch] = w[row][ch][r][s].
 // mode 1 (backward-data class): A[row=c][tap=(t,u)][ch=k] = w[k][c][r0 + sh*t][s0 + sw*u].
-__global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__ w, float *__restrict__ apk, int mode,
-                                                        int rows, int CH, int R, int S, int TR, int TS, int r0, int s0,
-                                                        int sh, int sw, int rowtiles, uint32_t *__restrict__ counters) {
-    if (blockIdx.x == 0 && threadIdx.x < 8) counters[threadIdx.x] = 0;   // tile counters of the persistent kernel
+// One launch lays out the filter for every class of a pass; blocks [first[j], first[j+1]) serve job j.
+struct PackJob {
+    float *apk;
+    uint32_t *counters;
+    int TR, TS, r0, s0;
+};
+struct PackMulti {
+    PackJob job[TAP_MAX_CLASSES];
+    uint32_t first[TAP_MAX_CLASSES + 1];
+    int njobs;
+};
+__global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__ w, PackMulti pm, int mode, int rows, int CH,
+                                                        int R, int S, int sh, int sw, int rowtiles) {
+    int ji = 0;
+    while (ji + 1 < pm.njobs && blockIdx.x >= pm.first[ji + 1]) ++ji;
+    const PackJob &j = pm.job[ji];
+    const uint32_t blk = blockIdx.x - pm.first[ji], nblk = pm.first[ji + 1] - pm.first[ji];
+    if (blk == 0 && threadIdx.x < 8) j.counters[threadIdx.x] = 0;   // tile counters of the persistent kernel
+    float *__restrict__ apk = j.apk;
+    const int TR = j.TR, TS = j.TS, r0 = j.r0, s0 = j.s0;
     const int nch = CH / KC;
     const int iters = TR * TS * nch;
     const size_t total = (size_t)rowtiles * iters * (TM * KC);
-    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+    for (size_t i = (size_t)blk * 256 + threadIdx.x; i < total; i += (size_t)nblk * 256) {
         int e = (int)(i & 3);
         int r64 = (int)((i >> 2) & 63);
         int q = (int)((i >> 8) & 7);
-        size_t blk = i >> 11;
-        int it = (int)(blk % iters);
-        int rt = (int)(blk / iters);
+        size_t cblk = i >> 11;
+        int it = (int)(cblk % iters);
+        int rt = (int)(cblk / iters);
         int cc = it % nch, tap = it / nch;
         int tr = tap / TS, ts = tap % TS;
         int ch = cc * KC + q * 4 + e;
@@ -689,10 +726,12 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
-void launch_tap(dim3 grid, hipStream_t st, TapParams p, int opts) {
+void launch_tap(hipStream_t st, TapMulti mp, int opts) {
     const int bf16 = opts & 1, counters_zeroed = !(opts & 2);   // the pack kernel zeroes the tile counters
+    const uint32_t tiles = mp.first[mp.ncls];
+    if (tiles == 0) return;
     if (bf16) {
-        hipLaunchKernelGGL(tap_igemm_bf16_kernel<3>, grid, dim3(256), 0, st, p);
+        hipLaunchKernelGGL(tap_igemm_bf16_kernel<3>, dim3(tiles), dim3(256), 0, st, mp);
         return;
     }
     static int stages_env = -1, persist = -1;
@@ -702,8 +741,6 @@ void launch_tap(dim3 grid, hipStream_t st, TapParams p, int opts) {
         e = getenv("XSMI_TAP_PERSIST");
         persist = e ? atoi(e) : 1;
     }
-    const int iters = p.TR * p.TS * p.nch;
-    const uint32_t tiles = grid.x * grid.y;
     // With at most one tile per CU a workgroup runs alone and the two-stage pipeline waits a full load
     // latency per chunk; a third stage in flight covers it (measured 104 -> 91 us on 32x512x7x7, 3x3).
     const int stages = stages_env ? stages_env : (tiles <= (uint32_t)xsmi::cu_count() ? 3 : TAP_STAGES);
@@ -711,20 +748,24 @@ void launch_tap(dim3 grid, hipStream_t st, TapParams p, int opts) {
     // code) the persistent kernel wins by 1-4 %; with more tiles the hardware's own workgroup
     // hand-over is as fast as the in-kernel one, and the plain kernel's dynamic dispatch balances better.
     const uint32_t resident = (uint32_t)xsmi::cu_count() * 4u;          // four workgroups per CU fit (registers)
-    if (persist && stages == 2 && iters >= 4 && (iters & 1) == 0 && tiles >= 16 &&
-        (tiles <= resident || (persist > 1 && counters_zeroed))) {
-        uint32_t g = tiles < resident ? tiles : resident;
-        g &= ~7u;
-        p.tiles = tiles;
-        p.rowtiles = (int)grid.y;
-        hipLaunchKernelGGL(tap_igemm_f32_persist_kernel, dim3(g), dim3(256), 0, st, p);
-        return;
+    if (mp.ncls == 1) {
+        TapParams p = mp.cls[0];
+        const int iters = p.TR * p.TS * p.nch;
+        if (persist && stages == 2 && iters >= 4 && (iters & 1) == 0 && tiles >= 16 &&
+            (tiles <= resident || (persist > 1 && counters_zeroed))) {
+            uint32_t g = tiles < resident ? tiles : resident;
+            g &= ~7u;
+            p.tiles = tiles;
+            p.rowtiles = mp.rowtiles;
+            hipLaunchKernelGGL(tap_igemm_f32_persist_kernel, dim3(g), dim3(256), 0, st, p);
+            return;
+        }
     }
     switch (stages) {
-        case 2: hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, grid, dim3(256), 0, st, p); break;
-        case 4: hipLaunchKernelGGL(tap_igemm_f32_kernel<4>, grid, dim3(256), 0, st, p); break;
-        case 5: hipLaunchKernelGGL(tap_igemm_f32_kernel<5>, grid, dim3(256), 0, st, p); break;
-        default: hipLaunchKernelGGL(tap_igemm_f32_kernel<3>, grid, dim3(256), 0, st, p); break;
+        case 2: hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, dim3(tiles), dim3(256), 0, st, mp); break;
+        case 4: hipLaunchKernelGGL(tap_igemm_f32_kernel<4>, dim3(tiles), dim3(256), 0, st, mp); break;
+        case 5: hipLaunchKernelGGL(tap_igemm_f32_kernel<5>, dim3(tiles), dim3(256), 0, st, mp); break;
+        default: hipLaunchKernelGGL(tap_igemm_f32_kernel<3>, dim3(tiles), dim3(256), 0, st, mp); break;
     }
 }
 
@@ -734,16 +775,30 @@ size_t tap_pack_bytes(int rows, int CH, int taps) {
 }
 uint32_t *tap_counters(float *apk, size_t pack_bytes) { return (uint32_t *)((char *)apk + pack_bytes - 256); }
 
-int launch_pack(hipStream_t st, const float *w, float *apk, int mode, int rows, int CH, int R, int S, int TR, int TS,
-                int r0, int s0, int sh, int sw) {
-    uint32_t *counters = tap_counters(apk, tap_pack_bytes(rows, CH, TR * TS));
+struct PackSpec { float *apk; int TR, TS, r0, s0; };
+
+int launch_pack(hipStream_t st, const float *w, const PackSpec *specs, int nspecs, int mode, int rows, int CH, int R, int S,
+                int sh, int sw) {
     const int rowtiles = xsmi::ceil_div(rows, TM);
-    size_t total = (size_t)rowtiles * TR * TS * (CH / KC) * TM * KC;
-    if (total == 0) return XSMI_OK;
-    int blocks = (int)((total + 255) / 256);
-    if (blocks > 2048) blocks = 2048;
-    hipLaunchKernelGGL(tap_pack_kernel, dim3(blocks), dim3(256), 0, st, w, apk, mode, rows, CH, R, S, TR, TS, r0, s0, sh,
-                       sw, rowtiles, counters);
+    PackMulti pm;
+    pm.njobs = 0;
+    uint32_t blocks = 0;
+    for (int i = 0; i < nspecs; ++i) {
+        const PackSpec &sp = specs[i];
+        size_t total = (size_t)rowtiles * sp.TR * sp.TS * (CH / KC) * TM * KC;
+        uint32_t nb = (uint32_t)((total + 255) / 256);
+        if (nb > 2048) nb = 2048;
+        if (nb == 0) nb = 1;                      // a class without taps still gets its counters cleared
+        PackJob &j = pm.job[pm.njobs];
+        j.apk = sp.apk; j.counters = tap_counters(sp.apk, tap_pack_bytes(rows, CH, sp.TR * sp.TS));
+        j.TR = sp.TR; j.TS = sp.TS; j.r0 = sp.r0; j.s0 = sp.s0;
+        pm.first[pm.njobs] = blocks;
+        blocks += nb;
+        ++pm.njobs;
+    }
+    if (pm.njobs == 0) return XSMI_OK;
+    pm.first[pm.njobs] = blocks;
+    hipLaunchKernelGGL(tap_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, mode, rows, CH, R, S, sh, sw, rowtiles);
     XSMI_LAUNCH_CHECK("tap_pack_kernel");
     return XSMI_OK;
 }
@@ -768,7 +823,8 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     hipStream_t st = stream();
     float *apk = (float *)workspace;
     if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
-        int rc = launch_pack(st, w, apk, 0, K, C, R, S, R, S, 0, 0, 1, 1);
+        PackSpec spec = {apk, R, S, 0, 0};
+        int rc = launch_pack(st, w, &spec, 1, 0, K, C, R, S, 1, 1);
         if (rc) return rc;
     }
     TapParams p;
@@ -781,11 +837,15 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     p.OY = OH; p.OX = OW; p.dOX = make_fastdiv(OW); p.dOY = make_fastdiv(OH);
     p.os_n = (long long)K * OH * OW; p.os_k = (long long)OH * OW; p.o_base = 0; p.os_y = OW; p.os_x = 1;
     p.accumulate = 0; p.relu = relu;
-    dim3 grid(ceil_div(p.M, BP), ceil_div(K, TM));
-    prof_begin();
+    p.tiles = 0; p.rowtiles = 0;
     p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
     p.counters = tap_counters(apk, tap_pack_bytes(K, C, R * S));
-    launch_tap(grid, st, p, opts);
+    TapMulti mp;
+    mp.ncls = 1; mp.rowtiles = ceil_div(K, TM);
+    mp.cls[0] = p;
+    mp.first[0] = 0; mp.first[1] = (uint32_t)ceil_div(p.M, BP) * (uint32_t)mp.rowtiles;
+    prof_begin();
+    launch_tap(st, mp, opts);
     prof_end();
     XSMI_LAUNCH_CHECK("tap_igemm kernel");
     return XSMI_OK;
@@ -795,8 +855,8 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
                       int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace) {
     hipStream_t st = stream();
     char *ws = (char *)workspace;
-    struct Plan { TapParams p; dim3 grid; };
-    Plan plans[64];
+    TapParams plans[64];
+    PackSpec specs[64];
     int nplans = 0;
     for (int ph = 0; ph < sh; ++ph) {
         const int OYc = ph < H ? ceil_div(H - ph, sh) : 0;
@@ -806,20 +866,19 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
         for (int pw = 0; pw < sw; ++pw) {
             const int OXc = pw < W ? ceil_div(W - pw, sw) : 0;
             if (OYc == 0 || OXc == 0) continue;
+            if (nplans == 64) return set_error("xsmi_conv2d_bwd_data: stride %dx%d has too many residue classes", sh, sw), XSMI_ERR_INVALID;
             const int s0 = (pw + pad) % sw;
             const int U = s0 < S ? ceil_div(S - s0, sw) : 0;
             const int cx = (pw + pad - s0) / sw;
             float *apk = (float *)ws;
             const size_t apk_bytes = tap_pack_bytes(C, K, T * U);
             ws += apk_bytes;
-            if (!(opts & 2)) {
-                int rc = launch_pack(st, w, apk, 1, C, K, R, S, T, U, r0, s0, sh, sw);
-                if (rc) return rc;
-            }
+            specs[nplans] = PackSpec{apk, T, U, r0, s0};
             TapParams p;
             p.in = dy; p.apk = apk; p.bias = nullptr; p.out = dx; p.mask = nullptr;
             p.apk_bytes = (uint32_t)apk_bytes;
             p.counters = tap_counters(apk, apk_bytes);
+            p.tiles = 0; p.rowtiles = 0;
             p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
             p.M = N * OYc * OXc; p.rows = C; p.nch = K / KC; p.TR = T; p.TS = U;
             p.dy0 = cy; p.dx0 = cx; p.dstep = -1;
@@ -829,14 +888,30 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             p.os_n = (long long)C * H * W; p.os_k = (long long)H * W; p.o_base = (long long)ph * W + pw;
             p.os_y = sh * W; p.os_x = sw;
             p.accumulate = accumulate; p.relu = 0;
-            plans[nplans].p = p;
-            plans[nplans].grid = dim3(ceil_div(p.M, BP), ceil_div(C, TM));
-            ++nplans;
+            plans[nplans++] = p;
+        }
+    }
+    // the residue classes of a pass run as one launch per TAP_MAX_CLASSES classes (stride 2: one launch)
+    if (!(opts & 2)) {
+        for (int i = 0; i < nplans; i += TAP_MAX_CLASSES) {
+            const int n = nplans - i < TAP_MAX_CLASSES ? nplans - i : TAP_MAX_CLASSES;
+            int rc = launch_pack(st, w, specs + i, n, 1, C, K, R, S, sh, sw);
+            if (rc) return rc;
         }
     }
     prof_begin();
-    for (int i = 0; i < nplans; ++i) {
-        launch_tap(plans[i].grid, st, plans[i].p, opts);
+    for (int i = 0; i < nplans; i += TAP_MAX_CLASSES) {
+        TapMulti mp;
+        mp.ncls = nplans - i < TAP_MAX_CLASSES ? nplans - i : TAP_MAX_CLASSES;
+        mp.rowtiles = ceil_div(C, TM);
+        uint32_t first = 0;
+        for (int c = 0; c < mp.ncls; ++c) {
+            mp.cls[c] = plans[i + c];
+            mp.first[c] = first;
+            first += (uint32_t)ceil_div(plans[i + c].M, BP) * (uint32_t)mp.rowtiles;
+        }
+        mp.first[mp.ncls] = first;
+        launch_tap(st, mp, opts);
         XSMI_LAUNCH_CHECK("tap_igemm kernel");
     }
     prof_end();
