@@ -928,12 +928,8 @@ void launch_tap(hipStream_t st, TapMulti mp, int opts) {
             return;
         }
     }
-    switch (stages) {
-        case 2: hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, dim3(tiles), dim3(256), 0, st, mp); break;
-        case 4: hipLaunchKernelGGL(tap_igemm_f32_kernel<4>, dim3(tiles), dim3(256), 0, st, mp); break;
-        case 5: hipLaunchKernelGGL(tap_igemm_f32_kernel<5>, dim3(tiles), dim3(256), 0, st, mp); break;
-        default: hipLaunchKernelGGL(tap_igemm_f32_kernel<3>, dim3(tiles), dim3(256), 0, st, mp); break;
-    }
+    if (stages == 2) hipLaunchKernelGGL(tap_igemm_f32_kernel<2>, dim3(tiles), dim3(256), 0, st, mp);
+    else hipLaunchKernelGGL(tap_igemm_f32_kernel<3>, dim3(tiles), dim3(256), 0, st, mp);
 }
 
 // packed filter + 256 bytes that hold the persistent kernel's eight tile counters

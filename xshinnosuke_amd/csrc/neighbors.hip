@@ -313,6 +313,26 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
     }
 }
 
+template <bool VEC>
+__global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta, const float *__restrict__ mean,
+                                                        const float *__restrict__ var, float *__restrict__ y, ChanIdx chan,
+                                                        uint32_t total, float eps, int relu) {
+    constexpr int W = VEC ? 4 : 1;
+    for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
+        const int c = chan(i);
+        const float g = gamma[c], bt = beta[c], mu = mean[c], rs = sqrtf(var[c] + eps);
+        float xv[W], yv[W];
+        if (VEC) *reinterpret_cast<float4 *>(xv) = *reinterpret_cast<const float4 *>(x + i); else xv[0] = x[i];
+#pragma unroll
+        for (int e = 0; e < W; ++e) {
+            const float v = g * ((xv[e] - mu) / rs) + bt;
+            yv[e] = (relu && v < 0.f) ? 0.f : v;
+        }
+        if (VEC) *reinterpret_cast<float4 *>(y + i) = *reinterpret_cast<float4 *>(yv); else y[i] = yv[0];
+    }
+}
+
 // ---- average pool over k x k blocks --------------------------------------------
 __global__ void __launch_bounds__(256) avgpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int H, int W,
                                                            int OH, int OW, int k, size_t total) {
@@ -547,17 +567,6 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     return XSMI_OK;
 }
 
-__global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
-                                                        const float *__restrict__ beta, const float *__restrict__ mean,
-                                                        const float *__restrict__ var, float *__restrict__ y, ChanIdx chan,
-                                                        uint32_t total, float eps, int relu) {
-    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
-        int c = chan(i);
-        float v = gamma[c] * ((x[i] - mean[c]) / sqrtf(var[c] + eps)) + beta[c];
-        y[i] = (relu && v < 0.f) ? 0.f : v;
-    }
-}
-
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
                   int N, int C, int HW, float eps, int relu) {
     XSMI_REQUIRE_INIT();
@@ -565,8 +574,12 @@ int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const f
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_infer: tensors of 2^29 elements or more are not supported");
     XSMI_CHECK_ARG(x && gamma && beta && mean && var && y, "xsmi_bn_infer: null pointer");
     size_t total = (size_t)N * C * HW;
-    hipLaunchKernelGGL(bn_infer_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean, var, y,
-                       make_chan(C, HW), (uint32_t)total, eps, relu);
+    if ((HW & 3) == 0 && aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(bn_infer_kernel<true>, grid_for(total / 4), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean,
+                           var, y, make_chan(C, HW), (uint32_t)total, eps, relu);
+    else
+        hipLaunchKernelGGL(bn_infer_kernel<false>, grid_for(total), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean,
+                           var, y, make_chan(C, HW), (uint32_t)total, eps, relu);
     XSMI_LAUNCH_CHECK("bn_infer_kernel");
     return XSMI_OK;
 }
