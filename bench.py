@@ -266,10 +266,14 @@ def traffic_run(be, reps=3):
     pdy = be.to_device(np.random.default_rng(5).standard_normal((p["N"], p["C"], p["H"] // 2, p["W"] // 2), dtype=np.float32))
     py = be.empty(pdy.shape); pidx = be.empty(pdy.shape, np.uint8); pgx = be.empty(px.shape)
     src = be.empty((px.size + pdy.size + pdy.size // 4,)); dst = be.empty(src.shape)
-    for _ in range(reps):
+    def conv_step():
         K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y)
         K.conv2d_bwd_data(ddy, dw_, x.shape, c["stride"], c["pad"], dx=gx)
         K.conv2d_bwd_weight(ddy, dx_, w.shape, c["stride"], c["pad"], dw=gw, db=gb)
+    preheat(be, conv_step, seconds=0.3)          # counters of the last dispatches are read at the sustained clock
+    for _ in range(reps):
+        conv_step()
+        K.conv2d_fwd(dx_, dw_, db_, c["stride"], c["pad"], out=y, bf16=True)
         K.maxpool2d_fwd(px, p["k"], p["stride"], p["pad"], out=py, idx=pidx)
         K.maxpool2d_bwd(pdy, pidx, px.shape, p["k"], p["stride"], p["pad"], dx=pgx)
         K.copy_kernel(dst, src)
