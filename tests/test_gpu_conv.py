@@ -103,7 +103,7 @@ BF16_CASES = [  # shapes whose reduction channels are a multiple of 32 take the 
     (2, 64, 28, 28, 128, 3, 3, 2, 2, 1),
     (2, 64, 28, 28, 128, 1, 1, 2, 2, 0),
     (3, 128, 14, 14, 130, 3, 3, 1, 1, 1),
-    (2, 3, 32, 32, 64, 7, 7, 2, 2, 3),     # stem: stays on the fp32 kernel, the flag only permits bf16
+    (2, 3, 32, 32, 64, 7, 7, 2, 2, 3),     # stem: channels padded to one octet in the channels-last forward
 ]
 
 
@@ -124,7 +124,7 @@ def test_conv_bf16_opt_in(gpu, n, c, h, w, k, r, s, sh, sw, pad):
     gx = K.conv2d_bwd_data(ddy, dw_, x.shape, (sh, sw), pad, bf16=True).numpy()
     assert rel_l2(y, y_ref) <= 1e-2
     assert rel_l2(gx, dx_ref) <= 1e-2
-    if c % 32 == 0:
+    if c % 32 == 0 or c <= 8:
         y_r, _ = oracle.conv2d_fwd(round_bf16(x), round_bf16(wt), b, (sh, sw), pad)
         assert rel_l2(y, y_r) <= TOL
         assert rel_l2(y, y_ref) > 1e-4            # the bf16 kernel really ran
@@ -137,6 +137,44 @@ def test_conv_bf16_opt_in(gpu, n, c, h, w, k, r, s, sh, sw, pad):
     gw, _ = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (sh, sw), pad, want_db=True, bf16=True)
     gw32, _ = K.conv2d_bwd_weight(ddy, dx_, wt.shape, (sh, sw), pad, want_db=True)
     np.testing.assert_array_equal(gw.numpy(), gw32.numpy())
+
+
+BF16_FWD_CASES = [  # n, c, h, w, k, r, s, sh, sw, pad: tile tails in rows and pixels, odd chunk counts, both tile shapes
+    (1, 32, 5, 7, 8, 1, 1, 1, 1, 0),
+    (3, 96, 9, 11, 70, 3, 3, 1, 1, 1),
+    (2, 32, 13, 13, 200, 5, 5, 2, 2, 2),
+    (5, 64, 17, 15, 64, 3, 3, 1, 1, 0),
+    (2, 128, 30, 30, 128, 3, 3, 1, 1, 1),
+    (4, 1, 28, 28, 8, 2, 2, 1, 1, 0),
+    (2, 8, 20, 18, 130, 3, 5, 1, 2, 2),
+    (1, 3, 224, 224, 64, 7, 7, 2, 2, 3),
+    (2, 512, 7, 7, 512, 3, 3, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", BF16_FWD_CASES)
+def test_conv_bf16_forward_channels_last(gpu, n, c, h, w, k, r, s, sh, sw, pad):
+    """bf16 forward through the channels-last copy, with the fused bias + ReLU epilogue and its sign mask:
+    against the oracle on operands rounded to bf16 only the fp32 accumulation order differs (<= 1e-5)."""
+    K = gpu.kernels
+    rng = np.random.default_rng(1000 + 7 * c + k)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    wt = he_normal(rng, (k, c, r, s))
+    b = rng.standard_normal((k,)).astype(np.float32)
+    pre_ref, _ = oracle.conv2d_fwd(round_bf16(x), round_bf16(wt), b, (sh, sw), pad)
+    dx_, dw_, db_ = gpu.to_device(x), gpu.to_device(wt), gpu.to_device(b)
+    y = K.conv2d_fwd(dx_, dw_, db_, (sh, sw), pad, bf16=True).numpy()
+    assert y.shape == pre_ref.shape
+    assert rel_l2(y, pre_ref) <= TOL
+    mask = gpu.empty(pre_ref.shape, np.uint8)
+    act = K.conv2d_fwd(dx_, dw_, db_, (sh, sw), pad, relu=True, neg_mask=mask, bf16=True).numpy()
+    np.testing.assert_array_equal(act, np.maximum(y, 0.0))
+    np.testing.assert_array_equal(mask.numpy(), (y < 0).astype(np.uint8))
+    # the filter may stay packed between calls; without a bias the epilogue adds nothing
+    y0 = K.conv2d_fwd(dx_, dw_, None, (sh, sw), pad, bf16=True).numpy()
+    y1 = K.conv2d_fwd(dx_, dw_, None, (sh, sw), pad, bf16=True, packed=True).numpy()
+    np.testing.assert_array_equal(y0, y1)
+    assert rel_l2(y0 + b.reshape(1, -1, 1, 1), pre_ref) <= TOL
 
 
 def test_conv_packed_workspace_flag(gpu):

@@ -337,6 +337,10 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd: workspace of %zu bytes needed, %zu given", need,
                    workspace_bytes);
+    if ((flags & XSMI_CONV_BF16) && xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad) &&
+        workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
+        return xsmi::nhwc_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
+                                   (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
     if (xsmi::tap_path_ok(C))
         return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
                                   (flags & XSMI_CONV_RELU) ? 1 : 0,

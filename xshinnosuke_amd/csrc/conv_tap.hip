@@ -833,6 +833,521 @@ __global__ void __launch_bounds__(256) tap_igemm_bf16_r128_kernel(TapMulti mp) {
     }
 }
 
+// bf16 tile kernel: operands are rounded to bf16 on their way INTO the LDS, so a stage holds bf16 in the
+// layout the matrix instruction consumes and every fragment is one 128-bit LDS read.
+//   tile   64*WR rows x 64*WC pixels per 256-thread workgroup, a wave owns 64 x 64 (2 x 2 blocks of 32 x 32)
+//   chunk  one tap x 32 channels = two v_mfma_f32_32x32x16_bf16 steps; step u, lane half h use channel group 2u + h
+//   stage  A [4 groups][ROWS][8 bf16], B [4 groups][PIX][8 bf16]; three stages
+// A is packed to bf16 in exactly that layout by tap_pack_bf16_kernel and arrives by LDS-direct loads.  B is
+// gathered from the fp32 tensor into registers (a thread = one pixel, 8*k consecutive channels, so every
+// wave-level load is 256 contiguous bytes), converted and written with 128-bit LDS stores.  The loads of
+// chunk i+2 are issued while chunk i multiplies; chunk i+1 is converted and stored during the same iteration.
+template <int WR, int WC>
+__global__ void __launch_bounds__(256) tap_bf16_tile_kernel(TapMulti mp) {
+    static_assert(WR * WC == 4, "four waves");
+    constexpr int ROWS = 64 * WR, PIX = 64 * WC;
+    constexpr int GROUPS = 256 / PIX;                 // thread groups that split a chunk's 32 channels
+    constexpr int CPT = KC / GROUPS;                  // channels per thread and chunk
+    constexpr int A_BYTES = ROWS * 64, B_BYTES = PIX * 64, STAGE = A_BYTES + B_BYTES;
+    constexpr int NLOADS = CPT + WR;                  // vector-memory loads per thread and chunk
+    __shared__ __attribute__((aligned(16))) unsigned char smem[3 * STAGE];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    uint32_t logical = xsmi::xcd_contiguous_id(blockIdx.x, gridDim.x);
+    int ci = 0;
+    while (ci + 1 < mp.ncls && logical >= mp.first[ci + 1]) ++ci;
+    const TapParams &p = mp.cls[ci];
+    logical -= mp.first[ci];
+    const uint32_t nrt = (uint32_t)mp.rowtiles;       // ROWS-row tiles
+    const int rowtile = nrt == 1 ? 0 : (int)(logical % nrt);
+    const int m0 = (int)(nrt == 1 ? logical : logical / nrt) * PIX;
+
+    // ---- gather role: pixel m0 + pl, channels grp*CPT .. grp*CPT + CPT-1 of each chunk ----
+    const int pl = t & (PIX - 1);
+    const int grp = __builtin_amdgcn_readfirstlane(t / PIX);
+    int iyb = 0, ixb = 0, nbase = 0;
+    const bool live = m0 + pl < p.M;
+    if (live) {
+        uint32_t m = (uint32_t)(m0 + pl);
+        uint32_t q = xsmi::fdiv(m, p.dOX);
+        int x = (int)m - (int)q * p.OX;
+        uint32_t n = xsmi::fdiv(q, p.dOY);
+        int y = (int)q - (int)n * p.OY;
+        iyb = y * p.sy + p.dy0;
+        ixb = x * p.sx + p.dx0;
+        nbase = (int)n * p.in_n_stride;
+    }
+    __amdgpu_buffer_rsrc_t rin = __builtin_amdgcn_make_buffer_rsrc((void *)p.in, 0, (int)p.in_bytes, 0x00020000);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(p.apk, p.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0];
+    const int iters = p.TR * p.TS * p.nch;
+    const uint32_t a_voff = (uint32_t)((wave * WR * 64 + lane) * 16);
+    // loop-invariant parameters in registers (p is indexed by class, so the compiler would re-read them)
+    const int dstep = p.dstep, IH = p.IH, IW = p.IW, nch = p.nch, TS = p.TS;
+    const uint32_t plane_bytes = p.plane_bytes;
+
+    // B runs three chunks ahead of the multiply (two register sets), A two chunks ahead (three LDS stages)
+    int r = 0, s = 0, cc = 0;                          // position of the next B chunk to load
+    uint32_t ld_asoff = (uint32_t)rowtile * (uint32_t)iters * (uint32_t)A_BYTES;
+    float breg[2][CPT];
+    auto load_b = [&](auto set_tag) {
+        constexpr int set = decltype(set_tag)::value;
+        int iy = iyb + r * dstep, ix = ixb + s * dstep;
+        bool ok = live && (unsigned)iy < (unsigned)IH && (unsigned)ix < (unsigned)IW;
+        const int voff = ok ? (nbase + iy * IW + ix) * 4 : (int)0x80000000u;
+        const uint32_t soff = (uint32_t)(cc * KC + grp * CPT) * plane_bytes;
+#pragma unroll
+        for (int e = 0; e < CPT; ++e)
+            breg[set][e] = __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(rin, voff, (int)(soff + (uint32_t)e * plane_bytes), 0));
+        if (++cc == nch) {
+            cc = 0;
+            if (++s == TS) { s = 0; ++r; }
+        }
+    };
+    auto issue_a = [&](uint32_t stage) {               // this wave's WR KB of the next chunk's packed rows
+#pragma unroll
+        for (int qa = 0; qa < WR; ++qa)
+            xsmi::load_lds_b128(rap, lds0 + stage + (uint32_t)((wave * WR + qa) * 1024), a_voff + (uint32_t)qa * 1024u, ld_asoff);
+        ld_asoff += (uint32_t)A_BYTES;
+    };
+    auto store_b = [&](auto set_tag, uint32_t stage) {
+        constexpr int set = decltype(set_tag)::value;
+#pragma unroll
+        for (int j = 0; j < CPT / 8; ++j) {
+            bf16x8 v;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) v[e] = (__bf16)breg[set][8 * j + e];
+            *reinterpret_cast<bf16x8 *>(smem + stage + A_BYTES + ((grp * (CPT / 8) + j) * PIX + pl) * 16) = v;
+        }
+    };
+
+    floatx16 acc[2][2];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave / WC, wc = wave % WC;
+    const int a_rd = (h * ROWS + wr * 64 + l31) * 16;                 // byte offset of group h, row block 0
+    const int b_rd = A_BYTES + (h * PIX + wc * 64 + l31) * 16;
+    using S0 = std::integral_constant<int, 0>;
+    using S1 = std::integral_constant<int, 1>;
+
+    uint32_t st_cur = 0, st_nxt = STAGE, st_nx2 = 2 * STAGE;
+    // prologue: chunk 0 in the LDS, B of chunks 1 and 2 and A of chunk 1 in flight (a class without taps has
+    // no chunks and writes zeros).  Loads retire in order: B0 A0 B1 A1 B2.
+    if (iters > 0) {
+        load_b(S0{});
+        issue_a(st_cur);
+        if (iters > 1) {
+            load_b(S1{});
+            issue_a(st_nxt);
+        }
+        store_b(S0{}, st_cur);
+        if (iters > 2) load_b(S0{});
+        constexpr int two = NLOADS + CPT < 63 ? NLOADS + CPT : 63;   // the counter holds 63 at most
+        if (iters > 2) xsmi::wait_vmcnt<two>();
+        else if (iters > 1) xsmi::wait_vmcnt<NLOADS>();
+        else xsmi::wait_vmcnt<0>();
+        xsmi::wait_lgkmcnt0();
+        xsmi::block_barrier();
+    }
+
+    // iteration `it` multiplies chunk it, moves chunk it+1 (register set (it+1) % 2) into the LDS, and issues
+    // B of chunk it+3 into that set and A of chunk it+2 into the stage that chunk it-1 has left
+    auto body = [&](auto next_set, int it) {
+        bf16x8 fa[2][2], fb[2][2];                    // [step][block]
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[u][i] = *reinterpret_cast<const bf16x8 *>(smem + st_cur + a_rd + (2 * u * ROWS + 32 * i) * 16);
+                fb[u][i] = *reinterpret_cast<const bf16x8 *>(smem + st_cur + b_rd + (2 * u * PIX + 32 * i) * 16);
+            }
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+        if (it + 1 < iters) store_b(next_set, st_nxt);
+        if (it + 3 < iters) load_b(next_set);
+        if (it + 2 < iters) issue_a(st_nx2);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j) acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[1][i], fb[1][j], acc[i][j], 0, 0, 0);
+        if (it + 1 < iters) {
+            // A of chunk it+1 has landed (only this iteration's loads may still be in flight); this wave's LDS
+            // stores and fragment reads are done
+            if (it + 3 < iters) xsmi::wait_vmcnt<NLOADS>();
+            else if (it + 2 < iters) xsmi::wait_vmcnt<WR>();
+            else xsmi::wait_vmcnt<0>();
+            xsmi::wait_lgkmcnt0();
+            xsmi::block_barrier();
+        }
+        const uint32_t tmp = st_cur;
+        st_cur = st_nxt; st_nxt = st_nx2; st_nx2 = tmp;
+    };
+    for (int it = 0; it < iters; it += 2) {
+        body(S1{}, it);
+        if (it + 1 < iters) body(S0{}, it + 1);
+    }
+
+    // ---- epilogue: register v of lane l in block (i, j) = row 32i + 8*(v/4) + 4*(l/32) + v%4, pixel 32j + l%32 ----
+    const int rbase = rowtile * ROWS + wr * 64 + 4 * h;
+#pragma unroll
+    for (int j = 0; j < 2; ++j) {
+        const int m = m0 + wc * 64 + 32 * j + l31;
+        if (m >= p.M) continue;
+        uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+        int x = m - (int)q * p.OX;
+        uint32_t n = xsmi::fdiv(q, p.dOY);
+        int y = (int)q - (int)n * p.OY;
+        const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                int row = rbase + 32 * i + 8 * (v >> 2) + (v & 3);
+                if (row < p.rows) {
+                    float val = acc[i][j][v];
+                    if (p.bias) val += p.bias[row];
+                    long long o = pix_off + (long long)row * p.os_k;
+                    if (p.relu) {
+                        if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
+                        val = val > 0.f ? val : 0.f;
+                    }
+                    if (p.accumulate) val += p.out[o];
+                    p.out[o] = val;
+                }
+            }
+    }
+}
+
+// ---- bf16 forward on a channels-last copy ------------------------------------------------------------
+// The fastest bf16 path first rewrites the activations as bf16 [N][H + 2 pad][W + 2 pad][CP] (CP = channels
+// rounded up to a multiple of 8) with a materialised zero border.  Eight consecutive channels of a pixel are
+// then 16 contiguous bytes, which is exactly one lane's operand of v_mfma_f32_32x32x16_bf16, so both operands
+// go global -> LDS with 128-bit LDS-direct loads: no registers, no conversion and no validity test in the
+// loop, a thread's pixel offset is fixed for the whole kernel and the (tap, channel) displacement is scalar.
+// A vector-memory instruction occupies the CU's address unit for 16 cycles whatever its width, so the
+// per-element dword gathers of the NCHW kernels (8-32 per thread and chunk) bound them; this form needs 4-5
+// loads per wave and chunk.
+//
+// The reduction index is a list of octets, o = tap * (CP / 8) + channel octet; a chunk is four consecutive
+// octets (group g = octet 4 * chunk + g).  With CP a multiple of 32 a chunk is 32 channels of one tap; with
+// CP = 8 (a 3-channel stem) it is four consecutive taps.
+struct NhwcParams {
+    const __bf16 *xp;
+    const float *apk;     // bf16 [row tile][chunk][group 4][ROWS][8]
+    const float *bias;
+    float *out;
+    uint8_t *mask;
+    uint32_t xp_bytes, apk_bytes;
+    int M, rows, nchunks;
+    int R, S, C8;         // taps, octets per tap
+    int Hp, Wp, sy, sx;
+    int OY, OX;
+    xsmi::FastDiv dOX, dOY;
+    long long os_n, os_k;
+    int relu;
+    int rowtiles;
+    uint32_t tiles;       // pixel tiles x row tiles
+};
+
+// x fp32 [N][C][H][W] -> xp bf16 [N][Hp][Wp][CP]; a workgroup converts WS pixels of one padded row.
+__global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ xp, int C, int H,
+                                                             int W, int CP, int pad, int Hp, int Wp, int WS, int nseg) {
+    extern __shared__ float tile[];                   // [C][WS | 1]
+    const int t = threadIdx.x;
+    const int seg = blockIdx.x % nseg;
+    const int rowid = blockIdx.x / nseg;              // n * Hp + hp
+    const int hp = rowid % Hp, n = rowid / Hp;
+    const int ih = hp - pad;
+    __bf16 *row = xp + (size_t)rowid * Wp * CP;
+    if (ih < 0 || ih >= H) {                          // border row: zeros (CP is a multiple of 8: 16-byte stores)
+        uint4 *r4 = reinterpret_cast<uint4 *>(row);
+        const int n16 = Wp * CP / 8;
+        for (int i = seg * 256 + t; i < n16; i += nseg * 256) r4[i] = make_uint4(0, 0, 0, 0);
+        return;
+    }
+    const int w0 = seg * WS;
+    const int wn = W - w0 < WS ? W - w0 : WS;
+    const int stride = WS | 1;
+    const float *src = x + (((size_t)n * C) * H + ih) * W + w0;
+    for (int i = t; i < C * wn; i += 256) {
+        int c = i / wn, wl = i - c * wn;
+        tile[c * stride + wl] = src[(size_t)c * H * W + wl];
+    }
+    __syncthreads();
+    const int CP2 = CP / 2;
+    uint32_t *dst = reinterpret_cast<uint32_t *>(row + (size_t)(pad + w0) * CP);
+    for (int i = t; i < wn * CP2; i += 256) {
+        int wl = i / CP2, c = 2 * (i - wl * CP2);
+        float v0 = c < C ? tile[c * stride + wl] : 0.f;
+        float v1 = c + 1 < C ? tile[(c + 1) * stride + wl] : 0.f;
+        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+        bf16x2 pk;
+        pk[0] = (__bf16)v0; pk[1] = (__bf16)v1;
+        dst[i] = __builtin_bit_cast(uint32_t, pk);
+    }
+    // left and right border pixels of the row
+    uint32_t *r32 = reinterpret_cast<uint32_t *>(row);
+    if (seg == 0)
+        for (int i = t; i < pad * CP2; i += 256) r32[i] = 0;
+    if (seg == nseg - 1)
+        for (int i = t; i < pad * CP2; i += 256) r32[(size_t)(pad + W) * CP2 + i] = 0;
+}
+
+// Filters for the channels-last kernel: bf16 [row tile][chunk][ROWS][4 slots][8], the LDS image of a stage's A
+// part.  Octet g of a row sits in slot g ^ ((row >> 2) & 3) (see the kernel); zero where the octet or the
+// channel does not exist.
+__global__ void __launch_bounds__(256) tap_pack_oct_kernel(const float *__restrict__ w, __bf16 *__restrict__ apk, int rows, int C,
+                                                            int R, int S, int C8, int nchunks, int rowtiles, int ROWS) {
+    const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
+    const int octets = R * S * C8;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        int e = (int)(i & 7);
+        int slot = (int)((i >> 3) & 3);
+        size_t rest = i >> 5;
+        int rr = (int)(rest % ROWS);
+        size_t cblk = rest / ROWS;
+        int it = (int)(cblk % nchunks);
+        int rt = (int)(cblk / nchunks);
+        int g = slot ^ ((rr >> 2) & 3);
+        int o = 4 * it + g;
+        int tap = o / C8, ch = (o - tap * C8) * 8 + e;
+        int row = rt * ROWS + rr;
+        float v = 0.f;
+        if (row < rows && o < octets && ch < C) v = w[((size_t)row * C + ch) * R * S + tap];
+        apk[i] = (__bf16)v;
+    }
+}
+
+// Persistent: the launch has at most as many workgroups as fit the chip at once, and a workgroup walks a
+// contiguous range of tiles as ONE stream of chunks.  The loads run three chunks ahead of the multiply across
+// tile boundaries, so a tile's first chunks arrive while the previous tile still multiplies and its output
+// stores drain behind the next tile's MFMAs; only a workgroup's very first chunk is waited for with nothing
+// else to do.  (Stores count in vmcnt like loads; the loop's waits stay correct with stores pending, because
+// loads complete in order among themselves: they just wait a little longer at a tile boundary.)
+template <int WR, int WC, bool STEM>
+__global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(NhwcParams p) {
+    static_assert(WR * WC == 4, "four waves");
+    constexpr int ROWS = 64 * WR, PIX = 64 * WC;
+    constexpr int STAGES = 3;
+    constexpr int NB = PIX / 64;                      // B loads per wave and chunk (16 pixels x 64 bytes each)
+    constexpr int A_BYTES = ROWS * 64, B_BYTES = PIX * 64, STAGE = A_BYTES + B_BYTES;
+    constexpr int NLOADS = NB + WR;
+    // A stage holds A [ROWS][64 bytes] and B [PIX][64 bytes]: the chunk's four octets of a row or pixel, octet g
+    // in 16-byte slot g ^ ((index >> 2) & 3).  A fragment read (32 consecutive rows or pixels, one octet) then
+    // covers 256 consecutive bytes' worth of banks with every 16 lanes (the LDS serves 256 bytes per clock), and a B load (16 consecutive pixels x 4 slots, lane = pixel * 4 +
+    // slot) reads 64 contiguous bytes per pixel and lands as one contiguous KB.
+    __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * STAGE];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t wg = xsmi::xcd_contiguous_id(blockIdx.x, gridDim.x);
+    // tiles [tile_begin, tile_end) of the launch's p.tiles, row tile fastest
+    const uint32_t tile_begin = (uint32_t)(((uint64_t)wg * p.tiles) / gridDim.x);
+    const uint32_t tile_end = (uint32_t)(((uint64_t)(wg + 1) * p.tiles) / gridDim.x);
+    const uint32_t nrt = (uint32_t)p.rowtiles;
+    const int S = p.S, R = p.R, C8 = p.C8, Wp = p.Wp;
+    const int iters = p.nchunks;
+    const int total = (int)(tile_end - tile_begin) * iters;       // chunks of this workgroup's stream
+
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(p.xp, p.xp_bytes);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(p.apk, p.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0];
+    const uint32_t a_voff = (uint32_t)((wave * WR * 64 + lane) * 16);
+
+    // ---- issue side: tile i_tile, chunk i_chunk; this lane's pixel and octet for each of its NB loads ----
+    uint32_t i_tile = tile_begin;
+    int i_chunk = 0;
+    uint32_t voff[NB];                                // byte offset of the lane's pixel (+ its octet when not STEM)
+    int oct[NB];                                      // the lane's octet of a chunk
+    uint32_t ld_asoff = 0, ld_stage = 0;
+    int r = 0, s = 0, c8 = 0;                          // chunk position when a chunk is one tap's 4 octets
+    int rj[NB], sj[NB];                                // per lane: tap position when an octet is a whole tap
+#pragma unroll
+    for (int j = 0; j < NB; ++j) oct[j] = (lane & 3) ^ ((((wave * NB + j) * 16 + (lane >> 2)) >> 2) & 3);
+    auto issue_tile = [&]() {                          // set the issue side up for tile i_tile
+        const uint32_t mt = nrt == 1 ? i_tile : i_tile / nrt;
+        const int rowtile = nrt == 1 ? 0 : (int)(i_tile - mt * nrt);
+        const int m0 = (int)mt * PIX;
+        ld_asoff = (uint32_t)rowtile * (uint32_t)iters * (uint32_t)A_BYTES;
+        r = 0; s = 0; c8 = 0;
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            const int m = m0 + (wave * NB + j) * 16 + (lane >> 2);
+            voff[j] = 0x80000000u;                    // pixels beyond M read zeros
+            if (m < p.M) {
+                uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+                int x = m - (int)q * p.OX;
+                uint32_t n = xsmi::fdiv(q, p.dOY);
+                int y = (int)q - (int)n * p.OY;
+                voff[j] = (uint32_t)((((int)n * p.Hp + y * p.sy) * Wp + x * p.sx) * C8) * 16u + (STEM ? 0u : (uint32_t)oct[j] * 16u);
+            }
+            if (STEM) {
+                rj[j] = oct[j] / S;
+                sj[j] = oct[j] - rj[j] * S;
+            }
+        }
+    };
+    auto issue = [&]() {
+        // a chunk past the filter (the chunk count is rounded up to even) meets zero rows of A: re-read tap 0
+        const uint32_t soff = (STEM || r >= R) ? 0u : (uint32_t)(((r * Wp + s) * C8 + c8) * 16);
+#pragma unroll
+        for (int j = 0; j < NB; ++j) {
+            uint32_t vo = voff[j];
+            if (STEM) {
+                // taps past the filter meet zero rows of A: read zeros
+                vo = rj[j] < R ? vo + (uint32_t)(rj[j] * Wp + sj[j]) * 16u : 0x80000000u;
+                sj[j] += 4;
+                while (sj[j] >= S) { sj[j] -= S; ++rj[j]; }
+            }
+            xsmi::load_lds_b128(rin, lds0 + ld_stage + (uint32_t)(A_BYTES + (wave * NB + j) * 1024), vo, soff);
+        }
+#pragma unroll
+        for (int qa = 0; qa < WR; ++qa)
+            xsmi::load_lds_b128(rap, lds0 + ld_stage + (uint32_t)((wave * WR + qa) * 1024), a_voff + (uint32_t)qa * 1024u, ld_asoff);
+        ld_asoff += (uint32_t)A_BYTES;
+        ld_stage += (uint32_t)STAGE;
+        if (ld_stage == (uint32_t)(STAGES * STAGE)) ld_stage = 0;
+        if (!STEM) {
+            c8 += 4;
+            if (c8 == C8) {
+                c8 = 0;
+                if (++s == S) { s = 0; ++r; }
+            }
+        }
+        if (++i_chunk == iters) {
+            i_chunk = 0;
+            if (++i_tile < tile_end) issue_tile();
+        }
+    };
+
+    // ---- multiply side ----
+    floatx16 acc[2][2];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
+    };
+    zero_acc();
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave / WC, wc = wave % WC;
+    // step u, lane half h read octet 2u + h: slot (2u) ^ xs with xs = h ^ ((l31 >> 2) & 3)
+    const int xs = h ^ ((l31 >> 2) & 3);
+    const int a_rd = (wr * 64 + l31) * 64;
+    const int b_rd = A_BYTES + (wc * 64 + l31) * 64;
+    uint32_t c_tile = tile_begin;
+
+    // register v of lane l in block (i, j) = row 32i + 8*(v/4) + 4*(l/32) + v%4, pixel 32j + l%32
+    auto epilogue = [&]() {
+        const uint32_t mt = nrt == 1 ? c_tile : c_tile / nrt;
+        const int rowtile = nrt == 1 ? 0 : (int)(c_tile - mt * nrt);
+        const int m0 = (int)mt * PIX;
+        const int rbase = rowtile * ROWS + wr * 64 + 4 * h;
+#pragma unroll
+        for (int j = 0; j < 2; ++j) {
+            const int m = m0 + wc * 64 + 32 * j + l31;
+            if (m >= p.M) continue;
+            uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+            int x = m - (int)q * p.OX;
+            uint32_t n = xsmi::fdiv(q, p.dOY);
+            int y = (int)q - (int)n * p.OY;
+            const long long pix_off = (long long)n * p.os_n + (long long)y * p.OX + x;
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    int row = rbase + 32 * i + 8 * (v >> 2) + (v & 3);
+                    if (row < p.rows) {
+                        float val = acc[i][j][v];
+                        if (p.bias) val += p.bias[row];
+                        long long o = pix_off + (long long)row * p.os_k;
+                        if (p.relu) {
+                            if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
+                            val = val > 0.f ? val : 0.f;
+                        }
+                        p.out[o] = val;
+                    }
+                }
+        }
+    };
+
+    // Software pipeline: the fragments of chunk g+1 are read while chunk g multiplies.  An iteration issues
+    // the first half of chunk g's MFMAs, then (while they execute) waits for chunk g+1, crosses the barrier,
+    // refills the stage that chunk g has left with chunk g+3 and reads chunk g+1's fragments, then issues
+    // the second half.  Every wave has read all of chunk g before that barrier (its fragments were complete
+    // before the first half), so three stages give a prefetch distance of three chunks.
+    bf16x8 fa[2][2][2], fb[2][2][2];                  // [buffer][step][block]
+    uint32_t rd_stage = 0;
+    auto read_frags = [&](auto buf_tag) {
+        constexpr int bf = decltype(buf_tag)::value;
+#pragma unroll
+        for (int u = 0; u < 2; ++u)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                fa[bf][u][i] = *reinterpret_cast<const bf16x8 *>(smem + rd_stage + a_rd + 2048 * i + ((2 * u) ^ xs) * 16);
+                fb[bf][u][i] = *reinterpret_cast<const bf16x8 *>(smem + rd_stage + b_rd + 2048 * i + ((2 * u) ^ xs) * 16);
+            }
+        rd_stage += (uint32_t)STAGE;
+        if (rd_stage == (uint32_t)(STAGES * STAGE)) rd_stage = 0;
+    };
+    using B0 = std::integral_constant<int, 0>;
+    using B1 = std::integral_constant<int, 1>;
+    auto body = [&](auto cur_tag, auto nxt_tag, int g) {
+        constexpr int cur = decltype(cur_tag)::value;
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][0][i], fb[cur][0][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+        if (g + 1 < total) {
+            if (g + 3 <= total) xsmi::wait_vmcnt<NLOADS>();         // chunk g+2 may still be in flight
+            else xsmi::wait_vmcnt<0>();
+            xsmi::wait_lgkmcnt0();
+            xsmi::block_barrier();
+            if (g + 3 < total) issue();
+            read_frags(nxt_tag);
+        }
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 2; ++j)
+                acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[cur][1][i], fb[cur][1][j], acc[i][j], 0, 0, 0);
+        __builtin_amdgcn_sched_barrier(0);
+    };
+    if (total > 0) {
+        issue_tile();
+        issue();
+        issue();                                       // a tile has an even number of chunks, at least two
+        xsmi::wait_vmcnt<NLOADS>();
+        xsmi::block_barrier();
+        if (total > 2) issue();
+        read_frags(B0{});
+    }
+    int g = 0;
+    for (; c_tile < tile_end; ++c_tile) {
+        for (int it = 0; it < iters; it += 2, g += 2) {
+            body(B0{}, B1{}, g);
+            body(B1{}, B0{}, g + 1);
+        }
+        epilogue();
+        zero_acc();
+    }
+}
+
 // Packs A for the tap-major kernel.  mode 0 (forward): A[row][tap=(r,s)][ch] = w[row][ch][r][s].
 // mode 1 (backward-data class): A[row=c][tap=(t,u)][ch=k] = w[k][c][r0 + sh*t][s0 + sw*u].
 // One launch lays out the filter for every class of a pass; blocks [first[j], first[j+1]) serve job j.
@@ -880,11 +1395,77 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
+// The same filters for tap_bf16_tile_kernel: bf16, [row tile][chunk][group 4][ROWS rows][8 channels], i.e. the
+// LDS image of a stage's A part per (row tile, chunk).
+__global__ void __launch_bounds__(256) tap_pack_bf16_kernel(const float *__restrict__ w, PackMulti pm, int mode, int rows, int CH,
+                                                             int R, int S, int sh, int sw, int rowtiles, int ROWS) {
+    int ji = 0;
+    while (ji + 1 < pm.njobs && blockIdx.x >= pm.first[ji + 1]) ++ji;
+    const PackJob &j = pm.job[ji];
+    const uint32_t blk = blockIdx.x - pm.first[ji], nblk = pm.first[ji + 1] - pm.first[ji];
+    if (blk == 0 && threadIdx.x < 8) j.counters[threadIdx.x] = 0;
+    __bf16 *__restrict__ apk = reinterpret_cast<__bf16 *>(j.apk);
+    const int TR = j.TR, TS = j.TS, r0 = j.r0, s0 = j.s0;
+    const int nch = CH / KC;
+    const int iters = TR * TS * nch;
+    const size_t per_block = (size_t)ROWS * KC;
+    const size_t total = (size_t)rowtiles * iters * per_block;
+    for (size_t i = (size_t)blk * 256 + threadIdx.x; i < total; i += (size_t)nblk * 256) {
+        int e = (int)(i & 7);
+        size_t rest = i >> 3;
+        int rr = (int)(rest % ROWS);
+        rest /= ROWS;
+        int g = (int)(rest & 3);
+        size_t cblk = rest >> 2;
+        int it = (int)(cblk % iters);
+        int rt = (int)(cblk / iters);
+        int cc = it % nch, tap = it / nch;
+        int tr = tap / TS, ts = tap % TS;
+        int ch = cc * KC + g * 8 + e;
+        int row = rt * ROWS + rr;
+        float v = 0.f;
+        if (row < rows) {
+            if (mode == 0)
+                v = w[(((size_t)row * CH + ch) * R + tr) * S + ts];
+            else
+                v = w[(((size_t)ch * rows + row) * R + (r0 + sh * tr)) * S + (s0 + sw * ts)];
+        }
+        apk[i] = (__bf16)v;
+    }
+}
+
+// Rows per tile of tap_bf16_tile_kernel for a layer with `rows` output rows; 0 = use the fp32-staged kernels.
+int bf16_tile_rows(int opts, int rows) {
+    static int on = -1;
+    if (on < 0) {
+        const char *e = getenv("XSMI_BF16_TILE");
+        on = e ? atoi(e) : 1;
+    }
+    if (!(opts & 1) || !on) return 0;
+    return rows <= 64 ? 64 : 128;
+}
+
 void launch_tap(hipStream_t st, TapMulti mp, int opts) {
     const int bf16 = opts & 1, counters_zeroed = !(opts & 2);   // the pack kernel zeroes the tile counters
     const uint32_t tiles = mp.first[mp.ncls];
     if (tiles == 0) return;
     if (bf16) {
+        const int trows = bf16_tile_rows(opts, mp.cls[0].rows);
+        if (trows) {
+            // tiles are 64 x 256 (one row tile) or 128 x 128; mp was built for 64 x 64
+            TapMulti m2 = mp;
+            m2.rowtiles = xsmi::ceil_div(mp.cls[0].rows, trows);
+            const int pix = trows == 64 ? 256 : 128;
+            uint32_t first = 0;
+            for (int c = 0; c < mp.ncls; ++c) {
+                m2.first[c] = first;
+                first += (uint32_t)xsmi::ceil_div(mp.cls[c].M, pix) * (uint32_t)m2.rowtiles;
+            }
+            m2.first[mp.ncls] = first;
+            if (trows == 64) hipLaunchKernelGGL((tap_bf16_tile_kernel<1, 4>), dim3(first), dim3(256), 0, st, m2);
+            else hipLaunchKernelGGL((tap_bf16_tile_kernel<2, 2>), dim3(first), dim3(256), 0, st, m2);
+            return;
+        }
         // an even number of 64-row tiles pairs up into 128-row tiles: half the activation loads per MFMA
         if ((mp.rowtiles & 1) == 0) {
             TapMulti m2 = mp;
@@ -941,14 +1522,15 @@ uint32_t *tap_counters(float *apk, size_t pack_bytes) { return (uint32_t *)((cha
 struct PackSpec { float *apk; int TR, TS, r0, s0; };
 
 int launch_pack(hipStream_t st, const float *w, const PackSpec *specs, int nspecs, int mode, int rows, int CH, int R, int S,
-                int sh, int sw) {
-    const int rowtiles = xsmi::ceil_div(rows, TM);
+                int sh, int sw, int opts) {
+    const int trows = bf16_tile_rows(opts, rows);
+    const int rowtiles = xsmi::ceil_div(rows, trows ? trows : TM);
     PackMulti pm;
     pm.njobs = 0;
     uint32_t blocks = 0;
     for (int i = 0; i < nspecs; ++i) {
         const PackSpec &sp = specs[i];
-        size_t total = (size_t)rowtiles * sp.TR * sp.TS * (CH / KC) * TM * KC;
+        size_t total = (size_t)rowtiles * sp.TR * sp.TS * (CH / KC) * (trows ? trows : TM) * KC;
         uint32_t nb = (uint32_t)((total + 255) / 256);
         if (nb > 2048) nb = 2048;
         if (nb == 0) nb = 1;                      // a class without taps still gets its counters cleared
@@ -961,7 +1543,10 @@ int launch_pack(hipStream_t st, const float *w, const PackSpec *specs, int nspec
     }
     if (pm.njobs == 0) return XSMI_OK;
     pm.first[pm.njobs] = blocks;
-    hipLaunchKernelGGL(tap_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, mode, rows, CH, R, S, sh, sw, rowtiles);
+    if (trows)
+        hipLaunchKernelGGL(tap_pack_bf16_kernel, dim3(blocks), dim3(256), 0, st, w, pm, mode, rows, CH, R, S, sh, sw, rowtiles, trows);
+    else
+        hipLaunchKernelGGL(tap_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, mode, rows, CH, R, S, sh, sw, rowtiles);
     XSMI_LAUNCH_CHECK("tap_pack_kernel");
     return XSMI_OK;
 }
@@ -987,7 +1572,7 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     float *apk = (float *)workspace;
     if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
         PackSpec spec = {apk, R, S, 0, 0};
-        int rc = launch_pack(st, w, &spec, 1, 0, K, C, R, S, 1, 1);
+        int rc = launch_pack(st, w, &spec, 1, 0, K, C, R, S, 1, 1, opts);
         if (rc) return rc;
     }
     TapParams p;
@@ -1011,6 +1596,91 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     launch_tap(st, mp, opts);
     prof_end();
     XSMI_LAUNCH_CHECK("tap_igemm kernel");
+    return XSMI_OK;
+}
+
+// ---- channels-last bf16 forward ----
+static int nhwc_cp(int C) { return (C + 7) / 8 * 8; }
+static int nhwc_rows(int K) { return K <= 64 ? 64 : 128; }
+static size_t nhwc_apk_bytes(int C, int K, int R, int S) {
+    const int ROWS = nhwc_rows(K);
+    const size_t nchunks = (size_t)(ceil_div(R * S * (nhwc_cp(C) / 8), 8) * 2);   // even
+    return align_up((size_t)ceil_div(K, ROWS) * nchunks * ROWS * 64, 256);
+}
+static size_t nhwc_xp_bytes(int N, int C, int H, int W, int pad) {
+    return align_up((size_t)N * (H + 2 * pad) * (W + 2 * pad) * nhwc_cp(C) * 2, 256);
+}
+
+bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad) {
+    static int on = -1;
+    if (on < 0) {
+        const char *e = getenv("XSMI_BF16_NHWC");
+        on = e ? atoi(e) : 1;
+    }
+    if (!on) return false;
+    if (!(C % 32 == 0 || C <= 8)) return false;
+    return nhwc_xp_bytes(N, C, H, W, pad) < ((size_t)1 << 31) && nhwc_apk_bytes(C, K, R, S) < ((size_t)1 << 32);
+}
+
+size_t nhwc_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int pad) {
+    return nhwc_apk_bytes(C, K, R, S) + nhwc_xp_bytes(N, C, H, W, pad);
+}
+
+int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                  int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace) {
+    hipStream_t st = stream();
+    const int CP = nhwc_cp(C), C8 = CP / 8, ROWS = nhwc_rows(K);
+    const int Hp = H + 2 * pad, Wp = W + 2 * pad;
+    const int nchunks = ceil_div(R * S * C8, 8) * 2, rowtiles = ceil_div(K, ROWS);   // the kernel takes chunks in pairs
+    __bf16 *apk = (__bf16 *)workspace;
+    __bf16 *xp = (__bf16 *)((char *)workspace + nhwc_apk_bytes(C, K, R, S));
+    if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
+        const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
+        int blocks = (int)((total + 255) / 256);
+        if (blocks > 2048) blocks = 2048;
+        hipLaunchKernelGGL(tap_pack_oct_kernel, dim3(blocks), dim3(256), 0, st, w, apk, K, C, R, S, C8, nchunks, rowtiles, ROWS);
+        XSMI_LAUNCH_CHECK("tap_pack_oct_kernel");
+    }
+    prof_begin();
+    {
+        // a workgroup converts WS pixels of one padded row through an LDS tile of C x (WS | 1) floats (<= 32 KB)
+        int WS = 8192 / C - 1;
+        if (WS > W) WS = W;
+        if (WS < 1) WS = 1;
+        const int nseg = ceil_div(W, WS);
+        const size_t lds = (size_t)C * (WS | 1) * sizeof(float);
+        hipLaunchKernelGGL(nhwc_pad_bf16_kernel, dim3((unsigned)(N * Hp * nseg)), dim3(256), lds, st, x, xp, C, H, W, CP, pad, Hp,
+                           Wp, WS, nseg);
+        XSMI_LAUNCH_CHECK("nhwc_pad_bf16_kernel");
+    }
+    NhwcParams p;
+    p.xp = xp; p.apk = (const float *)apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
+    p.xp_bytes = (uint32_t)((size_t)N * Hp * Wp * CP * 2);
+    p.apk_bytes = (uint32_t)nhwc_apk_bytes(C, K, R, S);
+    p.M = N * OH * OW; p.rows = K; p.nchunks = nchunks;
+    p.R = R; p.S = S; p.C8 = C8; p.Hp = Hp; p.Wp = Wp; p.sy = sh; p.sx = sw;
+    p.OY = OH; p.OX = OW; p.dOX = make_fastdiv(OW); p.dOY = make_fastdiv(OH);
+    p.os_n = (long long)K * OH * OW; p.os_k = (long long)OH * OW;
+    p.relu = relu; p.rowtiles = rowtiles;
+    const bool stem = C8 % 4 != 0;           // an octet list that does not split into whole-tap chunks (C <= 8)
+    p.tiles = (uint32_t)ceil_div(p.M, ROWS == 64 ? 256 : 128) * (uint32_t)rowtiles;
+    // as many workgroups as are resident at once (LDS: 48 KB per 128 x 128 tile, 60 KB per 64 x 256 tile)
+    const unsigned resident = (unsigned)cu_count() * (ROWS == 64 ? 2u : 3u);
+    static int persist = -1;
+    if (persist < 0) {
+        const char *e = getenv("XSMI_NHWC_PERSIST");
+        persist = e ? atoi(e) : 0;
+    }
+    const unsigned grid = (!persist || p.tiles < resident) ? p.tiles : resident;
+    if (ROWS == 64) {
+        if (stem) hipLaunchKernelGGL((tap_nhwc_bf16_kernel<1, 4, true>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((tap_nhwc_bf16_kernel<1, 4, false>), dim3(grid), dim3(256), 0, st, p);
+    } else {
+        if (stem) hipLaunchKernelGGL((tap_nhwc_bf16_kernel<2, 2, true>), dim3(grid), dim3(256), 0, st, p);
+        else hipLaunchKernelGGL((tap_nhwc_bf16_kernel<2, 2, false>), dim3(grid), dim3(256), 0, st, p);
+    }
+    prof_end();
+    XSMI_LAUNCH_CHECK("tap_nhwc_bf16_kernel");
     return XSMI_OK;
 }
 
@@ -1058,7 +1728,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
     if (!(opts & 2)) {
         for (int i = 0; i < nplans; i += TAP_MAX_CLASSES) {
             const int n = nplans - i < TAP_MAX_CLASSES ? nplans - i : TAP_MAX_CLASSES;
-            int rc = launch_pack(st, w, specs + i, n, 1, C, K, R, S, sh, sw);
+            int rc = launch_pack(st, w, specs + i, n, 1, C, K, R, S, sh, sw, opts);
             if (rc) return rc;
         }
     }

@@ -44,7 +44,13 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
     size_t b = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     size_t m = a > b ? a : b;
-    return m > c ? m : c;
+    m = m > c ? m : c;
+    // the bf16 forward takes its fastest form when the workspace also holds a channels-last copy of x
+    if (xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad)) {
+        size_t d = xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad);
+        m = m > d ? m : d;
+    }
+    return m;
 }
 
 int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size_t n, float beta) {

@@ -93,6 +93,13 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
                       int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace);
 
+// bf16 forward on a channels-last bf16 copy of the activations (conv_tap.hip): channels a multiple of 32, or
+// at most 8 (a stem); the workspace holds the packed filter followed by the copy
+bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad);
+size_t nhwc_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int pad);
+int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                  int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace);
+
 // tap-major backward-weight (conv_wgrad_tap.hip)
 bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW);
 size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW);
