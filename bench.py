@@ -249,8 +249,8 @@ def bench_resnet18_infer(be, steps, warmup):
     d = logits["bf16"] - logits["fp32"]
     out["resnet18_infer_bf16_logits_rel_l2_vs_fp32"] = float(np.linalg.norm(d) / np.linalg.norm(logits["fp32"]))
     out["resnet18_infer_workload"] = ("N=256x3x224x224, forward only, moving-statistics BN (fresh: mean 0, var 1), "
-                                      "fp32 tensors in HBM; bf16 = conv operands rounded to bf16 in registers, fp32 accumulate; "
-                                      "the 3-channel stem stays on the fp32 kernel")
+                                      "fp32 tensors in HBM, batch norm folded into the convolutions; bf16 = each conv rewrites "
+                                      "its input as a channels-last bf16 copy and multiplies bf16 operands with fp32 accumulation")
     return out
 
 

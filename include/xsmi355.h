@@ -194,6 +194,12 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
 /* Inference form with given statistics (xs/nn/functional.py:708-725); relu != 0 clips at zero. */
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
                   int N, int C, int HW, float eps, int relu);
+/* The same inference normalisation folded into the convolution that precedes it (the pair
+ * xs/layers/convolutional.py:69-78 then xs/nn/functional.py:708-725 collapses to one convolution):
+ * w_out[k][..] = w[k][..] * gamma[k] / sqrt(var[k] + eps), b_out[k] = beta[k] + (bias[k] - mean[k]) * that scale
+ * (bias may be NULL).  w is (K, per_k). */
+int xsmi_bn_fold(const float *w, const float *bias, const float *gamma, const float *beta, const float *mean,
+                 const float *var, float *w_out, float *b_out, int K, int per_k, float eps);
 /* Backward (xs/nn/grad_fn.py:379-411): dgamma = sum(dy*xhat), dbeta = sum(dy),
  * dx = gamma / (m*sqrtvar) * (m*dy - dbeta - xhat*dgamma), m = N*HW.  All three are overwritten.
  * With neg_mask (the byte mask of a fused ReLU) dy counts as 0 where the mask is set (strict mask,

@@ -323,3 +323,50 @@ def test_checkpoint_round_trip_from_the_device(tmp_path):
         np.testing.assert_allclose(h2['train_loss'], h1['train_loss'], rtol=1e-6)
     finally:
         xs.GLOBAL.USE_CUDA = False
+
+
+def test_inference_folds_batch_norm_into_the_convolution(gpu):
+    """Conv2D -> BatchNormalization [-> ReLU] in a Sequential, moving statistics, nothing to differentiate: the
+    normalisation is folded into the filter.  Same values as the layer-by-layer forward (which runs whenever
+    gradients are tracked), layer outputs shared, and the kernel-level fold against its closed form."""
+    from xshinnosuke_amd.layers import Conv2D, BatchNormalization, ReLU
+    K = gpu.kernels
+    rng = np.random.default_rng(31)
+    w = rng.standard_normal((5, 3, 3, 3)).astype(np.float32)
+    b = rng.standard_normal(5).astype(np.float32)
+    g, bt, mu = (rng.standard_normal(5).astype(np.float32) for _ in range(3))
+    var = rng.uniform(0.5, 2.0, 5).astype(np.float32)
+    w2, b2 = K.bn_fold(gpu.to_device(w), gpu.to_device(b), gpu.to_device(g), gpu.to_device(bt), gpu.to_device(mu),
+                       gpu.to_device(var), 1e-3)
+    scale = g / np.sqrt(var + np.float32(1e-3))
+    np.testing.assert_allclose(w2.numpy(), w * scale[:, None, None, None], rtol=1e-6)
+    np.testing.assert_allclose(b2.numpy(), bt + (b - mu) * scale, rtol=1e-5, atol=1e-6)
+    w3, b3 = K.bn_fold(gpu.to_device(w), None, gpu.to_device(g), gpu.to_device(bt), gpu.to_device(mu), gpu.to_device(var), 1e-3)
+    np.testing.assert_allclose(b3.numpy(), bt - mu * scale, rtol=1e-5, atol=1e-6)
+
+    np.random.seed(8)
+    xs.GLOBAL.USE_CUDA = True
+    try:
+        net = Sequential(Conv2D(8, 3, padding=1, input_shape=(3, 10, 12)), BatchNormalization(), ReLU(True),
+                         Conv2D(6, 3, stride=2, padding=1, use_bias=False), BatchNormalization())
+        x = xs.tensor(rng.standard_normal((4, 3, 10, 12)).astype(np.float32)).to('cuda')
+        with xs.no_grad():
+            net(x)                                   # creates the parameters
+        for layer in net._graph:
+            if isinstance(layer, BatchNormalization):
+                c = layer.moving_mean.shape[0] if hasattr(layer.moving_mean, 'shape') else len(layer.moving_mean)
+                layer.moving_mean = xs.tensor(rng.standard_normal(c).astype(np.float32)).to('cuda')
+                layer.moving_variance = xs.tensor(rng.uniform(0.5, 2.0, c).astype(np.float32)).to('cuda')
+                layer._parameters[0].eval = gpu.to_device(rng.standard_normal(c).astype(np.float32))
+                layer._parameters[1].eval = gpu.to_device(rng.standard_normal(c).astype(np.float32))
+        xs.GLOBAL.TRAINING = False
+        plain = net(x).numpy()                       # gradients tracked: layer by layer
+        with xs.no_grad():
+            folded = net(x)
+        assert rel_l2(folded.numpy(), plain) <= 1e-5
+        assert net._graph[0].data is net._graph[1].data is net._graph[2].data
+        assert net._graph[3].data is net._graph[4].data is folded
+        assert folded.grad_fn is None and not folded.requires_grad
+    finally:
+        xs.GLOBAL.TRAINING = True
+        xs.GLOBAL.USE_CUDA = False

@@ -75,6 +75,7 @@ SIGNATURES = {
     "xsmi_bn_workspace_bytes": (_sz, [_i]),
     "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f, _i]),
+    "xsmi_bn_fold": (_i, [_vp] * 8 + [_i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 8 + [_i, _i, _i, _vp, _sz]),
     "xsmi_avgpool_fwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
     "xsmi_avgpool_bwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),

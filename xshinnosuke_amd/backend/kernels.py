@@ -294,6 +294,21 @@ def bn_infer(x, gamma, beta, mean, var, eps, y=None, relu=False):
     return y
 
 
+def bn_fold(w, bias, gamma, beta, mean, var, eps):
+    """Filter and bias of the convolution that equals conv(w, bias) followed by the inference normalisation."""
+    _f32(w, "w")
+    k = w.shape[0]
+    for a in (gamma, beta, mean, var):
+        if a.size != k:
+            raise ValueError("bn_fold: %d statistics for %d filters" % (a.size, k))
+    if bias is not None and bias.size != k:
+        raise ValueError("bn_fold: bias has %d elements for %d filters" % (bias.size, k))
+    w_out, b_out = empty(w.shape), empty((k,))
+    lib.call("xsmi_bn_fold", w.cptr, bias.cptr if bias is not None else None, gamma.cptr, beta.cptr, mean.cptr, var.cptr,
+             w_out.cptr, b_out.cptr, k, w.size // k, float(eps))
+    return w_out, b_out
+
+
 def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=None):
     """dx, dgamma, dbeta; buffers passed in are overwritten completely.  ``neg_mask`` is the byte mask of a fused
     ReLU: the upstream gradient counts as 0 where it is set."""

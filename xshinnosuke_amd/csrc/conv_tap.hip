@@ -1058,11 +1058,15 @@ struct NhwcParams {
     uint32_t tiles;       // pixel tiles x row tiles
 };
 
-// x fp32 [N][C][H][W] -> xp bf16 [N][Hp][Wp][CP]; a workgroup converts WS pixels of one padded row.
+// x fp32 [N][C][H][W] -> xp bf16 [N][Hp][Wp][CP]; a workgroup converts WS pixels of one padded row through an
+// LDS tile.  Reading, a wave covers 64 >> wlog channels x (1 << wlog) pixels per step (runs of consecutive
+// pixels of one channel); writing, 64 >> clog pixels x (1 << clog) channel pairs (runs of consecutive channels
+// of one pixel): both sides move whole contiguous runs without an integer division.
 __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restrict__ x, __bf16 *__restrict__ xp, int C, int H,
-                                                             int W, int CP, int pad, int Hp, int Wp, int WS, int nseg) {
+                                                             int W, int CP, int pad, int Hp, int Wp, int WS, int nseg,
+                                                             int wlog, int clog) {
     extern __shared__ float tile[];                   // [C][WS | 1]
-    const int t = threadIdx.x;
+    const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
     const int seg = blockIdx.x % nseg;
     const int rowid = blockIdx.x / nseg;              // n * Hp + hp
     const int hp = rowid % Hp, n = rowid / Hp;
@@ -1077,29 +1081,54 @@ __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restr
     const int w0 = seg * WS;
     const int wn = W - w0 < WS ? W - w0 : WS;
     const int stride = WS | 1;
+    const size_t HW = (size_t)H * W;
     const float *src = x + (((size_t)n * C) * H + ih) * W + w0;
-    for (int i = t; i < C * wn; i += 256) {
-        int c = i / wn, wl = i - c * wn;
-        tile[c * stride + wl] = src[(size_t)c * H * W + wl];
+    {
+        const int WL = 1 << wlog, cpw = 64 >> wlog;
+        const int wl0 = lane & (WL - 1), cs = lane >> wlog;
+        constexpr int U = 8;                          // loads in flight per thread
+        for (int wl = wl0; wl < wn; wl += WL)
+            for (int c0 = wave * cpw + cs; c0 < C; c0 += 4 * cpw * U) {
+                float v[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int c = c0 + u * 4 * cpw;
+                    v[u] = c < C ? src[(size_t)c * HW + wl] : 0.f;
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const int c = c0 + u * 4 * cpw;
+                    if (c < C) tile[c * stride + wl] = v[u];
+                }
+            }
     }
     __syncthreads();
-    const int CP2 = CP / 2;
-    uint32_t *dst = reinterpret_cast<uint32_t *>(row + (size_t)(pad + w0) * CP);
-    for (int i = t; i < wn * CP2; i += 256) {
-        int wl = i / CP2, c = 2 * (i - wl * CP2);
-        float v0 = c < C ? tile[c * stride + wl] : 0.f;
-        float v1 = c + 1 < C ? tile[(c + 1) * stride + wl] : 0.f;
-        typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
-        bf16x2 pk;
-        pk[0] = (__bf16)v0; pk[1] = (__bf16)v1;
-        dst[i] = __builtin_bit_cast(uint32_t, pk);
+    {
+        const int CP2 = CP / 2;
+        const int CL = 1 << clog, ppw = 64 >> clog;
+        const int c20 = lane & (CL - 1), ps = lane >> clog;
+        uint32_t *dst = reinterpret_cast<uint32_t *>(row + (size_t)(pad + w0) * CP);
+#pragma unroll 4
+        for (int p0 = wave * ppw; p0 < wn; p0 += 4 * ppw) {
+            const int wl = p0 + ps;
+            if (wl < wn)
+                for (int c2 = c20; c2 < CP2; c2 += CL) {
+                    const int c = 2 * c2;
+                    float v0 = c < C ? tile[c * stride + wl] : 0.f;
+                    float v1 = c + 1 < C ? tile[(c + 1) * stride + wl] : 0.f;
+                    typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+                    bf16x2 pk;
+                    pk[0] = (__bf16)v0; pk[1] = (__bf16)v1;
+                    dst[wl * CP2 + c2] = __builtin_bit_cast(uint32_t, pk);
+                }
+        }
+        // left and right border pixels of the row
+        uint32_t *r32 = reinterpret_cast<uint32_t *>(row);
+        if (seg == 0)
+            for (int i = t; i < pad * CP2; i += 256) r32[i] = 0;
+        if (seg == nseg - 1)
+            for (int i = t; i < pad * CP2; i += 256) r32[(size_t)(pad + W) * CP2 + i] = 0;
     }
-    // left and right border pixels of the row
-    uint32_t *r32 = reinterpret_cast<uint32_t *>(row);
-    if (seg == 0)
-        for (int i = t; i < pad * CP2; i += 256) r32[i] = 0;
-    if (seg == nseg - 1)
-        for (int i = t; i < pad * CP2; i += 256) r32[(size_t)(pad + W) * CP2 + i] = 0;
 }
 
 // Filters for the channels-last kernel: bf16 [row tile][chunk][ROWS][4 slots][8], the LDS image of a stage's A
@@ -1649,8 +1678,11 @@ int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
         if (WS < 1) WS = 1;
         const int nseg = ceil_div(W, WS);
         const size_t lds = (size_t)C * (WS | 1) * sizeof(float);
+        int wlog = 0, clog = 0;
+        while ((1 << wlog) < WS && wlog < 6) ++wlog;         // pixels per wave step when reading
+        while ((1 << clog) < CP / 2 && clog < 6) ++clog;     // channel pairs per wave step when writing
         hipLaunchKernelGGL(nhwc_pad_bf16_kernel, dim3((unsigned)(N * Hp * nseg)), dim3(256), lds, st, x, xp, C, H, W, CP, pad, Hp,
-                           Wp, WS, nseg);
+                           Wp, WS, nseg, wlog, clog);
         XSMI_LAUNCH_CHECK("nhwc_pad_bf16_kernel");
     }
     NhwcParams p;

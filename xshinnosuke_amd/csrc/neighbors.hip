@@ -333,6 +333,23 @@ __global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__
     }
 }
 
+// Folds a moving-statistics batch norm that follows a convolution into the convolution: with
+// scale[k] = gamma[k] / sqrt(var[k] + eps), w_out[k][j] = w[k][j] * scale[k] and
+// b_out[k] = beta[k] + (bias[k] - mean[k]) * scale[k].
+__global__ void __launch_bounds__(256) bn_fold_kernel(const float *__restrict__ w, const float *__restrict__ bias,
+                                                       const float *__restrict__ gamma, const float *__restrict__ beta,
+                                                       const float *__restrict__ mean, const float *__restrict__ var,
+                                                       float *__restrict__ w_out, float *__restrict__ b_out, int K, int per_k,
+                                                       float eps) {
+    const size_t total = (size_t)K * per_k;
+    for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
+        const int k = (int)(i / per_k);
+        const float scale = gamma[k] / sqrtf(var[k] + eps);
+        w_out[i] = w[i] * scale;
+        if (i == (size_t)k * per_k) b_out[k] = beta[k] + ((bias ? bias[k] : 0.f) - mean[k]) * scale;
+    }
+}
+
 // ---- average pool over k x k blocks --------------------------------------------
 __global__ void __launch_bounds__(256) avgpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int H, int W,
                                                            int OH, int OW, int k, size_t total) {
@@ -581,6 +598,17 @@ int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const f
         hipLaunchKernelGGL(bn_infer_kernel<false>, grid_for(total), dim3(256), 0, xsmi::stream(), x, gamma, beta, mean,
                            var, y, make_chan(C, HW), (uint32_t)total, eps, relu);
     XSMI_LAUNCH_CHECK("bn_infer_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_bn_fold(const float *w, const float *bias, const float *gamma, const float *beta, const float *mean,
+                 const float *var, float *w_out, float *b_out, int K, int per_k, float eps) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(K > 0 && per_k > 0, "xsmi_bn_fold: empty filter");
+    XSMI_CHECK_ARG(w && gamma && beta && mean && var && w_out && b_out, "xsmi_bn_fold: null pointer");
+    hipLaunchKernelGGL(bn_fold_kernel, grid_for((size_t)K * per_k), dim3(256), 0, xsmi::stream(), w, bias, gamma, beta, mean,
+                       var, w_out, b_out, K, per_k, eps);
+    XSMI_LAUNCH_CHECK("bn_fold_kernel");
     return XSMI_OK;
 }
 

@@ -102,6 +102,37 @@ def conv2d(inputs, weight, bias=None, stride=(1, 1), padding=0, out=None, activa
     return out
 
 
+def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, beta, moving_mean, moving_variance,
+                                epsilon=1e-5, out=None, activation=None):
+    """``batch_norm(conv2d(inputs, ...), ..., training=False)`` (and the ReLU after it) on device tensors as ONE
+    convolution: with given statistics the normalisation is a per-filter scale and shift, which is folded into the
+    filter and the bias first (this package's extension; values equal the two-step form up to float rounding).
+    Forward only: the result carries no ``grad_fn``."""
+    _mark_input(inputs)
+    if activation not in (None, 'relu'):
+        raise ValueError("conv2d_batch_norm_inference can only fuse activation='relu'")
+    x = inputs.eval
+    if not is_device(x):
+        raise NotImplementedError('the folded convolution needs device tensors')
+    if len(x.shape) != 4 or len(weight.shape) != 4:
+        raise ValueError('conv2d expects NCHW input and KCRS weight, got %s and %s' % (x.shape, weight.shape))
+    stride = _pair(stride)
+    padding = int(padding)
+    stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]
+    b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
+    w2, b2 = K.bn_fold(_f32_device(weight.eval), b_dev, *stats, epsilon)
+    dst = out.eval if (out is not None and is_device(out.eval)) else None
+    y = K.conv2d_fwd(_f32_device(x), w2, b2, stride, padding, relu=activation == 'relu', out=dst, bf16=bool(GLOBAL.CONV_BF16))
+    if out is None:
+        out = Tensor(y)
+    elif y is not dst:
+        out.eval = y
+    out.requires_grad = False
+    out.grad_fn = None                               # a reused output tensor may carry one from a tracked forward
+    _wire(out, inputs, weight, bias)
+    return out
+
+
 def max_pool2d(inputs, kernel_size=2, stride=None, padding=0, out=None):
     """Max pooling with zero-valued padding that takes part in the max and first-maximum
     tie-breaking (reference xs/nn/functional.py:445-491).

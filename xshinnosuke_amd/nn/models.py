@@ -15,10 +15,12 @@ from ..core import autograd
 from ..core.base import Tensor, Parameter
 from ..layers.base import Layer
 from ..layers.normalize import BatchNormalization
+from ..layers.convolutional import Conv2D
 from ..layers.activators import ReLU
 from ..optim import get_optimizer
 from ..utils.data import DataSet, DataLoader
 from .objectives import get_objective
+from . import functional as F
 
 
 class _Base:
@@ -242,6 +244,30 @@ class Sequential(_Model):
                 x = layer.forward(x, fuse_relu=True)
                 nxt.data = x
                 i += 2
+            # Inference (moving statistics, nothing to differentiate) of Conv2D -> BatchNormalization [-> ReLU] on a
+            # device-resident dynamic graph: the normalisation is a per-filter scale and shift, folded into the
+            # convolution.  All the layers involved then hold the same output tensor.
+            elif (isinstance(layer, Conv2D) and layer.activation is None and isinstance(nxt, BatchNormalization) and
+                    nxt.axis == 1 and not GLOBAL.TRAINING and not GLOBAL.COMPUTE_GRAD and isinstance(x, Tensor) and
+                    x.is_dynamic and x.device == 'cuda' and len(layer._parameters) and len(nxt._parameters)):
+                relu = layers[i + 2] if i + 2 < n and isinstance(layers[i + 2], ReLU) else None
+                x.next_layers.append(layer)
+                weight, bias = layer._parameters[0], (layer._parameters[1] if layer.use_bias else None)
+                gamma, beta = nxt._parameters
+                # as in the layers' own calls, the previous output tensor is written again when it still fits
+                prev = layer.data if isinstance(layer.data, Tensor) and layer.data.device == 'cuda' else None
+                if prev is not None:
+                    oh, ow = F.K.conv_out_hw(x.shape[2], x.shape[3], weight.shape[2], weight.shape[3], layer.stride, layer.pad_size)
+                    if tuple(prev.shape) != (x.shape[0], weight.shape[0], oh, ow):
+                        prev = None
+                x = F.conv2d_batch_norm_inference(x, weight, bias, layer.stride, layer.pad_size, gamma, beta, nxt.moving_mean,
+                                                  nxt.moving_variance, nxt.epsilon, prev, 'relu' if relu is not None else None)
+                layer.data = x
+                nxt.data = x
+                i += 2
+                if relu is not None:
+                    relu.data = x
+                    i += 1
             else:
                 x = layer.forward(x)
                 i += 1
