@@ -134,6 +134,9 @@ __global__ void __launch_bounds__(256) igemm_f32_kernel(IgemmParams p) {
         fetch(0);
         stage(0);
     }
+    // the tile's bias through the LDS: one coalesced load instead of a dependent global load per output element
+    __shared__ float s_bias[TM];
+    if (p.bias && t < TM) s_bias[t] = rowtile * TM + t < p.rows ? p.bias[rowtile * TM + t] : 0.f;
     __syncthreads();
     for (int c = 0; c < p.nchunks; ++c) {
         const int cur = c & 1;
@@ -182,7 +185,7 @@ __global__ void __launch_bounds__(256) igemm_f32_kernel(IgemmParams p) {
             int row = rbase + it * 32 + 8 * (v >> 2) + (v & 3);
             if (row < p.rows) {
                 float val = it == 0 ? acc0[v] : acc1[v];
-                if (p.bias) val += p.bias[row];
+                if (p.bias) val += s_bias[row - rowtile * TM];
                 long long o = pix_off + (long long)row * p.os_k;
                 if (p.relu) {
                     if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;

@@ -94,6 +94,11 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
     const uint32_t nrt = (uint32_t)mp.rowtiles;
     const int rowtile = nrt == 1 ? 0 : (int)(logical % nrt);
     const int m0 = (int)(nrt == 1 ? logical : logical / nrt) * BP;
+    // The tile's bias goes through the LDS: one coalesced load here instead of a dependent global load per
+    // output element in the epilogue.  Only the forward pass has a bias, and it has at least one chunk, so a
+    // barrier of the main loop lies between this store and the epilogue's reads.
+    __shared__ float s_bias[TM];
+    if (p.bias && t < TM) s_bias[t] = rowtile * TM + t < p.rows ? p.bias[rowtile * TM + t] : 0.f;
 
     // ---- gather role: pixel m0 + lane, channels 8*wave .. 8*wave+7 of each chunk ----
     int iyb = 0, ixb = 0, nbase = 0;
@@ -274,7 +279,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
         int row = rbase + 8 * (v >> 2) + (v & 3);
         if (row < p.rows) {
             float val = acc[v];
-            if (p.bias) val += p.bias[row];
+            if (p.bias) val += s_bias[row - rowtile * TM];
             long long o = pix_off + (long long)row * p.os_k;
             if (p.relu) {
                 if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
@@ -298,6 +303,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
     constexpr int STAGES = 2;
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     __shared__ uint32_t s_next;
+    __shared__ float s_bias[2][TM];                   // bias of the current tile, alternating per tile
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -468,8 +474,12 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
 
     using T0 = std::integral_constant<int, 0>;
     using T1 = std::integral_constant<int, 1>;
+    int bias_buf = 0;
     for (;;) {
         const bool last_tile = !nxt_valid;                    // uniform over the workgroup
+        // one coalesced load of the tile's bias; the chunk loop's barriers publish it before the epilogue reads
+        // it, and the buffer is rewritten only two tiles later
+        if (p.bias && t < TM) s_bias[bias_buf][t] = cur_rowtile * TM + t < p.rows ? p.bias[cur_rowtile * TM + t] : 0.f;
         uint32_t fetched = 0;
         if (!last_tile && t == 0) fetched = atomicAdd(p.counters + xcd, 1u);   // tile after the next one
         // Every chunk runs the full body.  In a workgroup's last tile the two chunks "after the end" are
@@ -496,7 +506,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
                     int row = rbase + 8 * (v >> 2) + (v & 3);
                     if (row < p.rows) {
                         float val = acc[v];
-                        if (p.bias) val += p.bias[row];
+                        if (p.bias) val += s_bias[bias_buf][row - cur_rowtile * TM];
                         long long o = pix_off + (long long)row * p.os_k;
                         if (p.relu) {
                             if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
@@ -514,6 +524,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
         }
 #pragma unroll
         for (int v = 0; v < 16; ++v) { acc[v] = 0.f; acc2[v] = 0.f; }
+        bias_buf ^= 1;
 
         // the tile fetched at the top of this iteration becomes the next one; the issue side has
         // already moved into what was the next tile and now becomes the current one
@@ -1175,6 +1186,7 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
     // covers 256 consecutive bytes' worth of banks with every 16 lanes (the LDS serves 256 bytes per clock), and a B load (16 consecutive pixels x 4 slots, lane = pixel * 4 +
     // slot) reads 64 contiguous bytes per pixel and lands as one contiguous KB.
     __shared__ __attribute__((aligned(16))) unsigned char smem[STAGES * STAGE];
+    __shared__ float s_bias[ROWS];                    // the current tile's bias, staged once per tile
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -1284,6 +1296,13 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
         const int rowtile = nrt == 1 ? 0 : (int)(c_tile - mt * nrt);
         const int m0 = (int)mt * PIX;
         const int rbase = rowtile * ROWS + wr * 64 + 4 * h;
+        // one coalesced load of the tile's bias instead of a dependent global load per output element; the
+        // barrier also keeps a faster wave's next tile from overwriting it (a workgroup-uniform branch)
+        if (p.bias) {
+            if (t < ROWS) s_bias[t] = rowtile * ROWS + t < p.rows ? p.bias[rowtile * ROWS + t] : 0.f;
+            __syncthreads();
+        }
+        const int lrow = wr * 64 + 4 * h;
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int m = m0 + wc * 64 + 32 * j + l31;
@@ -1300,7 +1319,7 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
                     int row = rbase + 32 * i + 8 * (v >> 2) + (v & 3);
                     if (row < p.rows) {
                         float val = acc[i][j][v];
-                        if (p.bias) val += p.bias[row];
+                        if (p.bias) val += s_bias[lrow + 32 * i + 8 * (v >> 2) + (v & 3)];
                         long long o = pix_off + (long long)row * p.os_k;
                         if (p.relu) {
                             if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
