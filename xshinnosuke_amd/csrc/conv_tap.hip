@@ -1050,7 +1050,10 @@ __global__ void __launch_bounds__(256) tap_bf16_tile_kernel(TapMulti mp) {
 //
 // The reduction index is a list of octets, o = tap * (CP / 8) + channel octet; a chunk is four consecutive
 // octets (group g = octet 4 * chunk + g).  With CP a multiple of 32 a chunk is 32 channels of one tap; with
-// CP = 8 (a 3-channel stem) it is four consecutive taps.
+// CP = 8 (5 to 8 channels) it is four consecutive taps.  A stem of at most 4 channels and a filter at most 8
+// wide is copied with CP = 4 instead: 16 bytes are then two horizontally adjacent pixels, an octet is two
+// adjacent taps x 4 channels, and a chunk is one whole filter row (four tap pairs) -- 6 of 8 reduction slots
+// carry data for RGB instead of 3 of 8.
 struct NhwcParams {
     const __bf16 *xp;
     const float *apk;     // bf16 [row tile][chunk][group 4][ROWS][8]
@@ -1059,7 +1062,8 @@ struct NhwcParams {
     uint8_t *mask;
     uint32_t xp_bytes, apk_bytes;
     int M, rows, nchunks;
-    int R, S, C8;         // taps, octets per tap
+    int R, S, C8;         // filter rows, taps per filter row, octets per tap
+    uint32_t pix_bytes, tap_bytes, row_bytes;   // byte steps of the copy: next pixel, next tap, next filter row
     int Hp, Wp, sy, sx;
     int OY, OX;
     xsmi::FastDiv dOX, dOY;
@@ -1083,10 +1087,16 @@ __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restr
     const int hp = rowid % Hp, n = rowid / Hp;
     const int ih = hp - pad;
     __bf16 *row = xp + (size_t)rowid * Wp * CP;
-    if (ih < 0 || ih >= H) {                          // border row: zeros (CP is a multiple of 8: 16-byte stores)
-        uint4 *r4 = reinterpret_cast<uint4 *>(row);
-        const int n16 = Wp * CP / 8;
-        for (int i = seg * 256 + t; i < n16; i += nseg * 256) r4[i] = make_uint4(0, 0, 0, 0);
+    if (ih < 0 || ih >= H) {                          // border row: zeros
+        if ((CP & 7) == 0) {                          // rows are 16-byte multiples
+            uint4 *r4 = reinterpret_cast<uint4 *>(row);
+            const int n16 = Wp * CP / 8;
+            for (int i = seg * 256 + t; i < n16; i += nseg * 256) r4[i] = make_uint4(0, 0, 0, 0);
+        } else {
+            uint32_t *r1 = reinterpret_cast<uint32_t *>(row);
+            const int n4 = Wp * CP / 2;
+            for (int i = seg * 256 + t; i < n4; i += nseg * 256) r1[i] = 0;
+        }
         return;
     }
     const int w0 = seg * WS;
@@ -1142,13 +1152,36 @@ __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restr
     }
 }
 
+// The same copy for at most 4 channels (CP = 4): a thread converts one padded pixel, reads and writes are
+// both runs of consecutive pixels, no LDS.  blockIdx.y = n * Hp + hp.
+__global__ void __launch_bounds__(256) nhwc_pad_c4_kernel(const float *__restrict__ x, __bf16 *__restrict__ xp, int C, int H,
+                                                           int W, int pad, int Hp, int Wp) {
+    const int wp = blockIdx.x * 256 + threadIdx.x;
+    if (wp >= Wp) return;
+    const int rowid = blockIdx.y;
+    const int hp = rowid % Hp, n = rowid / Hp;
+    const int ih = hp - pad, iw = wp - pad;
+    float v[4] = {0.f, 0.f, 0.f, 0.f};
+    if (ih >= 0 && ih < H && iw >= 0 && iw < W) {
+        const float *src = x + (((size_t)n * C) * H + ih) * W + iw;
+#pragma unroll
+        for (int c = 0; c < 4; ++c)
+            if (c < C) v[c] = src[(size_t)c * H * W];
+    }
+    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+    bf16x4 pk;
+#pragma unroll
+    for (int c = 0; c < 4; ++c) pk[c] = (__bf16)v[c];
+    reinterpret_cast<uint2 *>(xp)[(size_t)rowid * Wp + wp] = __builtin_bit_cast(uint2, pk);
+}
+
 // Filters for the channels-last kernel: bf16 [row tile][chunk][ROWS][4 slots][8], the LDS image of a stage's A
 // part.  Octet g of a row sits in slot g ^ ((row >> 2) & 3) (see the kernel); zero where the octet or the
 // channel does not exist.
 __global__ void __launch_bounds__(256) tap_pack_oct_kernel(const float *__restrict__ w, __bf16 *__restrict__ apk, int rows, int C,
-                                                            int R, int S, int C8, int nchunks, int rowtiles, int ROWS) {
+                                                            int R, int S, int C8, int nchunks, int rowtiles, int ROWS, int pair) {
     const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
-    const int octets = R * S * C8;
+    const int octets = pair ? R * 4 : R * S * C8;
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
         int e = (int)(i & 7);
         int slot = (int)((i >> 3) & 3);
@@ -1159,10 +1192,20 @@ __global__ void __launch_bounds__(256) tap_pack_oct_kernel(const float *__restri
         int rt = (int)(cblk / nchunks);
         int g = slot ^ ((rr >> 2) & 3);
         int o = 4 * it + g;
-        int tap = o / C8, ch = (o - tap * C8) * 8 + e;
+        int tap, ch;
+        bool ok = o < octets;
+        if (pair) {                                   // chunk = filter row, group = tap pair, element = (tap, channel)
+            const int sx = 2 * g + (e >> 2);
+            tap = it * S + sx;
+            ch = e & 3;
+            ok = ok && sx < S;
+        } else {
+            tap = o / C8;
+            ch = (o - tap * C8) * 8 + e;
+        }
         int row = rt * ROWS + rr;
         float v = 0.f;
-        if (row < rows && o < octets && ch < C) v = w[((size_t)row * C + ch) * R * S + tap];
+        if (row < rows && ok && ch < C) v = w[((size_t)row * C + ch) * R * S + tap];
         apk[i] = (__bf16)v;
     }
 }
@@ -1197,6 +1240,7 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
     const uint32_t tile_end = (uint32_t)(((uint64_t)(wg + 1) * p.tiles) / gridDim.x);
     const uint32_t nrt = (uint32_t)p.rowtiles;
     const int S = p.S, R = p.R, C8 = p.C8, Wp = p.Wp;
+    const uint32_t row_bytes = p.row_bytes, tap_bytes = p.tap_bytes;
     const int iters = p.nchunks;
     const int total = (int)(tile_end - tile_begin) * iters;       // chunks of this workgroup's stream
 
@@ -1230,7 +1274,7 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
                 int x = m - (int)q * p.OX;
                 uint32_t n = xsmi::fdiv(q, p.dOY);
                 int y = (int)q - (int)n * p.OY;
-                voff[j] = (uint32_t)((((int)n * p.Hp + y * p.sy) * Wp + x * p.sx) * C8) * 16u + (STEM ? 0u : (uint32_t)oct[j] * 16u);
+                voff[j] = (uint32_t)(((int)n * p.Hp + y * p.sy) * Wp + x * p.sx) * p.pix_bytes + (STEM ? 0u : (uint32_t)oct[j] * 16u);
             }
             if (STEM) {
                 rj[j] = oct[j] / S;
@@ -1240,7 +1284,7 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
     };
     auto issue = [&]() {
         // a chunk past the filter (the chunk count is rounded up to even) meets zero rows of A: re-read tap 0
-        const uint32_t soff = (STEM || r >= R) ? 0u : (uint32_t)(((r * Wp + s) * C8 + c8) * 16);
+        const uint32_t soff = (STEM || r >= R) ? 0u : (uint32_t)r * row_bytes + (uint32_t)s * tap_bytes + (uint32_t)c8 * 16u;
 #pragma unroll
         for (int j = 0; j < NB; ++j) {
             uint32_t vo = voff[j];
@@ -1648,15 +1692,21 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
 }
 
 // ---- channels-last bf16 forward ----
-static int nhwc_cp(int C) { return (C + 7) / 8 * 8; }
+// pair mode: at most 4 channels and a filter at most 8 wide (see the kernel's header)
+static bool nhwc_pair(int C, int S) { return C <= 4 && S <= 8; }
+static int nhwc_cp(int C, int S) { return nhwc_pair(C, S) ? 4 : (C + 7) / 8 * 8; }
 static int nhwc_rows(int K) { return K <= 64 ? 64 : 128; }
+static int nhwc_chunks(int C, int R, int S) {           // even: the kernel takes chunks in pairs
+    const int octets = nhwc_pair(C, S) ? R * 4 : R * S * (nhwc_cp(C, S) / 8);
+    return ceil_div(octets, 8) * 2;
+}
 static size_t nhwc_apk_bytes(int C, int K, int R, int S) {
     const int ROWS = nhwc_rows(K);
-    const size_t nchunks = (size_t)(ceil_div(R * S * (nhwc_cp(C) / 8), 8) * 2);   // even
-    return align_up((size_t)ceil_div(K, ROWS) * nchunks * ROWS * 64, 256);
+    return align_up((size_t)ceil_div(K, ROWS) * nhwc_chunks(C, R, S) * ROWS * 64, 256);
 }
-static size_t nhwc_xp_bytes(int N, int C, int H, int W, int pad) {
-    return align_up((size_t)N * (H + 2 * pad) * (W + 2 * pad) * nhwc_cp(C) * 2, 256);
+static size_t nhwc_xp_bytes(int N, int C, int H, int W, int S, int pad) {
+    // one spare pixel: the last tap pair of a row may reach one pixel past the copy's end
+    return align_up(((size_t)N * (H + 2 * pad) * (W + 2 * pad) + 1) * nhwc_cp(C, S) * 2, 256);
 }
 
 bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad) {
@@ -1667,30 +1717,36 @@ bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad) {
     }
     if (!on) return false;
     if (!(C % 32 == 0 || C <= 8)) return false;
-    return nhwc_xp_bytes(N, C, H, W, pad) < ((size_t)1 << 31) && nhwc_apk_bytes(C, K, R, S) < ((size_t)1 << 32);
+    return nhwc_xp_bytes(N, C, H, W, S, pad) < ((size_t)1 << 31) && nhwc_apk_bytes(C, K, R, S) < ((size_t)1 << 32);
 }
 
 size_t nhwc_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int pad) {
-    return nhwc_apk_bytes(C, K, R, S) + nhwc_xp_bytes(N, C, H, W, pad);
+    return nhwc_apk_bytes(C, K, R, S) + nhwc_xp_bytes(N, C, H, W, S, pad);
 }
 
 int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
                   int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace) {
     hipStream_t st = stream();
-    const int CP = nhwc_cp(C), C8 = CP / 8, ROWS = nhwc_rows(K);
+    const bool pair = nhwc_pair(C, S);
+    const int CP = nhwc_cp(C, S), C8 = pair ? 4 : CP / 8, ROWS = nhwc_rows(K);
     const int Hp = H + 2 * pad, Wp = W + 2 * pad;
-    const int nchunks = ceil_div(R * S * C8, 8) * 2, rowtiles = ceil_div(K, ROWS);   // the kernel takes chunks in pairs
+    const int nchunks = nhwc_chunks(C, R, S), rowtiles = ceil_div(K, ROWS);
     __bf16 *apk = (__bf16 *)workspace;
     __bf16 *xp = (__bf16 *)((char *)workspace + nhwc_apk_bytes(C, K, R, S));
     if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
         const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 2048) blocks = 2048;
-        hipLaunchKernelGGL(tap_pack_oct_kernel, dim3(blocks), dim3(256), 0, st, w, apk, K, C, R, S, C8, nchunks, rowtiles, ROWS);
+        hipLaunchKernelGGL(tap_pack_oct_kernel, dim3(blocks), dim3(256), 0, st, w, apk, K, C, R, S, C8, nchunks, rowtiles, ROWS,
+                           pair ? 1 : 0);
         XSMI_LAUNCH_CHECK("tap_pack_oct_kernel");
     }
     prof_begin();
-    {
+    if (CP == 4) {
+        hipLaunchKernelGGL(nhwc_pad_c4_kernel, dim3((unsigned)ceil_div(Wp, 256), (unsigned)(N * Hp)), dim3(256), 0, st, x, xp, C, H,
+                           W, pad, Hp, Wp);
+        XSMI_LAUNCH_CHECK("nhwc_pad_c4_kernel");
+    } else {
         // a workgroup converts WS pixels of one padded row through an LDS tile of C x (WS | 1) floats (<= 32 KB)
         int WS = 8192 / C - 1;
         if (WS > W) WS = W;
@@ -1709,11 +1765,14 @@ int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
     p.xp_bytes = (uint32_t)((size_t)N * Hp * Wp * CP * 2);
     p.apk_bytes = (uint32_t)nhwc_apk_bytes(C, K, R, S);
     p.M = N * OH * OW; p.rows = K; p.nchunks = nchunks;
-    p.R = R; p.S = S; p.C8 = C8; p.Hp = Hp; p.Wp = Wp; p.sy = sh; p.sx = sw;
+    p.R = R; p.S = pair ? 1 : S; p.C8 = C8; p.Hp = Hp; p.Wp = Wp; p.sy = sh; p.sx = sw;
+    p.pix_bytes = (uint32_t)CP * 2u;
+    p.tap_bytes = (uint32_t)CP * 2u;
+    p.row_bytes = (uint32_t)Wp * (uint32_t)CP * 2u;
     p.OY = OH; p.OX = OW; p.dOX = make_fastdiv(OW); p.dOY = make_fastdiv(OH);
     p.os_n = (long long)K * OH * OW; p.os_k = (long long)OH * OW;
     p.relu = relu; p.rowtiles = rowtiles;
-    const bool stem = C8 % 4 != 0;           // an octet list that does not split into whole-tap chunks (C <= 8)
+    const bool stem = C8 % 4 != 0;           // an octet list that does not split into whole-tap chunks (5 to 8 channels)
     p.tiles = (uint32_t)ceil_div(p.M, ROWS == 64 ? 256 : 128) * (uint32_t)rowtiles;
     // as many workgroups as are resident at once (LDS: 48 KB per 128 x 128 tile, 60 KB per 64 x 256 tile)
     const unsigned resident = (unsigned)cu_count() * (ROWS == 64 ? 2u : 3u);
