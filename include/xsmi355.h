@@ -38,7 +38,14 @@ extern "C" {
 
 /* flags for the conv entry points */
 #define XSMI_CONV_RELU 0x1u      /* y = max(0, conv + bias)  (fused epilogue)            */
-#define XSMI_CONV_BF16 0x2u      /* opt-in: bf16 MFMA operands, fp32 accumulate          */
+#define XSMI_CONV_BF16 0x2u      /* opt-in: operands rounded to bf16 (nearest even), fp32
+                                    accumulate.  The forward (channels a multiple of 32, or at
+                                    most 8) first writes a channels-last bf16 copy of x with a
+                                    zero border into the workspace and multiplies from it; it
+                                    takes this form when the workspace has the size that
+                                    xsmi_conv2d_workspace_bytes reports, and a slower one that
+                                    gathers from x directly when it only has room for the filter.
+                                    The weight gradient ignores the flag.                     */
 #define XSMI_CONV_WS_PACKED 0x4u /* the workspace still holds what the previous call of the same
                                     entry point with the same geometry and the same filter values
                                     left there: the filter is not laid out again (inference loops).
