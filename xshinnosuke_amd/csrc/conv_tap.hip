@@ -787,8 +787,11 @@ __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restr
                                                              int wlog, int clog) {
     extern __shared__ float tile[];                   // [C][WS | 1]
     const int t = threadIdx.x, lane = t & 63, wave = t >> 6;
-    const int seg = blockIdx.x % nseg;
-    const int rowid = blockIdx.x / nseg;              // n * Hp + hp
+    // consecutive rows of an image go to the same XCD: input rows are short unaligned runs, and neighbouring rows
+    // share the memory blocks their ends straddle
+    const uint32_t bid = xsmi::xcd_contiguous_id(blockIdx.x, gridDim.x);
+    const int seg = (int)(bid % (uint32_t)nseg);
+    const int rowid = (int)(bid / (uint32_t)nseg);    // n * Hp + hp
     const int hp = rowid % Hp, n = rowid / Hp;
     const int ih = hp - pad;
     __bf16 *row = xp + (size_t)rowid * Wp * CP;
