@@ -253,6 +253,26 @@ def test_conv_full_size_adjoint_and_slice(gpu):
     assert rel_l2(gw, dw_ref) <= TOL
 
 
+@pytest.mark.parametrize("c,hw,k,r,st,pad", [(128, 28, 128, 3, 1, 1), (3, 224, 64, 7, 2, 3)])
+def test_conv_bf16_full_size_batch_slices(gpu, c, hw, k, r, st, pad):
+    """bf16 forward at the inference batch (N=256; a residual-stage layer and the stem): every image is
+    convolved independently and in one reduction order, so images cut from the big batch equal the same images
+    run as a small batch bit for bit, and the small batch meets the oracle on bf16-rounded operands."""
+    K = gpu.kernels
+    n = 256
+    rng = np.random.default_rng(40 + c)
+    x = rng.standard_normal((n, c, hw, hw), dtype=np.float32)
+    wt = he_normal(rng, (k, c, r, r))
+    b = rng.standard_normal((k,)).astype(np.float32)
+    dw_, db_ = gpu.to_device(wt), gpu.to_device(b)
+    y = K.conv2d_fwd(gpu.to_device(x), dw_, db_, (st, st), pad, relu=True, bf16=True).numpy()
+    for sl in (slice(0, 2), slice(101, 104), slice(254, 256)):
+        part = K.conv2d_fwd(gpu.to_device(x[sl]), dw_, db_, (st, st), pad, relu=True, bf16=True).numpy()
+        np.testing.assert_array_equal(y[sl], part)
+    ref, _ = oracle.conv2d_fwd(round_bf16(x[254:]), round_bf16(wt), b, (st, st), pad)
+    assert rel_l2(y[254:], np.maximum(ref, 0.0)) <= TOL
+
+
 def test_conv_rejects_bad_arguments(gpu):
     K = gpu.kernels
     x = gpu.zeros((1, 3, 4, 4)); w = gpu.zeros((2, 4, 3, 3))
