@@ -108,3 +108,43 @@ def test_softmax_cross_entropy(gpu):
         if reduction == "mean":
             gref /= 37
         assert rel_l2(g, gref) <= 1e-5
+
+
+def test_held_back_add_joins_the_in_place_relu(gpu):
+    """kernels.add(defer=True) launches nothing until the next library call: an in-place ReLU of the result runs
+    as one add+ReLU pass, anything else (a read, a write to an operand, another add) sees the plain sum."""
+    from xshinnosuke_amd.backend import capi
+    K = gpu.kernels
+    rng = np.random.default_rng(12)
+    a = rng.standard_normal((3, 5, 7, 9)).astype(np.float32)
+    b = rng.standard_normal((3, 5, 7, 9)).astype(np.float32)
+    da, db = gpu.to_device(a), gpu.to_device(b)
+    c = K.add(da, db, defer=True)
+    assert capi._deferred and capi._deferred[0][2] is c
+    r = K.relu_fwd(c, out=c)
+    assert r is c and not capi._deferred
+    np.testing.assert_array_equal(c.numpy(), np.maximum(a + b, 0.0))
+    c = K.add(da, db, defer=True)
+    np.testing.assert_array_equal(c.numpy(), a + b)                 # a read enqueues the add first
+    c = K.add(da, db, defer=True)
+    da.fill_zero()                                                   # so does a write to an operand
+    np.testing.assert_array_equal(c.numpy(), a + b)
+    np.testing.assert_array_equal(da.numpy(), np.zeros_like(a))
+    da.set(a)
+    c1 = K.add(da, db, defer=True)
+    c2 = K.add(c1, db, defer=True)                                   # and another held-back add
+    other = gpu.to_device(a)
+    K.relu_fwd(other, out=other)                                     # an in-place ReLU of something else
+    assert not capi._deferred
+    np.testing.assert_array_equal(c2.numpy(), (a + b) + b)
+    np.testing.assert_array_equal(other.numpy(), np.maximum(a, 0.0))
+    # through the tensor API: no_grad residual add + in-place ReLU layer
+    import xshinnosuke_amd as xs
+    from xshinnosuke_amd.layers import ReLU
+    ta, tb = xs.tensor(a).to('cuda'), xs.tensor(b).to('cuda')
+    with xs.no_grad():
+        out = ta + tb
+        out = ReLU(inplace=True)(out)
+    np.testing.assert_array_equal(out.numpy(), np.maximum(a + b, 0.0))
+    out2 = ta + tb                                                   # gradients tracked or not: same values
+    np.testing.assert_array_equal(out2.numpy(), a + b)

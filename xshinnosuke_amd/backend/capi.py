@@ -67,6 +67,7 @@ SIGNATURES = {
     "xsmi_axpy": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_axpy_multi": (_i, [_i, _c.POINTER(_vp), _c.POINTER(_vp), _c.POINTER(_sz), _f]),
     "xsmi_add": (_i, [_vp, _vp, _vp, _sz]),
+    "xsmi_add_relu": (_i, [_vp, _vp, _vp, _sz]),
     "xsmi_scale_shift": (_i, [_vp, _vp, _f, _f, _sz]),
     "xsmi_relu_fwd": (_i, [_vp, _vp, _sz]),
     "xsmi_relu_fwd_mask": (_i, [_vp, _vp, _vp, _sz]),
@@ -121,6 +122,8 @@ class _Lib:
 
     def call(self, name, *args):
         """Call an int-returning entry point; raise with the library's message on failure."""
+        if _deferred:
+            _flush_deferred()
         dll = self._open()
         rc = getattr(dll, name)(*args)
         if rc != 0:
@@ -131,6 +134,33 @@ class _Lib:
 
 
 lib = _Lib()
+
+# One element-wise add may be held back until the next call into the library: if that call is the in-place ReLU
+# of its result, both run as one pass (kernels.add / kernels.relu_fwd).  Every other call enqueues the add first,
+# so nothing can read or change the operands or the result between the add and the point where it was asked for.
+_deferred = []          # at most one (a, b, out) triple of device arrays
+
+
+def _flush_deferred():
+    a, b, out = _deferred.pop()
+    lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
+
+
+def defer_add(a, b, out):
+    if _deferred:
+        _flush_deferred()
+    _deferred.append((a, b, out))
+
+
+def take_deferred_add(out):
+    """The operands of the held-back add whose result is ``out``, or None (a different pending add is enqueued)."""
+    if not _deferred:
+        return None
+    if _deferred[0][2] is out:
+        a, b, _ = _deferred.pop()
+        return a, b
+    _flush_deferred()
+    return None
 
 
 def init(device=0):

@@ -8,6 +8,7 @@ import ctypes
 
 import numpy as np
 
+from . import capi
 from .capi import lib, CONV_RELU, CONV_BF16, CONV_WS_PACKED
 from .array import DeviceArray, Workspace, empty
 
@@ -212,8 +213,15 @@ def axpy_multi(ys, xs, a):
     lib.call("xsmi_axpy_multi", n, yp, xp, ns, float(a))
 
 
-def add(a, b, out=None):
+def add(a, b, out=None, defer=False):
+    """``defer=True`` (new result array only) holds the launch back until the next call into the library, so that
+    an in-place ReLU of the result can run in the same pass; any other call enqueues the add first."""
     _f32(a, "a"); _f32(b, "b")
+    if defer and out is None and a.size == b.size:
+        out = empty(a.shape)
+        a.ptr; b.ptr                                  # operands with a pending clear are cleared now
+        capi.defer_add(a, b, out)
+        return out
     out = _like(a, out)
     lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
     return out
@@ -232,6 +240,11 @@ def add_scalar(a, t, out=None):
 
 def relu_fwd(x, out=None):
     _f32(x, "x")
+    if out is x:                                      # in place: a held-back add that produced x joins this pass
+        ops = capi.take_deferred_add(x)
+        if ops is not None:
+            lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, x.size)
+            return x
     out = _like(x, out)
     lib.call("xsmi_relu_fwd", x.cptr, out.cptr, x.size)
     return out

@@ -50,6 +50,15 @@ struct AddF {
         reinterpret_cast<float4 *>(o)[j] = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
     }
 };
+struct AddReluF {
+    const float *a, *b; float *o;
+    __device__ static float f(float u, float v) { const float t = u + v; return t > 0.f ? t : 0.f; }
+    __device__ void one(size_t i) const { o[i] = f(a[i], b[i]); }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
+        reinterpret_cast<float4 *>(o)[j] = make_float4(f(u.x, v.x), f(u.y, v.y), f(u.z, v.z), f(u.w, v.w));
+    }
+};
 struct ScaleF {
     const float *a; float *o; float s, t;
     __device__ void one(size_t i) const { o[i] = s * a[i] + t; }
@@ -523,6 +532,11 @@ int xsmi_add(const float *a, const float *b, float *out, size_t n) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add: null pointer");
     return launch_ew("add", n, aligned16(a) && aligned16(b) && aligned16(out), AddF{a, b, out});
+}
+int xsmi_add_relu(const float *a, const float *b, float *out, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add_relu: null pointer");
+    return launch_ew("add_relu", n, aligned16(a) && aligned16(b) && aligned16(out), AddReluF{a, b, out});
 }
 int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n) {
     XSMI_REQUIRE_INIT();

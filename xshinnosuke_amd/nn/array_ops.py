@@ -40,11 +40,12 @@ def iadd(dst, src):
         np.add(dst, np.asarray(same_place(dst, src)).reshape(dst.shape), out=dst)
 
 
-def add(a, b, out=None):
+def add(a, b, out=None, defer=False):
+    """``defer`` (device arrays, new result): see kernels.add."""
     if is_device(a):
         b = same_place(a, b)
         if b.size == a.size:
-            return K.add(a, b, out)
+            return K.add(a, b, out, defer=defer)
         if b.size == 1:
             return K.add_scalar(a, float(b.numpy().reshape(-1)[0]), out)
         raise NotImplementedError('broadcast add of %s and %s on the device' % (a.shape, b.shape))
