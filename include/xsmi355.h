@@ -177,8 +177,9 @@ int xsmi_axpy_multi(int count, float *const *ys, const float *const *xs, const s
 /* out[i] = a[i] + b[i]                   (residual add, xs/nn/functional.py:6-21) */
 int xsmi_add(const float *a, const float *b, float *out, size_t n);
 /* out[i] = max(0, a[i] + b[i]): the residual add followed by the block's in-place ReLU
- * (xs/nn/functional.py:6-21 then xs/layers/activators.py:37-50) in one pass */
-int xsmi_add_relu(const float *a, const float *b, float *out, size_t n);
+ * (xs/nn/functional.py:6-21 then xs/layers/activators.py:37-50) in one pass; neg_mask (or NULL)
+ * receives 1 where the sum is < 0, the sign the ReLU's backward needs */
+int xsmi_add_relu(const float *a, const float *b, float *out, uint8_t *neg_mask, size_t n);
 /* out[i] = s * a[i] + t */
 int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n);
 /* y = max(0, x) (may be in place)        (xs/nn/td_functional.py:59-60) */

@@ -148,3 +148,11 @@ def test_held_back_add_joins_the_in_place_relu(gpu):
     np.testing.assert_array_equal(out.numpy(), np.maximum(a + b, 0.0))
     out2 = ta + tb                                                   # gradients tracked or not: same values
     np.testing.assert_array_equal(out2.numpy(), a + b)
+    # tracked: the fused pass also delivers the ReLU's sign mask, and the gradient reaches both operands masked
+    ta.requires_grad = True; tb.requires_grad = True
+    out3 = ReLU(inplace=True)(ta + tb)
+    np.testing.assert_array_equal(out3.numpy(), np.maximum(a + b, 0.0))
+    out3.backward(xs.tensor(np.ones_like(a)).to('cuda'))
+    expect = ((a + b) >= 0).astype(np.float32)
+    np.testing.assert_array_equal(ta.grad.numpy(), expect)
+    np.testing.assert_array_equal(tb.grad.numpy(), expect)

@@ -67,7 +67,7 @@ SIGNATURES = {
     "xsmi_axpy": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_axpy_multi": (_i, [_i, _c.POINTER(_vp), _c.POINTER(_vp), _c.POINTER(_sz), _f]),
     "xsmi_add": (_i, [_vp, _vp, _vp, _sz]),
-    "xsmi_add_relu": (_i, [_vp, _vp, _vp, _sz]),
+    "xsmi_add_relu": (_i, [_vp, _vp, _vp, _vp, _sz]),
     "xsmi_scale_shift": (_i, [_vp, _vp, _f, _f, _sz]),
     "xsmi_relu_fwd": (_i, [_vp, _vp, _sz]),
     "xsmi_relu_fwd_mask": (_i, [_vp, _vp, _vp, _sz]),

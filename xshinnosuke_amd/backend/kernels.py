@@ -243,7 +243,7 @@ def relu_fwd(x, out=None):
     if out is x:                                      # in place: a held-back add that produced x joins this pass
         ops = capi.take_deferred_add(x)
         if ops is not None:
-            lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, x.size)
+            lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, None, x.size)
             return x
     out = _like(x, out)
     lib.call("xsmi_relu_fwd", x.cptr, out.cptr, x.size)
@@ -253,6 +253,12 @@ def relu_fwd(x, out=None):
 def relu_fwd_mask(x, out=None):
     """Returns (max(0, x), uint8 mask of x < 0); ``out`` may be ``x`` itself."""
     _f32(x, "x")
+    if out is x:                                      # in place: a held-back add that produced x joins this pass
+        ops = capi.take_deferred_add(x)
+        if ops is not None:
+            mask = empty(x.shape, np.uint8)
+            lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, mask.cptr, x.size)
+            return x, mask
     out = _like(x, out)
     mask = empty(x.shape, np.uint8)
     lib.call("xsmi_relu_fwd_mask", x.cptr, out.cptr, mask.cptr, x.size)

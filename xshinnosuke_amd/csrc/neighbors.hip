@@ -51,12 +51,18 @@ struct AddF {
     }
 };
 struct AddReluF {
-    const float *a, *b; float *o;
-    __device__ static float f(float u, float v) { const float t = u + v; return t > 0.f ? t : 0.f; }
-    __device__ void one(size_t i) const { o[i] = f(a[i], b[i]); }
+    const float *a, *b; float *o; uint8_t *m;        // m (optional): 1 where the sum is < 0
+    __device__ static float f(float t) { return t > 0.f ? t : 0.f; }
+    __device__ void one(size_t i) const {
+        const float t = a[i] + b[i];
+        if (m) m[i] = t < 0.f ? 1 : 0;
+        o[i] = f(t);
+    }
     __device__ void quad(size_t j) const {
         float4 u = reinterpret_cast<const float4 *>(a)[j], v = reinterpret_cast<const float4 *>(b)[j];
-        reinterpret_cast<float4 *>(o)[j] = make_float4(f(u.x, v.x), f(u.y, v.y), f(u.z, v.z), f(u.w, v.w));
+        const float4 t = make_float4(u.x + v.x, u.y + v.y, u.z + v.z, u.w + v.w);
+        if (m) reinterpret_cast<uchar4 *>(m)[j] = make_uchar4(t.x < 0.f, t.y < 0.f, t.z < 0.f, t.w < 0.f);
+        reinterpret_cast<float4 *>(o)[j] = make_float4(f(t.x), f(t.y), f(t.z), f(t.w));
     }
 };
 struct ScaleF {
@@ -533,10 +539,11 @@ int xsmi_add(const float *a, const float *b, float *out, size_t n) {
     XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add: null pointer");
     return launch_ew("add", n, aligned16(a) && aligned16(b) && aligned16(out), AddF{a, b, out});
 }
-int xsmi_add_relu(const float *a, const float *b, float *out, size_t n) {
+int xsmi_add_relu(const float *a, const float *b, float *out, uint8_t *neg_mask, size_t n) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add_relu: null pointer");
-    return launch_ew("add_relu", n, aligned16(a) && aligned16(b) && aligned16(out), AddReluF{a, b, out});
+    return launch_ew("add_relu", n, aligned16(a) && aligned16(b) && aligned16(out) && (((uintptr_t)neg_mask & 3) == 0),
+                     AddReluF{a, b, out, neg_mask});
 }
 int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n) {
     XSMI_REQUIRE_INIT();

@@ -192,10 +192,10 @@ def _binary(lhs, rhs, fn, backward_fn, out):
 
 
 def add(lhs, rhs, out=None):
-    # With nothing to differentiate, the launch of a device add is held back until the next operation: the in-place
-    # ReLU of a residual block then computes max(0, lhs + rhs) in one pass (same values; see backend/kernels.add).
-    defer = out is None and not (GLOBAL.COMPUTE_GRAD and (lhs.requires_grad or rhs.requires_grad))
-    return _binary(lhs, rhs, lambda a, b, o: A.add(a, b, o, defer=defer), AddBackward, out)
+    # The launch of a device add into a new tensor is held back until the next operation: the in-place ReLU of a
+    # residual block then computes max(0, lhs + rhs) (and its sign mask) in one pass; anything else sees the plain
+    # sum (see backend/kernels.add).
+    return _binary(lhs, rhs, lambda a, b, o: A.add(a, b, o, defer=o is None), AddBackward, out)
 
 
 def sub(lhs, rhs, out=None):
