@@ -556,8 +556,10 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 //   stage  A [4 groups][ROWS][8 bf16], B [4 groups][PIX][8 bf16]; three stages
 // A is packed to bf16 in exactly that layout by tap_pack_bf16_kernel and arrives by LDS-direct loads.  B is
 // gathered from the fp32 tensor into registers (a thread = one pixel, 8*k consecutive channels, so every
-// wave-level load is 256 contiguous bytes), converted and written with 128-bit LDS stores.  The loads of
-// chunk i+2 are issued while chunk i multiplies; chunk i+1 is converted and stored during the same iteration.
+// wave-level load is 256 contiguous bytes), converted and written with 128-bit LDS stores.  While chunk i
+// multiplies, chunk i+1 is converted and stored, B of chunk i+3 is requested into the register set that frees and A
+// of chunk i+2 into the stage that chunk i-1 has left.  This is the forward's fallback when the workspace has no
+// room for a channels-last copy, and the bf16 backward-data kernel.
 template <int WR, int WC>
 __global__ void __launch_bounds__(256) tap_bf16_tile_kernel(TapMulti mp) {
     static_assert(WR * WC == 4, "four waves");
