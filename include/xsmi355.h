@@ -105,8 +105,8 @@ int xsmi_copy_kernel(void *dst, const void *src, size_t bytes);
  * x (N,C,H,W), w (K,C,R,S), bias (K) or NULL, y (N,K,OH,OW).
  */
 
-/* Workspace needed by the three conv entry points for this geometry (the
- * maximum over fwd / bwd_data / bwd_weight and over flags). */
+/* Workspace needed by the conv entry points for this geometry (the maximum
+ * over fwd / bwd_data / bwd_weight / bwd and over flags). */
 size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S,
                                    int sh, int sw, int pad);
 
@@ -138,6 +138,18 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
                            int N, int C, int H, int W, int K, int R, int S,
                            int sh, int sw, int pad, float beta, unsigned flags,
                            void *workspace, size_t workspace_bytes);
+
+/* Both backward passes of one layer in one call: what xsmi_conv2d_bwd_weight and
+ * xsmi_conv2d_bwd_data compute, with the same results bit for bit (Conv2DBackward,
+ * xs/nn/grad_fn.py:191-203, does the two one after the other).  The two share only
+ * their inputs, so the weight gradient runs on a second stream of the library beside
+ * the data gradient; the main stream waits for both before the call's successors.
+ * db may be NULL.  flags: XSMI_CONV_BF16 or 0. */
+int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w,
+                    float *dx, float *dw, float *db,
+                    int N, int C, int H, int W, int K, int R, int S,
+                    int sh, int sw, int pad, float beta_dx, float beta_dw, unsigned flags,
+                    void *workspace, size_t workspace_bytes);
 
 /* ---- max pooling ---------------------------------------------------------
  * x (N,C,H,W) -> y (N,C,OH,OW), square window k, zero-valued padding that takes

@@ -177,6 +177,29 @@ def test_conv_bf16_forward_channels_last(gpu, n, c, h, w, k, r, s, sh, sw, pad):
     assert rel_l2(y0 + b.reshape(1, -1, 1, 1), pre_ref) <= TOL
 
 
+@pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", [CASES[2], CASES[4], CASES[6], CASES[9], CASES[11]])
+@pytest.mark.parametrize("accumulate", [False, True])
+def test_conv_both_gradients_in_one_call(gpu, n, c, h, w, k, r, s, sh, sw, pad, accumulate):
+    """xsmi_conv2d_bwd runs the two backward kernels side by side on two streams: same bits as the two
+    calls one after the other, also when adding into gradients that are already there, and twice in a row
+    (the second call's kernels must wait for the first call's)."""
+    K = gpu.kernels
+    rng = np.random.default_rng(77 + c + k)
+    x = gpu.to_device(rng.standard_normal((n, c, h, w)).astype(np.float32))
+    wt = gpu.to_device(he_normal(rng, (k, c, r, s)))
+    oh, ow = K.conv_out_hw(h, w, r, s, (sh, sw), pad)
+    dys = [gpu.to_device(rng.standard_normal((n, k, oh, ow)).astype(np.float32)) for _ in range(2)]
+    init = [rng.standard_normal(shape).astype(np.float32) for shape in ((n, c, h, w), (k, c, r, s), (k,))]
+    a = [gpu.to_device(v) for v in init]
+    b = [gpu.to_device(v) for v in init]
+    for dy in dys:
+        K.conv2d_bwd_weight(dy, x, wt.shape, (sh, sw), pad, dw=a[1], db=a[2], accumulate=accumulate)
+        K.conv2d_bwd_data(dy, wt, x.shape, (sh, sw), pad, dx=a[0], accumulate=accumulate)
+        K.conv2d_bwd(dy, x, wt, b[0], b[1], b[2], (sh, sw), pad, accumulate=accumulate)
+    for u, v in zip(a, b):
+        assert np.array_equal(u.numpy(), v.numpy())
+
+
 def test_conv_packed_workspace_flag(gpu):
     """XSMI_CONV_WS_PACKED: a repeated forward / backward-data call may skip laying the filter out again."""
     K = gpu.kernels

@@ -61,6 +61,7 @@ SIGNATURES = {
     "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
     "xsmi_conv2d_bwd_data": (_i, [_vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
     "xsmi_conv2d_bwd_weight": (_i, [_vp, _vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
+    "xsmi_conv2d_bwd": (_i, [_vp] * 6 + _CONV_DIMS + [_f, _f, _u, _vp, _sz]),
     "xsmi_maxpool2d_fwd": (_i, [_vp, _vp, _vp] + [_i] * 8),
     "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
     "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),

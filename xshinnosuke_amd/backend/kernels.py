@@ -121,6 +121,27 @@ def conv2d_bwd_weight(dy, x, w_shape, stride=(1, 1), pad=0, dw=None, db=None, ac
     return dw, db
 
 
+def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False, bf16=False):
+    """Both gradients of one layer in one call, into existing device buffers; the two kernels run side by side.
+    Same results as ``conv2d_bwd_weight`` followed by ``conv2d_bwd_data``."""
+    _f32(dy, "dy"); _f32(x, "x"); _f32(w, "w")
+    dims = _dims(x.shape, w.shape, stride, pad)
+    n, c, h, wd, k, r, s = dims[:7]
+    oh, ow = conv_out_hw(h, wd, r, s, stride, pad)
+    if dy.shape != (n, k, oh, ow):
+        raise ValueError("conv2d backward: dy has shape %s, expected %s" % (dy.shape, (n, k, oh, ow)))
+    if dx.shape != tuple(x.shape) or dw.shape != tuple(w.shape):
+        raise ValueError("conv2d backward: dx %s / dw %s do not match x %s / w %s" % (dx.shape, dw.shape, x.shape, w.shape))
+    if db is not None and db.size != k:
+        raise ValueError("conv2d backward: db has %d elements for %d filters" % (db.size, k))
+    ws, ws_bytes = _workspace(dims)
+    beta_dw = _beta(accumulate, dw, db)
+    beta_dx = _beta(accumulate, dx)
+    lib.call("xsmi_conv2d_bwd", dy.cptr, x.cptr, w.cptr, dx.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
+             beta_dx, beta_dw, CONV_BF16 if bf16 else 0, ws, ws_bytes)
+    return dx, dw, db
+
+
 def pool_out_hw(h, w, k, stride, pad):
     if stride[0] < 1 or stride[1] < 1 or pad < 0:
         raise ValueError("stride must be positive and padding non-negative (got %s, %s)" % (stride, pad))

@@ -6,6 +6,9 @@
 namespace {
 thread_local char g_err[512] = "";
 hipStream_t g_stream = nullptr;
+hipStream_t g_side = nullptr;            // second stream for work that may overlap the main stream's
+hipStream_t g_current = nullptr;         // what stream() hands out: g_stream, or g_side inside a side section
+hipEvent_t g_fork = nullptr, g_join = nullptr;
 int g_device = -1;
 int g_cus = 0;
 bool g_ready = false;
@@ -21,14 +24,29 @@ void set_error(const char *fmt, ...) {
     vsnprintf(g_err, sizeof(g_err), fmt, ap);
     va_end(ap);
 }
-hipStream_t stream() { return g_stream; }
+hipStream_t stream() { return g_current; }
+// A side section runs the launches issued between side_begin() and side_end() on the second stream, ordered
+// after everything enqueued on the main stream so far; side_join() makes the main stream wait for them.  The
+// caller puts independent main-stream work between side_end() and side_join().
+int side_begin() {
+    XSMI_HIP(hipEventRecord(g_fork, g_stream));
+    XSMI_HIP(hipStreamWaitEvent(g_side, g_fork, 0));
+    g_current = g_side;
+    return XSMI_OK;
+}
+void side_end() { g_current = g_stream; }
+int side_join() {
+    XSMI_HIP(hipEventRecord(g_join, g_side));
+    XSMI_HIP(hipStreamWaitEvent(g_stream, g_join, 0));
+    return XSMI_OK;
+}
 bool ready() { return g_ready; }
 int cu_count() { return g_cus; }
 void prof_begin() {
-    if (g_profiling) (void)hipEventRecord(g_prof0, g_stream);
+    if (g_profiling && g_current == g_stream) (void)hipEventRecord(g_prof0, g_stream);
 }
 void prof_end() {
-    if (g_profiling) {
+    if (g_profiling && g_current == g_stream) {
         (void)hipEventRecord(g_prof1, g_stream);
         g_prof_valid = true;
     }
@@ -66,6 +84,10 @@ int xsmi_init(int device) {
         return XSMI_ERR_RUNTIME;
     }
     XSMI_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
+    XSMI_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
+    XSMI_HIP(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));
+    XSMI_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    g_current = g_stream;
     g_device = device;
     g_cus = prop.multiProcessorCount;
     g_ready = true;

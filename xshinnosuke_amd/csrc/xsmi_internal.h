@@ -9,8 +9,14 @@ namespace xsmi {
 
 // Thread-local error text returned by xsmi_last_error().
 void set_error(const char *fmt, ...);
-// Library stream; nullptr until xsmi_init succeeded.
+// The stream ops launch on: the library's main stream, or its second stream inside a side section.
+// nullptr until xsmi_init succeeded.
 hipStream_t stream();
+// Side section: launches between side_begin() and side_end() go to the second stream, ordered after all
+// earlier main-stream work; side_join() makes the main stream wait for them.
+int side_begin();
+void side_end();
+int side_join();
 bool ready();
 int cu_count();
 // With xsmi_profiling(1) every op brackets its main kernel(s) with two events on

@@ -58,6 +58,14 @@ def Conv2DBackward(outputs):
     w_dev = _f32_device(weight.eval)
     want_dw = weight.requires_grad
     want_db = bias is not None and bias.requires_grad
+    if want_dw and inputs.requires_grad:
+        dw_buf, dx_buf = weight.grad.eval, inputs.grad.eval
+        db_buf = bias.grad.eval if want_db else None
+        if is_device(dw_buf) and is_device(dx_buf) and (not want_db or is_device(db_buf)):
+            # all gradients live on the device: one call, the two kernels side by side
+            K.conv2d_bwd(dy, x_dev, w_dev, dx_buf, dw_buf, db_buf.reshape(-1) if want_db else None, stride, pad,
+                         accumulate=True, bf16=bf16)
+            return
     if want_dw or want_db:
         dw_buf = weight.grad.eval if want_dw else None
         db_buf = bias.grad.eval if want_db else None
