@@ -205,7 +205,7 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n);
 
 /* Batch normalisation over axis 1 of an (N, C, HW) tensor with batch statistics
  * (xs/nn/functional.py:676-707): y = gamma * xhat + beta, xhat = (x - mean) / sqrt(var + eps),
- * biased variance.  Outputs xhat (N*C*HW), sqrtvar/mean/var (C).  ws: xsmi_bn_workspace_bytes(C). */
+ * biased variance.  Outputs xhat (N*C*HW, or NULL to skip it), sqrtvar/mean/var (C).  ws: xsmi_bn_workspace_bytes(C). */
 size_t xsmi_bn_workspace_bytes(int C);
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
                 float *mean, float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask,
@@ -226,9 +226,14 @@ int xsmi_bn_fold(const float *w, const float *bias, const float *gamma, const fl
 /* Backward (xs/nn/grad_fn.py:379-411): dgamma = sum(dy*xhat), dbeta = sum(dy),
  * dx = gamma / (m*sqrtvar) * (m*dy - dbeta - xhat*dgamma), m = N*HW.  All three are overwritten.
  * With neg_mask (the byte mask of a fused ReLU) dy counts as 0 where the mask is set (strict mask,
- * xs/nn/grad_fn.py:146-157). */
-int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, const uint8_t *neg_mask,
-                float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes);
+ * xs/nn/grad_fn.py:146-157).
+ * mean == NULL: xhat is the normalised input that xsmi_bn_fwd stored.  mean != NULL: xsmi_bn_fwd was
+ * called with xhat == NULL, the `xhat` argument is the forward's input x, and (x - mean) / sqrtvar is
+ * formed again on the fly (the same float operations, hence the same bits, without the forward's
+ * extra write of a tensor of x's size). */
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const float *sqrtvar, const float *gamma,
+                const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws,
+                size_t ws_bytes);
 
 /* Mean over non-overlapping k x k blocks of an NCHW tensor and its gradient
  * (the live mode of avg_pool2d, xs/nn/functional.py:539-583, xs/nn/grad_fn.py:284-309). */
@@ -237,8 +242,13 @@ int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int
 
 /* C[M,N] = op(A) . op(B) (+ bias[N] broadcast over rows); row-major, float32.  op is a transpose when
  * trans_a / trans_b is non-zero: A is stored (K,M) resp. B is stored (N,K).
- * (Dense layer: xs/nn/functional.py:99-120, xs/nn/grad_fn.py:86-99.) */
-int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b);
+ * (Dense layer: xs/nn/functional.py:99-120, xs/nn/grad_fn.py:86-99.)
+ * workspace may be NULL.  With one, a product with few output tiles and a long K is split along K over
+ * up to one workgroup per compute unit (at most workspace_bytes / (4*M*N) splits, 4*M*N bytes each) and
+ * the partial products are added in ascending K order by a second kernel: the result does not depend on
+ * timing, only on the number of splits. */
+int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b,
+              void *workspace, size_t workspace_bytes);
 /* out[j] = sum_i a[i][j] over an (M, N) matrix */
 int xsmi_colsum(const float *a, float *out, int M, int N);
 /* out[0] = sum of all n elements (float64 accumulation, one workgroup) */

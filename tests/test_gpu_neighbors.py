@@ -51,6 +51,15 @@ def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     np.testing.assert_array_equal(dx2.numpy(), dx3.numpy())
     np.testing.assert_array_equal(dg2.numpy(), dg3.numpy())
     np.testing.assert_array_equal(db2.numpy(), db3.numpy())
+    # without the stored normalised input: the backward forms it again from x and the batch mean, same bits
+    xd = gpu.to_device(x)
+    y4, xh4, sqv4, mean4, _ = K.bn_fwd(xd, gpu.to_device(gamma), gpu.to_device(beta), eps, neg_mask=mask, want_xhat=False)
+    assert xh4 is None
+    np.testing.assert_array_equal(y4.numpy(), yr.numpy())
+    dx4, dg4, db4 = K.bn_bwd(gpu.to_device(dy), xd, sqv4, gpu.to_device(gamma), neg_mask=mask, mean=mean4)
+    np.testing.assert_array_equal(dx4.numpy(), dx2.numpy())
+    np.testing.assert_array_equal(dg4.numpy(), dg2.numpy())
+    np.testing.assert_array_equal(db4.numpy(), db2.numpy())
     # inference form with the given statistics (xs/nn/functional.py:708-725)
     yi = K.bn_infer(gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta), gpu.to_device(mm0), gpu.to_device(mv0), eps)
     yi_ref = gamma.reshape(b) * (x64 - mm0.reshape(b)) / np.sqrt(mv0.reshape(b) + eps) + beta.reshape(b)
@@ -81,7 +90,7 @@ def test_dense_gemm_all_transposes(gpu):
     """addmm forward and the two gradient products (xs/nn/functional.py:99-120, xs/nn/grad_fn.py:86-99)."""
     K = gpu.kernels
     rng = np.random.default_rng(3)
-    for (m, k, n) in ((32, 512, 1000), (7, 130, 33), (256, 64, 10), (1, 1, 1)):
+    for (m, k, n) in ((32, 512, 1000), (7, 130, 33), (256, 64, 10), (1, 1, 1), (5, 1001, 3)):
         a = rng.standard_normal((m, k)).astype(np.float32); b = rng.standard_normal((k, n)).astype(np.float32)
         bias = rng.standard_normal(n).astype(np.float32); g = rng.standard_normal((m, n)).astype(np.float32)
         da, db_, dg = gpu.to_device(a), gpu.to_device(b), gpu.to_device(g)

@@ -307,19 +307,22 @@ def _nchw3(shape):
     return int(n), int(c), int(hw)
 
 
-def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None):
+def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None, want_xhat=True):
     """``moving=(moving_mean, moving_var)`` device arrays are updated in place: m = momentum*m + (1-momentum)*stat.
-    A uint8 ``neg_mask`` of x's size fuses a ReLU: it receives pre-activation < 0 and y is clipped at 0."""
+    A uint8 ``neg_mask`` of x's size fuses a ReLU: it receives pre-activation < 0 and y is clipped at 0.
+    ``want_xhat=False`` skips the store of the normalised input (None is returned for it): ``bn_bwd`` forms it
+    again from x and the batch mean."""
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
-    y = _like(x, y); xhat = empty(x.shape)
+    y = _like(x, y); xhat = empty(x.shape) if want_xhat else None
     y.take_fresh()
     sqrtvar = empty((c,)); mean = empty((c,)); var = empty((c,))
     mm, mv = moving if moving is not None else (None, None)
     if mm is not None and (mm.size != c or mv.size != c):
         raise ValueError("bn_fwd: moving statistics must have %d elements" % c)
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
-    lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr, sqrtvar.cptr, mean.cptr, var.cptr,
+    lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr if want_xhat else None, sqrtvar.cptr,
+             mean.cptr, var.cptr,
              mm.cptr if mm is not None else None, mv.cptr if mv is not None else None, float(momentum),
              neg_mask.cptr if neg_mask is not None else None, n, c, hw, float(eps), ws, ws_bytes)
     return y, xhat, sqrtvar, mean, var
@@ -349,9 +352,12 @@ def bn_fold(w, bias, gamma, beta, mean, var, eps):
     return w_out, b_out
 
 
-def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=None):
+def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=None, mean=None):
     """dx, dgamma, dbeta; buffers passed in are overwritten completely.  ``neg_mask`` is the byte mask of a fused
-    ReLU: the upstream gradient counts as 0 where it is set."""
+    ReLU: the upstream gradient counts as 0 where it is set.  With ``mean`` (the batch mean of the forward),
+    ``xhat`` is the forward's input x instead of its normalised form."""
+    if xhat.size != dy.size or (mean is not None and mean.size != dy.shape[1]):
+        raise ValueError("bn_bwd: operands do not match %s" % (dy.shape,))
     n, c, hw = _nchw3(dy.shape)
     dx = empty(dy.shape) if dx is None else dx
     dgamma = empty((c,)) if dgamma is None else dgamma
@@ -361,7 +367,7 @@ def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=
     for o in (dx, dgamma, dbeta):
         o.take_fresh()
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
-    lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, sqrtvar.cptr, gamma.cptr,
+    lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, mean.cptr if mean is not None else None, sqrtvar.cptr, gamma.cptr,
              neg_mask.cptr if neg_mask is not None else None, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw, ws, ws_bytes)
     return dx, dgamma, dbeta
 
@@ -391,8 +397,10 @@ def gemm(a, b, bias=None, trans_a=False, trans_b=False, out=None):
         out = empty((m, n))
     elif out.size != m * n:
         raise ValueError("gemm: output has shape %s, expected %s" % (out.shape, (m, n)))
+    # room for a split of K over the chip when the output is small (the dense layer's batch of rows)
+    ws, ws_bytes = _ws.get(min(64 * m * n * 4, 1 << 24))
     lib.call("xsmi_gemm", a.cptr, b.cptr, bias.cptr if bias is not None else None, out.cptr, int(m), int(n), int(k),
-             1 if trans_a else 0, 1 if trans_b else 0)
+             1 if trans_a else 0, 1 if trans_b else 0, ws, ws_bytes)
     return out
 
 

@@ -179,43 +179,54 @@ inline ChanIdx make_chan(int C, int HW) {
 // ---- batch norm --------------------------------------------------------------
 // pass 1: per (channel, split) partial sums of a and a*b over the N*HW elements of the channel
 // `zero` (optional, one byte per element): elements whose byte is set count as a == 0 (the gradient of a fused
-// ReLU that was clipped)
+// ReLU that was clipped).  A channel's elements are numbered image by image in load units (float4 when VEC:
+// HW % 4 == 0, so planes are 16-byte aligned; else floats); split sp owns units [sp*per, (sp+1)*per), a fixed
+// assignment, so the sums do not depend on timing.  Each thread issues four independent loads per operand
+// before it adds: a block has only a few units per thread, and one load at a time would leave it waiting on
+// memory latency for most of its life.
+template <bool VEC>
 __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict__ a, const float *__restrict__ b,
                                                           const uint8_t *__restrict__ zero, double *__restrict__ part,
-                                                          int N, int C, int HW, int nsplit) {
+                                                          int C, int HW, xsmi::FastDiv dU, uint32_t total, uint32_t per,
+                                                          const float *__restrict__ mean, const float *__restrict__ sqrtvar) {
+    constexpr int W = VEC ? 4 : 1, UNR = 4;
     __shared__ double sm[4];
     const int c = blockIdx.x, sp = blockIdx.y;
+    // with `mean`, b holds the values before normalisation and (b - mean) / sqrtvar is formed here
+    const float mu = mean ? mean[c] : 0.f, rs = mean ? sqrtvar[c] : 1.f;
+    const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
     double s0 = 0.0, s1 = 0.0;
-    // split sp takes images sp, sp + nsplit, ... (a fixed assignment: deterministic sums) and walks
-    // them as one flat range of float4 (planes are 16-byte aligned when HW % 4 == 0) or float units
-    const int nimg = sp < N ? (N - sp + nsplit - 1) / nsplit : 0;
-    if ((HW & 3) == 0) {
-        const uint32_t U = (uint32_t)HW >> 2, total = (uint32_t)nimg * U;
-        for (uint32_t e = threadIdx.x; e < total; e += 256) {
-            const uint32_t j = e / U, i = e - j * U;
-            const size_t base = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW;
-            float4 u = reinterpret_cast<const float4 *>(a + base)[i];
-            if (zero) {
-                const uchar4 z = reinterpret_cast<const uchar4 *>(zero + base)[i];
-                if (z.x) u.x = 0.f;
-                if (z.y) u.y = 0.f;
-                if (z.z) u.z = 0.f;
-                if (z.w) u.w = 0.f;
+    for (uint32_t e0 = beg + threadIdx.x; e0 < end; e0 += 256 * UNR) {
+        float u[UNR][W], v[UNR][W];
+        unsigned char z[UNR][W];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const uint32_t e = e0 + 256u * k;
+            const bool ok = e < end;
+            const uint32_t j = xsmi::fdiv(e, dU), i = e - j * dU.d;
+            const size_t off = ((size_t)j * C + c) * (size_t)HW + (size_t)i * W;
+            if (VEC) {
+                *reinterpret_cast<float4 *>(u[k]) = ok ? *reinterpret_cast<const float4 *>(a + off) : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (b) *reinterpret_cast<float4 *>(v[k]) = ok ? *reinterpret_cast<const float4 *>(b + off) : make_float4(0.f, 0.f, 0.f, 0.f);
+                if (zero) *reinterpret_cast<uchar4 *>(z[k]) = ok ? *reinterpret_cast<const uchar4 *>(zero + off) : make_uchar4(0, 0, 0, 0);
+            } else {
+                u[k][0] = ok ? a[off] : 0.f;
+                if (b) v[k][0] = ok ? b[off] : 0.f;
+                if (zero) z[k][0] = ok ? zero[off] : 0;
             }
-            const float4 v = b ? reinterpret_cast<const float4 *>(b + base)[i] : u;
-            s0 += ((double)u.x + (double)u.y) + ((double)u.z + (double)u.w);
-            s1 += ((double)u.x * (double)v.x + (double)u.y * (double)v.y) +
-                  ((double)u.z * (double)v.z + (double)u.w * (double)v.w);
         }
-    } else {
-        const uint32_t U = (uint32_t)HW, total = (uint32_t)nimg * U;
-        for (uint32_t e = threadIdx.x; e < total; e += 256) {
-            const uint32_t j = e / U, i = e - j * U;
-            const size_t off = ((size_t)(sp + (int)j * nsplit) * C + c) * (size_t)HW + i;
-            const float u = (zero && zero[off]) ? 0.f : a[off];
-            const float v = b ? b[off] : u;
-            s0 += (double)u;
-            s1 += (double)u * (double)v;
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            double t0 = 0.0, t1 = 0.0;
+#pragma unroll
+            for (int q = 0; q < W; ++q) {
+                const float uu = (zero && z[k][q]) ? 0.f : u[k][q];
+                const float vv = b ? (mean ? (v[k][q] - mu) / rs : v[k][q]) : uu;
+                t0 += (double)uu;
+                t1 += (double)uu * (double)vv;
+            }
+            s0 += t0;
+            s1 += t1;
         }
     }
     s0 = block_sum(s0, sm);
@@ -225,14 +236,29 @@ __global__ void __launch_bounds__(256) bn_partial_kernel(const float *__restrict
         part[((size_t)c * BN_SPLIT + sp) * 2 + 1] = s1;
     }
 }
-// number of partial reductions per channel: enough work per block (about 1024 load units) to hide latency
-static int bn_splits(int N, int HW) {
-    const long long units = (long long)N * ((HW & 3) == 0 ? HW >> 2 : HW);
-    long long s = units / 1024;
+// Split of a channel's N*HW elements over up to BN_SPLIT blocks: at least 512 load units per block.
+struct BnSplit { int nsplit; uint32_t total, per; xsmi::FastDiv dU; bool vec; };
+static BnSplit bn_split(int N, int HW, bool vec) {
+    BnSplit r;
+    r.vec = vec;
+    const uint32_t U = vec ? (uint32_t)HW >> 2 : (uint32_t)HW;
+    r.total = (uint32_t)N * U;
+    uint32_t s = r.total / 512;
     if (s < 1) s = 1;
-    if (s > BN_SPLIT) s = BN_SPLIT;
-    if (s > N) s = N;
-    return (int)s;
+    if (s > (uint32_t)BN_SPLIT) s = BN_SPLIT;
+    r.per = (r.total + s - 1) / s;
+    r.nsplit = (int)((r.total + r.per - 1) / r.per);
+    r.dU = xsmi::make_fastdiv(U);
+    return r;
+}
+static void launch_bn_partial(hipStream_t st, const float *a, const float *b, const uint8_t *zero, double *part, int C, int HW,
+                              const BnSplit &sp, const float *mean, const float *sqrtvar) {
+    if (sp.vec)
+        hipLaunchKernelGGL(bn_partial_kernel<true>, dim3(C, sp.nsplit), dim3(256), 0, st, a, b, zero, part, C, HW, sp.dU,
+                           sp.total, sp.per, mean, sqrtvar);
+    else
+        hipLaunchKernelGGL(bn_partial_kernel<false>, dim3(C, sp.nsplit), dim3(256), 0, st, a, b, zero, part, C, HW, sp.dU,
+                           sp.total, sp.per, mean, sqrtvar);
 }
 __global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar, float *mean, float *var, int C, double m,
                                 float eps, int nsplit, float *moving_mean, float *moving_var, float momentum) {
@@ -303,11 +329,13 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
                                                             const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
                                                             const float *__restrict__ dgamma, const float *__restrict__ dbeta,
                                                             const uint8_t *__restrict__ zero, float *__restrict__ dx,
-                                                            ChanIdx chan, uint32_t total, float m) {
+                                                            ChanIdx chan, uint32_t total, float m,
+                                                            const float *__restrict__ mean) {
     constexpr int W = VEC ? 4 : 1;
     for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
         const int c = chan(i);
-        const float g = gamma[c], db = dbeta[c], dg = dgamma[c], den = m * sqrtvar[c];
+        const float rs = sqrtvar[c], mu = mean ? mean[c] : 0.f;
+        const float g = gamma[c], db = dbeta[c], dg = dgamma[c], den = m * rs;
         float gv[W], hv[W], ov[W];
         unsigned char zv[W];
         if (VEC) {
@@ -321,6 +349,7 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
 #pragma unroll
         for (int e = 0; e < W; ++e) {
             const float d = (zero && zv[e]) ? 0.f : gv[e];
+            if (mean) hv[e] = (hv[e] - mu) / rs;     // xhat holds the values before normalisation
             // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
             ov[e] = g * (m * d - db - hv[e] * dg) / den;
         }
@@ -401,12 +430,16 @@ __global__ void __launch_bounds__(256) avgpool_bwd_kernel(const float *__restric
 constexpr int GEMM_KC = 128;
 __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                     const float *__restrict__ bias, float *__restrict__ C, int M, int N,
-                                                    int K, int ta, int tb) {
+                                                    int K, int ta, int tb, int chunks_per_split) {
     __shared__ float As[32][GEMM_KC + 1], Bs[GEMM_KC][33];
     const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
     float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
-    for (int k0 = 0; k0 < K; k0 += GEMM_KC) {
+    // split z multiplies K range [kbeg, kend) and writes its own M x N slab of C (C is then the partial buffer)
+    const int kbeg = blockIdx.z * chunks_per_split * GEMM_KC;
+    const int kend = min(K, kbeg + chunks_per_split * GEMM_KC);
+    C += (size_t)blockIdx.z * M * N;
+    for (int k0 = kbeg; k0 < kend; k0 += GEMM_KC) {
         // all loads of the chunk first (independent, so their latencies overlap), then the LDS stores
         float ra[GEMM_KC / 8], rb[GEMM_KC / 8];
 #pragma unroll
@@ -414,17 +447,17 @@ __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, 
             const int i = threadIdx.x + 256 * u;
             if (ta) {                                   // A stored (K, M): lanes along m
                 const int kk = i >> 5, r = i & 31;
-                ra[u] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(k0 + kk) * M + m0 + r] : 0.f;
+                ra[u] = (m0 + r < M && k0 + kk < kend) ? A[(size_t)(k0 + kk) * M + m0 + r] : 0.f;
             } else {                                    // A stored (M, K): lanes along k
                 const int r = i / GEMM_KC, kk = i % GEMM_KC;
-                ra[u] = (m0 + r < M && k0 + kk < K) ? A[(size_t)(m0 + r) * K + k0 + kk] : 0.f;
+                ra[u] = (m0 + r < M && k0 + kk < kend) ? A[(size_t)(m0 + r) * K + k0 + kk] : 0.f;
             }
             if (tb) {                                   // B stored (N, K): lanes along k
                 const int c = i / GEMM_KC, kk = i % GEMM_KC;
-                rb[u] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(n0 + c) * K + k0 + kk] : 0.f;
+                rb[u] = (n0 + c < N && k0 + kk < kend) ? B[(size_t)(n0 + c) * K + k0 + kk] : 0.f;
             } else {                                    // B stored (K, N): lanes along n
                 const int kk = i >> 5, c = i & 31;
-                rb[u] = (n0 + c < N && k0 + kk < K) ? B[(size_t)(k0 + kk) * N + n0 + c] : 0.f;
+                rb[u] = (n0 + c < N && k0 + kk < kend) ? B[(size_t)(k0 + kk) * N + n0 + c] : 0.f;
             }
         }
 #pragma unroll
@@ -447,6 +480,15 @@ __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, 
             int m = m0 + ty * 2 + i, n = n0 + tx * 2 + j;
             if (m < M && n < N) C[(size_t)m * N + n] = acc[i][j] + (bias ? bias[n] : 0.f);
         }
+}
+// C = bias + the K-split partial products, added in ascending split order
+__global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *__restrict__ part, const float *__restrict__ bias,
+                                                           float *__restrict__ C, uint32_t MN, int N, int splits) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= MN) return;
+    float s = part[i];
+    for (int z = 1; z < splits; ++z) s += part[(size_t)z * MN + i];
+    C[i] = s + (bias ? bias[i % (uint32_t)N] : 0.f);
 }
 
 __global__ void __launch_bounds__(256) colsum_kernel(const float *__restrict__ a, float *__restrict__ out, int M, int N) {
@@ -585,9 +627,9 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
-    const int nsplit = bn_splits(N, HW);
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, x, (const float *)nullptr,
-                       (const uint8_t *)nullptr, part, N, C, HW, nsplit);
+    const BnSplit split = bn_split(N, HW, (HW & 3) == 0 && aligned16(x));
+    const int nsplit = split.nsplit;
+    launch_bn_partial(st, x, nullptr, nullptr, part, C, HW, split, nullptr, nullptr);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
                        (double)N * HW, eps, nsplit, moving_mean, moving_var, momentum);
@@ -633,8 +675,9 @@ int xsmi_bn_fold(const float *w, const float *bias, const float *gamma, const fl
     return XSMI_OK;
 }
 
-int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const float *gamma, const uint8_t *neg_mask,
-                float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws, size_t ws_bytes) {
+int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const float *sqrtvar, const float *gamma,
+                const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws,
+                size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_bwd: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_bwd: tensors of 2^29 elements or more are not supported");
@@ -642,8 +685,10 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const 
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd: workspace too small");
     hipStream_t st = xsmi::stream();
     double *part = (double *)ws;
-    const int nsplit = bn_splits(N, HW);
-    hipLaunchKernelGGL(bn_partial_kernel, dim3(C, nsplit), dim3(256), 0, st, dy, xhat, neg_mask, part, N, C, HW, nsplit);
+    const BnSplit split = bn_split(N, HW, (HW & 3) == 0 && aligned16(dy) && aligned16(xhat) &&
+                                              (!neg_mask || ((uintptr_t)neg_mask & 3) == 0));
+    const int nsplit = split.nsplit;
+    launch_bn_partial(st, dy, xhat, neg_mask, part, C, HW, split, mean, sqrtvar);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C, nsplit);
     XSMI_LAUNCH_CHECK("bn_bwd_stats_kernel");
@@ -652,10 +697,10 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *sqrtvar, const 
                      (!neg_mask || ((uintptr_t)neg_mask & 3) == 0);
     if (vec)
         hipLaunchKernelGGL(bn_bwd_apply_kernel<true>, grid_for(total / 4), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
-                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
+                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW), mean);
     else
         hipLaunchKernelGGL(bn_bwd_apply_kernel<false>, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
-                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW));
+                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW), mean);
     XSMI_LAUNCH_CHECK("bn_bwd_apply_kernel");
     return XSMI_OK;
 }
@@ -682,13 +727,38 @@ int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int
     return XSMI_OK;
 }
 
-int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b) {
+int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M, int N, int K, int trans_a, int trans_b,
+              void *ws, size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(M > 0 && N > 0 && K > 0, "xsmi_gemm: empty matrix");
     XSMI_CHECK_ARG(A && B && C, "xsmi_gemm: null pointer");
-    hipLaunchKernelGGL(gemm_kernel, dim3((N + 31) / 32, (M + 31) / 32), dim3(256), 0, xsmi::stream(), A, B, bias, C, M, N,
-                       K, trans_a, trans_b);
+    XSMI_CHECK_ARG((double)M * N < 2147483648.0, "xsmi_gemm: outputs of 2^31 elements or more are not supported");
+    // A skinny product (a batch of 32 rows) has few 32 x 32 output tiles and a long K: with a workspace, K is
+    // split over enough workgroups to occupy the chip and the partial products are added in a second pass.
+    const int tiles = ((N + 31) / 32) * ((M + 31) / 32), chunks = (K + GEMM_KC - 1) / GEMM_KC;
+    int splits = 1;
+    if (ws && chunks > 1 && tiles < xsmi::cu_count()) {
+        splits = (xsmi::cu_count() + tiles - 1) / tiles;
+        if (splits > chunks) splits = chunks;
+        const size_t fit = ws_bytes / ((size_t)M * N * sizeof(float));
+        if ((size_t)splits > fit) splits = (int)fit;
+        if (splits < 1) splits = 1;
+    }
+    const int cps = (chunks + splits - 1) / splits;
+    splits = (chunks + cps - 1) / cps;
+    hipStream_t st = xsmi::stream();
+    if (splits == 1) {
+        hipLaunchKernelGGL(gemm_kernel, dim3((N + 31) / 32, (M + 31) / 32, 1), dim3(256), 0, st, A, B, bias, C, M, N, K,
+                           trans_a, trans_b, chunks);
+        XSMI_LAUNCH_CHECK("gemm_kernel");
+        return XSMI_OK;
+    }
+    hipLaunchKernelGGL(gemm_kernel, dim3((N + 31) / 32, (M + 31) / 32, splits), dim3(256), 0, st, A, B,
+                       (const float *)nullptr, (float *)ws, M, N, K, trans_a, trans_b, cps);
     XSMI_LAUNCH_CHECK("gemm_kernel");
+    const uint32_t MN = (uint32_t)((size_t)M * N);
+    hipLaunchKernelGGL(gemm_reduce_kernel, dim3((MN + 255) / 256), dim3(256), 0, st, (const float *)ws, bias, C, MN, N, splits);
+    XSMI_LAUNCH_CHECK("gemm_reduce_kernel");
     return XSMI_OK;
 }
 

@@ -411,7 +411,7 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
         neg_mask = dev.empty(x.shape, np.uint8) if relu else None
         y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst,
                                                            (mm.reshape(-1), mv.reshape(-1)) if fused else None, momentum,
-                                                           neg_mask)
+                                                           neg_mask, want_xhat=False)
         if not track:
             neg_mask = None
         if not fused:
@@ -435,6 +435,8 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
     if GLOBAL.COMPUTE_GRAD and out.requires_grad and training:
         out.cache['sqrtvar'] = sqrtvar
         out.cache['normalized_x'] = xhat
+        # on the device the normalised input is not stored: the backward forms it again from x and the mean
+        out.cache['batch_mean'] = mean_ if xhat is None else None
         if neg_mask is not None:
             out.cache['neg_mask'] = neg_mask
         else:

@@ -242,10 +242,14 @@ def BatchNormBackward(outputs):
     if is_device(dy):
         out_dx, out_dg, out_db = _fresh_grad(inputs), _fresh_grad(gamma), _fresh_grad(beta)
         gam = A.same_place(dy, gamma.eval)
-        dx, dgamma, dbeta = K.bn_bwd(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gam,
+        xhat, mean = outputs.cache['normalized_x'], outputs.cache.get('batch_mean')
+        if xhat is None:                             # not stored by the forward: x and the batch mean stand in
+            xhat = inputs.eval
+        dx, dgamma, dbeta = K.bn_bwd(dy, xhat, outputs.cache['sqrtvar'], gam,
                                      dx=out_dx, dgamma=None if out_dg is None else out_dg.reshape(-1),
                                      dbeta=None if out_db is None else out_db.reshape(-1),
-                                     neg_mask=outputs.cache.get('neg_mask'))       # fused ReLU: strict mask on dy
+                                     neg_mask=outputs.cache.get('neg_mask'),       # fused ReLU: strict mask on dy
+                                     mean=mean if outputs.cache['normalized_x'] is None else None)
     else:
         out_dx = out_dg = out_db = None
         dx, dgamma, dbeta = A.batch_norm_backward(dy, outputs.cache['normalized_x'], outputs.cache['sqrtvar'], gamma.eval)
