@@ -260,100 +260,149 @@ static void launch_bn_partial(hipStream_t st, const float *a, const float *b, co
         hipLaunchKernelGGL(bn_partial_kernel<false>, dim3(C, sp.nsplit), dim3(256), 0, st, a, b, zero, part, C, HW, sp.dU,
                            sp.total, sp.per, mean, sqrtvar);
 }
-__global__ void bn_stats_kernel(const double *__restrict__ part, float *sqrtvar, float *mean, float *var, int C, double m,
-                                float eps, int nsplit, float *moving_mean, float *moving_var, float momentum) {
-    int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
-    double s0 = 0.0, s1 = 0.0;
-    for (int sp = 0; sp < nsplit; ++sp) {
-        s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
-        s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
+// Sums of one channel's partials: the same fixed tree in every block of the channel, so all of them (and the one
+// that stores the statistics) work with identical values.  sm: two doubles of LDS.
+__device__ __forceinline__ void bn_channel_sums(const double *__restrict__ part, int c, int nsplit, double *sm, double &s0,
+                                                double &s1) {
+    if (threadIdx.x < 64) {
+        double a = 0.0, b = 0.0;
+        if ((int)threadIdx.x < nsplit) {
+            a = part[((size_t)c * BN_SPLIT + threadIdx.x) * 2 + 0];
+            b = part[((size_t)c * BN_SPLIT + threadIdx.x) * 2 + 1];
+        }
+        a = wave_sum(a);
+        b = wave_sum(b);
+        if (threadIdx.x == 0) { sm[0] = a; sm[1] = b; }
     }
-    double mu = s0 / m;
-    double v = s1 / m - mu * mu;
-    if (v < 0.0) v = 0.0;
-    mean[c] = (float)mu;
-    var[c] = (float)v;
-    sqrtvar[c] = (float)sqrt(v + (double)eps);
-    if (moving_mean) {                               // m = momentum*m + (1-momentum)*cur, as xsmi_lerp computes it
-        moving_mean[c] = momentum * moving_mean[c] + (1.f - momentum) * (float)mu;
-        moving_var[c] = momentum * moving_var[c] + (1.f - momentum) * (float)v;
-    }
+    __syncthreads();
+    s0 = sm[0];
+    s1 = sm[1];
 }
-// VEC: four consecutive elements per thread (HW % 4 == 0, so they share a channel and planes are 16-byte
-// aligned).  neg_mask != nullptr fuses a ReLU: mask = pre-activation < 0, y = max(pre-activation, 0).
+// pass 2 of the forward: block (c, sp) turns the channel's partial sums into mean and sqrt(var + eps) (block sp == 0
+// also stores them and updates the moving statistics: m = momentum*m + (1-momentum)*cur, as xsmi_lerp computes it)
+// and normalises its units of the channel, numbered as in bn_partial_kernel.  neg_mask != nullptr fuses a ReLU:
+// mask = pre-activation < 0, y = max(pre-activation, 0).
+struct BnFwdOut {
+    float *y, *xhat, *sqrtvar, *mean, *var, *moving_mean, *moving_var;
+    uint8_t *neg_mask;
+};
 template <bool VEC>
 __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
-                                                        const float *__restrict__ beta, const float *__restrict__ mean,
-                                                        const float *__restrict__ sqrtvar, float *__restrict__ y,
-                                                        float *__restrict__ xhat, uint8_t *__restrict__ neg_mask,
-                                                        ChanIdx chan, uint32_t total) {
-    constexpr int W = VEC ? 4 : 1;
-    for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
-        const int c = chan(i);
-        const float mu = mean[c], rs = sqrtvar[c], g = gamma[c], bt = beta[c];
-        float xv[W], hv[W], yv[W];
-        unsigned char mv[W];
-        if (VEC) *reinterpret_cast<float4 *>(xv) = *reinterpret_cast<const float4 *>(x + i); else xv[0] = x[i];
+                                                        const float *__restrict__ beta, const double *__restrict__ part,
+                                                        int nsplit_part, double m, float eps, float momentum, BnFwdOut o,
+                                                        int C, int HW, xsmi::FastDiv dU, uint32_t total, uint32_t per) {
+    constexpr int W = VEC ? 4 : 1, UNR = 4;
+    __shared__ double sm[2];
+    const int c = blockIdx.x, sp = blockIdx.y;
+    double s0, s1;
+    bn_channel_sums(part, c, nsplit_part, sm, s0, s1);
+    const double mu_d = s0 / m;
+    double v = s1 / m - mu_d * mu_d;
+    if (v < 0.0) v = 0.0;
+    const float mu = (float)mu_d, rs = (float)sqrt(v + (double)eps), g = gamma[c], bt = beta[c];
+    if (sp == 0 && threadIdx.x == 0) {
+        o.mean[c] = mu;
+        o.var[c] = (float)v;
+        o.sqrtvar[c] = rs;
+        if (o.moving_mean) {
+            o.moving_mean[c] = momentum * o.moving_mean[c] + (1.f - momentum) * mu;
+            o.moving_var[c] = momentum * o.moving_var[c] + (1.f - momentum) * (float)v;
+        }
+    }
+    const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
+    for (uint32_t e0 = beg + threadIdx.x; e0 < end; e0 += 256 * UNR) {
+        float xv[UNR][W];
+        size_t off[UNR];
 #pragma unroll
-        for (int e = 0; e < W; ++e) {
-            hv[e] = (xv[e] - mu) / rs;
-            const float pre = g * hv[e] + bt;
-            mv[e] = pre < 0.f ? 1 : 0;
-            yv[e] = (neg_mask && pre < 0.f) ? 0.f : pre;
+        for (int k = 0; k < UNR; ++k) {
+            const uint32_t e = e0 + 256u * k;
+            const uint32_t j = xsmi::fdiv(e, dU), i = e - j * dU.d;
+            off[k] = ((size_t)j * C + c) * (size_t)HW + (size_t)i * W;
+            if (e < end) {
+                if (VEC) *reinterpret_cast<float4 *>(xv[k]) = *reinterpret_cast<const float4 *>(x + off[k]); else xv[k][0] = x[off[k]];
+            }
         }
-        if (VEC) {
-            if (xhat) *reinterpret_cast<float4 *>(xhat + i) = *reinterpret_cast<float4 *>(hv);
-            *reinterpret_cast<float4 *>(y + i) = *reinterpret_cast<float4 *>(yv);
-            if (neg_mask) *reinterpret_cast<uchar4 *>(neg_mask + i) = make_uchar4(mv[0], mv[1], mv[2], mv[3]);
-        } else {
-            if (xhat) xhat[i] = hv[0];
-            y[i] = yv[0];
-            if (neg_mask) neg_mask[i] = mv[0];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            if (e0 + 256u * k >= end) break;
+            float hv[W], yv[W];
+            unsigned char mv[W];
+#pragma unroll
+            for (int q = 0; q < W; ++q) {
+                hv[q] = (xv[k][q] - mu) / rs;
+                const float pre = g * hv[q] + bt;
+                mv[q] = pre < 0.f ? 1 : 0;
+                yv[q] = (o.neg_mask && pre < 0.f) ? 0.f : pre;
+            }
+            if (VEC) {
+                if (o.xhat) *reinterpret_cast<float4 *>(o.xhat + off[k]) = *reinterpret_cast<float4 *>(hv);
+                *reinterpret_cast<float4 *>(o.y + off[k]) = *reinterpret_cast<float4 *>(yv);
+                if (o.neg_mask) *reinterpret_cast<uchar4 *>(o.neg_mask + off[k]) = make_uchar4(mv[0], mv[1], mv[2], mv[3]);
+            } else {
+                if (o.xhat) o.xhat[off[k]] = hv[0];
+                o.y[off[k]] = yv[0];
+                if (o.neg_mask) o.neg_mask[off[k]] = mv[0];
+            }
         }
     }
 }
-__global__ void bn_bwd_stats_kernel(const double *__restrict__ part, float *dgamma, float *dbeta, int C, int nsplit) {
-    int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= C) return;
-    double s0 = 0.0, s1 = 0.0;
-    for (int sp = 0; sp < nsplit; ++sp) {
-        s0 += part[((size_t)c * BN_SPLIT + sp) * 2 + 0];
-        s1 += part[((size_t)c * BN_SPLIT + sp) * 2 + 1];
-    }
-    dbeta[c] = (float)s0;
-    dgamma[c] = (float)s1;
-}
+// pass 2 of the backward: block (c, sp) turns the partial sums into dbeta = sum(dy) and dgamma = sum(dy*xhat) (block
+// sp == 0 stores them) and writes dx for its units of the channel.  With `mean`, xhat holds the values before
+// normalisation and (xhat - mean) / sqrtvar is formed here.
 template <bool VEC>
 __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
                                                             const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
-                                                            const float *__restrict__ dgamma, const float *__restrict__ dbeta,
-                                                            const uint8_t *__restrict__ zero, float *__restrict__ dx,
-                                                            ChanIdx chan, uint32_t total, float m,
-                                                            const float *__restrict__ mean) {
-    constexpr int W = VEC ? 4 : 1;
-    for (uint32_t i = (blockIdx.x * 256u + threadIdx.x) * W; i < total; i += gridDim.x * 256u * W) {
-        const int c = chan(i);
-        const float rs = sqrtvar[c], mu = mean ? mean[c] : 0.f;
-        const float g = gamma[c], db = dbeta[c], dg = dgamma[c], den = m * rs;
-        float gv[W], hv[W], ov[W];
-        unsigned char zv[W];
-        if (VEC) {
-            *reinterpret_cast<float4 *>(gv) = *reinterpret_cast<const float4 *>(dy + i);
-            *reinterpret_cast<float4 *>(hv) = *reinterpret_cast<const float4 *>(xhat + i);
-            if (zero) *reinterpret_cast<uchar4 *>(zv) = *reinterpret_cast<const uchar4 *>(zero + i);
-        } else {
-            gv[0] = dy[i]; hv[0] = xhat[i];
-            if (zero) zv[0] = zero[i];
+                                                            const double *__restrict__ part, int nsplit_part,
+                                                            float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                            const uint8_t *__restrict__ zero, float *__restrict__ dx, float m,
+                                                            const float *__restrict__ mean, int C, int HW, xsmi::FastDiv dU,
+                                                            uint32_t total, uint32_t per) {
+    constexpr int W = VEC ? 4 : 1, UNR = 4;
+    __shared__ double sm[2];
+    const int c = blockIdx.x, sp = blockIdx.y;
+    double s0, s1;
+    bn_channel_sums(part, c, nsplit_part, sm, s0, s1);
+    const float db = (float)s0, dg = (float)s1;
+    if (sp == 0 && threadIdx.x == 0) {
+        dbeta[c] = db;
+        dgamma[c] = dg;
+    }
+    const float rs = sqrtvar[c], mu = mean ? mean[c] : 0.f, g = gamma[c], den = m * rs;
+    const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
+    for (uint32_t e0 = beg + threadIdx.x; e0 < end; e0 += 256 * UNR) {
+        float gv[UNR][W], hv[UNR][W];
+        unsigned char zv[UNR][W];
+        size_t off[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const uint32_t e = e0 + 256u * k;
+            const uint32_t j = xsmi::fdiv(e, dU), i = e - j * dU.d;
+            off[k] = ((size_t)j * C + c) * (size_t)HW + (size_t)i * W;
+            if (e < end) {
+                if (VEC) {
+                    *reinterpret_cast<float4 *>(gv[k]) = *reinterpret_cast<const float4 *>(dy + off[k]);
+                    *reinterpret_cast<float4 *>(hv[k]) = *reinterpret_cast<const float4 *>(xhat + off[k]);
+                    if (zero) *reinterpret_cast<uchar4 *>(zv[k]) = *reinterpret_cast<const uchar4 *>(zero + off[k]);
+                } else {
+                    gv[k][0] = dy[off[k]];
+                    hv[k][0] = xhat[off[k]];
+                    if (zero) zv[k][0] = zero[off[k]];
+                }
+            }
         }
 #pragma unroll
-        for (int e = 0; e < W; ++e) {
-            const float d = (zero && zv[e]) ? 0.f : gv[e];
-            if (mean) hv[e] = (hv[e] - mu) / rs;     // xhat holds the values before normalisation
-            // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
-            ov[e] = g * (m * d - db - hv[e] * dg) / den;
+        for (int k = 0; k < UNR; ++k) {
+            if (e0 + 256u * k >= end) break;
+            float ov[W];
+#pragma unroll
+            for (int q = 0; q < W; ++q) {
+                const float d = (zero && zv[k][q]) ? 0.f : gv[k][q];
+                const float h = mean ? (hv[k][q] - mu) / rs : hv[k][q];
+                // gamma*(m*dy - sum(dy) - xhat*sum(dy*xhat)) / (m*sqrtvar); the sums carry one factor gamma in the reference
+                ov[q] = g * (m * d - db - h * dg) / den;
+            }
+            if (VEC) *reinterpret_cast<float4 *>(dx + off[k]) = *reinterpret_cast<float4 *>(ov); else dx[off[k]] = ov[0];
         }
-        if (VEC) *reinterpret_cast<float4 *>(dx + i) = *reinterpret_cast<float4 *>(ov); else dx[i] = ov[0];
     }
 }
 
@@ -631,18 +680,15 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     const int nsplit = split.nsplit;
     launch_bn_partial(st, x, nullptr, nullptr, part, C, HW, split, nullptr, nullptr);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
-    hipLaunchKernelGGL(bn_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, sqrtvar, mean, var, C,
-                       (double)N * HW, eps, nsplit, moving_mean, moving_var, momentum);
-    XSMI_LAUNCH_CHECK("bn_stats_kernel");
-    size_t total = (size_t)N * C * HW;
-    const bool vec = (HW & 3) == 0 && aligned16(x) && aligned16(y) && (!xhat || aligned16(xhat)) &&
-                     (!neg_mask || ((uintptr_t)neg_mask & 3) == 0);
-    if (vec)
-        hipLaunchKernelGGL(bn_apply_kernel<true>, grid_for(total / 4), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y,
-                           xhat, neg_mask, make_chan(C, HW), (uint32_t)total);
+    const BnSplit ap = bn_split(N, HW, (HW & 3) == 0 && aligned16(x) && aligned16(y) && (!xhat || aligned16(xhat)) &&
+                                           (!neg_mask || ((uintptr_t)neg_mask & 3) == 0));
+    const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask};
+    if (ap.vec)
+        hipLaunchKernelGGL(bn_apply_kernel<true>, dim3(C, ap.nsplit), dim3(256), 0, st, x, gamma, beta, part, nsplit,
+                           (double)N * HW, eps, momentum, o, C, HW, ap.dU, ap.total, ap.per);
     else
-        hipLaunchKernelGGL(bn_apply_kernel<false>, grid_for(total), dim3(256), 0, st, x, gamma, beta, mean, sqrtvar, y,
-                           xhat, neg_mask, make_chan(C, HW), (uint32_t)total);
+        hipLaunchKernelGGL(bn_apply_kernel<false>, dim3(C, ap.nsplit), dim3(256), 0, st, x, gamma, beta, part, nsplit,
+                           (double)N * HW, eps, momentum, o, C, HW, ap.dU, ap.total, ap.per);
     XSMI_LAUNCH_CHECK("bn_apply_kernel");
     return XSMI_OK;
 }
@@ -690,17 +736,14 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
     const int nsplit = split.nsplit;
     launch_bn_partial(st, dy, xhat, neg_mask, part, C, HW, split, mean, sqrtvar);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
-    hipLaunchKernelGGL(bn_bwd_stats_kernel, dim3((C + 255) / 256), dim3(256), 0, st, part, dgamma, dbeta, C, nsplit);
-    XSMI_LAUNCH_CHECK("bn_bwd_stats_kernel");
-    size_t total = (size_t)N * C * HW;
-    const bool vec = (HW & 3) == 0 && aligned16(dy) && aligned16(xhat) && aligned16(dx) &&
-                     (!neg_mask || ((uintptr_t)neg_mask & 3) == 0);
-    if (vec)
-        hipLaunchKernelGGL(bn_bwd_apply_kernel<true>, grid_for(total / 4), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
-                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW), mean);
+    const BnSplit ap = bn_split(N, HW, split.vec && aligned16(dx));
+    const float m = (float)((double)N * HW);
+    if (ap.vec)
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<true>, dim3(C, ap.nsplit), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, part,
+                           nsplit, dgamma, dbeta, neg_mask, dx, m, mean, C, HW, ap.dU, ap.total, ap.per);
     else
-        hipLaunchKernelGGL(bn_bwd_apply_kernel<false>, grid_for(total), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma,
-                           dbeta, neg_mask, dx, make_chan(C, HW), (uint32_t)total, (float)((double)N * HW), mean);
+        hipLaunchKernelGGL(bn_bwd_apply_kernel<false>, dim3(C, ap.nsplit), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, part,
+                           nsplit, dgamma, dbeta, neg_mask, dx, m, mean, C, HW, ap.dU, ap.total, ap.per);
     XSMI_LAUNCH_CHECK("bn_bwd_apply_kernel");
     return XSMI_OK;
 }
