@@ -192,6 +192,8 @@ int xsmi_add(const float *a, const float *b, float *out, size_t n);
  * (xs/nn/functional.py:6-21 then xs/layers/activators.py:37-50) in one pass; neg_mask (or NULL)
  * receives 1 where the sum is < 0, the sign the ReLU's backward needs */
 int xsmi_add_relu(const float *a, const float *b, float *out, uint8_t *neg_mask, size_t n);
+/* out[i] = value */
+int xsmi_fill(float *out, float value, size_t n);
 /* out[i] = s * a[i] + t */
 int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n);
 /* y = max(0, x) (may be in place)        (xs/nn/td_functional.py:59-60) */
@@ -258,8 +260,11 @@ int xsmi_sum_all(const float *a, float *out, size_t n);
  * (xs/nn/functional.py:984-1010): sm = softmax(logits), loss[0] = mean or sum of -log sm[i, label[i]].
  * `loss` must hold 1 + M floats (loss[1..M] receives the per-row terms). */
 int xsmi_softmax_ce_fwd(const float *logits, const int64_t *labels, float *sm, float *loss, int M, int N, int mean);
-/* dlogits = (sm - onehot(labels)) * scale      (xs/nn/grad_fn.py:604-620) */
-int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, float *dlogits, int M, int N, float scale);
+/* dlogits = (sm - onehot(labels)) * scale * (upstream ? upstream[0] : 1)      (xs/nn/grad_fn.py:604-620)
+ * upstream: the loss's own gradient as one float in device memory (or NULL), so that the caller need not
+ * read it back to the host. */
+int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, const float *upstream, float *dlogits, int M, int N,
+                        float scale);
 
 #ifdef __cplusplus
 }

@@ -85,7 +85,8 @@ SIGNATURES = {
     "xsmi_colsum": (_i, [_vp, _vp, _i, _i]),
     "xsmi_sum_all": (_i, [_vp, _vp, _sz]),
     "xsmi_softmax_ce_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
-    "xsmi_softmax_ce_bwd": (_i, [_vp, _vp, _vp, _i, _i, _f]),
+    "xsmi_softmax_ce_bwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
+    "xsmi_fill": (_i, [_vp, _f, _sz]),
 }
 
 CONV_RELU = 0x1

@@ -439,10 +439,22 @@ def softmax_ce_fwd(logits, labels, reduction):
 
 
 def softmax_ce_bwd(sm, labels, reduction, upstream):
+    """``upstream``: the loss's gradient, a host scalar or a one-element device array (read on the device, so
+    the host does not wait for the forward to finish)."""
     m, n = sm.reshape(-1, sm.shape[-1]).shape
     labels = _labels(labels)
-    up = float(np.asarray(upstream).reshape(-1)[0])
+    up_dev = upstream if isinstance(upstream, DeviceArray) else None
+    if up_dev is not None and (up_dev.dtype != np.float32 or up_dev.size != 1):
+        raise ValueError("softmax_ce_bwd: upstream must be one float32")
+    up = 1.0 if up_dev is not None else float(np.asarray(upstream).reshape(-1)[0])
     scale_ = up / m if reduction == 'mean' else up
     dz = empty(sm.shape)
-    lib.call("xsmi_softmax_ce_bwd", sm.cptr, labels.cptr, dz.cptr, int(m), int(n), scale_)
+    lib.call("xsmi_softmax_ce_bwd", sm.cptr, labels.cptr, up_dev.cptr if up_dev is not None else None, dz.cptr,
+             int(m), int(n), scale_)
     return dz
+
+
+def full(shape, value):
+    out = empty(shape)
+    lib.call("xsmi_fill", out.cptr, float(value), out.size)
+    return out

@@ -340,8 +340,12 @@ class Tensor(object):
                 self._grad = Tensor(g)
         elif self._data.size == 1:
             if self._grad is None:
-                one = np.array(1., dtype=self._data.dtype).reshape(self._data.shape)
-                self._grad = Tensor(to_device(one) if is_device(self._data) else one)
+                if is_device(self._data) and self._data.dtype == np.float32:
+                    from ..backend import kernels as K
+                    self._grad = Tensor(K.full(self._data.shape, 1.0))      # written on the device: no host wait
+                else:
+                    one = np.array(1., dtype=self._data.dtype).reshape(self._data.shape)
+                    self._grad = Tensor(to_device(one) if is_device(self._data) else one)
         else:
             raise ValueError('grad can be implicitly created only for scalar outputs')
         GLOBAL.OUTPUTS = self

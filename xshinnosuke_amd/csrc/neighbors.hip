@@ -42,6 +42,11 @@ struct AxpyF {
         reinterpret_cast<float4 *>(y)[j] = o;
     }
 };
+struct FillF {
+    float *o; float v;
+    __device__ void one(size_t i) const { o[i] = v; }
+    __device__ void quad(size_t j) const { reinterpret_cast<float4 *>(o)[j] = make_float4(v, v, v, v); }
+};
 struct AddF {
     const float *a, *b; float *o;
     __device__ void one(size_t i) const { o[i] = a[i] + b[i]; }
@@ -583,7 +588,9 @@ __global__ void __launch_bounds__(256) nll_reduce_kernel(const float *__restrict
     if (threadIdx.x == 0) loss[0] = (float)(mean ? s / (double)M : s);
 }
 __global__ void __launch_bounds__(256) softmax_ce_bwd_kernel(const float *__restrict__ sm, const int64_t *__restrict__ lab,
-                                                              float *__restrict__ dz, int N, size_t total, float scale) {
+                                                              float *__restrict__ dz, int N, size_t total, float scale,
+                                                              const float *__restrict__ upstream) {
+    if (upstream) scale *= upstream[0];
     for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += (size_t)gridDim.x * 256) {
         size_t row = i / N;
         int j = (int)(i - row * N);
@@ -635,6 +642,11 @@ int xsmi_add_relu(const float *a, const float *b, float *out, uint8_t *neg_mask,
     XSMI_CHECK_ARG(n == 0 || (a && b && out), "xsmi_add_relu: null pointer");
     return launch_ew("add_relu", n, aligned16(a) && aligned16(b) && aligned16(out) && (((uintptr_t)neg_mask & 3) == 0),
                      AddReluF{a, b, out, neg_mask});
+}
+int xsmi_fill(float *out, float value, size_t n) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || out, "xsmi_fill: null pointer");
+    return launch_ew("fill", n, aligned16(out), FillF{out, value});
 }
 int xsmi_scale_shift(const float *a, float *out, float s, float t, size_t n) {
     XSMI_REQUIRE_INIT();
@@ -833,12 +845,13 @@ int xsmi_softmax_ce_fwd(const float *logits, const int64_t *labels, float *sm, f
     return XSMI_OK;
 }
 
-int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, float *dlogits, int M, int N, float scale) {
+int xsmi_softmax_ce_bwd(const float *sm, const int64_t *labels, const float *upstream, float *dlogits, int M, int N,
+                        float scale) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(M > 0 && N > 0 && sm && labels && dlogits, "xsmi_softmax_ce_bwd: bad argument");
     size_t total = (size_t)M * N;
     hipLaunchKernelGGL(softmax_ce_bwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), sm, labels, dlogits, N, total,
-                       scale);
+                       scale, upstream);
     XSMI_LAUNCH_CHECK("softmax_ce_bwd_kernel");
     return XSMI_OK;
 }

@@ -266,8 +266,10 @@ def CrossEntropyLossBackward(outputs):
     logits, labels = outputs.in_bounds
     if not logits.requires_grad:
         return
-    g = A.softmax_cross_entropy_grad(logits.cache['softmax'].eval, labels.eval, outputs.cache['reduction'],
-                                     outputs.grad.eval if not is_device(outputs.grad.eval) else outputs.grad.eval.numpy())
+    up = outputs.grad.eval
+    if is_device(up) and not is_device(logits.cache['softmax'].eval):
+        up = up.numpy()
+    g = A.softmax_cross_entropy_grad(logits.cache['softmax'].eval, labels.eval, outputs.cache['reduction'], up)
     if logits.grad is None:
         logits.grad = Tensor(g)
     else:
