@@ -173,6 +173,11 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx,
  * dx = beta*dx + (neg_mask ? 0 : dy) over n elements.  Replaces ReLUBackward
  * (xs/nn/grad_fn.py:146-157) for the fused conv epilogue. dx may alias dy. */
 int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size_t n, float beta);
+/* The same masked gradient into two tensors in one pass: dx1 = beta1*dx1 + g, dx2 = beta2*dx2 + g with
+ * g = neg_mask ? 0 : dy.  For a ReLU applied in place to a sum (a residual block's end,
+ * xs/nn/grad_fn.py:146-157 followed by AddBackward, xs/nn/grad_fn.py:14-22): both addends receive it.
+ * dy, dx1, dx2 16-byte aligned, neg_mask 4-byte aligned; dx1 != dx2. */
+int xsmi_relu_mask_bwd2(const float *dy, const uint8_t *neg_mask, float *dx1, float beta1, float *dx2, float beta2, size_t n);
 
 /* ---- neighbours of conv / pool in a network (device-resident tensors) --------
  * Small element-wise, normalisation and reduction kernels so that activations need not

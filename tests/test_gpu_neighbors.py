@@ -165,3 +165,29 @@ def test_held_back_add_joins_the_in_place_relu(gpu):
     expect = ((a + b) >= 0).astype(np.float32)
     np.testing.assert_array_equal(ta.grad.numpy(), expect)
     np.testing.assert_array_equal(tb.grad.numpy(), expect)
+    # a second sweep adds into the gradients that are already there
+    g2 = rng.standard_normal(a.shape).astype(np.float32)
+    out4 = ReLU(inplace=True)(ta + tb)
+    out4.backward(xs.tensor(g2).to('cuda'))
+    np.testing.assert_array_equal(ta.grad.numpy(), expect + g2 * expect)
+    np.testing.assert_array_equal(tb.grad.numpy(), expect + g2 * expect)
+
+
+def test_masked_gradient_into_two_tensors(gpu):
+    """xsmi_relu_mask_bwd2 against two single calls, overwrite and accumulate, with a ragged tail."""
+    K = gpu.kernels
+    rng = np.random.default_rng(21)
+    n = 4 * 1000 + 3
+    dy = rng.standard_normal(n).astype(np.float32)
+    mask = (rng.random(n) < 0.4).astype(np.uint8)
+    o1, o2 = rng.standard_normal(n).astype(np.float32), rng.standard_normal(n).astype(np.float32)
+    ddy, dm = gpu.to_device(dy), gpu.to_device(mask)
+    for acc in (False, True):
+        d1, d2 = gpu.to_device(o1), gpu.to_device(o2)
+        K.relu_mask_bwd2(ddy, dm, d1, d2, accumulate=acc)
+        e1, e2 = gpu.to_device(o1), gpu.to_device(o2)
+        K.relu_mask_bwd(ddy, dm, dx=e1, accumulate=acc)
+        K.relu_mask_bwd(ddy, dm, dx=e2, accumulate=acc)
+        np.testing.assert_array_equal(d1.numpy(), e1.numpy())
+        np.testing.assert_array_equal(d2.numpy(), e2.numpy())
+        np.testing.assert_array_equal(d1.numpy(), (o1 if acc else 0) + np.where(mask != 0, np.float32(0), dy))

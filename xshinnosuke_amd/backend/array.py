@@ -106,6 +106,11 @@ class DeviceArray:
             lib.call("xsmi_memset", ctypes.c_void_p(blk.ptr), 0, blk.nbytes)
         return blk.ptr + self._offset
 
+    def address(self):
+        """The device address as an integer; unlike ``ptr`` it leaves a pending clear pending (for alignment and
+        aliasing checks)."""
+        return self._block.ptr + self._offset
+
     def is_fresh(self):
         """True if the array is a whole allocation whose clear is still pending."""
         blk = self._block

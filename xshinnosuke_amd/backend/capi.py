@@ -65,6 +65,7 @@ SIGNATURES = {
     "xsmi_maxpool2d_fwd": (_i, [_vp, _vp, _vp] + [_i] * 8),
     "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
     "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),
+    "xsmi_relu_mask_bwd2": (_i, [_vp, _vp, _vp, _f, _vp, _f, _sz]),
     "xsmi_axpy": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_axpy_multi": (_i, [_i, _c.POINTER(_vp), _c.POINTER(_vp), _c.POINTER(_sz), _f]),
     "xsmi_add": (_i, [_vp, _vp, _vp, _sz]),

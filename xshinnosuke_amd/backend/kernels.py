@@ -192,6 +192,16 @@ def relu_mask_bwd(dy, neg_mask, dx=None, accumulate=False):
     return dx
 
 
+def relu_mask_bwd2(dy, neg_mask, dx1, dx2, accumulate=True):
+    """The masked gradient (0 where neg_mask is set, else dy) added into (or written over) two tensors at once."""
+    _f32(dy, "dy")
+    if dx1.size != dy.size or dx2.size != dy.size or dx1 is dx2:
+        raise ValueError("relu_mask_bwd2: needs two different outputs of dy's size")
+    b1, b2 = _beta(accumulate, dx1), _beta(accumulate, dx2)
+    lib.call("xsmi_relu_mask_bwd2", dy.cptr, neg_mask.cptr, dx1.cptr, b1, dx2.cptr, b2, dy.size)
+    return dx1, dx2
+
+
 def copy_kernel(dst, src):
     lib.call("xsmi_copy_kernel", dst.cptr, src.cptr, src.nbytes)
 

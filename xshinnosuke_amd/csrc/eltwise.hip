@@ -32,6 +32,35 @@ __global__ void __launch_bounds__(256) relu_mask_bwd_kernel(const float *__restr
     }
 }
 
+// the same masked gradient delivered to two tensors at once (both inputs of the addition in front of the ReLU)
+__global__ void __launch_bounds__(256) relu_mask_bwd2_kernel(const float *__restrict__ dy, const uint8_t *__restrict__ mask,
+                                                              float *dx1, float *dx2, size_t n, int acc1, int acc2) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= n) return;
+    if (i + 4 <= n) {
+        float4 g = *reinterpret_cast<const float4 *>(dy + i);
+        uchar4 m = *reinterpret_cast<const uchar4 *>(mask + i);
+        const float4 o = make_float4(m.x ? 0.f : g.x, m.y ? 0.f : g.y, m.z ? 0.f : g.z, m.w ? 0.f : g.w);
+        float4 o1 = o, o2 = o;
+        if (acc1) {
+            float4 d = *reinterpret_cast<const float4 *>(dx1 + i);
+            o1.x += d.x; o1.y += d.y; o1.z += d.z; o1.w += d.w;
+        }
+        if (acc2) {
+            float4 d = *reinterpret_cast<const float4 *>(dx2 + i);
+            o2.x += d.x; o2.y += d.y; o2.z += d.z; o2.w += d.w;
+        }
+        *reinterpret_cast<float4 *>(dx1 + i) = o1;
+        *reinterpret_cast<float4 *>(dx2 + i) = o2;
+    } else {
+        for (; i < n; ++i) {
+            const float o = mask[i] ? 0.f : dy[i];
+            dx1[i] = acc1 ? dx1[i] + o : o;
+            dx2[i] = acc2 ? dx2[i] + o : o;
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -97,6 +126,21 @@ int xsmi_relu_mask_bwd(const float *dy, const uint8_t *neg_mask, float *dx, size
     hipLaunchKernelGGL(relu_mask_bwd_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, xsmi::stream(), dy,
                        neg_mask, dx, n, beta == 1.f ? 1 : 0);
     XSMI_LAUNCH_CHECK("relu_mask_bwd_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_relu_mask_bwd2(const float *dy, const uint8_t *neg_mask, float *dx1, float beta1, float *dx2, float beta2, size_t n) {
+    XSMI_REQUIRE_INIT();
+    if (n == 0) return XSMI_OK;
+    XSMI_CHECK_ARG(dy && neg_mask && dx1 && dx2, "xsmi_relu_mask_bwd2: null pointer");
+    XSMI_CHECK_ARG(dx1 != dx2, "xsmi_relu_mask_bwd2: the two outputs must differ");
+    XSMI_CHECK_ARG((beta1 == 0.f || beta1 == 1.f) && (beta2 == 0.f || beta2 == 1.f), "xsmi_relu_mask_bwd2: beta must be 0 or 1");
+    XSMI_CHECK_ARG((((uintptr_t)dy | (uintptr_t)dx1 | (uintptr_t)dx2) & 15) == 0 && ((uintptr_t)neg_mask & 3) == 0,
+                   "xsmi_relu_mask_bwd2: tensors must be 16-byte aligned (mask: 4)");
+    size_t threads = (n + 3) / 4;
+    hipLaunchKernelGGL(relu_mask_bwd2_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, xsmi::stream(), dy,
+                       neg_mask, dx1, dx2, n, beta1 == 1.f ? 1 : 0, beta2 == 1.f ? 1 : 0);
+    XSMI_LAUNCH_CHECK("relu_mask_bwd2_kernel");
     return XSMI_OK;
 }
 

@@ -110,19 +110,38 @@ def ReLUBackward(outputs):
     """Reference xs/nn/grad_fn.py:146-157, both the in-place and the out-of-place form."""
     if outputs.cache.get('inplace'):
         g, mask = outputs.grad.eval, outputs.cache['neg_mask_inplace']
+        prev = outputs.cache['grad_fn'].pop()
+        outputs.cache['inplace'] = bool(outputs.cache['grad_fn'])
+        outputs.grad_fn = prev
+        if prev is AddBackward and is_device(g) and not outputs.retain_grad() and _both_addends_on_device(outputs, g):
+            # ReLU applied in place to a sum: the masked gradient goes to both addends in one pass
+            a, b = outputs.in_bounds
+            K.relu_mask_bwd2(g, mask, a.grad.eval, b.grad.eval, accumulate=True)
+            return
         if is_device(g):
             K.relu_mask_bwd(g, mask, dx=g)                 # in place on the gradient
         else:
             g[mask] = 0
-        prev = outputs.cache['grad_fn'].pop()
-        outputs.cache['inplace'] = bool(outputs.cache['grad_fn'])
-        outputs.grad_fn = prev
         if prev is not None:
             prev(outputs)
     else:
         inputs, = outputs.in_bounds
         if inputs.requires_grad:
             _accumulate(inputs, A.relu_grad(outputs.grad.eval, inputs.eval))
+
+
+def _both_addends_on_device(outputs, g):
+    """Two distinct addends of the output's shape that both want a gradient and keep it in aligned device memory."""
+    if len(outputs.in_bounds) != 2:
+        return False
+    a, b = outputs.in_bounds
+    if a is b or not (a.requires_grad and b.requires_grad):
+        return False
+    for t in (a, b):
+        d = t.grad.eval if t.grad is not None else None
+        if d is None or not is_device(d) or d.dtype != np.float32 or tuple(t.shape) != tuple(outputs.shape) or d.address() % 16:
+            return False
+    return a.grad.eval.address() != b.grad.eval.address() and g.address() % 16 == 0
 
 
 def AddBackward(outputs):
