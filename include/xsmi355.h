@@ -12,8 +12,10 @@
  *     partials) is a caller-provided workspace sized by the matching
  *     *_workspace_bytes query.  The workspace contents are dead after the call
  *     has completed on the stream.
- *   - All work is enqueued on one library-owned stream; results are visible to
- *     the host after xsmi_sync() or a (blocking) xsmi_memcpy_d2h.
+ *   - All work is enqueued in order on one library-owned stream (xsmi_conv2d_bwd
+ *     forks part of its work to a second one and joins it again before the
+ *     call's successors); results are visible to the host after xsmi_sync() or
+ *     a (blocking) xsmi_memcpy_d2h.  Calls are not re-entrant across threads.
  *   - Window geometry follows the reference: symmetric integer zero padding
  *     `pad`, stride (sh, sw), OH = (H + 2*pad - R)/sh + 1 (floor), no dilation,
  *     no groups.
