@@ -220,7 +220,7 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
                 float *mean, float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask,
                 int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
 /* moving_mean / moving_var (both or neither): m = momentum*m + (1-momentum)*batch statistic, the update the
- * reference performs after the forward (xs/nn/functional.py:700-707), done by the statistics kernel.
+ * reference performs after the forward (xs/nn/functional.py:700-707), done by the normalisation kernel.
  * neg_mask (or NULL) fuses the ReLU that follows the normalisation in a residual block
  * (xs/layers/activators.py:37-50): neg_mask[i] = pre-activation < 0, y = max(pre-activation, 0). */
 /* Inference form with given statistics (xs/nn/functional.py:708-725); relu != 0 clips at zero. */

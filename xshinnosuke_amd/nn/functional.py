@@ -406,7 +406,7 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
     dst = None if out is None else out.eval
     if training:
         mm, mv = moving_mean.eval, moving_variance.eval
-        fused = is_device(x) and is_device(mm) and is_device(mv)      # the statistics kernel updates them
+        fused = is_device(x) and is_device(mm) and is_device(mv)      # the normalisation kernel updates them
         track = GLOBAL.COMPUTE_GRAD and bool(inputs.requires_grad or gamma.requires_grad or beta.requires_grad)
         neg_mask = dev.empty(x.shape, np.uint8) if relu else None
         y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst,
