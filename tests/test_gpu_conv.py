@@ -179,10 +179,13 @@ def test_conv_bf16_forward_channels_last(gpu, n, c, h, w, k, r, s, sh, sw, pad):
 
 @pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", [CASES[2], CASES[4], CASES[6], CASES[9], CASES[11]])
 @pytest.mark.parametrize("accumulate", [False, True])
-def test_conv_both_gradients_in_one_call(gpu, n, c, h, w, k, r, s, sh, sw, pad, accumulate):
-    """xsmi_conv2d_bwd runs the two backward kernels side by side on two streams: same bits as the two
-    calls one after the other, also when adding into gradients that are already there, and twice in a row
-    (the second call's kernels must wait for the first call's)."""
+@pytest.mark.parametrize("async_dw", [False, True])
+def test_conv_both_gradients_in_one_call(gpu, n, c, h, w, k, r, s, sh, sw, pad, accumulate, async_dw):
+    """xsmi_conv2d_bwd runs the two backward kernels on two streams: same bits as the two calls one after the
+    other, also when adding into gradients that are already there, and twice in a row (the second call's kernels
+    must wait for the first call's).  With async_dw the weight gradient is still on the second stream when the call
+    returns; reading it back joins first."""
+    from xshinnosuke_amd.backend import capi
     K = gpu.kernels
     rng = np.random.default_rng(77 + c + k)
     x = gpu.to_device(rng.standard_normal((n, c, h, w)).astype(np.float32))
@@ -195,9 +198,49 @@ def test_conv_both_gradients_in_one_call(gpu, n, c, h, w, k, r, s, sh, sw, pad, 
     for dy in dys:
         K.conv2d_bwd_weight(dy, x, wt.shape, (sh, sw), pad, dw=a[1], db=a[2], accumulate=accumulate)
         K.conv2d_bwd_data(dy, wt, x.shape, (sh, sw), pad, dx=a[0], accumulate=accumulate)
-        K.conv2d_bwd(dy, x, wt, b[0], b[1], b[2], (sh, sw), pad, accumulate=accumulate)
+    for dy in dys:
+        K.conv2d_bwd(dy, x, wt, b[0], b[1], b[2], (sh, sw), pad, accumulate=accumulate, async_dw=async_dw)
+        assert capi.side_pending() == async_dw
     for u, v in zip(a, b):
         assert np.array_equal(u.numpy(), v.numpy())
+    assert not capi.side_pending()
+
+
+def test_conv_async_weight_gradient_is_joined_before_use(gpu):
+    """Whatever touches the weight gradient after an asynchronous xsmi_conv2d_bwd (an optimizer update, the plain
+    weight-gradient entry point adding into the same buffer) sees it complete; the passes of a backward sweep that
+    cannot touch it do not wait."""
+    from xshinnosuke_amd.backend import capi
+    K = gpu.kernels
+    rng = np.random.default_rng(5)
+    n, c, h, k = 8, 64, 28, 64
+    x = gpu.to_device(rng.standard_normal((n, c, h, h)).astype(np.float32))
+    wt = gpu.to_device(he_normal(rng, (k, c, 3, 3)))
+    dy = gpu.to_device(rng.standard_normal((n, k, h, h)).astype(np.float32))
+    ref_dw, _ = K.conv2d_bwd_weight(dy, x, wt.shape, (1, 1), 1)
+    ref = ref_dw.numpy()
+    twice = gpu.to_device(ref)
+    K.conv2d_bwd_weight(dy, x, wt.shape, (1, 1), 1, dw=twice, accumulate=True)
+    for use in ("axpy", "bwd_weight", "sync"):
+        dx, dw = gpu.empty(x.shape), gpu.empty(wt.shape)
+        other = gpu.empty(x.shape)
+        mask = gpu.to_device(np.zeros(x.shape, np.uint8))
+        K.conv2d_bwd(dy, x, wt, dx, dw, None, (1, 1), 1, async_dw=True)
+        K.relu_mask_bwd(dx, mask, dx=other)                  # a pass of the sweep: does not join
+        assert capi.side_pending()
+        if use == "axpy":
+            p = gpu.to_device(np.zeros(wt.shape, np.float32))
+            K.axpy(p, dw, 1.0)
+            assert not capi.side_pending()
+            np.testing.assert_array_equal(p.numpy(), ref)
+        elif use == "bwd_weight":
+            K.conv2d_bwd_weight(dy, x, wt.shape, (1, 1), 1, dw=dw, accumulate=True)
+            assert not capi.side_pending()
+            np.testing.assert_array_equal(dw.numpy(), twice.numpy())
+        else:
+            gpu.synchronize()
+            assert not capi.side_pending()
+            np.testing.assert_array_equal(dw.numpy(), ref)
 
 
 def test_conv_packed_workspace_flag(gpu):

@@ -270,6 +270,10 @@ class Workspace:
     def __init__(self):
         self._block = None
 
+    def holds(self, nbytes):
+        """True if ``get(nbytes)`` would hand out the present block (no reallocation)."""
+        return self._block is not None and self._block.nbytes >= nbytes
+
     def get(self, nbytes):
         if self._block is None or self._block.nbytes < nbytes:
             self._block = None

@@ -61,7 +61,8 @@ SIGNATURES = {
     "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
     "xsmi_conv2d_bwd_data": (_i, [_vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
     "xsmi_conv2d_bwd_weight": (_i, [_vp, _vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
-    "xsmi_conv2d_bwd": (_i, [_vp] * 6 + _CONV_DIMS + [_f, _f, _u, _vp, _sz]),
+    "xsmi_conv2d_bwd": (_i, [_vp] * 6 + _CONV_DIMS + [_f, _f, _u, _vp, _sz, _vp, _sz]),
+    "xsmi_conv2d_bwd_join": (_i, []),
     "xsmi_maxpool2d_fwd": (_i, [_vp, _vp, _vp] + [_i] * 8),
     "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
     "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),
@@ -93,6 +94,7 @@ SIGNATURES = {
 CONV_RELU = 0x1
 CONV_BF16 = 0x2
 CONV_WS_PACKED = 0x4
+CONV_DW_ASYNC = 0x8
 
 
 def library_path():
@@ -127,6 +129,8 @@ class _Lib:
         """Call an int-returning entry point; raise with the library's message on failure."""
         if _deferred:
             _flush_deferred()
+        if _side_hold and name not in _SIDE_SAFE:
+            join_side()
         dll = self._open()
         rc = getattr(dll, name)(*args)
         if rc != 0:
@@ -137,6 +141,32 @@ class _Lib:
 
 
 lib = _Lib()
+
+# Weight gradients that xsmi_conv2d_bwd left on the library's second stream (XSMI_CONV_DW_ASYNC).  The arrays they
+# read and write are kept alive here, so their memory cannot be handed out again, and every call into the library
+# joins the second stream first unless it is one of the passes of a backward sweep listed below: those write
+# activation gradients only, never a filter gradient, a forward activation or an upstream gradient already consumed.
+_side_hold = []
+_SIDE_SAFE = frozenset(("xsmi_conv2d_bwd", "xsmi_bn_bwd", "xsmi_relu_mask_bwd", "xsmi_relu_mask_bwd2", "xsmi_relu_bwd",
+                        "xsmi_maxpool2d_bwd", "xsmi_avgpool_bwd", "xsmi_conv2d_bwd_join"))
+
+
+def hold_side(*arrays):
+    _side_hold.append(arrays)
+
+
+def side_pending():
+    return bool(_side_hold)
+
+
+def join_side():
+    """The main stream waits for the weight gradients on the second stream; their operands are released."""
+    if _side_hold:
+        try:
+            lib.call("xsmi_conv2d_bwd_join")
+        finally:
+            del _side_hold[:]
+
 
 # One element-wise add may be held back until the next call into the library: if that call is the in-place ReLU
 # of its result, both run as one pass (kernels.add / kernels.relu_fwd).  Every other call enqueues the add first,

@@ -9,10 +9,11 @@ import ctypes
 import numpy as np
 
 from . import capi
-from .capi import lib, CONV_RELU, CONV_BF16, CONV_WS_PACKED
+from .capi import lib, CONV_RELU, CONV_BF16, CONV_WS_PACKED, CONV_DW_ASYNC
 from .array import DeviceArray, Workspace, empty
 
 _ws = Workspace()
+_ws_dw = Workspace()        # weight-gradient scratch of conv2d_bwd: lives beside _ws because the two kernels overlap
 
 
 def conv_out_hw(h, w, r, s, stride, pad):
@@ -121,9 +122,11 @@ def conv2d_bwd_weight(dy, x, w_shape, stride=(1, 1), pad=0, dw=None, db=None, ac
     return dw, db
 
 
-def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False, bf16=False):
-    """Both gradients of one layer in one call, into existing device buffers; the two kernels run side by side.
-    Same results as ``conv2d_bwd_weight`` followed by ``conv2d_bwd_data``."""
+def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False, bf16=False, async_dw=False):
+    """Both gradients of one layer in one call, into existing device buffers.  Same results as ``conv2d_bwd_weight``
+    followed by ``conv2d_bwd_data``.  ``async_dw=True`` leaves the weight gradient running on the library's second
+    stream beside whatever is enqueued next; dw and db are complete after ``capi.join_side()``, which every call into
+    the library performs by itself except the passes of a backward sweep that cannot touch them."""
     _f32(dy, "dy"); _f32(x, "x"); _f32(w, "w")
     dims = _dims(x.shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -134,11 +137,18 @@ def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False
         raise ValueError("conv2d backward: dx %s / dw %s do not match x %s / w %s" % (dx.shape, dw.shape, x.shape, w.shape))
     if db is not None and db.size != k:
         raise ValueError("conv2d backward: db has %d elements for %d filters" % (db.size, k))
-    ws, ws_bytes = _workspace(dims)
+    need = lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
+    if capi.side_pending() and not _ws_dw.holds(need):
+        capi.join_side()                        # the block about to be replaced may still be in use
+    ws, ws_bytes = _ws.get(need)
+    ws_dw, ws_dw_bytes = _ws_dw.get(need)
     beta_dw = _beta(accumulate, dw, db)
     beta_dx = _beta(accumulate, dx)
+    flags = (CONV_BF16 if bf16 else 0) | (CONV_DW_ASYNC if async_dw else 0)
     lib.call("xsmi_conv2d_bwd", dy.cptr, x.cptr, w.cptr, dx.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
-             beta_dx, beta_dw, CONV_BF16 if bf16 else 0, ws, ws_bytes)
+             beta_dx, beta_dw, flags, ws, ws_bytes, ws_dw, ws_dw_bytes)
+    if async_dw:
+        capi.hold_side(dy, x, dw, db)
     return dx, dw, db
 
 

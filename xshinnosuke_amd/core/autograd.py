@@ -1,6 +1,7 @@
 """Reverse-mode sweep over the dynamic graph (counterpart of xs/core/autograd.py:5-45)."""
 from . import state as GLOBAL
 from .base import Parameter
+from ..backend import capi as _capi
 
 
 def topological_sort(ins, outs):
@@ -26,8 +27,7 @@ def topological_sort(ins, outs):
     return order
 
 
-def backward(outputs, inputs, retain_graph=False):
-    graph = topological_sort(inputs, outputs)
+def _sweep(graph, retain_graph):
     for node in reversed(graph):
         if node.grad_fn is not None:
             node.grad_fn(node)
@@ -41,6 +41,14 @@ def backward(outputs, inputs, retain_graph=False):
         else:
             node.free_memory()
             node.reset_(**kwargs)
+
+
+def backward(outputs, inputs, retain_graph=False):
+    graph = topological_sort(inputs, outputs)
+    try:
+        _sweep(graph, retain_graph)
+    finally:
+        _capi.join_side()        # weight gradients that conv layers left on the backend's second stream
     if retain_graph:
         GLOBAL.GRAPH = graph
     else:

@@ -263,6 +263,12 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
     const size_t need = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need,
                    "xsmi_conv2d_bwd_weight: workspace of %zu bytes needed, %zu given", need, workspace_bytes);
+    // called on the main stream while weight gradients of xsmi_conv2d_bwd are still on the second one: they may
+    // add into the same dw, so they come first
+    if (!xsmi::on_side_stream()) {
+        int rj = xsmi::side_join();
+        if (rj) return rj;
+    }
 
     if (xsmi::wgrad_tap_ok(dy, x, C, K, OH, OW))
         return xsmi::wgrad_tap(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, OH, OW, beta == 1.f ? 1 : 0, workspace);

@@ -74,9 +74,6 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
     size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     size_t m = a > b ? a : b;
     m = m > c ? m : c;
-    // xsmi_conv2d_bwd runs both backward kernels at once, each in a part of its own
-    size_t both = xsmi::align_up(b, 256) + c;
-    m = m > both ? m : both;
     // the bf16 forward takes its fastest form when the workspace also holds a channels-last copy of x
     if (xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad)) {
         size_t d = xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad);
@@ -87,33 +84,42 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
 
 int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w, float *dx, float *dw, float *db, int N, int C, int H,
                     int W, int K, int R, int S, int sh, int sw, int pad, float beta_dx, float beta_dw, unsigned flags,
-                    void *workspace, size_t workspace_bytes) {
+                    void *workspace, size_t workspace_bytes, void *workspace_dw, size_t workspace_dw_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && K > 0 && R > 0 && S > 0 && sh > 0 && sw > 0 && pad >= 0 &&
                        H + 2 * pad >= R && W + 2 * pad >= S,
                    "xsmi_conv2d_bwd: bad geometry");
     XSMI_CHECK_ARG(dy && x && w && dx && dw, "xsmi_conv2d_bwd: null tensor pointer");
     XSMI_CHECK_ARG((beta_dx == 0.f || beta_dx == 1.f) && (beta_dw == 0.f || beta_dw == 1.f), "xsmi_conv2d_bwd: beta must be 0 or 1");
-    XSMI_CHECK_ARG((flags & ~XSMI_CONV_BF16) == 0, "xsmi_conv2d_bwd: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_DW_ASYNC)) == 0, "xsmi_conv2d_bwd: unknown flags 0x%x", flags);
     const int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
-    const size_t data_part = xsmi::align_up(xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw), 256);
-    const size_t weight_part = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
-    XSMI_CHECK_ARG(workspace && workspace_bytes >= data_part + weight_part,
-                   "xsmi_conv2d_bwd: workspace of %zu bytes needed, %zu given", data_part + weight_part, workspace_bytes);
-    // The two kernels share only their inputs.  Where the data gradient's grid (128-pixel x 64-channel tiles)
-    // leaves compute units idle, the weight gradient runs beside it on the second stream: 6-9 % less time for
-    // both at 7x7 and 14x14 feature maps.  Grids that fill the chip alone only get in each other's way
-    // (15 % more time at 56x56), so they run one after the other on the main stream.
+    const size_t data_need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
+    const size_t weight_need = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
+    XSMI_CHECK_ARG(workspace && workspace_bytes >= data_need, "xsmi_conv2d_bwd: workspace of %zu bytes needed, %zu given",
+                   data_need, workspace_bytes);
+    XSMI_CHECK_ARG(workspace_dw && workspace_dw_bytes >= weight_need,
+                   "xsmi_conv2d_bwd: weight-gradient workspace of %zu bytes needed, %zu given", weight_need, workspace_dw_bytes);
+    XSMI_CHECK_ARG((char *)workspace + workspace_bytes <= (char *)workspace_dw ||
+                       (char *)workspace_dw + workspace_dw_bytes <= (char *)workspace,
+                   "xsmi_conv2d_bwd: the two workspaces overlap");
+    const unsigned kflags = flags & XSMI_CONV_BF16;
+    // The two kernels share only their inputs.  XSMI_CONV_DW_ASYNC: the weight gradient goes to the second stream
+    // and stays there; the main stream runs on (data gradient, then whatever the caller enqueues next: the
+    // memory-bound passes between two convolutions of a backward sweep fit beside a matrix-bound kernel) until
+    // xsmi_conv2d_bwd_join.  Without the flag the call is complete in main-stream order when it returns: where the
+    // data gradient's grid (128-pixel x 64-channel tiles) leaves compute units idle the weight gradient still runs
+    // beside it (6-9 % less time for both at 7x7 and 14x14 feature maps) and is joined at once; grids that fill the
+    // chip alone only get in each other's way (15 % more time at 56x56) and run one after the other.
     const long long tiles = (((long long)N * H * W + 127) / 128) * xsmi::ceil_div(C, 64);
-    const bool beside = tiles <= xsmi::cu_count();
-    int rc = beside ? xsmi::side_begin() : XSMI_OK;
+    const bool async = (flags & XSMI_CONV_DW_ASYNC) != 0;
+    const bool beside = async || tiles <= xsmi::cu_count();
+    int rc = beside ? xsmi::side_begin() : xsmi::side_join();    // in main-stream order: after any earlier async work
     if (rc) return rc;
-    rc = xsmi_conv2d_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, beta_dw, flags,
-                                (char *)workspace + data_part, weight_part);
+    rc = xsmi_conv2d_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, beta_dw, kflags, workspace_dw, weight_need);
     if (beside) xsmi::side_end();
     if (rc == XSMI_OK)
-        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, flags, workspace, data_part);
-    const int rj = beside ? xsmi::side_join() : XSMI_OK;
+        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, kflags, workspace, data_need);
+    const int rj = (beside && !async) || rc ? xsmi::side_join() : XSMI_OK;
     return rc ? rc : rj;
 }
 

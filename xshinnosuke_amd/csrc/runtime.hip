@@ -9,6 +9,7 @@ hipStream_t g_stream = nullptr;
 hipStream_t g_side = nullptr;            // second stream for work that may overlap the main stream's
 hipStream_t g_current = nullptr;         // what stream() hands out: g_stream, or g_side inside a side section
 hipEvent_t g_fork = nullptr, g_join = nullptr;
+bool g_side_pending = false;             // the second stream holds work the main stream has not waited for yet
 int g_device = -1;
 int g_cus = 0;
 bool g_ready = false;
@@ -32,14 +33,19 @@ int side_begin() {
     XSMI_HIP(hipEventRecord(g_fork, g_stream));
     XSMI_HIP(hipStreamWaitEvent(g_side, g_fork, 0));
     g_current = g_side;
+    g_side_pending = true;
     return XSMI_OK;
 }
 void side_end() { g_current = g_stream; }
 int side_join() {
+    if (!g_side_pending) return XSMI_OK;
     XSMI_HIP(hipEventRecord(g_join, g_side));
     XSMI_HIP(hipStreamWaitEvent(g_stream, g_join, 0));
+    g_side_pending = false;
     return XSMI_OK;
 }
+bool side_pending() { return g_side_pending; }
+bool on_side_stream() { return g_current == g_side; }
 bool ready() { return g_ready; }
 int cu_count() { return g_cus; }
 void prof_begin() {
@@ -188,8 +194,15 @@ int xsmi_memset(void *dst, int byte_value, size_t bytes) {
     return XSMI_OK;
 }
 
+int xsmi_conv2d_bwd_join(void) {
+    XSMI_REQUIRE_INIT();
+    return xsmi::side_join();
+}
+
 int xsmi_sync(void) {
     XSMI_REQUIRE_INIT();
+    int rc = xsmi::side_join();                      // weight gradients still on the second stream
+    if (rc) return rc;
     XSMI_HIP(hipStreamSynchronize(g_stream));
     return XSMI_OK;
 }

@@ -13,10 +13,13 @@ void set_error(const char *fmt, ...);
 // nullptr until xsmi_init succeeded.
 hipStream_t stream();
 // Side section: launches between side_begin() and side_end() go to the second stream, ordered after all
-// earlier main-stream work; side_join() makes the main stream wait for them.
+// earlier main-stream work; side_join() makes the main stream wait for them (it may come much later:
+// until then the main stream runs on beside them).
 int side_begin();
 void side_end();
-int side_join();
+int side_join();              // no-op when the second stream holds nothing the main stream has not waited for
+bool side_pending();
+bool on_side_stream();
 bool ready();
 int cu_count();
 // With xsmi_profiling(1) every op brackets its main kernel(s) with two events on

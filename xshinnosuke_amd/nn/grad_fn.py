@@ -62,9 +62,10 @@ def Conv2DBackward(outputs):
         dw_buf, dx_buf = weight.grad.eval, inputs.grad.eval
         db_buf = bias.grad.eval if want_db else None
         if is_device(dw_buf) and is_device(dx_buf) and (not want_db or is_device(db_buf)):
-            # all gradients live on the device: one call, the two kernels side by side
+            # all gradients live on the device: one call; the weight gradient keeps running on the second
+            # stream beside the rest of the sweep (the backend joins it before anything else can touch it)
             K.conv2d_bwd(dy, x_dev, w_dev, dx_buf, dw_buf, db_buf.reshape(-1) if want_db else None, stride, pad,
-                         accumulate=True, bf16=bf16)
+                         accumulate=True, bf16=bf16, async_dw=True)
             return
     if want_dw or want_db:
         dw_buf = weight.grad.eval if want_dw else None
