@@ -99,24 +99,30 @@ def test_dense_gemm_all_transposes(gpu):
         assert rel_l2(K.gemm(da, dg, trans_a=True).numpy(), a.T.astype(np.float64) @ g) <= 1e-5
 
 
-def test_softmax_cross_entropy(gpu):
-    """xs/nn/functional.py:984-1010 and xs/nn/grad_fn.py:604-620."""
+@pytest.mark.parametrize("m,n", [(37, 100), (32, 1000), (3, 2500)])
+def test_softmax_cross_entropy(gpu, m, n):
+    """xs/nn/functional.py:984-1010 and xs/nn/grad_fn.py:604-620; rows longer than what a workgroup keeps in
+    registers (2048 classes) take the second form of the loops."""
     K = gpu.kernels
-    rng = np.random.default_rng(4)
-    logits = (rng.standard_normal((37, 100)) * 3).astype(np.float32); labels = rng.integers(0, 100, size=37)
+    rng = np.random.default_rng(4 + n)
+    logits = (rng.standard_normal((m, n)) * 3).astype(np.float32); labels = rng.integers(0, n, size=m)
     z = logits.astype(np.float64); z -= z.max(axis=1, keepdims=True)
     sm = np.exp(z); sm /= sm.sum(axis=1, keepdims=True)
     for reduction in ("mean", "sum"):
         dl = gpu.to_device(labels.astype(np.int64), np.int64)
         loss, smd = K.softmax_ce_fwd(gpu.to_device(logits), dl, reduction)
-        ref = -np.log(sm[np.arange(37), labels])
+        assert rel_l2(smd.numpy(), sm) <= 1e-6
+        ref = -np.log(sm[np.arange(m), labels])
         ref = ref.mean() if reduction == "mean" else ref.sum()
         assert abs(float(np.asarray(loss.numpy()).reshape(-1)[0]) - ref) <= 1e-5 * abs(ref)
         g = K.softmax_ce_bwd(smd, dl, reduction, 1.0).numpy()
-        gref = sm.copy(); gref[np.arange(37), labels] -= 1.0
+        gref = sm.copy(); gref[np.arange(m), labels] -= 1.0
         if reduction == "mean":
-            gref /= 37
+            gref /= m
         assert rel_l2(g, gref) <= 1e-5
+        up = gpu.to_device(np.array([0.5], np.float32))          # the loss's own gradient read on the device
+        g2 = K.softmax_ce_bwd(smd, dl, reduction, up).numpy()
+        assert rel_l2(g2, 0.5 * gref) <= 1e-5
 
 
 def test_held_back_add_joins_the_in_place_relu(gpu):
@@ -191,3 +197,22 @@ def test_masked_gradient_into_two_tensors(gpu):
         np.testing.assert_array_equal(d1.numpy(), e1.numpy())
         np.testing.assert_array_equal(d2.numpy(), e2.numpy())
         np.testing.assert_array_equal(d1.numpy(), (o1 if acc else 0) + np.where(mask != 0, np.float32(0), dy))
+
+
+@pytest.mark.parametrize("n,c,h,w,k", [(3, 5, 6, 6, 2), (4, 70, 7, 7, 7), (2, 3, 7, 8, 3), (1, 2, 13, 13, 13)])
+def test_average_pool_blocks(gpu, n, c, h, w, k):
+    """Mean over non-overlapping k x k blocks and its gradient (xs/nn/functional.py:539-583,
+    xs/nn/grad_fn.py:284-309); k == H == W is the global pool in front of ResNet's dense layer."""
+    K = gpu.kernels
+    rng = np.random.default_rng(n + c + h + k)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    oh, ow = h // k, w // k
+    ref = x[:, :, :oh * k, :ow * k].astype(np.float64).reshape(n, c, oh, k, ow, k).mean(axis=(3, 5))
+    y = K.avgpool_fwd(gpu.to_device(x), k).numpy()
+    assert y.shape == (n, c, oh, ow)
+    np.testing.assert_allclose(y, ref, rtol=1e-6, atol=1e-7)
+    dy = rng.standard_normal((n, c, oh, ow)).astype(np.float32)
+    dx = K.avgpool_bwd(gpu.to_device(dy), x.shape, k).numpy()
+    dref = np.zeros_like(x)
+    dref[:, :, :oh * k, :ow * k] = np.repeat(np.repeat(dy, k, axis=2), k, axis=3) / np.float32(k * k)
+    np.testing.assert_allclose(dx, dref, rtol=1e-6, atol=0)

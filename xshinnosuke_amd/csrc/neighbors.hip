@@ -463,6 +463,18 @@ __global__ void __launch_bounds__(256) avgpool_fwd_kernel(const float *__restric
         y[o] = (float)(s / (double)(k * k));
     }
 }
+// the window is the whole plane (global pooling): one wavefront per plane, lanes along the plane's contiguous elements
+__global__ void __launch_bounds__(256) avgpool_plane_kernel(const float *__restrict__ x, float *__restrict__ y, int HW,
+                                                             uint32_t planes) {
+    const uint32_t pl = blockIdx.x * 4u + (threadIdx.x >> 6);
+    if (pl >= planes) return;
+    const int lane = threadIdx.x & 63;
+    const float *p = x + (size_t)pl * HW;
+    double s = 0.0;
+    for (int i = lane; i < HW; i += 64) s += (double)p[i];
+    s = wave_sum(s);
+    if (lane == 0) y[pl] = (float)(s / (double)HW);
+}
 __global__ void __launch_bounds__(256) avgpool_bwd_kernel(const float *__restrict__ dy, float *__restrict__ dx, int H, int W,
                                                            int OH, int OW, int k, size_t total) {
     for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
@@ -561,19 +573,40 @@ __global__ void __launch_bounds__(256) sum_all_kernel(const float *__restrict__ 
     if (threadIdx.x == 0) out[0] = (float)s;
 }
 
-// ---- softmax cross-entropy: one wavefront per row ------------------------------------
-__global__ void __launch_bounds__(64) softmax_rows_kernel(const float *__restrict__ z, const int64_t *__restrict__ lab,
-                                                           float *__restrict__ sm, float *__restrict__ nll, int M, int N) {
-    const int row = blockIdx.x, lane = threadIdx.x;
+// ---- softmax cross-entropy: one workgroup per row --------------------------------------
+// exp() in float64, once per element: a thread keeps up to SOFTMAX_KEEP of its elements' exponentials in
+// registers between the sum and the division (rows of up to 256 * SOFTMAX_KEEP classes); beyond that they
+// are computed again.
+constexpr int SOFTMAX_KEEP = 8;
+__global__ void __launch_bounds__(256) softmax_rows_kernel(const float *__restrict__ z, const int64_t *__restrict__ lab,
+                                                            float *__restrict__ sm, float *__restrict__ nll, int M, int N) {
+    __shared__ double red[4];
+    __shared__ float redf[4];
+    const int row = blockIdx.x, t = threadIdx.x;
     const float *zr = z + (size_t)row * N;
     float mx = -3.402823466e38f;
-    for (int j = lane; j < N; j += 64) mx = fmaxf(mx, zr[j]);
+    for (int j = t; j < N; j += 256) mx = fmaxf(mx, zr[j]);
     for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if ((t & 63) == 0) redf[t >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
+    double e[SOFTMAX_KEEP];
     double s = 0.0;
-    for (int j = lane; j < N; j += 64) s += exp((double)(zr[j] - mx));
-    s = wave_sum(s);
-    for (int j = lane; j < N; j += 64) sm[(size_t)row * N + j] = (float)(exp((double)(zr[j] - mx)) / s);
-    if (lane == 0) {
+#pragma unroll
+    for (int u = 0; u < SOFTMAX_KEEP; ++u) {
+        const int j = t + 256 * u;
+        e[u] = j < N ? exp((double)(zr[j] - mx)) : 0.0;
+        s += e[u];
+    }
+    for (int j = t + 256 * SOFTMAX_KEEP; j < N; j += 256) s += exp((double)(zr[j] - mx));
+    s = block_sum(s, red);
+#pragma unroll
+    for (int u = 0; u < SOFTMAX_KEEP; ++u) {
+        const int j = t + 256 * u;
+        if (j < N) sm[(size_t)row * N + j] = (float)(e[u] / s);
+    }
+    for (int j = t + 256 * SOFTMAX_KEEP; j < N; j += 256) sm[(size_t)row * N + j] = (float)(exp((double)(zr[j] - mx)) / s);
+    if (t == 0) {
         int64_t l = lab[row];
         double p = (l >= 0 && l < N) ? exp((double)(zr[l] - mx)) / s : 1.0;
         nll[row] = (float)(-log(p));
@@ -766,7 +799,11 @@ int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k
     XSMI_CHECK_ARG(x && y, "xsmi_avgpool_fwd: null pointer");
     int OH = H / k, OW = W / k;
     size_t total = (size_t)N * C * OH * OW;
-    hipLaunchKernelGGL(avgpool_fwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, y, H, W, OH, OW, k, total);
+    if (k == H && k == W && total < 0x7fffffffu)
+        hipLaunchKernelGGL(avgpool_plane_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, xsmi::stream(), x, y, H * W,
+                           (uint32_t)total);
+    else
+        hipLaunchKernelGGL(avgpool_fwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, y, H, W, OH, OW, k, total);
     XSMI_LAUNCH_CHECK("avgpool_fwd_kernel");
     return XSMI_OK;
 }
@@ -838,7 +875,7 @@ int xsmi_softmax_ce_fwd(const float *logits, const int64_t *labels, float *sm, f
     XSMI_CHECK_ARG(M > 0 && N > 0 && logits && labels && sm && loss, "xsmi_softmax_ce_fwd: bad argument");
     hipStream_t st = xsmi::stream();
     // `loss` has room for 1 + M floats: loss[0] is the result, loss[1..M] the per-row terms
-    hipLaunchKernelGGL(softmax_rows_kernel, dim3(M), dim3(64), 0, st, logits, labels, sm, loss + 1, M, N);
+    hipLaunchKernelGGL(softmax_rows_kernel, dim3(M), dim3(256), 0, st, logits, labels, sm, loss + 1, M, N);
     XSMI_LAUNCH_CHECK("softmax_rows_kernel");
     hipLaunchKernelGGL(nll_reduce_kernel, dim3(1), dim3(256), 0, st, loss + 1, loss, M, mean);
     XSMI_LAUNCH_CHECK("nll_reduce_kernel");
