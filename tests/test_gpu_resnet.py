@@ -100,6 +100,43 @@ def test_resnet18_trains_on_device():
     assert np.isfinite(losses).all() and losses[-1] < losses[0]
 
 
+def test_resnet18_steps_do_not_depend_on_the_weight_gradient_overlap(monkeypatch):
+    """Conv layers leave their weight gradients running on the backend's second stream across the backward sweep.
+    Three SGD steps with that overlap and three with every weight gradient joined at once end in the same bits."""
+    from xshinnosuke_amd.backend import kernels as K
+
+    def run(overlap):
+        if not overlap:
+            plain = K.conv2d_bwd
+            monkeypatch.setattr(K, "conv2d_bwd", lambda *a, **kw: plain(*a, **dict(kw, async_dw=False)))
+        np.random.seed(3)
+        X = np.random.randn(8, 3, 64, 64).astype(np.float32)
+        Y = np.random.randint(0, 10, (8,))
+        net = ResNet18(classes=10, pool=2).to('cuda')
+        x, y = xs.tensor(X).to('cuda'), xs.tensor(Y).to('cuda')
+        net(x)
+        xs.GLOBAL.INPUTS = None
+        opt = SGD(net.parameters(), lr=0.05)
+        crit = xs.nn.CrossEntropyLoss()
+        losses = []
+        for _ in range(3):
+            opt.zero_grad()
+            loss = crit(net(x), y)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        out = [p.numpy().copy() for p in _named_params(net)]
+        monkeypatch.undo()
+        xs.GLOBAL.INPUTS = None
+        return losses, out
+
+    la, pa = run(True)
+    lb, pb = run(False)
+    assert la == lb
+    for u, v in zip(pa, pb):
+        np.testing.assert_array_equal(u, v)
+
+
 def _oracle_forward(net, x):
     """ResNet-18 inference (moving-statistics batch norm) in NumPy: convolutions and the max-pool through the
     oracle (float64 GEMM, one rounding), the rest in float64 rounded to float32 per op."""
