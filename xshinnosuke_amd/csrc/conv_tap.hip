@@ -1196,6 +1196,51 @@ __global__ void __launch_bounds__(256) tap_pack_kernel(const float *__restrict__
     }
 }
 
+// The 3x3 stride-1 case of the layout above with wide accesses: a thread takes one row and the four channels of one
+// quad, i.e. 36 floats of w (mode 0: one contiguous run, read as nine float4; mode 1: four runs of nine), and
+// stores one float4 per tap; the lanes of a wavefront are consecutive rows, so every store instruction writes 1 KB
+// of one tap's block.  Twelve times fewer cache-line requests than one float per thread.
+__global__ void __launch_bounds__(64) tap_pack_3x3_kernel(const float *__restrict__ w, float *__restrict__ apk,
+                                                            uint32_t *__restrict__ counters, int mode, int rows, int CH,
+                                                            int rowtiles) {
+    if (blockIdx.x == 0 && threadIdx.x < 8) counters[threadIdx.x] = 0;   // tile counters of the persistent kernel
+    const int nch = CH / KC;
+    const uint32_t i = blockIdx.x * 64u + threadIdx.x;         // one wavefront per block: 64 rows of one quad
+    const int r64 = (int)(i & 63), q = (int)((i >> 6) & 7);
+    const uint32_t cblk = i >> 9;
+    const int cc = (int)(cblk % (uint32_t)nch), rt = (int)(cblk / (uint32_t)nch);
+    const int ch0 = cc * KC + q * 4, row = rt * TM + r64;
+    float v[4][9];
+    if (row < rows) {
+        if (mode == 0) {
+            const float4 *src = reinterpret_cast<const float4 *>(w + ((size_t)row * CH + ch0) * 9);
+            float buf[36];
+#pragma unroll
+            for (int u = 0; u < 9; ++u) *reinterpret_cast<float4 *>(buf + 4 * u) = src[u];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int t = 0; t < 9; ++t) v[e][t] = buf[e * 9 + t];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float *src = w + ((size_t)(ch0 + e) * rows + row) * 9;
+#pragma unroll
+                for (int t = 0; t < 9; ++t) v[e][t] = src[t];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int t = 0; t < 9; ++t) v[e][t] = 0.f;
+    }
+    float *dst = apk + ((size_t)rt * 9 * nch + cc) * (TM * KC) + q * (TM * 4) + r64 * 4;
+#pragma unroll
+    for (int t = 0; t < 9; ++t)
+        *reinterpret_cast<float4 *>(dst + (size_t)t * nch * (TM * KC)) = make_float4(v[0][t], v[1][t], v[2][t], v[3][t]);
+}
+
 // The same filters for tap_bf16_tile_kernel: bf16, [row tile][chunk][group 4][ROWS rows][8 channels], i.e. the
 // LDS image of a stage's A part per (row tile, chunk).
 __global__ void __launch_bounds__(256) tap_pack_bf16_kernel(const float *__restrict__ w, PackMulti pm, int mode, int rows, int CH,
@@ -1323,6 +1368,15 @@ int launch_pack(hipStream_t st, const float *w, const PackSpec *specs, int nspec
     }
     if (pm.njobs == 0) return XSMI_OK;
     pm.first[pm.njobs] = blocks;
+    if (!trows && nspecs == 1 && R == 3 && S == 3 && sh == 1 && sw == 1 && specs[0].TR == 3 && specs[0].TS == 3 &&
+        ((uintptr_t)w & 15) == 0 && (size_t)rows * CH >= 65536) {
+        // whole 3x3 filters of 2.4 MB and more (smaller ones are bound by the launch, not by the gather)
+        const uint32_t nb = (uint32_t)(rowtiles * (CH / KC) * 8);
+        hipLaunchKernelGGL(tap_pack_3x3_kernel, dim3(nb), dim3(64), 0, st, w, pm.job[0].apk, pm.job[0].counters, mode, rows,
+                           CH, rowtiles);
+        XSMI_LAUNCH_CHECK("tap_pack_3x3_kernel");
+        return XSMI_OK;
+    }
     if (trows)
         hipLaunchKernelGGL(tap_pack_bf16_kernel, dim3(blocks), dim3(256), 0, st, w, pm, mode, rows, CH, R, S, sh, sw, rowtiles, trows);
     else
