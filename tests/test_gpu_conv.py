@@ -349,3 +349,38 @@ def test_conv_rejects_bad_arguments(gpu):
         K.conv2d_fwd(x, w)                       # filter larger than the input
     with pytest.raises(ValueError):
         K.conv2d_fwd(x, gpu.zeros((2, 3, 3, 3)), stride=(0, 1))
+
+
+def test_conv_combined_backward_rejects_bad_arguments(gpu):
+    """The C ABI refuses what it cannot run safely: unknown flags, a missing or too small workspace, two workspaces
+    that overlap; the wrappers refuse mismatched buffers before anything is enqueued."""
+    import ctypes
+    from xshinnosuke_amd.backend import capi
+    K = gpu.kernels
+    x = gpu.zeros((2, 64, 8, 8)); w = gpu.zeros((64, 64, 3, 3)); dy = gpu.zeros((2, 64, 8, 8))
+    dx = gpu.zeros(x.shape); dw = gpu.zeros(w.shape)
+    dims = [2, 64, 8, 8, 64, 3, 3, 1, 1, 1]
+    need = capi.lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
+    ws = gpu.empty((2 * need // 4 + 64,))
+    base = ws.cptr.value
+    a, b = ctypes.c_void_p(base), ctypes.c_void_p(base + (need + 255) // 256 * 256)
+    args = [dy.cptr, x.cptr, w.cptr, dx.cptr, dw.cptr, None] + dims + [0.0, 0.0]
+    capi.lib.call("xsmi_conv2d_bwd", *args, 0, a, need, b, need)                 # the well-formed call
+    with pytest.raises(ValueError, match="unknown flags"):
+        capi.lib.call("xsmi_conv2d_bwd", *args, 0x40, a, need, b, need)
+    with pytest.raises(ValueError, match="workspace"):
+        capi.lib.call("xsmi_conv2d_bwd", *args, 0, a, need, None, 0)
+    with pytest.raises(ValueError, match="workspace"):
+        capi.lib.call("xsmi_conv2d_bwd", *args, 0, a, 16, b, need)
+    with pytest.raises(ValueError, match="overlap"):
+        capi.lib.call("xsmi_conv2d_bwd", *args, 0, a, need, ctypes.c_void_p(base + 256), need)
+    with pytest.raises(ValueError, match="beta"):
+        capi.lib.call("xsmi_conv2d_bwd", *(args[:-2] + [0.5, 0.0]), 0, a, need, b, need)
+    with pytest.raises(ValueError):
+        K.conv2d_bwd(dy, x, w, gpu.zeros((2, 64, 8, 9)), dw)                      # dx of another shape
+    with pytest.raises(ValueError):
+        K.conv2d_bwd(gpu.zeros((2, 64, 7, 8)), x, w, dx, dw)                      # dy of another shape
+    with pytest.raises(ValueError):
+        K.relu_mask_bwd2(dy, gpu.zeros(dy.shape, np.uint8), dx, dx)               # one buffer given twice
+    gpu.synchronize()
+    assert not capi.side_pending()
