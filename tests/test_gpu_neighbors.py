@@ -8,7 +8,9 @@ from util import rel_l2
 pytestmark = pytest.mark.gpu
 
 
-@pytest.mark.parametrize("shape", [(4, 8, 6, 6), (32, 64, 14, 14), (5, 3, 7, 7), (2, 130, 9, 5), (64, 16)])
+# per channel up to 8192 elements: one kernel does both passes; beyond: partial sums + apply (float4 or scalar form)
+@pytest.mark.parametrize("shape", [(4, 8, 6, 6), (32, 64, 14, 14), (5, 3, 7, 7), (2, 130, 9, 5), (64, 16),
+                                   (8, 16, 40, 40), (6, 5, 37, 41), (32, 8, 16, 16), (33, 4, 16, 16)])
 def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     """xs/nn/functional.py:676-707 and xs/nn/grad_fn.py:379-411."""
     K = gpu.kernels

@@ -411,6 +411,95 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
     }
 }
 
+// Small layers (a channel's N*HW elements fit a workgroup's registers): both passes in one kernel, one workgroup
+// per channel.  The elements are read once, summed in float64 (fixed order: per thread in element order, then
+// block_sum), normalised from the registers and written; a launch and a read of the tensor less than the two-kernel
+// form, which matters where a launch costs as much as the data movement (14x14 and 7x7 feature maps).
+constexpr int BN_SMALL_PER = 32;                      // elements per thread kept in registers
+constexpr int BN_SMALL_MAX = 256 * BN_SMALL_PER;      // 8192 elements per channel
+__device__ __forceinline__ size_t bn_small_off(uint32_t e, int c, int C, int HW, const xsmi::FastDiv &dHW) {
+    const uint32_t j = xsmi::fdiv(e, dHW), i = e - j * (uint32_t)HW;
+    return ((size_t)j * C + c) * (size_t)HW + i;
+}
+__global__ void __launch_bounds__(256) bn_fwd_small_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                            const float *__restrict__ beta, double m, float eps, float momentum,
+                                                            BnFwdOut o, int C, int HW, xsmi::FastDiv dHW, uint32_t total) {
+    __shared__ double sm[4];
+    const int c = blockIdx.x;
+    float v[BN_SMALL_PER];
+    double s0 = 0.0, s1 = 0.0;
+#pragma unroll
+    for (int u = 0; u < BN_SMALL_PER; ++u) {
+        const uint32_t e = threadIdx.x + 256u * u;
+        v[u] = e < total ? x[bn_small_off(e, c, C, HW, dHW)] : 0.f;
+        s0 += (double)v[u];
+        s1 += (double)v[u] * (double)v[u];
+    }
+    s0 = block_sum(s0, sm);
+    s1 = block_sum(s1, sm);
+    const double mu_d = s0 / m;
+    double var = s1 / m - mu_d * mu_d;
+    if (var < 0.0) var = 0.0;
+    const float mu = (float)mu_d, rs = (float)sqrt(var + (double)eps), g = gamma[c], bt = beta[c];
+    if (threadIdx.x == 0) {
+        o.mean[c] = mu;
+        o.var[c] = (float)var;
+        o.sqrtvar[c] = rs;
+        if (o.moving_mean) {
+            o.moving_mean[c] = momentum * o.moving_mean[c] + (1.f - momentum) * mu;
+            o.moving_var[c] = momentum * o.moving_var[c] + (1.f - momentum) * (float)var;
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < BN_SMALL_PER; ++u) {
+        const uint32_t e = threadIdx.x + 256u * u;
+        if (e >= total) break;
+        const size_t off = bn_small_off(e, c, C, HW, dHW);
+        const float hv = (v[u] - mu) / rs;
+        const float pre = g * hv + bt;
+        if (o.xhat) o.xhat[off] = hv;
+        o.y[off] = (o.neg_mask && pre < 0.f) ? 0.f : pre;
+        if (o.neg_mask) o.neg_mask[off] = pre < 0.f ? 1 : 0;
+    }
+}
+__global__ void __launch_bounds__(256) bn_bwd_small_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
+                                                            const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
+                                                            float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                            const uint8_t *__restrict__ zero, float *__restrict__ dx, float m,
+                                                            const float *__restrict__ mean, int C, int HW, xsmi::FastDiv dHW,
+                                                            uint32_t total) {
+    __shared__ double sm[4];
+    const int c = blockIdx.x;
+    const float rs = sqrtvar[c], mu = mean ? mean[c] : 0.f, g = gamma[c], den = m * rs;
+    float d[BN_SMALL_PER], h[BN_SMALL_PER];
+    double s0 = 0.0, s1 = 0.0;
+#pragma unroll
+    for (int u = 0; u < BN_SMALL_PER; ++u) {
+        const uint32_t e = threadIdx.x + 256u * u;
+        d[u] = 0.f; h[u] = 0.f;
+        if (e < total) {
+            const size_t off = bn_small_off(e, c, C, HW, dHW);
+            d[u] = (zero && zero[off]) ? 0.f : dy[off];
+            h[u] = mean ? (xhat[off] - mu) / rs : xhat[off];
+        }
+        s0 += (double)d[u];
+        s1 += (double)d[u] * (double)h[u];
+    }
+    s0 = block_sum(s0, sm);
+    s1 = block_sum(s1, sm);
+    const float db = (float)s0, dg = (float)s1;
+    if (threadIdx.x == 0) {
+        dbeta[c] = db;
+        dgamma[c] = dg;
+    }
+#pragma unroll
+    for (int u = 0; u < BN_SMALL_PER; ++u) {
+        const uint32_t e = threadIdx.x + 256u * u;
+        if (e >= total) break;
+        dx[bn_small_off(e, c, C, HW, dHW)] = g * (m * d[u] - db - h[u] * dg) / den;
+    }
+}
+
 template <bool VEC>
 __global__ void __launch_bounds__(256) bn_infer_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                         const float *__restrict__ beta, const float *__restrict__ mean,
@@ -720,6 +809,13 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     XSMI_CHECK_ARG((moving_mean == nullptr) == (moving_var == nullptr), "xsmi_bn_fwd: give both moving statistics or neither");
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
     hipStream_t st = xsmi::stream();
+    if ((size_t)N * HW <= (size_t)BN_SMALL_MAX) {
+        const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask};
+        hipLaunchKernelGGL(bn_fwd_small_kernel, dim3(C), dim3(256), 0, st, x, gamma, beta, (double)N * HW, eps, momentum, o, C,
+                           HW, xsmi::make_fastdiv(HW), (uint32_t)(N * HW));
+        XSMI_LAUNCH_CHECK("bn_fwd_small_kernel");
+        return XSMI_OK;
+    }
     double *part = (double *)ws;
     const BnSplit split = bn_split(N, HW, (HW & 3) == 0 && aligned16(x));
     const int nsplit = split.nsplit;
@@ -775,6 +871,12 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
     XSMI_CHECK_ARG(dy && xhat && sqrtvar && gamma && dx && dgamma && dbeta, "xsmi_bn_bwd: null pointer");
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd: workspace too small");
     hipStream_t st = xsmi::stream();
+    if ((size_t)N * HW <= (size_t)BN_SMALL_MAX) {
+        hipLaunchKernelGGL(bn_bwd_small_kernel, dim3(C), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, neg_mask, dx,
+                           (float)((double)N * HW), mean, C, HW, xsmi::make_fastdiv(HW), (uint32_t)(N * HW));
+        XSMI_LAUNCH_CHECK("bn_bwd_small_kernel");
+        return XSMI_OK;
+    }
     double *part = (double *)ws;
     const BnSplit split = bn_split(N, HW, (HW & 3) == 0 && aligned16(dy) && aligned16(xhat) &&
                                               (!neg_mask || ((uintptr_t)neg_mask & 3) == 0));
