@@ -367,6 +367,37 @@ def test_inference_folds_batch_norm_into_the_convolution(gpu):
         assert net._graph[0].data is net._graph[1].data is net._graph[2].data
         assert net._graph[3].data is net._graph[4].data is folded
         assert folded.grad_fn is None and not folded.requires_grad
+        # The folded and packed filters are kept while the parameters are untouched: the next forward launches no
+        # fold, and the same values come out for another (smaller) batch; a changed statistic, scale or filter is seen.
+        from xshinnosuke_amd.backend import capi
+        calls = []
+        real = capi.lib.call
+        capi.lib.call = lambda name, *a: (calls.append(name), real(name, *a))[1]
+        try:
+            with xs.no_grad():
+                again = net(x).numpy()
+        finally:
+            capi.lib.call = real
+        assert "xsmi_bn_fold" not in calls and calls.count("xsmi_conv2d_fwd") == 2
+        np.testing.assert_array_equal(again, folded.numpy())
+        x2 = xs.tensor(x.numpy()[:2]).to('cuda')
+        with xs.no_grad():
+            part = net(x2).numpy()
+        np.testing.assert_array_equal(part, again[:2])
+        conv2, bn2 = net._graph[3], net._graph[4]
+        for change in ("mean", "gamma", "filter", "bf16"):
+            if change == "mean":
+                bn2.moving_mean.eval = gpu.to_device(rng.standard_normal(6).astype(np.float32))
+            elif change == "gamma":
+                K.scale(bn2._parameters[0].eval, 2.0, out=bn2._parameters[0].eval)      # in place, through a kernel
+            elif change == "filter":
+                conv2._parameters[0].eval.fill_zero(lazy=True)                          # only a pending clear
+            with xs.conv_precision('bf16' if change == "bf16" else 'fp32'), xs.no_grad():
+                out = net(x).numpy()                 # first: nothing else has looked at the parameters since the change
+            plain = net(x).numpy()
+            assert rel_l2(out, plain) <= (1e-2 if change == "bf16" else 1e-5), change
+            if change == "filter":
+                assert np.abs(plain).max() > 0 and np.array_equal(out[:, :, 0, 0], out[:, :, 1, 1])   # bias only
     finally:
         xs.GLOBAL.TRAINING = True
         xs.GLOBAL.USE_CUDA = False

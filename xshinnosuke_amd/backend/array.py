@@ -36,12 +36,13 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version")
 
     def __init__(self, nbytes):
         ensure_init()
         self.logical = int(nbytes)
         self.lazy_zero = False
+        self.version = 0                     # counts every hand-out of the address and every pending clear
         size = _round_size(nbytes)
         free = _POOL.get(size)
         if free:
@@ -101,10 +102,17 @@ class DeviceArray:
     @property
     def ptr(self):
         blk = self._block
+        blk.version += 1                     # whoever takes the address may write through it
         if blk.lazy_zero:                    # logically zero, memory not cleared yet: clear it on first use
             blk.lazy_zero = False
             lib.call("xsmi_memset", ctypes.c_void_p(blk.ptr), 0, blk.nbytes)
         return blk.ptr + self._offset
+
+    def state(self):
+        """(allocation, version): equal to an earlier value exactly when the address has not been handed out (to a
+        kernel, a copy, the host) and no clear was scheduled since, i.e. the contents cannot have changed.  Lets
+        results derived from an array (a packed or folded filter) be kept for the next call."""
+        return id(self._block), self._block.version
 
     def address(self):
         """The device address as an integer; unlike ``ptr`` it leaves a pending clear pending (for alignment and
@@ -190,6 +198,7 @@ class DeviceArray:
         blk = self._block
         if lazy and self._offset == 0 and self.nbytes >= blk.logical:
             blk.lazy_zero = True
+            blk.version += 1
             return self
         if self.nbytes:
             lib.call("xsmi_memset", self.cptr, 0, self.nbytes)

@@ -30,6 +30,11 @@ def _dims(x_shape, w_shape, stride, pad):
     return [int(v) for v in (n, c, h, w, k, r, s, stride[0], stride[1], pad)]
 
 
+def conv2d_workspace_bytes(x_shape, w_shape, stride, pad):
+    """Bytes of workspace the conv entry points want for this geometry."""
+    return lib.raw("xsmi_conv2d_workspace_bytes")(*_dims(x_shape, w_shape, stride, pad))
+
+
 def _workspace(dims):
     need = lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
     return _ws.get(need)
@@ -41,9 +46,11 @@ def _f32(a, what):
     return a
 
 
-def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False, packed=False):
-    """``packed=True`` promises that the previous conv call was this same forward with the same geometry and
-    filter values (the shared workspace still holds the filter's packed form), so it is not laid out again."""
+def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False, packed=False,
+               workspace=None):
+    """``packed=True`` promises that the previous conv call on this workspace was this same forward with the same
+    geometry and filter values (the workspace still holds the filter's packed form), so it is not laid out again.
+    ``workspace``: a ``Workspace`` of the caller's instead of the shared one (a layer that keeps its packed filter)."""
     _f32(x, "x"); _f32(w, "w")
     dims = _dims(x.shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -61,7 +68,7 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
     if neg_mask is not None and (neg_mask.dtype != np.uint8 or neg_mask.size != out.size):
         raise ValueError("conv2d: neg_mask must be uint8 with one byte per output element")
     flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0)
-    ws, ws_bytes = _workspace(dims)
+    ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(lib.raw("xsmi_conv2d_workspace_bytes")(*dims))
     lib.call("xsmi_conv2d_fwd", x.cptr, w.cptr, bias.cptr if bias is not None else None, out.cptr,
              neg_mask.cptr if neg_mask is not None else None, *dims, flags, ws, ws_bytes)
     return out

@@ -118,11 +118,34 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
         raise ValueError('conv2d expects NCHW input and KCRS weight, got %s and %s' % (x.shape, weight.shape))
     stride = _pair(stride)
     padding = int(padding)
-    stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]
-    b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
-    w2, b2 = K.bn_fold(_f32_device(weight.eval), b_dev, *stats, epsilon)
     dst = out.eval if (out is not None and is_device(out.eval)) else None
-    y = K.conv2d_fwd(_f32_device(x), w2, b2, stride, padding, relu=activation == 'relu', out=dst, bf16=bool(GLOBAL.CONV_BF16))
+    bf16 = bool(GLOBAL.CONV_BF16)
+    relu = activation == 'relu'
+    sources = [t.eval for t in (weight, bias, gamma, beta, moving_mean, moving_variance) if t is not None]
+    kept = getattr(weight, '_folded_filter', None)
+    x = _f32_device(x)
+    if all(is_device(a) and a.dtype == np.float32 for a in sources):
+        # Frozen parameters: the folded filter, its bias and its packed form (in a workspace of this filter's own) are
+        # kept while nobody has taken the address of a parameter since they were made (DeviceArray.state).
+        now = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape[1:]))
+        need = K.conv2d_workspace_bytes(x.shape, weight.shape, stride, padding)
+        if kept is not None and kept['key'] == now and kept['ws'].holds(need):
+            y = K.conv2d_fwd(x, kept['w'], kept['b'], stride, padding, relu=relu, out=dst, bf16=bf16, packed=True,
+                             workspace=kept['ws'])
+        else:
+            stats = [a.reshape(-1) for a in sources[-4:]]
+            b_dev = None if bias is None else bias.eval.reshape(-1)
+            w2, b2 = K.bn_fold(weight.eval, b_dev, *stats, epsilon)
+            ws = kept['ws'] if kept is not None else K.Workspace()
+            y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, workspace=ws)
+            # the fold has read the parameters: their state as of now is what the kept filter belongs to
+            key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape[1:]))
+            weight._folded_filter = {'key': key, 'w': w2, 'b': b2, 'ws': ws, 'of': sources}   # 'of' keeps the ids in the key alive
+    else:
+        stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]
+        b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
+        w2, b2 = K.bn_fold(_f32_device(weight.eval), b_dev, *stats, epsilon)
+        y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16)
     if out is None:
         out = Tensor(y)
     elif y is not dst:
