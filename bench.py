@@ -30,6 +30,7 @@ import numpy as np
 
 ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
+sys.path.insert(1, os.path.join(ROOT, "tests"))      # the ResNet-18 workload (tests/resnet18.py) is a caller of the package
 
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
@@ -174,7 +175,7 @@ def bench_resnet18(be, steps, warmup):
     """ResNet-18 (BasicBlock [2,2,2,2], 7x7/2 stem, 3x3/2 max-pool, global avg pool, FC 1000) fwd+bwd+SGD through the
     layer API on device-resident tensors: N=32x3x224x224 fp32, He-normal weights, random labels."""
     import xshinnosuke_amd as xs
-    from xshinnosuke_amd.utils.resnet import ResNet18
+    from resnet18 import ResNet18
     from xshinnosuke_amd.optim import SGD
     np.random.seed(6)
     x = xs.tensor(np.random.default_rng(6).standard_normal((32, 3, 224, 224), dtype=np.float32)).to('cuda')
@@ -216,7 +217,7 @@ def bench_resnet18_infer(be, steps, warmup):
     """ResNet-18 N=256 forward only, moving-statistics BN, convolutions allowed to use bf16 MFMA operands; the fp32
     forward of the same weights and input runs beside it and gives the logits' relative L2 distance."""
     import xshinnosuke_amd as xs
-    from xshinnosuke_amd.utils.resnet import ResNet18
+    from resnet18 import ResNet18
     xs.GLOBAL.INPUTS = None
     X = np.random.default_rng(7).standard_normal((256, 3, 224, 224), dtype=np.float32)
     x = xs.tensor(X).to('cuda')

@@ -229,6 +229,12 @@ int xsmi_relu_fwd(const float *x, float *y, size_t n);
 int xsmi_relu_fwd_mask(const float *x, float *y, uint8_t *neg_mask, size_t n);
 /* dx[i] = pre[i] < 0 ? 0 : dy[i]         (strict mask, xs/nn/grad_fn.py:146-157); dx may alias dy */
 int xsmi_relu_bwd(const float *dy, const float *pre, float *dx, size_t n);
+/* y = 1 / (1 + exp(-x)) for kind 1, tanh(x) for kind 2 (may be in place): the other two activations a layer's
+ * `activation=` argument names (xs/nn/td_functional.py:63-70, xs/layers/activators.py:62-87) */
+int xsmi_act_fwd(const float *x, float *y, size_t n, int kind);
+/* dx = dy * y * (1 - y) for kind 1, dy * (1 - y^2) for kind 2, y being the forward's output
+ * (xs/nn/grad_fn.py:161-170); dx may alias dy */
+int xsmi_act_bwd(const float *dy, const float *y, float *dx, size_t n, int kind);
 /* m[i] = momentum * m[i] + (1 - momentum) * cur[i]   (moving statistics, xs/nn/functional.py:700-707) */
 int xsmi_lerp(float *m, const float *cur, float momentum, size_t n);
 

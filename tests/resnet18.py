@@ -4,8 +4,8 @@
 ``pool`` and ``classes`` choose the tail: the reference script uses AvgPooling2D(2) and 100 classes on 56x56
 inputs; the 224x224 benchmark configuration uses a global 7x7 average pool and 1000 classes.
 """
-from ..layers import Conv2D, BatchNormalization, ReLU, MaxPooling2D, AvgPooling2D, Flatten, Dense
-from ..nn.models import Module, Sequential
+from xshinnosuke_amd.layers import Conv2D, BatchNormalization, ReLU, MaxPooling2D, AvgPooling2D, Flatten, Dense
+from xshinnosuke_amd.nn.models import Module, Sequential
 
 
 class BasicBlock(Module):

@@ -300,6 +300,33 @@ def test_device_fit_matches_host_fit_batch_for_batch():
         xs.GLOBAL.USE_CUDA = False
 
 
+def test_device_fit_allocates_nothing_in_the_steady_state():
+    """Static graph on the device: from the third step on, a training step calls neither the device allocator
+    nor the pinned-memory allocator (blocks come from the size-keyed pool, layer outputs are preallocated)."""
+    from xshinnosuke_amd.backend import capi
+    rng = np.random.default_rng(15)
+    x = rng.standard_normal((96, 1, 12, 12)).astype(np.float32)
+    labels = rng.integers(0, 4, size=96)
+    np.random.seed(5)
+    xs.GLOBAL.USE_CUDA = True
+    calls = []
+    real = capi.lib.call
+    try:
+        m = _small_cnn(); m.compile(SGD(lr=0.05), 'cross_entropy')
+        capi.lib.call = lambda name, *a: (calls.append(name), real(name, *a))[1]
+        m.fit(x, labels, batch_size=16, epochs=1, verbose=0, shuffle=False)       # six steps of 16
+    finally:
+        capi.lib.call = real
+        xs.GLOBAL.USE_CUDA = False
+    steps = [i for i, name in enumerate(calls) if name == "xsmi_axpy_multi"]       # one optimizer step each
+    assert len(steps) == 6
+    steady = calls[steps[1] + 1:steps[5] + 1]                                       # steps 3..6
+    assert "xsmi_conv2d_fwd" in steady and "xsmi_conv2d_bwd_weight" in steady or "xsmi_conv2d_bwd" in steady
+    for name in ("xsmi_malloc", "xsmi_free", "xsmi_host_alloc", "xsmi_host_free"):
+        assert name not in steady, (name, steady.count(name))
+    assert "xsmi_malloc" in calls[:steps[0]]                                       # the counter does see allocations
+
+
 def test_checkpoint_round_trip_from_the_device(tmp_path):
     """save() writes host arrays; load() puts them back on the device; predictions and the next epoch agree."""
     rng = np.random.default_rng(6)
@@ -322,6 +349,35 @@ def test_checkpoint_round_trip_from_the_device(tmp_path):
         h2 = m2.fit(x, labels, batch_size=16, epochs=1, verbose=0, shuffle=False)
         np.testing.assert_allclose(h2['train_loss'], h1['train_loss'], rtol=1e-6)
     finally:
+        xs.GLOBAL.USE_CUDA = False
+
+
+def test_checkpoint_of_a_conv_batch_norm_model_after_inference(tmp_path):
+    """fit with validation and predict run the folded Conv2D -> BatchNormalization inference path, which keeps
+    folded filters between forwards; a checkpoint written afterwards holds parameters only, and the loaded
+    model predicts the same values."""
+    from xshinnosuke_amd.layers import BatchNormalization
+    rng = np.random.default_rng(16)
+    x = rng.standard_normal((48, 2, 10, 10)).astype(np.float32)
+    labels = rng.integers(0, 3, size=48)
+    np.random.seed(9)
+    xs.GLOBAL.USE_CUDA = True
+    try:
+        m = Sequential(Conv2D(6, 3, padding=1, input_shape=(2, 10, 10)), BatchNormalization(), ReLU(True),
+                       MaxPooling2D(2), Flatten(), Dense(3))
+        m.compile(SGD(lr=0.05), 'cross_entropy')
+        m.fit(x, labels, batch_size=16, epochs=2, verbose=0, validation_data=(x[:16], labels[:16]))
+        p1 = m.predict(x).numpy()
+        m.save(str(tmp_path / 'ckbn'))
+        raw = open(str(tmp_path / 'ckbn.pkl'), 'rb').read()
+        assert b'_Block' not in raw and b'Workspace' not in raw and b'_folded_filter' not in raw
+        m2 = Sequential(); m2.load(str(tmp_path / 'ckbn'))
+        assert m2._device == 'cuda'
+        p2 = m2.predict(x).numpy()
+        np.testing.assert_array_equal(p2, p1)
+        np.testing.assert_array_equal(m.predict(x).numpy(), p1)      # the saved model still works, too
+    finally:
+        xs.GLOBAL.TRAINING = True
         xs.GLOBAL.USE_CUDA = False
 
 

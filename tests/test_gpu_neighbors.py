@@ -218,3 +218,56 @@ def test_average_pool_blocks(gpu, n, c, h, w, k):
     dref = np.zeros_like(x)
     dref[:, :, :oh * k, :ow * k] = np.repeat(np.repeat(dy, k, axis=2), k, axis=3) / np.float32(k * k)
     np.testing.assert_allclose(dx, dref, rtol=1e-6, atol=0)
+
+
+@pytest.mark.parametrize("kind", ["sigmoid", "tanh"])
+@pytest.mark.parametrize("n", [1, 7, 4096, 100003])
+def test_sigmoid_and_tanh_kernels(gpu, kind, n):
+    """xs/nn/td_functional.py:63-70 and xs/nn/grad_fn.py:161-170, float32 kernels against float64 formulas."""
+    K = gpu.kernels
+    rng = np.random.default_rng(n)
+    x = (rng.standard_normal(n) * 3).astype(np.float32)
+    dy = rng.standard_normal(n).astype(np.float32)
+    x64 = x.astype(np.float64)
+    y_ref = 1 / (1 + np.exp(-x64)) if kind == "sigmoid" else np.tanh(x64)
+    y = K.act_fwd(gpu.to_device(x), kind)
+    np.testing.assert_allclose(y.numpy(), y_ref, rtol=2e-6, atol=1e-7)
+    y32 = y.numpy().astype(np.float64)
+    dx_ref = dy * y32 * (1 - y32) if kind == "sigmoid" else dy * (1 - y32 * y32)
+    dx = K.act_bwd(gpu.to_device(dy), y, kind)
+    np.testing.assert_allclose(dx.numpy(), dx_ref, rtol=2e-6, atol=1e-7)
+
+
+def test_conv2d_layer_with_a_named_activation(gpu):
+    """Conv2D(activation='tanh' | 'sigmoid') appends the named activation to the convolution (reference
+    xs/layers/convolutional.py:16,76-77): values and gradients of a dynamic forward / backward on the device
+    against the oracle convolution followed by the closed form."""
+    import oracle
+    import xshinnosuke_amd as xs
+    from xshinnosuke_amd.layers import Conv2D
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((3, 4, 9, 9)).astype(np.float32)
+    up = rng.standard_normal((3, 6, 9, 9)).astype(np.float32)
+    try:
+        for name in ("tanh", "sigmoid"):
+            xs.GLOBAL.INPUTS = None
+            xs.GLOBAL.USE_CUDA = True
+            layer = Conv2D(6, 3, padding=1, activation=name)
+            xt = xs.tensor(x, requires_grad=True).to('cuda')
+            xt.retain_grad(True)
+            out = layer(xt)
+            w, b = (p.numpy() for p in layer.parameters())
+            pre, col = oracle.conv2d_fwd(x, w.astype(np.float32), b.reshape(-1).astype(np.float32), (1, 1), 1)
+            act = np.tanh(pre.astype(np.float64)) if name == "tanh" else 1 / (1 + np.exp(-pre.astype(np.float64)))
+            assert out.device == 'cuda' and rel_l2(out.numpy(), act) <= 1e-5
+            assert layer.data is out
+            out.backward(xs.tensor(up).to('cuda'))
+            dpre = up * ((1 - act ** 2) if name == "tanh" else act * (1 - act))
+            dx, dw, db = oracle.conv2d_bwd(dpre.astype(np.float32), x.shape, w.astype(np.float32), col, (1, 1), 1,
+                                           np.zeros_like(x), np.zeros(w.shape, np.float32), np.zeros(6, np.float32))
+            assert rel_l2(xt.grad.numpy(), dx) <= 1e-5
+            assert rel_l2(layer.parameters()[0].grad.numpy(), dw) <= 1e-5
+            assert rel_l2(layer.parameters()[1].grad.numpy().reshape(-1), db) <= 1e-5
+    finally:
+        xs.GLOBAL.INPUTS = None
+        xs.GLOBAL.USE_CUDA = False

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import xshinnosuke_amd as xs
-from xshinnosuke_amd.utils.resnet import ResNet18
+from resnet18 import ResNet18
 from xshinnosuke_amd.optim import SGD
 from util import rel_l2
 

@@ -4,7 +4,7 @@ import math
 
 import numpy as np
 
-from .capi import lib, ensure_init
+from .capi import lib, ensure_init, XsmiError
 
 
 _DTYPE_CLASS = np.dtype(np.float32).__class__
@@ -58,6 +58,10 @@ class _Block:
             self.ptr = p.value
         self.nbytes = size
 
+    def __reduce__(self):
+        # a device address means nothing in another process; arrays pickle as host copies (DeviceArray.__reduce__)
+        raise TypeError("a device memory block cannot be pickled")
+
     def __del__(self):
         try:
             if self.ptr:
@@ -73,11 +77,13 @@ class _Block:
 
 def _rebuild_array(host):
     """Unpickling side of DeviceArray.__reduce__: back onto the device when one can be used, else the
-    host array itself (tensors then simply live on the host)."""
+    host array itself (tensors then simply live on the host).  Only "no library / no gfx950 device" selects
+    the host: a failed allocation or copy is an error, not a reason to scatter a model over two places."""
     try:
-        return to_device(host, host.dtype)
-    except Exception:
+        ensure_init()
+    except (XsmiError, ValueError):              # library missing, no device, or device 0 out of range
         return host
+    return to_device(host, host.dtype)
 
 
 class DeviceArray:
@@ -278,6 +284,9 @@ class Workspace:
 
     def __init__(self):
         self._block = None
+
+    def __reduce__(self):
+        raise TypeError("a device workspace cannot be pickled")
 
     def holds(self, nbytes):
         """True if ``get(nbytes)`` would hand out the present block (no reallocation)."""

@@ -75,6 +75,8 @@ SIGNATURES = {
     "xsmi_relu_fwd": (_i, [_vp, _vp, _sz]),
     "xsmi_relu_fwd_mask": (_i, [_vp, _vp, _vp, _sz]),
     "xsmi_relu_bwd": (_i, [_vp, _vp, _vp, _sz]),
+    "xsmi_act_fwd": (_i, [_vp, _vp, _sz, _i]),
+    "xsmi_act_bwd": (_i, [_vp, _vp, _vp, _sz, _i]),
     "xsmi_lerp": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_bn_workspace_bytes": (_sz, [_i]),
     "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
@@ -123,6 +125,10 @@ class _Lib:
         return dll
 
     def raw(self, name):
+        """The bare ctypes function of a query that enqueues nothing and touches no device memory.  Everything
+        else must go through ``call``, which is where a held-back add is enqueued and the second stream joined."""
+        if name not in _QUERIES:
+            raise XsmiError("%s launches work: call it through lib.call" % name)
         return getattr(self._open(), name)
 
     def call(self, name, *args):
@@ -139,6 +145,8 @@ class _Lib:
                 raise ValueError(msg)
             raise XsmiError(msg)
 
+
+_QUERIES = frozenset(("xsmi_conv2d_workspace_bytes", "xsmi_bn_workspace_bytes", "xsmi_is_initialized", "xsmi_last_error"))
 
 lib = _Lib()
 

@@ -320,6 +320,27 @@ def relu_bwd(dy, pre, dx=None):
     return dx
 
 
+ACT_KINDS = {'sigmoid': 1, 'tanh': 2}
+
+
+def act_fwd(x, kind, out=None):
+    """sigmoid or tanh of x (``out`` may be x)."""
+    _f32(x, "x")
+    out = _like(x, out)
+    lib.call("xsmi_act_fwd", x.cptr, out.cptr, x.size, ACT_KINDS[kind])
+    return out
+
+
+def act_bwd(dy, y, kind, dx=None):
+    """Gradient of sigmoid / tanh through the forward's output y."""
+    _f32(dy, "dy"); _f32(y, "y")
+    if y.size != dy.size:
+        raise ValueError("act_bwd: %s vs %s" % (dy.shape, y.shape))
+    dx = _like(dy, dx)
+    lib.call("xsmi_act_bwd", dy.cptr, y.cptr, dx.cptr, dy.size, ACT_KINDS[kind])
+    return dx
+
+
 def lerp_(m, cur, momentum):
     """m = momentum*m + (1-momentum)*cur"""
     lib.call("xsmi_lerp", m.cptr, cur.cptr, float(momentum), m.size)

@@ -7,6 +7,8 @@ either a ``numpy.ndarray`` (host) or a :class:`DeviceArray` (MI355X HBM); the
 static graph re-uses one preallocated buffer for a shorter last batch
 (xs/layers/base.py:88-104).
 """
+import weakref
+
 import numpy as np
 
 from . import state as GLOBAL
@@ -160,7 +162,18 @@ class Tensor(object):
 
     @property
     def out_bounds(self):
-        return self._out_bounds
+        """The tensors computed from this one that are still alive.  The links are weak: a tensor that outlives a
+        training loop (a loader's batch tensor, a static layer output feeding the loss) must not keep every
+        result ever derived from it, and that result's device memory, alive."""
+        live = [t for t in (r() for r in self._out_bounds) if t is not None]
+        if len(live) != len(self._out_bounds):
+            self._out_bounds = [weakref.ref(t) for t in live]
+        return live
+
+    def __getstate__(self):
+        state = dict(self.__dict__)
+        state['_out_bounds'] = []                # weak links are rebuilt by the next forward
+        return state
 
     def add_in_bounds(self, *ins):
         for i in ins:
@@ -171,10 +184,14 @@ class Tensor(object):
 
     def add_out_bounds(self, *outs):
         for o in outs:
-            if isinstance(o, Tensor):
-                self._out_bounds.append(o)
-            else:
+            if not isinstance(o, Tensor):
                 raise TypeError('Not a Tensor')
+            refs = self._out_bounds
+            if refs and refs[-1]() is o:         # a reused output tensor, wired again by the next forward
+                continue
+            if len(refs) >= 32:
+                refs[:] = [r for r in refs if r() is not None]
+            refs.append(weakref.ref(o))
 
     def requires_grad_(self, flag):
         self.requires_grad = flag

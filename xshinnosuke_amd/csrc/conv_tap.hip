@@ -863,12 +863,13 @@ __global__ void __launch_bounds__(256) nhwc_pad_bf16_kernel(const float *__restr
 }
 
 // The same copy for at most 4 channels (CP = 4): a thread converts one padded pixel, reads and writes are
-// both runs of consecutive pixels, no LDS.  blockIdx.y = n * Hp + hp.
+// both runs of consecutive pixels, no LDS.  Block b serves columns 256 * (b % nwb) .. of padded row b / nwb
+// (= n * Hp + hp); the grid is one-dimensional so that the row count is not bound by the 65535 limit of grid.y.
 __global__ void __launch_bounds__(256) nhwc_pad_c4_kernel(const float *__restrict__ x, __bf16 *__restrict__ xp, int C, int H,
-                                                           int W, int pad, int Hp, int Wp) {
-    const int wp = blockIdx.x * 256 + threadIdx.x;
+                                                           int W, int pad, int Hp, int Wp, int nwb) {
+    const int rowid = (int)(blockIdx.x / (uint32_t)nwb);
+    const int wp = (int)(blockIdx.x - (uint32_t)rowid * (uint32_t)nwb) * 256 + threadIdx.x;
     if (wp >= Wp) return;
-    const int rowid = blockIdx.y;
     const int hp = rowid % Hp, n = rowid / Hp;
     const int ih = hp - pad, iw = wp - pad;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
@@ -1479,8 +1480,9 @@ int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
     }
     prof_begin();
     if (CP == 4) {
-        hipLaunchKernelGGL(nhwc_pad_c4_kernel, dim3((unsigned)ceil_div(Wp, 256), (unsigned)(N * Hp)), dim3(256), 0, st, x, xp, C, H,
-                           W, pad, Hp, Wp);
+        const int nwb = ceil_div(Wp, 256);
+        hipLaunchKernelGGL(nhwc_pad_c4_kernel, dim3((unsigned)nwb * (unsigned)(N * Hp)), dim3(256), 0, st, x, xp, C, H,
+                           W, pad, Hp, Wp, nwb);
         XSMI_LAUNCH_CHECK("nhwc_pad_c4_kernel");
     } else {
         // a workgroup converts WS pixels of one padded row through an LDS tile of C x (WS | 1) floats (<= 32 KB)

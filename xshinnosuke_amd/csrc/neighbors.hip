@@ -106,6 +106,25 @@ struct ReluBwdF {
                                                         p.w < 0.f ? 0.f : g.w);
     }
 };
+// sigmoid (kind 1) and tanh (kind 2), forward and the backward written in terms of the forward's output y
+struct ActF {
+    const float *x; float *y; int kind;
+    __device__ float f(float v) const { return kind == 1 ? 1.f / (1.f + expf(-v)) : tanhf(v); }
+    __device__ void one(size_t i) const { y[i] = f(x[i]); }
+    __device__ void quad(size_t j) const {
+        float4 u = reinterpret_cast<const float4 *>(x)[j];
+        reinterpret_cast<float4 *>(y)[j] = make_float4(f(u.x), f(u.y), f(u.z), f(u.w));
+    }
+};
+struct ActBwdF {
+    const float *dy, *y; float *dx; int kind;
+    __device__ float g(float d, float o) const { return kind == 1 ? d * o * (1.f - o) : d * (1.f - o * o); }
+    __device__ void one(size_t i) const { dx[i] = g(dy[i], y[i]); }
+    __device__ void quad(size_t j) const {
+        float4 d = reinterpret_cast<const float4 *>(dy)[j], o = reinterpret_cast<const float4 *>(y)[j];
+        reinterpret_cast<float4 *>(dx)[j] = make_float4(g(d.x, o.x), g(d.y, o.y), g(d.z, o.z), g(d.w, o.w));
+    }
+};
 struct LerpF {
     float *m; const float *c; float mom;
     __device__ void one(size_t i) const { m[i] = mom * m[i] + (1.f - mom) * c[i]; }
@@ -790,6 +809,18 @@ int xsmi_relu_bwd(const float *dy, const float *pre, float *dx, size_t n) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(n == 0 || (dy && pre && dx), "xsmi_relu_bwd: null pointer");
     return launch_ew("relu_bwd", n, aligned16(dy) && aligned16(pre) && aligned16(dx), ReluBwdF{dy, pre, dx});
+}
+int xsmi_act_fwd(const float *x, float *y, size_t n, int kind) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (x && y), "xsmi_act_fwd: null pointer");
+    XSMI_CHECK_ARG(kind == 1 || kind == 2, "xsmi_act_fwd: kind must be 1 (sigmoid) or 2 (tanh)");
+    return launch_ew("act_fwd", n, aligned16(x) && aligned16(y), ActF{x, y, kind});
+}
+int xsmi_act_bwd(const float *dy, const float *y, float *dx, size_t n, int kind) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(n == 0 || (dy && y && dx), "xsmi_act_bwd: null pointer");
+    XSMI_CHECK_ARG(kind == 1 || kind == 2, "xsmi_act_bwd: kind must be 1 (sigmoid) or 2 (tanh)");
+    return launch_ew("act_bwd", n, aligned16(dy) && aligned16(y) && aligned16(dx), ActBwdF{dy, y, dx, kind});
 }
 int xsmi_lerp(float *m, const float *cur, float momentum, size_t n) {
     XSMI_REQUIRE_INIT();

@@ -1,66 +1,119 @@
-"""Layer base class (counterpart of xs/layers/base.py:6-134).
+"""Layer, the node type of both graph styles (the role of the reference's xs/layers/base.py:6-134).
 
-A layer is called either with a Tensor (eager: create parameters lazily from the
-input shape, run ``call``) or with another Layer (graph building: infer the
-output shape and link).  In a static graph every layer owns one preallocated
-output Tensor sized for the largest batch, re-sliced for a shorter last batch and
-written in place through the ``out=`` argument of the functional op.
+Applied to a Tensor a layer works eagerly: parameters are created from the input's shape on first use and
+``call`` runs the functional op.  Applied to another Layer it only records the edge and its output shape; the
+model later drives ``forward`` / ``backward`` over those edges, with one preallocated output tensor per layer
+(``static_buffer``).
 """
-from ..core import state as GLOBAL
-from ..core.base import Tensor, Parameter
-from ..nn.initializers import Zeros
-from ..nn import functional as F
+from ..core.base import Tensor, Parameter            # noqa: F401  (re-exported to the layer modules)
+from ..nn import functional as F                     # noqa: F401
+from . import static_buffer
 
 
 class Layer:
     def __init__(self, trainable=True, name=None, in_bounds=None, input_shape=None, shape=None, parameters=None,
                  **kwargs):
-        self.trainable = trainable
-        self._in_bounds = list(in_bounds) if in_bounds is not None else []
-        self._out_bounds = []
-        self._input_shape = input_shape
         self.name = str(name)
-        self._shape = shape
-        self._parameters = parameters if parameters is not None else []
+        self.trainable = trainable
+        self._shape, self._input_shape = shape, input_shape
+        self._parameters = [] if parameters is None else parameters
+        self._in_bounds = [] if in_bounds is None else list(in_bounds)
+        self._out_bounds = []
         self._data = None
 
+    # ------------------------------------------------------------------ applying a layer
     def __call__(self, x, *args, **kwargs):
-        if isinstance(x, Tensor):
-            if len(self._parameters) == 0:
-                self.init_params(tuple(x.shape[1:]))
-            x.next_layers.append(self)
-            return self.call(x, *args, **kwargs)
-        self._shape = self.compute_output_shape(x.shape)
-        self._in_bounds.append(x)
-        self._input_shape = x.shape
-        x.add_out_bounds(self)
+        if not isinstance(x, Tensor):
+            return self._chain_after(x)
+        return self._run(x, args, kwargs, dynamic=True)
+
+    def forward(self, x=None, *args, **kwargs):
+        """Static graphs call this without an argument: the input is then the output of the layer's last inbound
+        layer.  A Tensor argument is the dynamic form, as in ``__call__``."""
+        src = self._in_bounds[-1] if x is None else x
+        if isinstance(src, Tensor):
+            return self._run(src, args, kwargs, dynamic=src.is_dynamic)
+        if not self._parameters:
+            self.init_params(None)
+        return self.call(src.data, *args, **kwargs)
+
+    def _run(self, x, args, kwargs, dynamic):
+        if not self._parameters:
+            self.init_params(tuple(x.shape[1:]))
+        if dynamic:
+            self._forget_stale_output(x)
+            x.next_layers.append(self)           # autograd clears this layer's output after the backward sweep
+        return self.call(x, *args, **kwargs)
+
+    def _forget_stale_output(self, x):
+        """A dynamic forward hands the previous output tensor to the op as ``out=`` so that it is written again.
+        After a forward without backward (inference) that tensor is still there; when the batch size has
+        changed since, it cannot be reused and a new one is made (the reference raises a shape error here)."""
+        d = self._data
+        if isinstance(d, Tensor) and d.is_dynamic and d.eval is not None and len(d.shape) and d.shape[0] != x.shape[0]:
+            self._data = None
+
+    def _chain_after(self, inbound):
+        """Graph building, ``layer(previous_layer)``: record the edge, infer the output shape, return self."""
+        self._input_shape = inbound.shape
+        self._shape = self.compute_output_shape(inbound.shape)
+        self._in_bounds.append(inbound)
+        inbound.add_out_bounds(self)
         return self
 
     def connect(self, inbound=None):
-        if inbound is None:
-            if self._input_shape is None:
-                raise ValueError('must specify input_shape')
-        else:
+        """``Sequential.compile`` links consecutive layers with this; the first layer needs ``input_shape``."""
+        if inbound is not None:
             self._input_shape = inbound.shape
+        elif self._input_shape is None:
+            raise ValueError('must specify input_shape')
         self._shape = self.compute_output_shape(self._input_shape)
         if inbound is not None:
             self._in_bounds.append(inbound)
             inbound.add_out_bounds(self)
 
-    def params_count(self):
-        return sum(v.eval.size for v in self._parameters if v is not None)
+    def call(self, x, *args, **kwargs):
+        raise NotImplementedError
 
-    @property
-    def shape(self):
+    def backward(self, gradients=None):
+        """Static-graph backward of this layer: run the output tensor's grad_fn (which adds into the inputs'
+        gradients), then clear the output's own gradient for the next step."""
+        out = self._data
+        if gradients is not None:
+            if not isinstance(gradients, Tensor) or gradients.shape != out.shape:
+                raise ValueError('gradients must be a Tensor of the output shape %s' % (out.shape,))
+            out.grad = gradients
+        if out.grad_fn is not None:
+            out.grad_fn(out)
+            out.zero_grad()
+
+    # ------------------------------------------------------------------ shapes, parameters, buffers
+    def init_params(self, input_shape=None, *args):
+        pass
+
+    def compute_output_shape(self, input_shape=None):
+        self._shape = (input_shape,) if isinstance(input_shape, int) else tuple(input_shape)
         return self._shape
 
-    @property
-    def out_bounds(self):
-        return self._out_bounds
+    def init_layer_out_tensor(self, x=None):
+        if x is None:
+            x = self._in_bounds[0].data
+        self._data = static_buffer.fit_to_batch(self, self._data, x)
 
-    @property
-    def in_bounds(self):
-        return self._in_bounds
+    def parameters(self, parameters=None):
+        if parameters is None:
+            return self._parameters
+        self._parameters = parameters
+
+    def params_count(self):
+        return sum(p.eval.size for p in self._parameters if p is not None)
+
+    def add_out_bounds(self, *outs):
+        self._out_bounds.extend(o for o in outs if isinstance(o, Layer))
+
+    shape = property(lambda self: self._shape)
+    in_bounds = property(lambda self: self._in_bounds)
+    out_bounds = property(lambda self: self._out_bounds)
 
     @property
     def data(self):
@@ -69,69 +122,3 @@ class Layer:
     @data.setter
     def data(self, v):
         self._data = v
-
-    def parameters(self, parameters=None):
-        if parameters is None:
-            return self._parameters
-        self._parameters = parameters
-
-    def add_out_bounds(self, *outs):
-        for out in outs:
-            if isinstance(out, Layer):
-                self._out_bounds.append(out)
-
-    def init_params(self, input_shape=None, *args):
-        pass
-
-    def _new_out_tensor(self, x):
-        t = Zeros()((x.shape[0],) + tuple(self.shape), requires_grad=self.trainable)
-        if x.device == 'cuda' and t.device != 'cuda':
-            t.cuda_()
-        elif x.device == 'cpu' and t.device != 'cpu':
-            t.cpu_()
-        t.to('static')
-        return t
-
-    def init_layer_out_tensor(self, x=None):
-        x = self._in_bounds[0].data if x is None else x
-        if self._data is None or x.shape[0] > self._data.shape_capacity[0] or \
-                (x.shape[0] < self._data.shape_capacity[0] and not GLOBAL.TRAINING):
-            self._data = self._new_out_tensor(x)
-            self._data.add_in_bounds(x)
-            self._data.add_in_bounds(*self.parameters())
-        else:
-            if x.shape[0] < self._data.shape_capacity[0]:
-                self._data.slices(slice(None, x.shape[0], None))
-            else:
-                self._data.slices(slice(None, None, None))
-            # a reused output tensor must read from the tensor that feeds it now: the reference keeps the
-            # tensor it was created with (xs/layers/base.py:88-104), which goes stale as soon as a new
-            # loader hands in different batch tensors (fit after predict, a second fit)
-            if self._data.in_bounds and self._data.in_bounds[0] is not x:
-                self._data.in_bounds[0] = x
-
-    def compute_output_shape(self, input_shape=None):
-        self._shape = (input_shape,) if isinstance(input_shape, int) else tuple(input_shape)
-        return self._shape
-
-    def call(self, x, *args, **kwargs):
-        raise NotImplementedError
-
-    def forward(self, x=None, *args, **kwargs):
-        if x is None:
-            x = self._in_bounds[-1]
-        if len(self._parameters) == 0:
-            self.init_params(tuple(x.shape[1:]) if isinstance(x, Tensor) else None)
-        if isinstance(x, Tensor):
-            if x.is_dynamic:
-                x.next_layers.append(self)
-            return self.call(x, *args, **kwargs)
-        return self.call(x.data, *args, **kwargs)
-
-    def backward(self, gradients=None):
-        if gradients is not None:
-            assert isinstance(gradients, Tensor) and gradients.shape == self._data.shape
-            self._data.grad = gradients
-        if self._data.grad_fn is not None:
-            self._data.grad_fn(self._data)
-            self._data.zero_grad()

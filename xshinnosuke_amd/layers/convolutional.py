@@ -1,5 +1,6 @@
 """Conv2D layer (counterpart of xs/layers/convolutional.py:7-83)."""
 from .base import Layer, F, Parameter
+from .activators import FusedActivation
 from ..nn.initializers import get_initializer
 
 
@@ -9,14 +10,16 @@ def _size2(v):
     return tuple(int(i) for i in v)
 
 
-class Conv2D(Layer):
+class Conv2D(FusedActivation, Layer):
     """``Conv2D(out_channels, kernel_size, use_bias=True, stride=1, padding=0, activation=None, ...)``.
 
     weight ``(Cout, Cin, KH, KW)``, bias ``(1, Cout)``; parameters are created lazily from the first
     input.  ``padding`` is an int or 'same' / 'valid'.  With ``activation='relu'`` the activation is
     fused into the convolution kernel's epilogue and differentiated with the strict ``pre < 0`` mask,
     in static graphs as well (the reference applies it in a second pass and, in static graphs,
-    loses it for downstream layers, xs/layers/base.py:66-68).
+    loses it for downstream layers, xs/layers/base.py:66-68).  'sigmoid' and 'tanh' run as a child
+    activation layer on the convolution's output; an unknown name means no activation, as in the
+    reference (xs/layers/activators.py:74-87).
     """
 
     def __init__(self, out_channels, kernel_size, use_bias=True, stride=1, padding=0, activation=None,
@@ -26,9 +29,7 @@ class Conv2D(Layer):
         self.use_bias = use_bias
         self.stride = _size2(stride)
         self.padding = padding
-        if activation is not None and str(activation).lower() != 'relu':
-            raise ValueError("Conv2D fuses activation='relu' only; add other activations as layers")
-        self.activation = None if activation is None else 'relu'
+        self._set_activation(activation, fuse_relu=True)
         self.kernel_initializer = get_initializer(kernel_initializer)
         self.bias_initializer = get_initializer(bias_initializer)
         self.pad_size = padding if isinstance(padding, int) else 0
@@ -71,4 +72,12 @@ class Conv2D(Layer):
     def call(self, x, *args, **kwargs):
         weight, bias = self._parameters[0], (self._parameters[1] if self.use_bias else None)
         self._data = F.conv2d(x, weight, bias, self.stride, self.pad_size, self._data, activation=self.activation)
-        return self._data
+        return self._activate(self._data)
+
+    def init_layer_out_tensor(self, x=None):
+        super().init_layer_out_tensor(x)
+        self._static_act_buffer()
+
+    def backward(self, gradients=None):
+        self._act_backward()
+        super().backward(gradients)

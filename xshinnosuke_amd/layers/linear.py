@@ -1,12 +1,14 @@
 """Dense and Flatten (counterpart of xs/layers/linear.py)."""
-from functools import reduce
+import math
 
 from .base import Layer, F, Parameter
+from .activators import FusedActivation
 from ..nn.initializers import get_initializer
 
 
-class Dense(Layer):
-    """``y = x @ W + b`` with W ``(in, out)`` and b ``(1, out)``."""
+class Dense(FusedActivation, Layer):
+    """``y = act(x @ W + b)``, W ``(in, out)``, b ``(1, out)``; ``activation`` names 'relu', 'sigmoid' or
+    'tanh' (a child activation layer on the product's output)."""
 
     def __init__(self, out_features, activation=None, use_bias=True, kernel_initializer='normal',
                  bias_initializer='zeros', **kwargs):
@@ -14,9 +16,7 @@ class Dense(Layer):
         self.use_bias = use_bias
         self.kernel_initializer = get_initializer(kernel_initializer)
         self.bias_initializer = get_initializer(bias_initializer)
-        if activation is not None and str(activation).lower() != 'relu':
-            raise ValueError("Dense supports activation='relu' or None")
-        self.activation = None if activation is None else 'relu'
+        self._set_activation(activation, fuse_relu=False)
         super().__init__(**kwargs)
 
     def compute_output_shape(self, input_shape=None):
@@ -26,20 +26,26 @@ class Dense(Layer):
     def init_params(self, input_shape=None, *args):
         if input_shape is not None:
             self._input_shape = tuple(input_shape)
-        self._parameters.append(Parameter(self.kernel_initializer(tuple(self._input_shape) + (self.out_features,),
-                                                                  requires_grad=True)))
+        w_shape = tuple(self._input_shape) + (self.out_features,)
+        self._parameters.append(Parameter(self.kernel_initializer(w_shape, requires_grad=True)))
         if self.use_bias:
             self._parameters.append(Parameter(self.bias_initializer((1, self.out_features), requires_grad=True)))
 
+    def init_layer_out_tensor(self, x=None):
+        super().init_layer_out_tensor(x)
+        self._static_act_buffer()
+
     def call(self, x, *args, **kwargs):
+        weight = self._parameters[0]
         if self.use_bias:
-            weight, bias = self._parameters
-            self._data = F.addmm(bias, x, weight, self._data)
+            self._data = F.addmm(self._parameters[1], x, weight, self._data)
         else:
-            self._data = F.mm(x, self._parameters[0], self._data)
-        if self.activation == 'relu':
-            return F.relu(self._data)
-        return self._data
+            self._data = F.mm(x, weight, self._data)
+        return self._activate(self._data)
+
+    def backward(self, gradients=None):
+        self._act_backward()
+        super().backward(gradients)
 
 
 class Flatten(Layer):
@@ -50,8 +56,8 @@ class Flatten(Layer):
         super().__init__(**kwargs)
 
     def compute_output_shape(self, input_shape=None):
-        flat = reduce(lambda a, b: a * b, input_shape[self.start_dim - 1:])
-        self._shape = tuple(input_shape[:self.start_dim - 1]) + (flat,)
+        keep = self.start_dim - 1
+        self._shape = tuple(input_shape[:keep]) + (math.prod(input_shape[keep:]),)
         return self._shape
 
     def call(self, x, *args, **kwargs):

@@ -75,6 +75,25 @@ def relu_grad(dy, pre):
     return g
 
 
+def activation(x, kind, out=None):
+    """sigmoid / tanh as the reference computes them (xs/nn/td_functional.py:63-70)."""
+    if is_device(x):
+        return K.act_fwd(x, kind, out)
+    r = 1. / (1. + np.exp(-x)) if kind == 'sigmoid' else np.tanh(x)
+    if out is not None:
+        out[...] = r
+        return out
+    return r.astype(x.dtype, copy=False)
+
+
+def activation_grad(dy, y, kind):
+    """dy * y * (1 - y) for sigmoid, dy * (1 - y^2) for tanh (xs/nn/grad_fn.py:161-170)."""
+    if is_device(dy):
+        return K.act_bwd(dy, same_place(dy, y), kind)
+    y = np.asarray(same_place(dy, y))
+    return dy * y * (1 - y) if kind == 'sigmoid' else dy * (1 - np.square(y))
+
+
 def reshape(a, shape):
     return a.reshape(shape)
 

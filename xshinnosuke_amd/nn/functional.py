@@ -11,6 +11,8 @@ The remaining functions are the small set of neighbours the README networks and
 ResNet-18 need; they run in NumPy for host tensors and through element-wise /
 reduction kernels for device tensors.
 """
+import weakref
+
 import numpy as np
 
 from ..core import state as GLOBAL
@@ -20,6 +22,12 @@ from ..backend import array as dev
 from . import array_ops as A
 from .grad_fn import *  # noqa: F401,F403  (backward functions are part of this module's namespace, as in the reference)
 from .grad_fn import initialize_ops_grad, _f32_device
+
+
+# Folded (conv + inference batch norm) filters kept between forwards, keyed by the conv's weight Parameter.  They
+# live here and not on the Parameter: a checkpoint pickles the graph, and a kept filter holds device addresses
+# that mean nothing in another process.
+_FOLDED = weakref.WeakKeyDictionary()
 
 
 def _mark_input(t):
@@ -122,12 +130,13 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
     bf16 = bool(GLOBAL.CONV_BF16)
     relu = activation == 'relu'
     sources = [t.eval for t in (weight, bias, gamma, beta, moving_mean, moving_variance) if t is not None]
-    kept = getattr(weight, '_folded_filter', None)
+    kept = _FOLDED.get(weight)
     x = _f32_device(x)
     if all(is_device(a) and a.dtype == np.float32 for a in sources):
         # Frozen parameters: the folded filter, its bias and its packed form (in a workspace of this filter's own) are
         # kept while nobody has taken the address of a parameter since they were made (DeviceArray.state).
-        now = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape[1:]))
+        # (the batch size is part of the key: it decides which kernel, hence which packed layout, the library picks)
+        now = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape))
         need = K.conv2d_workspace_bytes(x.shape, weight.shape, stride, padding)
         if kept is not None and kept['key'] == now and kept['ws'].holds(need):
             y = K.conv2d_fwd(x, kept['w'], kept['b'], stride, padding, relu=relu, out=dst, bf16=bf16, packed=True,
@@ -139,8 +148,8 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
             ws = kept['ws'] if kept is not None else K.Workspace()
             y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, workspace=ws)
             # the fold has read the parameters: their state as of now is what the kept filter belongs to
-            key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape[1:]))
-            weight._folded_filter = {'key': key, 'w': w2, 'b': b2, 'ws': ws, 'of': sources}   # 'of' keeps the ids in the key alive
+            key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape))
+            _FOLDED[weight] = {'key': key, 'w': w2, 'b': b2, 'ws': ws, 'of': sources}   # 'of' keeps the ids in the key alive
     else:
         stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]
         b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
@@ -320,6 +329,29 @@ def relu(inputs, inplace=False, out=None):
         out.grad_fn = ReLUBackward
         initialize_ops_grad(inputs)
     return out
+
+
+def _activation(inputs, kind, backward_fn, out):
+    _mark_input(inputs)
+    res = A.activation(inputs.eval, kind, None if out is None else out.eval)
+    if out is None:
+        out = Tensor(res)
+    out.requires_grad = inputs.requires_grad
+    _wire(out, inputs)
+    if GLOBAL.COMPUTE_GRAD and out.requires_grad:
+        out.grad_fn = backward_fn
+        initialize_ops_grad(inputs)
+    return out
+
+
+def sigmoid(inputs, out=None):
+    """1 / (1 + exp(-x)) (reference xs/nn/functional.py:316-329)."""
+    return _activation(inputs, 'sigmoid', SigmoidBackward, out)
+
+
+def tanh(inputs, out=None):
+    """Reference xs/nn/functional.py:332-345."""
+    return _activation(inputs, 'tanh', TanhBackward, out)
 
 
 def flatten(inputs, start=1, out=None):

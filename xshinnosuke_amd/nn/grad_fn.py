@@ -131,6 +131,20 @@ def ReLUBackward(outputs):
             _accumulate(inputs, A.relu_grad(outputs.grad.eval, inputs.eval))
 
 
+def SigmoidBackward(outputs):
+    """Reference xs/nn/grad_fn.py:161-164."""
+    inputs, = outputs.in_bounds
+    if inputs.requires_grad:
+        _accumulate(inputs, A.activation_grad(outputs.grad.eval, outputs.eval, 'sigmoid'))
+
+
+def TanhBackward(outputs):
+    """Reference xs/nn/grad_fn.py:167-170."""
+    inputs, = outputs.in_bounds
+    if inputs.requires_grad:
+        _accumulate(inputs, A.activation_grad(outputs.grad.eval, outputs.eval, 'tanh'))
+
+
 def _both_addends_on_device(outputs, g):
     """Two distinct addends of the output's shape that both want a gradient and keep it in aligned device memory."""
     if len(outputs.in_bounds) != 2:

@@ -189,6 +189,14 @@ class _Model(_Base):
         return '\n'.join(rows)
 
 
+def _owns_static_output(*layers):
+    """True if one of the layers holds a preallocated static-graph output tensor.  fit / evaluate / predict give
+    every layer one before the first forward; such layers are driven one by one (their outputs are distinct
+    buffers that the layer-wise backward relies on), so the fused forms below leave them alone -- also when the
+    graph's first input, a loader's batch tensor, is a dynamic tensor."""
+    return any(isinstance(l, Layer) and isinstance(l._data, Tensor) and l._data.is_static for l in layers)
+
+
 class Sequential(_Model):
     def __init__(self, *layers):
         super().__init__()
@@ -240,16 +248,18 @@ class Sequential(_Model):
             # both (same values and gradients as the two layers; the ReLU layer's output is the same tensor, as
             # an in-place activation's is).  Static graphs drive the layers' backward one by one and are left alone.
             if (isinstance(layer, BatchNormalization) and isinstance(nxt, ReLU) and nxt.inplace and
-                    isinstance(x, Tensor) and x.is_dynamic and x.device == 'cuda'):
+                    isinstance(x, Tensor) and x.is_dynamic and x.device == 'cuda' and not _owns_static_output(layer, nxt)):
                 x = layer.forward(x, fuse_relu=True)
                 nxt.data = x
                 i += 2
             # Inference (moving statistics, nothing to differentiate) of Conv2D -> BatchNormalization [-> ReLU] on a
             # device-resident dynamic graph: the normalisation is a per-filter scale and shift, folded into the
             # convolution.  All the layers involved then hold the same output tensor.
-            elif (isinstance(layer, Conv2D) and layer.activation is None and isinstance(nxt, BatchNormalization) and
+            elif (isinstance(layer, Conv2D) and layer.activation is None and layer._act_layer is None and
+                    isinstance(nxt, BatchNormalization) and
                     nxt.axis == 1 and not GLOBAL.TRAINING and not GLOBAL.COMPUTE_GRAD and isinstance(x, Tensor) and
-                    x.is_dynamic and x.device == 'cuda' and len(layer._parameters) and len(nxt._parameters)):
+                    x.is_dynamic and x.device == 'cuda' and len(layer._parameters) and len(nxt._parameters) and
+                    not _owns_static_output(layer, nxt, layers[i + 2] if i + 2 < n else None)):
                 relu = layers[i + 2] if i + 2 < n and isinstance(layers[i + 2], ReLU) else None
                 x.next_layers.append(layer)
                 weight, bias = layer._parameters[0], (layer._parameters[1] if layer.use_bias else None)
