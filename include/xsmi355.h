@@ -127,6 +127,18 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
                     int sh, int sw, int pad, unsigned flags,
                     void *workspace, size_t workspace_bytes);
 
+/* The forward for callers that cannot allocate device memory or pass a workspace: code under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same kernels,
+ * arguments and results as xsmi_conv2d_fwd (flags: XSMI_CONV_RELU, XSMI_CONV_BF16); the scratch memory is a static
+ * device array of XSMI_NOALLOC_SCRATCH_BYTES (16 MiB) inside the library, one per GPU, held
+ * until the process ends.  Geometries whose workspace (xsmi_conv2d_workspace_bytes of the forward alone: the
+ * packed filter) exceeds it are refused with XSMI_ERR_INVALID.  All calls on a GPU share that array: calls that
+ * overlap on one GPU (two host threads, two streams) race.  Calls no hipMalloc / hipFree. */
+int xsmi_conv2d_fwd_noalloc(const float *x, const float *w, const float *bias, float *y,
+                            uint8_t *neg_mask, int N, int C, int H, int W, int K, int R, int S,
+                            int sh, int sw, int pad, unsigned flags);
+#define XSMI_NOALLOC_SCRATCH_BYTES ((size_t)16 << 20)
+
 /* Backward w.r.t. the input: dx = beta*dx + fold(dy^T . w).  Replaces the dcol
  * GEMM + col2im of Conv2DBackward (xs/nn/grad_fn.py:199-203, xs/utils/common.py:49-65).
  * beta must be 0 (overwrite) or 1 (accumulate, what the reference always does). */

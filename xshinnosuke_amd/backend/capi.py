@@ -59,6 +59,7 @@ SIGNATURES = {
     "xsmi_copy_kernel": (_i, [_vp, _vp, _sz]),
     "xsmi_conv2d_workspace_bytes": (_sz, _CONV_DIMS),
     "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
+    "xsmi_conv2d_fwd_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u]),
     "xsmi_conv2d_bwd_data": (_i, [_vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
     "xsmi_conv2d_bwd_weight": (_i, [_vp, _vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
     "xsmi_conv2d_bwd": (_i, [_vp] * 6 + _CONV_DIMS + [_f, _f, _u, _vp, _sz, _vp, _sz]),
@@ -97,6 +98,7 @@ CONV_RELU = 0x1
 CONV_BF16 = 0x2
 CONV_WS_PACKED = 0x4
 CONV_DW_ASYNC = 0x8
+NOALLOC_SCRATCH_BYTES = 16 << 20      # XSMI_NOALLOC_SCRATCH_BYTES of the header
 
 
 def library_path():

@@ -89,6 +89,8 @@ int xsmi_init(int device) {
         xsmi::set_error("xsmi_init: device %d is %s; this library holds gfx950 code only", device, prop.gcnArchName);
         return XSMI_ERR_RUNTIME;
     }
+    int rc = xsmi::noalloc_setup(device);                // address of this GPU's copy of the static scratch array
+    if (rc) return rc;
     XSMI_HIP(hipStreamCreateWithFlags(&g_stream, hipStreamNonBlocking));
     XSMI_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
     XSMI_HIP(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));

@@ -22,6 +22,8 @@ bool side_pending();
 bool on_side_stream();
 bool ready();
 int cu_count();
+// conv_noalloc.hip: resolves the device address of the static scratch array for `device` (the current device)
+int noalloc_setup(int device);
 // With xsmi_profiling(1) every op brackets its main kernel(s) with two events on
 // the library stream; xsmi_last_kernel_ms reads them back.
 void prof_begin();
