@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark of the conv / max-pool hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--no-cpu] [--no-extra] [--per-layer]
 
 A step is one pass of the conv hot path over one synthetic batch that is already
 resident in HBM: forward, backward-data and backward-weight (+ bias gradient) of
@@ -15,7 +15,12 @@ duration of that launch, taken from event pairs the library records directly
 around the kernel in a second pass over the same K steps.
 
 `cpu_baseline` times the NumPy restatement of the reference algorithm (the
-parity oracle) on the host cores of this machine, on the same workload.
+parity oracle) on the host cores of this machine, on the same workload; its
+`other_workloads` hold the same for the max-pool, README-net, ResNet-18 training
+and ResNet-18 inference configurations, each beside the GPU figure in `extra`.
+
+`--per-layer` times every distinct ResNet-18 convolution (N=32) pass by pass and
+prints one JSON line with a row per (layer, pass).
 
 Everything goes through libxsmi355.so; there is no fallback path.
 """
@@ -39,6 +44,21 @@ HBM_PEAK_GBPS = 8000.0
 CONV = dict(N=32, C=64, H=56, W=56, K=64, R=3, S=3, stride=(1, 1), pad=1)
 # BASELINE max-pool config
 POOL = dict(N=32, C=64, H=112, W=112, k=3, stride=(2, 2), pad=1)
+
+# The 11 distinct convolutions of ResNet-18 at N=32, 224x224 input: name, count, Cin, Cout, H_in, k, stride, pad
+RESNET18_CONVS = [
+    ("stem 3->64 7x7/2 224", 1, 3, 64, 224, 7, 2, 3),
+    ("layer1 64->64 3x3 56", 4, 64, 64, 56, 3, 1, 1),
+    ("layer2.0a 64->128 3x3/2 56", 1, 64, 128, 56, 3, 2, 1),
+    ("layer2.0s 64->128 1x1/2 56", 1, 64, 128, 56, 1, 2, 0),
+    ("layer2 128->128 3x3 28", 3, 128, 128, 28, 3, 1, 1),
+    ("layer3.0a 128->256 3x3/2 28", 1, 128, 256, 28, 3, 2, 1),
+    ("layer3.0s 128->256 1x1/2 28", 1, 128, 256, 28, 1, 2, 0),
+    ("layer3 256->256 3x3 14", 3, 256, 256, 14, 3, 1, 1),
+    ("layer4.0a 256->512 3x3/2 14", 1, 256, 512, 14, 3, 2, 1),
+    ("layer4.0s 256->512 1x1/2 14", 1, 256, 512, 14, 1, 2, 0),
+    ("layer4 512->512 3x3 7", 3, 512, 512, 7, 3, 1, 1),
+]
 
 
 # HBM bytes per launch of tap_igemm_f32_kernel on the CONV workload, from two hardware-counter runs
@@ -133,42 +153,175 @@ def bench_conv(be, steps, warmup):
     return ms / steps, wall_ms / steps, per
 
 
-def bench_pool(be, steps, warmup):
-    K = be.kernels
-    p = POOL
+def make_pool_inputs(p):
     rng = np.random.default_rng(4)
     x = rng.standard_normal((p["N"], p["C"], p["H"], p["W"]), dtype=np.float32)
     flat = x.reshape(-1, p["W"])
-    pick = rng.choice(flat.size, size=flat.size // 20, replace=False)
+    pick = rng.choice(flat.size, size=flat.size // 20, replace=False)      # 5 % ties with the right-hand neighbour
     r, col = np.divmod(pick, p["W"])
     flat[r, col] = flat[r, (col + 1) % p["W"]]
     oh = (p["H"] + 2 * p["pad"] - p["k"]) // p["stride"][0] + 1
     ow = (p["W"] + 2 * p["pad"] - p["k"]) // p["stride"][1] + 1
     dy = np.random.default_rng(5).standard_normal((p["N"], p["C"], oh, ow), dtype=np.float32)
-    dx_, ddy = be.to_device(x), be.to_device(dy)
-    y = be.empty(dy.shape); idx = be.empty(dy.shape, np.uint8); gx = be.empty(x.shape)
-    def pair():
-        K.maxpool2d_fwd(dx_, p["k"], p["stride"], p["pad"], out=y, idx=idx)
-        K.maxpool2d_bwd(ddy, idx, x.shape, p["k"], p["stride"], p["pad"], dx=gx)
-    preheat(be, pair)
-    for _ in range(warmup):
-        pair()
-    be.synchronize()
-    fm = batch_ms(be, lambda: K.maxpool2d_fwd(dx_, p["k"], p["stride"], p["pad"], out=y, idx=idx), steps)
-    bm = batch_ms(be, lambda: K.maxpool2d_bwd(ddy, idx, x.shape, p["k"], p["stride"], p["pad"], dx=gx), steps)
-    # plain copy of the same number of bytes, for the achievable-bandwidth reference
-    src = be.empty((x.size + dy.size + dy.size // 4,)); dst = be.empty(src.shape)
-    for _ in range(warmup):
-        K.copy_kernel(dst, src)
-    cm = batch_ms(be, lambda: K.copy_kernel(dst, src), steps)
+    return x, dy
+
+
+POOL_SETS = 5        # disjoint buffer sets the memory-bound kernels rotate over
+
+
+def bench_pool(be, steps, warmup):
+    """Max-pool forward / backward and the plain copy kernel, HBM-true: consecutive launches work on POOL_SETS
+    disjoint buffer sets (5 x 135 MB per direction and kernel, far beyond the 256 MB of last-level cache), so no
+    launch finds its operands cached by the previous one.  The "warm" figures repeat one set and are cache-assisted;
+    they are reported for comparison only."""
+    K = be.kernels
+    p = POOL
+    x, dy = make_pool_inputs(p)
+    sets = []
+    for _ in range(POOL_SETS):
+        sets.append(dict(x=be.to_device(x), dy=be.to_device(dy), y=be.empty(dy.shape), idx=be.empty(dy.shape, np.uint8),
+                         gx=be.empty(x.shape)))
+    nel = x.size + dy.size + dy.size // 4
+    copies = [(be.empty((nel,)), be.empty((nel,))) for _ in range(POOL_SETS)]
+    for c_src, _ in copies:
+        c_src.fill_zero()
+    state = {"i": 0}
+
+    def nxt():
+        state["i"] = (state["i"] + 1) % POOL_SETS
+        return state["i"]
+
+    def fwd(b):
+        K.maxpool2d_fwd(b["x"], p["k"], p["stride"], p["pad"], out=b["y"], idx=b["idx"])
+
+    def bwd(b):
+        K.maxpool2d_bwd(b["dy"], b["idx"], x.shape, p["k"], p["stride"], p["pad"], dx=b["gx"])
+
+    for b in sets:
+        fwd(b); bwd(b)
+    for c_src, c_dst in copies:                          # every buffer has been written once before anything is timed
+        K.copy_kernel(c_dst, c_src)
+    preheat(be, lambda: (fwd(sets[nxt()]), bwd(sets[nxt()]), K.copy_kernel(*copies[nxt()][::-1])))
+    n = max(steps, 4 * POOL_SETS)
+    n -= n % POOL_SETS
+    fm = batch_ms(be, lambda: fwd(sets[nxt()]), n)
+    bm = batch_ms(be, lambda: bwd(sets[nxt()]), n)
+    cm = batch_ms(be, lambda: K.copy_kernel(*copies[nxt()][::-1]), n)
+    fm_w = batch_ms(be, lambda: fwd(sets[0]), n)
+    bm_w = batch_ms(be, lambda: bwd(sets[0]), n)
+    cm_w = batch_ms(be, lambda: K.copy_kernel(copies[0][1], copies[0][0]), n)
     bytes_alg = x.nbytes + dy.nbytes + dy.size          # x + y + 1-byte index  (fwd);  dy + idx + dx  (bwd)
+    gbps = lambda ms: bytes_alg / ms / 1e6
     return {
-        "maxpool_workload": "N=32 C=64 112x112, 3x3 stride 2 pad 1, fp32, 5% ties",
+        "maxpool_workload": "N=32 C=64 112x112, 3x3 stride 2 pad 1, fp32, 5%% ties; launches rotate over %d disjoint buffer "
+                            "sets (%.0f MB in total per kernel)" % (POOL_SETS, POOL_SETS * bytes_alg / 1e6),
         "maxpool_algorithmic_MB": bytes_alg / 1e6,
-        "maxpool_fwd_ms": fm, "maxpool_fwd_GBps": bytes_alg / fm / 1e6, "maxpool_fwd_frac_hbm": bytes_alg / fm / 1e6 / HBM_PEAK_GBPS,
-        "maxpool_bwd_ms": bm, "maxpool_bwd_GBps": bytes_alg / bm / 1e6, "maxpool_bwd_frac_hbm": bytes_alg / bm / 1e6 / HBM_PEAK_GBPS,
-        "copy_kernel_GBps": 2 * src.nbytes / cm / 1e6, "copy_kernel_MB_each_way": src.nbytes / 1e6,
+        "maxpool_fwd_ms": fm, "maxpool_fwd_GBps": gbps(fm), "maxpool_fwd_frac_hbm": gbps(fm) / HBM_PEAK_GBPS,
+        "maxpool_bwd_ms": bm, "maxpool_bwd_GBps": gbps(bm), "maxpool_bwd_frac_hbm": gbps(bm) / HBM_PEAK_GBPS,
+        "copy_kernel_GBps": 2 * 4 * nel / cm / 1e6, "copy_kernel_MB_each_way": 4 * nel / 1e6,
+        "same_buffers_cache_assisted": {"maxpool_fwd_GBps": gbps(fm_w), "maxpool_bwd_GBps": gbps(bm_w),
+                                        "copy_kernel_GBps": 2 * 4 * nel / cm_w / 1e6},
     }
+
+
+def bench_per_layer(be, reps):
+    """Every distinct ResNet-18 convolution at N=32, pass by pass (forward incl. bias, backward-data,
+    backward-weight incl. bias gradient): whole ops as the training step issues them (filter layout kernels and split
+    reductions included), `reps` launches back to back between two events after a clock ramp."""
+    K = be.kernels
+    rows = []
+    rng = np.random.default_rng(11)
+    for name, count, c, k, h, r, st, pad in RESNET18_CONVS:
+        oh = (h + 2 * pad - r) // st + 1
+        x = be.to_device(rng.standard_normal((32, c, h, h), dtype=np.float32))
+        w = be.to_device((rng.standard_normal((k, c, r, r)) * np.sqrt(2.0 / (c * r * r))).astype(np.float32))
+        b = be.to_device(np.zeros((k,), np.float32))
+        dy = be.to_device(rng.standard_normal((32, k, oh, oh), dtype=np.float32))
+        y = be.empty(dy.shape); gx = be.empty(x.shape); gw = be.empty(w.shape); gb = be.empty((k,))
+        flops = 2.0 * 32 * oh * oh * k * c * r * r
+        passes = {
+            "fwd": lambda: K.conv2d_fwd(x, w, b, (st, st), pad, out=y),
+            "bwd_data": lambda: K.conv2d_bwd_data(dy, w, x.shape, (st, st), pad, dx=gx),
+            "bwd_weight": lambda: K.conv2d_bwd_weight(dy, x, w.shape, (st, st), pad, dw=gw, db=gb),
+        }
+        for pname, fn in passes.items():
+            if pname == "bwd_data" and c == 3:
+                continue                                  # the network input needs no gradient
+            preheat(be, fn, seconds=0.25)
+            ms = batch_ms(be, fn, reps)
+            tf = flops / (ms * 1e-3) / 1e12
+            rows.append({"layer": name, "count": count, "pass": pname, "ms": ms, "gflop": flops / 1e9, "tflops": tf,
+                         "frac_fp32_mfma_peak": tf / FP32_MFMA_PEAK_TFLOPS})
+        del x, w, b, dy, y, gx, gw, gb
+    total_ms = sum(r_["ms"] * r_["count"] for r_ in rows)
+    total_gflop = sum(r_["gflop"] * r_["count"] for r_ in rows)
+    return {"per_layer": rows, "conv_ms_per_training_step": total_ms, "conv_gflop_per_training_step": total_gflop,
+            "conv_tflops_whole_network": total_gflop / total_ms, "reps": reps,
+            "frac_fp32_mfma_peak_whole_network": total_gflop / total_ms / FP32_MFMA_PEAK_TFLOPS}
+
+
+README_N = 256
+
+
+def make_readme_inputs():
+    """README functional net: x 256x1x28x28 ~N(0,1), Conv2D(8, 2x2) He-normal + ReLU, MaxPool 2x2, Dense 1352->10
+    ~N(0, 0.1), uniform labels."""
+    rng = np.random.default_rng(0)
+    x = rng.standard_normal((README_N, 1, 28, 28), dtype=np.float32)
+    wc = (rng.standard_normal((8, 1, 2, 2)) * np.sqrt(2.0 / 4)).astype(np.float32)
+    wd = (rng.standard_normal((1352, 10)) * 0.1).astype(np.float32)
+    labels = rng.integers(0, 10, size=(README_N,))
+    return x, wc, wd, labels
+
+
+def bench_readme_net(be, steps, warmup):
+    """README net, one fwd+bwd+SGD step through the layer API on device-resident tensors (launch-bound: 11.9 MFLOP)."""
+    import xshinnosuke_amd as xs
+    from xshinnosuke_amd.layers import Conv2D, MaxPooling2D, Flatten, Dense
+    from xshinnosuke_amd.nn.models import Sequential
+    from xshinnosuke_amd.optim import SGD
+    x, wc, wd, labels = make_readme_inputs()
+    xs.GLOBAL.INPUTS = None
+    xs.GLOBAL.USE_CUDA = True
+    try:
+        net = Sequential(Conv2D(8, 2, activation='relu'), MaxPooling2D(2), Flatten(), Dense(10))
+        xt, yt = xs.tensor(x).to('cuda'), xs.tensor(labels).to('cuda')
+        with xs.no_grad():
+            net(xt)
+        xs.GLOBAL.INPUTS = None
+        conv, dense = net._graph[0], net._graph[3]
+        conv.parameters()[0].eval = be.to_device(wc)
+        dense.parameters()[0].eval = be.to_device(wd)
+        params = [q for l in (conv, dense) for q in l.parameters() if q is not None]
+        opt = SGD(params, lr=0.01)
+        crit = xs.nn.CrossEntropyLoss()
+
+        def step():
+            opt.zero_grad()
+            loss = crit(net(xt), yt)
+            loss.backward()
+            opt.step()
+            return loss
+
+        for _ in range(warmup + 5):
+            step()
+        be.synchronize()
+        e0, e1 = be.Event(), be.Event()
+        t0 = time.perf_counter()
+        e0.record()
+        for _ in range(steps):
+            loss = step()
+        e1.record()
+        ms = e0.elapsed_ms(e1)
+        be.synchronize()
+        wall = (time.perf_counter() - t0) * 1e3
+        return {"readme_net_ms_per_step": ms / steps, "readme_net_wall_ms_per_step": wall / steps,
+                "readme_net_images_per_sec": README_N * steps / (ms * 1e-3), "readme_net_last_loss": loss.item(),
+                "readme_net_workload": "N=256x1x28x28, Conv2D(8, 2x2, relu) + MaxPool 2x2 + Flatten + Dense(10), cross-entropy, "
+                                       "SGD lr 0.01; fwd+bwd+step through the layer API, device-resident"}
+    finally:
+        xs.GLOBAL.USE_CUDA = False
+        xs.GLOBAL.INPUTS = None
 
 
 def bench_resnet18(be, steps, warmup):
@@ -213,16 +366,25 @@ def bench_resnet18(be, steps, warmup):
             "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
 
 
-def bench_resnet18_infer(be, steps, warmup):
+def bench_resnet18_infer(be, steps, warmup, with_oracle=True):
     """ResNet-18 N=256 forward only, moving-statistics BN, convolutions allowed to use bf16 MFMA operands; the fp32
-    forward of the same weights and input runs beside it and gives the logits' relative L2 distance."""
+    forward of the same weights and input runs beside it.  With `with_oracle` the NumPy/oracle forward of the first
+    and the last image (the images of a batch are independent under moving statistics) is timed on the host and
+    gives the logits' relative L2 distance for both precisions."""
     import xshinnosuke_amd as xs
     from resnet18 import ResNet18
     xs.GLOBAL.INPUTS = None
-    X = np.random.default_rng(7).standard_normal((256, 3, 224, 224), dtype=np.float32)
-    x = xs.tensor(X).to('cuda')
-    net = ResNet18(classes=1000, pool=7).to('cuda')
     out = {}
+    ref = None
+    if with_oracle:
+        sec, ref, net, X, pick = cpu_resnet18_inference(2)
+        out["resnet18_infer_cpu_oracle"] = {"sec_for_images": sec, "images": len(pick), "images_per_sec": len(pick) / sec,
+                                            "cores": _blas_threads(), "sample": "oracle forward of images 0 and 255 of the batch"}
+    else:
+        np.random.seed(7)
+        X = np.random.default_rng(7).standard_normal((256, 3, 224, 224), dtype=np.float32)
+        net = ResNet18(classes=1000, pool=7).to('cuda')
+    x = xs.tensor(X).to('cuda')
     xs.GLOBAL.TRAINING = False
     try:
         with xs.no_grad():
@@ -248,7 +410,12 @@ def bench_resnet18_infer(be, steps, warmup):
         xs.GLOBAL.USE_CUDA = False
         xs.GLOBAL.INPUTS = None
     d = logits["bf16"] - logits["fp32"]
-    out["resnet18_infer_bf16_logits_rel_l2_vs_fp32"] = float(np.linalg.norm(d) / np.linalg.norm(logits["fp32"]))
+    out["resnet18_infer_bf16_logits_rel_l2_vs_fp32_kernels"] = float(np.linalg.norm(d) / np.linalg.norm(logits["fp32"]))
+    if ref is not None:
+        r64 = ref.astype(np.float64)
+        for mode in ("fp32", "bf16"):
+            out["resnet18_infer_%s_logits_rel_l2_vs_oracle" % mode] = float(
+                np.linalg.norm(logits[mode][pick] - r64) / np.linalg.norm(r64))
     out["resnet18_infer_workload"] = ("N=256x3x224x224, forward only, moving-statistics BN (fresh: mean 0, var 1), "
                                       "fp32 tensors in HBM, batch norm folded into the convolutions; bf16 = each conv rewrites "
                                       "its input as a channels-last bf16 copy and multiplies bf16 operands with fp32 accumulation")
@@ -287,31 +454,159 @@ def traffic_run(be, reps=3):
     return {"traffic_run": reps, "copy_kernel_bytes_each_way": src.nbytes}
 
 
-def cpu_baseline():
-    """Oracle (NumPy restatement of the reference algorithm) on the host cores, same workload."""
-    import oracle
+def _blas_threads():
     try:
         from threadpoolctl import threadpool_info
-        threads = max([p.get("num_threads", 1) for p in threadpool_info()] or [1])
+        return int(max([p.get("num_threads", 1) for p in threadpool_info()] or [1]))
     except Exception:
-        threads = os.cpu_count() or 1
-    c = CONV
-    x, w, b, dy = make_conv_inputs(c)
+        return int(os.cpu_count() or 1)
+
+
+def _median_after_warmup(fn, timed=3):
     times = []
-    for i in range(3):                       # 1 warm-up + 2 timed
+    for _ in range(timed + 1):                 # the first run is the warm-up
         t0 = time.perf_counter()
+        fn()
+        times.append(time.perf_counter() - t0)
+    return statistics.median(times[1:]), times[1:]
+
+
+def cpu_conv_step(c):
+    import oracle
+    x, w, b, dy = make_conv_inputs(c)
+
+    def step():
         y, col = oracle.conv2d_fwd(x, w, b.reshape(1, -1), c["stride"], c["pad"])
         oracle.conv2d_bwd(dy, x.shape, w, col, c["stride"], c["pad"],
                           np.zeros_like(x), np.zeros_like(w), np.zeros((1, c["K"]), dtype=np.float32))
-        times.append(time.perf_counter() - t0)
-        del y, col
-    sec = statistics.mean(times[1:])
-    return {
-        "value": 3 * conv_flops(c) / sec / 1e12, "unit": "TFLOP/s", "cores": int(threads), "kind": "port",
-        "sample": "full workload (N=32 conv fwd+bwd), 1 warm-up + 2 timed steps, NumPy %s float64 im2col+GEMM+col2im; "
-                  "os.cpu_count=%s" % (np.__version__, os.cpu_count()),
-        "sec_per_step": sec,
+    return _median_after_warmup(step)
+
+
+def cpu_pool_step():
+    import oracle
+    p = POOL
+    x, dy = make_pool_inputs(p)
+
+    def step():
+        y, am = oracle.max_pool2d_fwd(x, p["k"], p["stride"], p["pad"])
+        oracle.max_pool2d_bwd(dy, am, x.shape, p["k"], p["stride"], p["pad"], np.zeros_like(x))
+    return _median_after_warmup(step)
+
+
+def cpu_readme_step():
+    """README net fwd+bwd+SGD: conv / ReLU / max-pool through the oracle, dense + cross-entropy in NumPy float64."""
+    import oracle
+    x, wc, wd, labels = make_readme_inputs()
+    bc = np.zeros((8,), np.float32); bd = np.zeros((1, 10))
+    wd64 = wd.astype(np.float64)
+    rows = np.arange(len(labels))
+
+    def step():
+        y1, col = oracle.conv2d_fwd(x, wc, bc, (1, 1), 0)
+        a1 = oracle.relu_fwd(y1)
+        p1, am = oracle.max_pool2d_fwd(a1, 2, None, 0)
+        flat = p1.reshape(p1.shape[0], -1).astype(np.float64)
+        z = flat @ wd64 + bd
+        z -= z.max(axis=1, keepdims=True)
+        sm = np.exp(z); sm /= sm.sum(axis=1, keepdims=True)
+        g = sm; g[rows, labels] -= 1; g /= len(labels)
+        dwd = flat.T @ g; dbd = g.sum(axis=0, keepdims=True)
+        dflat = (g @ wd64.T).astype(np.float32)
+        da1 = oracle.max_pool2d_bwd(dflat.reshape(p1.shape), am, a1.shape, 2, (2, 2), 0, np.zeros_like(a1))
+        dy1 = oracle.relu_bwd(da1, y1)
+        _, dwc, dbc = oracle.conv2d_bwd(dy1, x.shape, wc, col, (1, 1), 0, None, np.zeros_like(wc), np.zeros_like(bc))
+        return wc - 0.01 * dwc, bc - 0.01 * dbc, wd64 - 0.01 * dwd, bd - 0.01 * dbd
+    return _median_after_warmup(step)
+
+
+def cpu_resnet18_hot_path():
+    """The conv / max-pool share of one ResNet-18 N=32 training step on the CPU path: forward + backward of each of the
+    11 distinct convolutions (oracle, float64 im2col + GEMM + col2im) timed once after a warm-up on the first one and
+    weighted by how often the layer occurs, plus the 3x3/2 max-pool forward + backward.  Batch norm, ReLU, residual
+    adds, the dense tail and the optimizer are not in this sample."""
+    import oracle
+    rng = np.random.default_rng(12)
+    total, per = 0.0, {}
+    first = True
+    for name, count, c, k, h, r, st, pad in RESNET18_CONVS:
+        oh = (h + 2 * pad - r) // st + 1
+        x = rng.standard_normal((32, c, h, h), dtype=np.float32)
+        w = (rng.standard_normal((k, c, r, r)) * np.sqrt(2.0 / (c * r * r))).astype(np.float32)
+        b = np.zeros((1, k), np.float32)
+        dy = rng.standard_normal((32, k, oh, oh), dtype=np.float32)
+
+        def step():
+            y, col = oracle.conv2d_fwd(x, w, b, (st, st), pad)
+            oracle.conv2d_bwd(dy, x.shape, w, col, (st, st), pad, None if c == 3 else np.zeros_like(x),
+                              np.zeros_like(w), np.zeros((1, k), np.float32))
+        if first:
+            step()
+            first = False
+        t0 = time.perf_counter()
+        step()
+        per[name] = time.perf_counter() - t0
+        total += count * per[name]
+        del x, w, dy
+    px, pdy = make_pool_inputs(POOL)
+    t0 = time.perf_counter()
+    y, am = oracle.max_pool2d_fwd(px, 3, (2, 2), 1)
+    oracle.max_pool2d_bwd(pdy, am, px.shape, 3, (2, 2), 1, np.zeros_like(px))
+    per["max-pool 3x3/2 112"] = time.perf_counter() - t0
+    total += per["max-pool 3x3/2 112"]
+    return total, per
+
+
+def cpu_resnet18_inference(images=2):
+    """Oracle forward of ResNet-18 (moving-statistics batch norm) on `images` images of the N=256 inference input;
+    returns (seconds, logits, the network) so that the GPU logits of the same images can be compared."""
+    import xshinnosuke_amd as xs
+    from resnet18 import ResNet18, oracle_forward
+    np.random.seed(7)
+    X = np.random.default_rng(7).standard_normal((256, 3, 224, 224), dtype=np.float32)
+    pick = [0, 255][:images]
+    xs.GLOBAL.INPUTS = None
+    net = ResNet18(classes=1000, pool=7).to('cuda')
+    with xs.no_grad():
+        net(xs.tensor(X[:1]).to('cuda'))
+    xs.GLOBAL.INPUTS = None
+    t0 = time.perf_counter()
+    ref = oracle_forward(net, X[pick])
+    sec = time.perf_counter() - t0
+    return sec, ref, net, X, pick
+
+
+def cpu_baseline(extra):
+    """Oracle (NumPy restatement of the reference algorithm) on the host cores.  The headline entry is the conv
+    workload (median of 3 steps after a warm-up); `other_workloads` hold the other configurations, each with the GPU
+    figure measured earlier in this run beside it."""
+    threads = _blas_threads()
+    c = CONV
+    sec, all_sec = cpu_conv_step(c)
+    out = {
+        "value": 3 * conv_flops(c) / sec / 1e12, "unit": "TFLOP/s", "cores": threads, "kind": "port",
+        "sample": "full workload (N=32 conv fwd+bwd), 1 warm-up + 3 timed steps (median), NumPy %s float64 "
+                  "im2col+GEMM+col2im; os.cpu_count=%s" % (np.__version__, os.cpu_count()),
+        "sec_per_step": sec, "sec_all": all_sec,
     }
+    others = {}
+    psec, _ = cpu_pool_step()
+    bytes_alg = 2 * (POOL["N"] * POOL["C"] * (POOL["H"] * POOL["W"] + (POOL["H"] // 2) * (POOL["W"] // 2) * 1.25) * 4)
+    others["maxpool_fwd_bwd"] = {"sec_per_step": psec, "GBps_algorithmic": bytes_alg / psec / 1e9, "cores": threads,
+                                 "sample": "full workload (fwd + bwd), 1 warm-up + 3 timed (median)",
+                                 "gpu_ms_fwd_plus_bwd": (extra or {}).get("maxpool_fwd_ms", float("nan")) +
+                                                        (extra or {}).get("maxpool_bwd_ms", float("nan"))}
+    rsec, _ = cpu_readme_step()
+    others["readme_net_step"] = {"sec_per_step": rsec, "images_per_sec": README_N / rsec, "cores": threads,
+                                 "sample": "full workload (N=256 fwd+bwd+SGD), 1 warm-up + 3 timed (median)",
+                                 "gpu_ms_per_step": (extra or {}).get("readme_net_ms_per_step")}
+    hsec, per = cpu_resnet18_hot_path()
+    others["resnet18_train_hot_path"] = {
+        "sec_per_step": hsec, "images_per_sec": 32 / hsec, "cores": threads, "per_layer_sec": per,
+        "sample": "conv + max-pool fwd+bwd of one N=32 step: each distinct conv geometry timed once (after one warm-up), "
+                  "weighted by its count; batch norm / ReLU / add / dense / optimizer not included",
+        "gpu_ms_per_whole_step": (extra or {}).get("resnet18_ms_per_step")}
+    out["other_workloads"] = others
+    return out
 
 
 def main():
@@ -322,7 +617,9 @@ def main():
     ap.add_argument("--no-cpu", action="store_true", help="skip the host-side NumPy baseline")
     ap.add_argument("--traffic-run", action="store_true",
                     help="run a short fixed kernel sequence (conv, max-pool, calibration copy) for counter collection and exit")
-    ap.add_argument("--no-extra", action="store_true", help="skip the max-pool / copy measurements")
+    ap.add_argument("--no-extra", action="store_true", help="skip the max-pool / copy / README-net / ResNet-18 measurements")
+    ap.add_argument("--per-layer", action="store_true",
+                    help="time every distinct ResNet-18 convolution (N=32) pass by pass, print one JSON line and exit")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs on one GPU only (got --gpus %d); the conv/pool path is data-parallel "
@@ -333,6 +630,9 @@ def main():
     info = be.device_info()
     if args.traffic_run:
         print(json.dumps(traffic_run(be)))
+        return
+    if args.per_layer:
+        print(json.dumps(bench_per_layer(be, max(10, args.steps // 10))))
         return
 
     ms_step, wall_ms_step, per = bench_conv(be, args.steps, args.warmup)
@@ -361,12 +661,14 @@ def main():
     }
     if not args.no_extra:
         out["extra"] = bench_pool(be, max(args.steps, 20), args.warmup)
+        be.release_cached_memory()
+        out["extra"].update(bench_readme_net(be, max(20, args.steps), args.warmup))
         out["extra"].update(bench_resnet18(be, max(5, args.steps // 5), 3))
         be.release_cached_memory()
-        out["extra"].update(bench_resnet18_infer(be, 3, 1))
+        out["extra"].update(bench_resnet18_infer(be, 3, 1, with_oracle=not args.no_cpu))
         be.release_cached_memory()
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline()
+        out["cpu_baseline"] = cpu_baseline(out.get("extra"))
     else:
         out["cpu_baseline"] = None
     print(json.dumps(out))

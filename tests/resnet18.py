@@ -4,6 +4,8 @@
 ``pool`` and ``classes`` choose the tail: the reference script uses AvgPooling2D(2) and 100 classes on 56x56
 inputs; the 224x224 benchmark configuration uses a global 7x7 average pool and 1000 classes.
 """
+import numpy as np
+
 from xshinnosuke_amd.layers import Conv2D, BatchNormalization, ReLU, MaxPooling2D, AvgPooling2D, Flatten, Dense
 from xshinnosuke_amd.nn.models import Module, Sequential
 
@@ -63,3 +65,43 @@ class ResNet18(Module):
         x = self.pool2(x)
         x = self.flat(x)
         return self.fc(x)
+
+
+def oracle_forward(net, x):
+    """ResNet-18 inference (moving-statistics batch norm) in NumPy: convolutions and the max-pool through the
+    oracle (float64 GEMM, one rounding), the rest in float64 rounded to float32 per op."""
+    import oracle            # the CPU checker: test / benchmark-baseline use only
+
+    def bn(layer, a):
+        g, b = (p.numpy().astype(np.float64).reshape(1, -1, 1, 1) for p in layer.parameters())
+        mm = layer.moving_mean.numpy().astype(np.float64).reshape(1, -1, 1, 1)
+        mv = layer.moving_variance.numpy().astype(np.float64).reshape(1, -1, 1, 1)
+        return (g * (a - mm) / np.sqrt(mv + layer.epsilon) + b).astype(np.float32)
+
+    def run(layer, a):
+        name = type(layer).__name__
+        if name == 'Sequential':
+            for sub in layer._graph:
+                a = run(sub, a)
+            return a
+        if name == 'BasicBlock':
+            out = run(layer.conv1, a) + run(layer.shortcut, a)
+            return np.maximum(out, 0)
+        if name == 'Conv2D':
+            w, b = (p.numpy() for p in layer.parameters())
+            return oracle.conv2d_fwd(a, w.astype(np.float32), b.reshape(-1).astype(np.float32), layer.stride, layer.pad_size)[0]
+        if name == 'BatchNormalization':
+            return bn(layer, a)
+        if name == 'ReLU':
+            return np.maximum(a, 0)
+        raise AssertionError(name)
+
+    a = run(net.conv1, x)
+    a = oracle.max_pool2d_fwd(a, 3, (2, 2), 1)[0]
+    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
+        a = run(stage, a)
+    k = net.pool2.kernel_size
+    n, c, h, w = a.shape
+    a = a.astype(np.float64).reshape(n, c, h // k, k, w // k, k).mean(axis=(3, 5)).astype(np.float32)
+    wfc, bfc = (p.numpy().astype(np.float64) for p in net.fc.parameters())
+    return (a.reshape(n, -1).astype(np.float64) @ wfc + bfc).astype(np.float32)

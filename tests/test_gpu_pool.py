@@ -20,6 +20,8 @@ CASES = [  # n c h w k sh sw pad
     (1, 2, 11, 13, 5, 2, 3, 2),
     (1, 1, 3, 3, 3, 1, 1, 0),        # single window
     (2, 3, 14, 10, 3, 2, 2, 1),      # W % 4 != 0 -> generic path
+    (3, 2, 6, 8, 3, 2, 2, 1),        # W % 8 == 0: eight gradient columns per thread, one thread per row pair
+    (1, 3, 4, 136, 3, 2, 2, 1),      # ... rows longer than one wavefront's 64 x 8 columns... and a lane at the wave edge
 ]
 
 

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import xshinnosuke_amd as xs
-from resnet18 import ResNet18
+from resnet18 import ResNet18, oracle_forward as _oracle_forward
 from xshinnosuke_amd.optim import SGD
 from util import rel_l2
 
@@ -135,46 +135,6 @@ def test_resnet18_steps_do_not_depend_on_the_weight_gradient_overlap(monkeypatch
     assert la == lb
     for u, v in zip(pa, pb):
         np.testing.assert_array_equal(u, v)
-
-
-def _oracle_forward(net, x):
-    """ResNet-18 inference (moving-statistics batch norm) in NumPy: convolutions and the max-pool through the
-    oracle (float64 GEMM, one rounding), the rest in float64 rounded to float32 per op."""
-    import oracle
-
-    def bn(layer, a):
-        g, b = (p.numpy().astype(np.float64).reshape(1, -1, 1, 1) for p in layer.parameters())
-        mm = layer.moving_mean.numpy().astype(np.float64).reshape(1, -1, 1, 1)
-        mv = layer.moving_variance.numpy().astype(np.float64).reshape(1, -1, 1, 1)
-        return (g * (a - mm) / np.sqrt(mv + layer.epsilon) + b).astype(np.float32)
-
-    def run(layer, a):
-        name = type(layer).__name__
-        if name == 'Sequential':
-            for sub in layer._graph:
-                a = run(sub, a)
-            return a
-        if name == 'BasicBlock':
-            out = run(layer.conv1, a) + run(layer.shortcut, a)
-            return np.maximum(out, 0)
-        if name == 'Conv2D':
-            w, b = (p.numpy() for p in layer.parameters())
-            return oracle.conv2d_fwd(a, w.astype(np.float32), b.reshape(-1).astype(np.float32), layer.stride, layer.pad_size)[0]
-        if name == 'BatchNormalization':
-            return bn(layer, a)
-        if name == 'ReLU':
-            return np.maximum(a, 0)
-        raise AssertionError(name)
-
-    a = run(net.conv1, x)
-    a = oracle.max_pool2d_fwd(a, 3, (2, 2), 1)[0]
-    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
-        a = run(stage, a)
-    k = net.pool2.kernel_size
-    n, c, h, w = a.shape
-    a = a.astype(np.float64).reshape(n, c, h // k, k, w // k, k).mean(axis=(3, 5)).astype(np.float32)
-    wfc, bfc = (p.numpy().astype(np.float64) for p in net.fc.parameters())
-    return (a.reshape(n, -1).astype(np.float64) @ wfc + bfc).astype(np.float32)
 
 
 def test_resnet18_bf16_inference_against_oracle():

@@ -21,8 +21,9 @@ def _forward_both(gpu, n, c, h, w, k, r, s, sh, sw, pad, relu, seed):
     dims = [n, c, h, w, k, r, s, sh, sw, pad]
     flags = capi.CONV_RELU if relu else 0
     y_ref, m_ref = gpu.empty((n, k, oh, ow)), gpu.empty((n, k, oh, ow), np.uint8)
-    need = capi.lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
-    ws = gpu.empty((need // 4 + 64,))
+    # a workspace of the static array's size: the library picks its kernels by the room it is given, and the same
+    # kernels give the same bits
+    ws = gpu.empty((capi.NOALLOC_SCRATCH_BYTES // 4,))
     capi.lib.call("xsmi_conv2d_fwd", x.cptr, wt.cptr, b.cptr, y_ref.cptr, m_ref.cptr if relu else None, *dims, flags,
                   ws.cptr, ws.nbytes)
     y, m = gpu.empty((n, k, oh, ow)), gpu.empty((n, k, oh, ow), np.uint8)

@@ -344,6 +344,10 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
         workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
         return xsmi::nhwc_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
                                    (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
+    if (!(flags & XSMI_CONV_BF16) && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * g.OH * g.OW, K, R, S, sh, sw) &&
+        workspace_bytes >= xsmi::sk_fwd_ws_bytes(C, K, R, S))
+        return xsmi::sk_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
+                                 (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
     if (xsmi::tap_path_ok(C))
         return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
                                   (flags & XSMI_CONV_RELU) ? 1 : 0,
@@ -394,6 +398,10 @@ int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int 
     const size_t need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_bwd_data: workspace of %zu bytes needed, %zu given",
                    need, workspace_bytes);
+    if (!(flags & XSMI_CONV_BF16) && xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw) &&
+        xsmi::sk_bwd_data_pays(N * H * W, C, R, S, sh, sw) && workspace_bytes >= xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw))
+        return xsmi::sk_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
+                                      (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
     if (xsmi::tap_path_ok(K))
         return xsmi::tap_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
                                        ((flags & XSMI_CONV_BF16) ? 1 : 0) | ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0), workspace);

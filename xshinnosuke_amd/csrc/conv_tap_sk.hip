@@ -1,0 +1,798 @@
+// Tap-major implicit-GEMM convolution (forward and backward-data), fp32 MFMA, second generation:
+// 64 x 64 outputs per wave and an even split of the launch's work over the resident workgroups.
+//
+// Same reduction order and data path as conv_tap.hip (reduction index = (tap, channel); global -> LDS
+// directly; zero border through the buffer range check), with two changes that the measurements of
+// that kernel asked for:
+//
+//  * A wave owns 64 rows x 64 pixels = 2 x 2 blocks of v_mfma_f32_32x32x2_f32.  One reduction step
+//    feeds four MFMAs from two A and two B registers, so LDS reads, global -> LDS loads, address
+//    arithmetic and workgroup barriers per MFMA are half of what the 32 x 32 wave tile needs.
+//    Workgroup tile: 128 rows x 128 pixels (2 x 2 waves), or 64 rows x 256 pixels when the layer has
+//    at most 64 rows.
+//
+//  * Work is counted in chunks (one tap x KC channels of one tile).  The launch has exactly as many
+//    workgroups as fit on the chip at once and workgroup g takes the contiguous range
+//    [g * U / G, (g + 1) * U / G) of the U chunks of all tiles, walking it as one software-pipelined
+//    stream.  Every compute unit therefore gets the same amount of matrix work whatever the tile
+//    count is (ResNet-18 at N=32 has 1.5 to 6.1 tiles of the old size per CU: up to a quarter of the
+//    machine idled in the last round of tiles).  A tile whose chunks are split between workgroups is
+//    finished by the workgroup that holds its first chunk: the others store their 64 x 64 x 4
+//    accumulators to the workspace and raise a flag, the owner adds them in ascending chunk order and
+//    runs the epilogue.  The summation order is a function of the geometry and the grid size only:
+//    results are reproducible bit for bit, there are no float atomics.
+//
+// Forward progress: a workgroup waits only for workgroups with a higher logical id, and each of those
+// stores its partial tile right after its first (at most one tile long) segment, before it can wait
+// for anything itself.  Workgroups start in id order, so whatever is resident either finishes or
+// waits for something that has already started.  The wait is bounded all the same (spin_limit).
+#include "xsmi_internal.h"
+#include <stdlib.h>
+#include <string.h>
+#include <type_traits>
+#include <utility>
+
+namespace {
+
+typedef float floatx16 __attribute__((ext_vector_type(16)));
+
+constexpr int SK_MAX_CLASSES = 4;
+constexpr int SK_MAX_GRID = 1024;           // upper bound of resident workgroups the workspace is sized for
+constexpr int SK_MAX_GRID_BIG = 768;        // ... of the kernels with 64 x 64 wave tiles (64 KB of partial tile each)
+
+// One parameter set: the layer (forward) or one residue class of a strided backward-data pass.
+struct SkClass {
+    uint32_t apk_off;      // bytes from the common packed-filter base to this class's [rowtile][chunk][quad][row][4]
+    int M, rows;
+    int nch, TR, TS;       // channel chunks per tap, taps
+    int dy0, dx0, dstep;   // input row for tap r: y * sy + dy0 + r * dstep
+    int IH, IW, sy, sx;
+    int in_n_stride;       // elements
+    uint32_t plane_bytes;
+    int OY, OX;
+    xsmi::FastDiv dOX, dOY, dIT;
+    long long os_n, os_k, o_base;
+    int os_y, os_x;
+    uint32_t first_unit;   // first chunk of the class in the launch's chunk numbering
+    uint32_t iters;        // chunks per tile = TR * TS * nch
+};
+
+struct SkParams {
+    SkClass cls[SK_MAX_CLASSES];
+    uint32_t end_unit[SK_MAX_CLASSES];     // first_unit of the next class
+    const float *in;
+    const float *apk;
+    const float *bias;
+    float *out;
+    uint8_t *mask;
+    float *part;           // [grid][64 accumulator registers][256 threads]
+    uint32_t *flags;       // [grid], zero between launches
+    uint32_t in_bytes, apk_bytes;
+    uint32_t units;        // chunks of all tiles of all classes
+    uint32_t spin_limit;
+    int ncls, rowtiles, accumulate, relu;
+};
+
+template <int N>
+using IC = std::integral_constant<int, N>;
+
+template <typename F, int... Is>
+__device__ __forceinline__ void static_for_impl(F &&f, std::integer_sequence<int, Is...>) {
+    (f(IC<Is>{}), ...);
+}
+template <int N, typename F>
+__device__ __forceinline__ void static_for(F &&f) {
+    static_for_impl(f, std::make_integer_sequence<int, N>{});
+}
+
+__device__ __forceinline__ float comp4(const float4 &v, int t) { return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w; }
+
+__device__ __forceinline__ void agent_store(float *p, float v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ float agent_load(const float *p) {
+    return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+}
+
+// ROWS x PIX outputs per 256-thread workgroup, KC reduction channels per chunk (a multiple of 16); a wave owns
+// BLK x BLK blocks of 32 x 32 (BLK = 2: the 64 x 64 wave tile described above; BLK = 1: the first-generation
+// kernel's 32 x 32 wave tile and loop body under the same even split of the work, for launches whose tiles are
+// so few that large partial tiles and the final burst of output stores would cost more than they save).
+template <int ROWS, int PIX, int KC, int BLK>
+__global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkParams sp) {
+    constexpr int WRn = ROWS / (32 * BLK), WCn = PIX / (32 * BLK);   // waves along rows / pixels
+    static_assert(WRn * WCn == 4, "four waves");
+    static_assert(BLK == 2 || KC == 32, "the 32 x 32 wave tile's loop body is written for 32-channel chunks");
+    constexpr int RT = ROWS / 64, PT = PIX / 64;     // 64-row / 64-pixel blocks of the tile (units of one wave-load)
+    constexpr int QUADS = KC / 4;                    // 16-byte channel groups of a chunk
+    constexpr int GROUPS = KC / 8;                   // BLK = 2: a group = 4 reduction steps of both lane halves = 16 MFMAs per wave
+    constexpr int A_FLOATS = ROWS * KC, B_FLOATS = PIX * KC, STAGE_FLOATS = A_FLOATS + B_FLOATS;
+    constexpr int NA = QUADS * RT / 4;               // A wave-loads (64 rows x 16 bytes) per wave and chunk
+    constexpr int NB = KC * PT / 4;                  // B wave-loads (64 pixels of one channel) per wave and chunk
+    constexpr int NI = NB + NA + 2;                  // issue items per chunk: prepare, B loads, A loads, advance
+    constexpr int NOUT = BLK * BLK;                  // accumulator blocks a lane holds of the output tile
+    static_assert(NA >= 1 && (BLK == 1 || NI <= 12 + 16 * (GROUPS - 1)), "the issue items must fit the slots of one chunk");
+    __shared__ __attribute__((aligned(16))) float smem[2][STAGE_FLOATS];
+    __shared__ float s_bias[2][ROWS];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t G = gridDim.x;
+    const uint32_t g = xsmi::xcd_contiguous_id(blockIdx.x, G);       // neighbours in chunk order share an L2
+    const uint32_t u0 = (uint32_t)(((uint64_t)g * sp.units) / G);
+    const uint32_t u1 = (uint32_t)(((uint64_t)(g + 1) * sp.units) / G);
+    const int rowtiles = sp.rowtiles;
+
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(sp.in, sp.in_bytes);
+    const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(sp.apk, sp.apk_bytes);
+    const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];
+
+    // ------------------------------------------------------------------ issue side
+    // position of the next chunk to load: unit iu; inside a tile (r, s, cc) and the packed-filter offset
+    const int pb = wave % PT;                          // pixel block (64 pixels) this wave gathers
+    const int chan0 = (wave / PT) * NB;                // first of the NB channels of a chunk this wave gathers
+    uint32_t iu = u0;
+    uint32_t i_left = 0;                               // chunks left in the segment being issued
+    int r = 0, s = 0, cc = 0;
+    int i_nch = 1, i_TS = 1, i_dstep = 0, i_IH = 0, i_IW = 0;
+    uint32_t i_plane = 0;
+    int iyb = 0, ixb = 0, nbase = 0;
+    bool live = false;
+    uint32_t ld_asoff = 0, ld_stage = lds0, ld_voff = 0, ld_soff = 0;
+    const uint32_t a_lane = (uint32_t)lane * 16u;
+
+    auto issue_segment = [&]() {                       // set up for the segment that starts at unit iu (iu < u1)
+        int ci = 0;
+        while (ci + 1 < sp.ncls && iu >= sp.end_unit[ci]) ++ci;
+        const SkClass &c = sp.cls[ci];
+        const uint32_t ul = iu - c.first_unit;
+        const uint32_t tile = xsmi::fdiv(ul, c.dIT);
+        const uint32_t ch = ul - tile * c.iters;
+        const uint32_t mt = rowtiles == 1 ? tile : tile / (uint32_t)rowtiles;
+        const uint32_t rt = rowtiles == 1 ? 0u : tile - mt * (uint32_t)rowtiles;
+        uint32_t n_seg = c.iters - ch;
+        if (n_seg > u1 - iu) n_seg = u1 - iu;
+        i_left = n_seg;
+        i_nch = c.nch; i_TS = c.TS; i_dstep = c.dstep; i_IH = c.IH; i_IW = c.IW; i_plane = c.plane_bytes;
+        const uint32_t tap = ch / (uint32_t)c.nch;
+        cc = (int)(ch - tap * (uint32_t)c.nch);
+        r = (int)(tap / (uint32_t)c.TS);
+        s = (int)(tap - (uint32_t)r * (uint32_t)c.TS);
+        ld_asoff = c.apk_off + (rt * c.iters + ch) * (uint32_t)(ROWS * KC * 4);
+        const int m = (int)mt * PIX + pb * 64 + lane;
+        live = m < c.M;
+        iyb = 0; ixb = 0; nbase = 0;
+        if (live) {
+            uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
+            int x = m - (int)q * c.OX;
+            uint32_t n = xsmi::fdiv(q, c.dOY);
+            int y = (int)q - (int)n * c.OY;
+            iyb = y * c.sy + c.dy0;
+            ixb = x * c.sx + c.dx0;
+            nbase = (int)n * c.in_n_stride;
+        }
+    };
+    auto issue_prep = [&]() {
+        int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
+        bool ok = live && (unsigned)iy < (unsigned)i_IH && (unsigned)ix < (unsigned)i_IW;
+        ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
+        ld_soff = (uint32_t)(cc * KC + chan0) * i_plane;
+    };
+    auto issue_b = [&](int e) {                        // channel chan0 + e of the chunk, this wave's 64 pixels
+        xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((A_FLOATS + (chan0 + e) * PIX + pb * 64) * 4), ld_voff,
+                           ld_soff + (uint32_t)e * i_plane);
+    };
+    auto issue_a = [&](int e) {                        // 64 rows of one quad
+        const int f = wave * NA + e, q = f / RT, rh = f % RT;
+        const uint32_t off = (uint32_t)((q * ROWS + rh * 64) * 16);
+        xsmi::load_lds_b128(rap, ld_stage + off, a_lane + off, ld_asoff);
+    };
+    auto issue_advance = [&]() {
+        ld_stage = ld_stage == lds0 ? lds0 + (uint32_t)(STAGE_FLOATS * 4) : lds0;
+        if (i_left == 0) return;                       // past the end of the range: dummy chunks, nothing to advance
+        ++iu;
+        ld_asoff += (uint32_t)(ROWS * KC * 4);
+        if (++cc == i_nch) {
+            cc = 0;
+            if (++s == i_TS) { s = 0; ++r; }
+        }
+        if (--i_left == 0) {
+            if (iu < u1) {
+                issue_segment();
+            } else {
+                // Past the range every chunk still runs the full loop body; its loads are given no live pixel
+                // (they touch no memory and fill the stage with zeros) and re-read the first filter block.
+                live = false; ld_asoff = 0; r = 0; s = 0; cc = 0;
+            }
+        }
+    };
+    auto issue_item = [&](auto ic) {
+        constexpr int n = decltype(ic)::value;
+        if constexpr (n == 0) issue_prep();
+        else if constexpr (n >= 1 && n <= NB) issue_b(n - 1);
+        else if constexpr (n > NB && n <= NB + NA) issue_a(n - 1 - NB);
+        else if constexpr (n == NB + NA + 1) issue_advance();
+    };
+    auto issue_all = [&]() { static_for<NI>([&](auto ic) { issue_item(ic); }); };
+
+    // ------------------------------------------------------------------ multiply side
+    // BLK = 2: acc[2 i + j] is block (i, j).  BLK = 1: two accumulators take alternate reduction steps of the one
+    // block and are added when a segment ends.
+    constexpr int NACC = BLK == 2 ? 4 : 2;
+    floatx16 acc[NACC];
+    auto zero_acc = [&]() {
+#pragma unroll
+        for (int a = 0; a < NACC; ++a)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[a][v] = 0.f;
+    };
+    zero_acc();
+    const int h = lane >> 5, l31 = lane & 31;
+    const int wr = wave / WCn, wc = wave % WCn;
+    // lane half h takes channels (KC/2) h .. of a chunk: quad (KC/8) h + group, channel (KC/2) h + 4 group + step
+    const int a_rd = ((GROUPS * h) * ROWS + wr * (32 * BLK) + l31) * 4;
+    const int b_rd = A_FLOATS + (KC / 2) * h * PIX + wc * (32 * BLK) + l31;
+    // BLK = 2: fragments of one group, two buffers.  BLK = 1: fragments of a whole chunk, two buffers.
+    float4 fa[2][BLK == 2 ? 2 : 4];                    // BLK = 2: [buffer][row block]; BLK = 1: [buffer][quad]
+    float fb[2][BLK == 2 ? 8 : 16];                    // BLK = 2: [buffer][2 step + pixel block]; BLK = 1: [buffer][channel]
+    int rd_off = 0;                                    // float offset of the stage the fragments are read from
+    auto read_item = [&](auto rt_, auto buf_, auto grp_) {          // BLK = 2 only
+        constexpr int n = decltype(rt_)::value, bf = decltype(buf_)::value, gn = decltype(grp_)::value;
+        const float *base = &smem[0][0] + rd_off;
+        if constexpr (n < 2) {
+            fa[bf][n] = *reinterpret_cast<const float4 *>(base + a_rd + (gn * ROWS + 32 * n) * 4);
+        } else {
+            constexpr int st = n - 2;
+            fb[bf][2 * st] = base[b_rd + (4 * gn + st) * PIX];
+            fb[bf][2 * st + 1] = base[b_rd + (4 * gn + st) * PIX + 32];
+        }
+    };
+
+    // compute-side cursor
+    uint32_t cu = u0;
+    uint32_t c_left = 0;                               // chunks left in the current segment
+    int c_ci = 0, c_m0 = 0, c_rt = 0;
+    bool c_head = false, c_complete = false;           // segment holds the tile's first chunk / its last chunk
+    uint32_t c_tile_end = 0;                           // unit after the tile's last chunk
+    int bias_buf = 0;
+    bool flag_pending = false;                         // a partial tile has been stored, its flag not raised yet
+    auto compute_segment = [&]() {
+        int ci = 0;
+        while (ci + 1 < sp.ncls && cu >= sp.end_unit[ci]) ++ci;
+        const SkClass &c = sp.cls[ci];
+        const uint32_t ul = cu - c.first_unit;
+        const uint32_t tile = xsmi::fdiv(ul, c.dIT);
+        const uint32_t ch = ul - tile * c.iters;
+        const uint32_t mt = rowtiles == 1 ? tile : tile / (uint32_t)rowtiles;
+        const uint32_t rt = rowtiles == 1 ? 0u : tile - mt * (uint32_t)rowtiles;
+        uint32_t n_seg = c.iters - ch;
+        if (n_seg > u1 - cu) n_seg = u1 - cu;
+        c_left = n_seg;
+        c_ci = ci; c_m0 = (int)mt * PIX; c_rt = (int)rt;
+        c_head = ch == 0;
+        c_complete = ch + n_seg == c.iters;
+        c_tile_end = cu + (c.iters - ch);
+        // the tile's bias goes through the LDS (one coalesced load); the chunk loop's barriers publish it
+        bias_buf ^= 1;
+        if (sp.bias && c_head && t < ROWS) s_bias[bias_buf][t] = c_rt * ROWS + t < c.rows ? sp.bias[c_rt * ROWS + t] : 0.f;
+    };
+
+    // accumulator register v of lane l in block (i, j): row 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, pixel 32 j + l % 32
+    auto store_tile = [&]() {
+        const SkClass &c = sp.cls[c_ci];
+        const int lrow = wr * (32 * BLK) + 4 * h;
+        const int rbase = c_rt * ROWS + lrow;
+#pragma unroll
+        for (int j = 0; j < BLK; ++j) {
+            const int m = c_m0 + wc * (32 * BLK) + 32 * j + l31;
+            if (m >= c.M) continue;
+            uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
+            int x = m - (int)q * c.OX;
+            uint32_t n = xsmi::fdiv(q, c.dOY);
+            int y = (int)q - (int)n * c.OY;
+            const long long pix_off = (long long)n * c.os_n + (long long)y * c.os_y + (long long)x * c.os_x + c.o_base;
+#pragma unroll
+            for (int i = 0; i < BLK; ++i)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) {
+                    const int ro = 32 * i + 8 * (v >> 2) + (v & 3);
+                    if (rbase + ro < c.rows) {
+                        float val = acc[i * BLK + j][v];
+                        if (sp.bias) val += s_bias[bias_buf][lrow + ro];
+                        long long o = pix_off + (long long)(rbase + ro) * c.os_k;
+                        if (sp.relu) {
+                            if (sp.mask) sp.mask[o] = val < 0.f ? 1 : 0;
+                            val = val > 0.f ? val : 0.f;
+                        }
+                        if (sp.accumulate) val += sp.out[o];
+                        sp.out[o] = val;
+                    }
+                }
+        }
+    };
+    auto end_segment = [&]() {
+        if constexpr (BLK == 1) acc[0] += acc[1];
+        if (!c_head) {
+            // not this workgroup's tile: hand the accumulators to the workgroup that holds the tile's first chunk
+            float *dst = sp.part + (size_t)g * (NOUT * 16 * 256) + t;
+#pragma unroll
+            for (int a = 0; a < NOUT; ++a)
+#pragma unroll
+                for (int v = 0; v < 16; ++v) agent_store(dst + (a * 16 + v) * 256, acc[a][v]);
+            if (cu < u1) {
+                // More chunks follow: the next chunk's body waits for all outstanding memory operations of every wave
+                // (vmcnt(0), then the workgroup barrier) before it reads the next stage, which covers these stores;
+                // the flag is raised after that body instead of stalling the workgroup for the write-through here.
+                flag_pending = true;
+            } else {
+                xsmi::wait_vmcnt<0>();                 // this thread's stores have been written through
+                __syncthreads();                       // ... and everybody else's
+                if (t == 0) __hip_atomic_store(sp.flags + g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+            return;
+        }
+        if (!c_complete) {
+            // the rest of the tile was multiplied by the workgroups that follow: add their parts in chunk order
+            for (uint32_t j = g + 1; j < G; ++j) {
+                const uint32_t js = (uint32_t)(((uint64_t)j * sp.units) / G);
+                if (js >= c_tile_end) break;
+                if (t == 0) {
+                    uint32_t spins = 0;
+                    while (__hip_atomic_load(sp.flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u &&
+                           ++spins < sp.spin_limit)
+                        __builtin_amdgcn_s_sleep(2);
+                }
+                __syncthreads();
+                const float *src = sp.part + (size_t)j * (NOUT * 16 * 256) + t;
+#pragma unroll
+                for (int a = 0; a < NOUT; ++a)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) acc[a][v] += agent_load(src + (a * 16 + v) * 256);
+                __syncthreads();                       // everybody has read the part before its flag is cleared
+                if (t == 0) __hip_atomic_store(sp.flags + j, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            }
+        }
+        store_tile();
+    };
+    auto chunk_done = [&]() {
+        if (flag_pending) {                            // uniform: the partial tile stored before this chunk is complete
+            flag_pending = false;
+            if (t == 0) __hip_atomic_store(sp.flags + g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        ++cu;
+        if (--c_left == 0) {
+            end_segment();
+            zero_acc();
+            if (cu < u1) compute_segment();
+        }
+    };
+
+    const uint32_t total = u1 - u0;
+    if (total == 0) return;
+#define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
+#define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
+    if constexpr (BLK == 2) {
+        // One group = 16 MFMAs on the fragments in buffer `g & 1`.  Each MFMA is followed in program order by at most
+        // one LDS fragment read of the next group and one issue item of the chunk after next, so that this work enters
+        // the pipes while the matrix unit is busy; sched_barrier pins the order.  In the chunk's last group the first
+        // four MFMAs are followed by the wait for the next chunk's loads and the workgroup barrier: after it every wave
+        // has all fragments of the current chunk in registers, so the current stage is free for the chunk after next,
+        // and the next chunk's first group can be read.
+        auto group = [&](auto gt) {
+            constexpr int gi = decltype(gt)::value;
+            constexpr int cur = gi & 1, nxt = cur ^ 1;
+            constexpr bool last = gi == GROUPS - 1;
+            static_for<16>([&](auto kt) {
+                constexpr int k = decltype(kt)::value;
+                constexpr int st = k >> 2, i = (k >> 1) & 1, j = k & 1;
+                XSMI_MFMA(acc[2 * i + j], comp4(fa[cur][i], st), fb[cur][2 * st + j]);
+                if constexpr (last && k == 3) {
+                    XSMI_PIN();
+                    xsmi::wait_vmcnt<0>();
+                    xsmi::wait_lgkmcnt0();             // this wave's fragment reads of the current stage have returned
+                    xsmi::block_barrier();
+                    rd_off = STAGE_FLOATS - rd_off;
+                    XSMI_PIN();
+                }
+                constexpr int rbase = last ? 4 : 0;
+                if constexpr (k >= rbase && k < rbase + 6) read_item(IC<k - rbase>{}, IC<nxt>{}, IC<(last ? 0 : gi + 1)>{});
+                constexpr int item = last ? k - 4 : 12 + 16 * gi + k;
+                if constexpr (item >= 0 && item < NI) issue_item(IC<item>{});
+                XSMI_PIN();
+            });
+        };
+        // prologue: chunk 0 of the range landed and its first group in registers; of chunk 1 the issue items that the
+        // last group of a loop iteration would have issued (the loop's first groups issue the rest)
+        issue_segment();
+        issue_all();
+        static_for<12>([&](auto ic) { issue_item(ic); });
+        compute_segment();
+        constexpr int EARLY_LOADS = NB + NA < 11 ? NB + NA : 11;     // loads among the items 1..11 of chunk 1
+        xsmi::wait_vmcnt<EARLY_LOADS>();
+        xsmi::block_barrier();
+        static_for<6>([&](auto n) { read_item(n, IC<0>{}, IC<0>{}); });
+        for (uint32_t k = 0; k < total; ++k) {
+            static_for<GROUPS>([&](auto gt) { group(gt); });
+            chunk_done();
+        }
+    } else {
+        // The first-generation loop body: the fragments of two consecutive chunks live in registers.  A chunk is 16
+        // MFMAs on the current fragments; after the first four it waits for the next chunk and crosses the barrier
+        // (every wave then holds the current chunk in registers, so its stage is free), and every later MFMA is
+        // followed by one slice of the remaining work: LDS fragment reads of the next chunk, LDS-direct loads of the
+        // chunk after next.
+        static_assert(BLK == 2 || (NB == 8 && NA == 2), "32 x 32 wave tile: 64 x 64 workgroup tile, 32-channel chunks");
+        auto read_chunk = [&](auto buf_) {
+            constexpr int bf = decltype(buf_)::value;
+            const float *base = &smem[0][0] + rd_off;
+#pragma unroll
+            for (int q4 = 0; q4 < 4; ++q4) fa[bf][q4] = *reinterpret_cast<const float4 *>(base + a_rd + q4 * ROWS * 4);
+#pragma unroll
+            for (int jj = 0; jj < 16; ++jj) fb[bf][jj] = base[b_rd + jj * PIX];
+        };
+        auto body = [&](auto buf_) {
+            constexpr int cur = decltype(buf_)::value, nxt = cur ^ 1;
+            XSMI_MFMA(acc[0], fa[cur][0].x, fb[cur][0]);
+            XSMI_MFMA(acc[1], fa[cur][0].y, fb[cur][1]);
+            XSMI_MFMA(acc[0], fa[cur][0].z, fb[cur][2]);
+            XSMI_MFMA(acc[1], fa[cur][0].w, fb[cur][3]);
+            XSMI_PIN();
+            xsmi::wait_vmcnt<0>();
+            xsmi::block_barrier();
+            rd_off = STAGE_FLOATS - rd_off;
+            XSMI_PIN();
+            const float *base = &smem[0][0] + rd_off;
+            XSMI_MFMA(acc[0], fa[cur][1].x, fb[cur][4]);
+            fa[nxt][0] = *reinterpret_cast<const float4 *>(base + a_rd);
+            issue_item(IC<0>{});
+            XSMI_PIN();
+            XSMI_MFMA(acc[1], fa[cur][1].y, fb[cur][5]);
+            fa[nxt][1] = *reinterpret_cast<const float4 *>(base + a_rd + ROWS * 4);
+            issue_item(IC<1>{});
+            XSMI_PIN();
+            XSMI_MFMA(acc[0], fa[cur][1].z, fb[cur][6]);
+            fa[nxt][2] = *reinterpret_cast<const float4 *>(base + a_rd + 2 * ROWS * 4);
+            issue_item(IC<2>{});
+            XSMI_PIN();
+            XSMI_MFMA(acc[1], fa[cur][1].w, fb[cur][7]);
+            fa[nxt][3] = *reinterpret_cast<const float4 *>(base + a_rd + 3 * ROWS * 4);
+            issue_item(IC<3>{});
+            XSMI_PIN();
+#define XSMI_SLOT(A, AV, J)                                           \
+            XSMI_MFMA(acc[A], AV, fb[cur][J]);                       \
+            fb[nxt][2 * (J - 8)] = base[b_rd + (2 * (J - 8)) * PIX];     \
+            fb[nxt][2 * (J - 8) + 1] = base[b_rd + (2 * (J - 8) + 1) * PIX]; \
+            issue_item(IC<J - 4>{});                                 \
+            XSMI_PIN();
+            XSMI_SLOT(0, fa[cur][2].x, 8)
+            XSMI_SLOT(1, fa[cur][2].y, 9)
+            XSMI_SLOT(0, fa[cur][2].z, 10)
+            XSMI_SLOT(1, fa[cur][2].w, 11)
+            XSMI_SLOT(0, fa[cur][3].x, 12)
+            XSMI_SLOT(1, fa[cur][3].y, 13)
+            XSMI_SLOT(0, fa[cur][3].z, 14)
+            XSMI_SLOT(1, fa[cur][3].w, 15)
+#undef XSMI_SLOT
+        };
+        // prologue: chunk 0 landed and in registers, chunk 1 in flight
+        issue_segment();
+        issue_all();
+        compute_segment();
+        xsmi::wait_vmcnt<0>();
+        xsmi::block_barrier();
+        read_chunk(IC<0>{});
+        issue_all();
+        for (uint32_t k = 0; k < total; k += 2) {
+            body(IC<0>{});
+            chunk_done();
+            if (k + 1 < total) {
+                body(IC<1>{});
+                chunk_done();
+            }
+        }
+    }
+#undef XSMI_MFMA
+#undef XSMI_PIN
+    xsmi::wait_vmcnt<0>();                             // the dummy chunks' loads target this workgroup's LDS
+}
+
+// ---- filter layout --------------------------------------------------------------------------------------------
+// [rowtile][chunk = tap * nch + cc][quad KC/4][row ROWS][4 channels]: the LDS image of a stage's A part.
+// mode 0 (forward): A[row][tap = (r, s)][ch] = w[row][ch][r][s].
+// mode 1 (backward-data class): A[row = c][tap = (t, u)][ch = k] = w[k][c][r0 + sh t][s0 + sw u].
+struct SkPackJob {
+    float *apk;
+    int TR, TS, r0, s0;
+};
+struct SkPackMulti {
+    SkPackJob job[SK_MAX_CLASSES];
+    uint32_t first[SK_MAX_CLASSES + 1];
+    int njobs;
+};
+__global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ w, SkPackMulti pm, uint32_t *__restrict__ flags,
+                                                       int nflags, int mode, int rows, int CH, int R, int S, int sh, int sw,
+                                                       int rowtiles, int ROWS, int KC) {
+    // the flags of the multiply kernel start at zero (it also leaves them at zero)
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < nflags; i += gridDim.x * 256) flags[i] = 0;
+    int ji = 0;
+    while (ji + 1 < pm.njobs && blockIdx.x >= pm.first[ji + 1]) ++ji;
+    const SkPackJob &j = pm.job[ji];
+    const uint32_t blk = blockIdx.x - pm.first[ji], nblk = pm.first[ji + 1] - pm.first[ji];
+    float *__restrict__ apk = j.apk;
+    const int TR = j.TR, TS = j.TS, r0 = j.r0, s0 = j.s0;
+    const int nch = CH / KC;
+    const int iters = TR * TS * nch;
+    const size_t total4 = (size_t)rowtiles * iters * ROWS * (KC / 4);          // float4 groups
+    for (size_t i = (size_t)blk * 256 + threadIdx.x; i < total4; i += (size_t)nblk * 256) {
+        const int rr = (int)(i % ROWS);
+        size_t rest = i / ROWS;
+        const int q = (int)(rest % (KC / 4));
+        rest /= (KC / 4);
+        const int it = (int)(rest % iters);
+        const int rt = (int)(rest / iters);
+        const int cc = it % nch, tap = it / nch;
+        const int tr = tap / TS, ts = tap % TS;
+        const int ch = cc * KC + q * 4;
+        const int row = rt * ROWS + rr;
+        float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+        if (row < rows) {
+            const size_t cstride = mode == 0 ? (size_t)R * S : (size_t)rows * R * S;
+            const float *src = mode == 0 ? w + (((size_t)row * CH + ch) * R + tr) * S + ts
+                                         : w + (((size_t)ch * rows + row) * R + (r0 + sh * tr)) * S + (s0 + sw * ts);
+            v = make_float4(src[0], src[cstride], src[2 * cstride], src[3 * cstride]);
+        }
+        reinterpret_cast<float4 *>(apk)[i] = v;
+    }
+}
+
+struct SkShape { int rows_tile, pix_tile, kc, blk; };
+int sk_env() {
+    static int v = -1;
+    if (v < 0) {
+        const char *e = getenv("XSMI_TAP_SK");
+        v = e ? atoi(e) : 1;
+    }
+    return v;
+}
+// 64 x 64 tiles with 32 x 32 per wave by default; XSMI_TAP_SK=2 selects the 64 x 64 wave tile
+// (128 x 128 tiles, or 64 x 256 for layers of at most 64 rows)
+SkShape sk_shape(int rows) {
+    if (sk_env() == 2) {
+        if (rows <= 64) return SkShape{64, 256, 16, 2};
+        return SkShape{128, 128, 32, 2};
+    }
+    return SkShape{64, 64, 32, 1};
+}
+
+size_t sk_pack_bytes(int rows, int CH, int taps, const SkShape &sh) {
+    return xsmi::align_up((size_t)xsmi::ceil_div(rows, sh.rows_tile) * taps * (CH / sh.kc) * sh.rows_tile * sh.kc * sizeof(float), 256);
+}
+constexpr size_t SK_FLAG_BYTES = (size_t)SK_MAX_GRID * 4;
+constexpr size_t SK_PART_BYTES = (size_t)SK_MAX_GRID_BIG * 64 * 256 * sizeof(float);     // >= SK_MAX_GRID x 16 KB
+
+// resident workgroups of the kernel variant (occupancy x compute units), cached per variant
+template <typename K>
+int sk_resident(K kernel, int *cache, int cap) {
+    if (*cache == 0) {
+        int per_cu = 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, 0) != hipSuccess || per_cu < 1) per_cu = 1;
+        int gsz = per_cu * xsmi::cu_count();
+        if (gsz > cap) gsz = cap;
+        *cache = gsz & ~7;
+        if (*cache < 8) *cache = 8;
+    }
+    return *cache;
+}
+
+int sk_launch(hipStream_t st, SkParams &p, const SkShape &shp) {
+    static int res_a = 0, res_b = 0, res_c = 0;
+    int resident;
+    if (shp.blk == 1) resident = sk_resident(tap_sk_f32_kernel<64, 64, 32, 1>, &res_c, SK_MAX_GRID);
+    else if (shp.rows_tile == 64) resident = sk_resident(tap_sk_f32_kernel<64, 256, 16, 2>, &res_a, SK_MAX_GRID_BIG);
+    else resident = sk_resident(tap_sk_f32_kernel<128, 128, 32, 2>, &res_b, SK_MAX_GRID_BIG);
+    uint32_t gsz = (uint32_t)resident;
+    if (gsz > p.units) gsz = p.units;                  // every workgroup gets at least one chunk
+    if (gsz == 0) return XSMI_OK;
+    static long spin = -1;
+    if (spin < 0) {
+        const char *e = getenv("XSMI_SK_SPIN_LIMIT");
+        spin = e ? atol(e) : (1L << 22);
+    }
+    p.spin_limit = (uint32_t)spin;
+    if (shp.blk == 1) hipLaunchKernelGGL((tap_sk_f32_kernel<64, 64, 32, 1>), dim3(gsz), dim3(256), 0, st, p);
+    else if (shp.rows_tile == 64) hipLaunchKernelGGL((tap_sk_f32_kernel<64, 256, 16, 2>), dim3(gsz), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL((tap_sk_f32_kernel<128, 128, 32, 2>), dim3(gsz), dim3(256), 0, st, p);
+    XSMI_LAUNCH_CHECK("tap_sk_f32_kernel");
+    return XSMI_OK;
+}
+
+}  // namespace
+
+namespace xsmi {
+
+// Usable when the reduction channels split into whole chunks of the tile shape.
+bool sk_path_ok(int reduce_channels, int rows) {
+    if (!sk_env()) return false;
+    const SkShape s = sk_shape(rows);
+    return reduce_channels % s.kc == 0 && reduce_channels % 32 == 0;
+}
+
+// Where the even split pays (measured on ResNet-18's layers at N=32 against the first-generation kernels, whose
+// workgroups take whole tiles): the exchange of partial tiles and the simultaneous end of all workgroups cost about
+// 5 us per launch, which is won back when whole tiles leave compute units idle (no more tiles than CUs: 512 -> 512
+// at 7 x 7, +17 %) or a last, mostly empty round (three or more tiles per CU: 64 -> 64 at 56 x 56, +6 %), and by
+// every strided backward-data pass, whose four residue classes of different lengths then share one balanced
+// launch (+20 to +26 %).  Strided forwards and 1 x 1 filters (a handful of chunks per tile) stay on whole tiles.
+bool sk_fwd_pays(int M, int rows, int R, int S, int sh, int sw) {
+    if (sk_env() >= 3) return true;                    // forced, for tests and measurements
+    if (sh != 1 || sw != 1 || R * S < 4) return false;
+    const long long tiles = (long long)ceil_div(M, 64) * ceil_div(rows, 64);
+    const int cus = cu_count() > 0 ? cu_count() : 256;
+    return tiles <= cus || tiles >= 3LL * cus;
+}
+bool sk_bwd_data_pays(int M, int rows, int R, int S, int sh, int sw) {
+    if (sk_env() >= 3) return true;
+    if (R * S < 4) return false;
+    if (sh == 1 && sw == 1) return sk_fwd_pays(M, rows, R, S, 1, 1);
+    return true;
+}
+
+size_t sk_fwd_ws_bytes(int C, int K, int R, int S) {
+    return sk_pack_bytes(K, C, R * S, sk_shape(K)) + SK_FLAG_BYTES + SK_PART_BYTES;
+}
+
+size_t sk_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
+    const SkShape s = sk_shape(C);
+    size_t total = 0;
+    for (int ph = 0; ph < sh; ++ph)
+        for (int pw = 0; pw < sw; ++pw) total += sk_pack_bytes(C, K, ceil_div(R, sh) * ceil_div(S, sw), s);
+    return total + SK_FLAG_BYTES + SK_PART_BYTES;
+}
+
+static void sk_fill_class(SkClass &c, const SkShape &shp, int rowtiles) {
+    c.iters = (uint32_t)(c.TR * c.TS * c.nch);
+    c.dIT = make_fastdiv(c.iters ? c.iters : 1);
+    (void)shp; (void)rowtiles;
+}
+
+int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace) {
+    hipStream_t st = stream();
+    const SkShape shp = sk_shape(K);
+    const int rowtiles = ceil_div(K, shp.rows_tile);
+    const size_t pack = sk_pack_bytes(K, C, R * S, shp);
+    float *apk = (float *)workspace;
+    uint32_t *flags = (uint32_t *)((char *)workspace + pack);
+    float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
+    if (!(opts & 2)) {
+        SkPackMulti pm;
+        pm.njobs = 1;
+        pm.job[0] = SkPackJob{apk, R, S, 0, 0};
+        size_t total4 = pack / 16;
+        uint32_t nb = (uint32_t)((total4 + 255) / 256);
+        if (nb > 4096) nb = 4096;
+        if (nb < 4) nb = 4;
+        pm.first[0] = 0; pm.first[1] = nb;
+        hipLaunchKernelGGL(sk_pack_kernel, dim3(nb), dim3(256), 0, st, w, pm, flags, SK_MAX_GRID, 0, K, C, R, S, 1, 1, rowtiles,
+                           shp.rows_tile, shp.kc);
+        XSMI_LAUNCH_CHECK("sk_pack_kernel");
+    }
+    SkParams p;
+    memset(&p, 0, sizeof(p));
+    SkClass &c = p.cls[0];
+    c.apk_off = 0;
+    c.M = N * OH * OW; c.rows = K; c.nch = C / shp.kc; c.TR = R; c.TS = S;
+    c.dy0 = -pad; c.dx0 = -pad; c.dstep = 1;
+    c.IH = H; c.IW = W; c.sy = sh; c.sx = sw;
+    c.in_n_stride = C * H * W; c.plane_bytes = (uint32_t)(H * W * 4);
+    c.OY = OH; c.OX = OW; c.dOX = make_fastdiv(OW); c.dOY = make_fastdiv(OH);
+    c.os_n = (long long)K * OH * OW; c.os_k = (long long)OH * OW; c.o_base = 0; c.os_y = OW; c.os_x = 1;
+    sk_fill_class(c, shp, rowtiles);
+    c.first_unit = 0;
+    const uint32_t tiles = (uint32_t)ceil_div(c.M, shp.pix_tile) * (uint32_t)rowtiles;
+    p.units = tiles * c.iters;
+    p.end_unit[0] = p.units;
+    p.in = x; p.apk = apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
+    p.part = part; p.flags = flags;
+    p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
+    p.apk_bytes = (uint32_t)pack;
+    p.ncls = 1; p.rowtiles = rowtiles; p.accumulate = 0; p.relu = relu;
+    prof_begin();
+    int rc = sk_launch(st, p, shp);
+    prof_end();
+    return rc;
+}
+
+int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
+                     int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace) {
+    hipStream_t st = stream();
+    const SkShape shp = sk_shape(C);
+    const int rowtiles = ceil_div(C, shp.rows_tile);
+    SkClass plans[SK_MAX_CLASSES];
+    SkPackJob jobs[SK_MAX_CLASSES];
+    int nplans = 0;
+    size_t off = 0;
+    for (int ph = 0; ph < sh; ++ph) {
+        const int OYc = ph < H ? ceil_div(H - ph, sh) : 0;
+        const int r0 = (ph + pad) % sh;
+        const int T = r0 < R ? ceil_div(R - r0, sh) : 0;
+        const int cy = (ph + pad - r0) / sh;
+        for (int pw = 0; pw < sw; ++pw) {
+            const int OXc = pw < W ? ceil_div(W - pw, sw) : 0;
+            if (OYc == 0 || OXc == 0) continue;
+            if (nplans == SK_MAX_CLASSES) return set_error("sk_conv_bwd_data: more than %d residue classes", SK_MAX_CLASSES), XSMI_ERR_INVALID;
+            const int s0 = (pw + pad) % sw;
+            const int U = s0 < S ? ceil_div(S - s0, sw) : 0;
+            const int cx = (pw + pad - s0) / sw;
+            SkClass c;
+            memset(&c, 0, sizeof(c));
+            c.apk_off = (uint32_t)off;
+            jobs[nplans] = SkPackJob{(float *)((char *)workspace + off), T, U, r0, s0};
+            off += sk_pack_bytes(C, K, T * U, shp);
+            c.M = N * OYc * OXc; c.rows = C; c.nch = K / shp.kc; c.TR = T; c.TS = U;
+            c.dy0 = cy; c.dx0 = cx; c.dstep = -1;
+            c.IH = OH; c.IW = OW; c.sy = 1; c.sx = 1;
+            c.in_n_stride = K * OH * OW; c.plane_bytes = (uint32_t)(OH * OW * 4);
+            c.OY = OYc; c.OX = OXc; c.dOX = make_fastdiv(OXc); c.dOY = make_fastdiv(OYc);
+            c.os_n = (long long)C * H * W; c.os_k = (long long)H * W; c.o_base = (long long)ph * W + pw;
+            c.os_y = sh * W; c.os_x = sw;
+            sk_fill_class(c, shp, rowtiles);
+            plans[nplans++] = c;
+        }
+    }
+    const size_t pack = off;
+    uint32_t *flags = (uint32_t *)((char *)workspace + pack);
+    float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
+    if (!(opts & 2)) {
+        SkPackMulti pm;
+        pm.njobs = nplans;
+        uint32_t blocks = 0;
+        for (int i = 0; i < nplans; ++i) {
+            size_t total4 = sk_pack_bytes(C, K, plans[i].TR * plans[i].TS, shp) / 16;
+            uint32_t nb = (uint32_t)((total4 + 255) / 256);
+            if (nb > 2048) nb = 2048;
+            if (nb < 1) nb = 1;
+            pm.job[i] = jobs[i];
+            pm.first[i] = blocks;
+            blocks += nb;
+        }
+        pm.first[nplans] = blocks;
+        hipLaunchKernelGGL(sk_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, flags, SK_MAX_GRID, 1, C, K, R, S, sh, sw,
+                           rowtiles, shp.rows_tile, shp.kc);
+        XSMI_LAUNCH_CHECK("sk_pack_kernel");
+    }
+    SkParams p;
+    memset(&p, 0, sizeof(p));
+    uint32_t units = 0;
+    int ncls = 0;
+    for (int i = 0; i < nplans; ++i) {
+        SkClass c = plans[i];
+        // A class without taps (a stride larger than the filter) multiplies nothing: its outputs are zero (or kept,
+        // when accumulating).  It gets one all-zero chunk per tile so that the epilogue runs: not needed for the
+        // layers this path serves (filter >= stride), so such geometries stay on the first-generation kernels.
+        if (c.iters == 0) return set_error("sk_conv_bwd_data: residue class without taps"), XSMI_ERR_INVALID;
+        c.first_unit = units;
+        units += (uint32_t)ceil_div(c.M, shp.pix_tile) * (uint32_t)rowtiles * c.iters;
+        p.end_unit[ncls] = units;
+        p.cls[ncls++] = c;
+    }
+    for (int i = ncls; i < SK_MAX_CLASSES; ++i) p.end_unit[i] = units;
+    p.units = units;
+    p.in = dy; p.apk = (const float *)workspace; p.bias = nullptr; p.out = dx; p.mask = nullptr;
+    p.part = part; p.flags = flags;
+    p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
+    p.apk_bytes = (uint32_t)pack;
+    p.ncls = ncls; p.rowtiles = rowtiles; p.accumulate = accumulate; p.relu = 0;
+    prof_begin();
+    int rc = sk_launch(st, p, shp);
+    prof_end();
+    return rc;
+}
+
+// backward-data geometries the second-generation kernel serves: every residue class has at least one tap
+bool sk_bwd_data_ok(int C, int K, int R, int S, int sh, int sw) {
+    return sk_path_ok(K, C) && sh * sw <= SK_MAX_CLASSES && R >= sh && S >= sw;
+}
+
+}  // namespace xsmi

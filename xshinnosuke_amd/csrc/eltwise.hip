@@ -74,6 +74,15 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
     size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     size_t m = a > b ? a : b;
     m = m > c ? m : c;
+    // the second-generation fp32 kernels are chosen when the workspace also has room for their partial tiles
+    if (xsmi::sk_path_ok(C, K)) {
+        size_t e = xsmi::sk_fwd_ws_bytes(C, K, R, S);
+        m = m > e ? m : e;
+    }
+    if (xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw)) {
+        size_t e = xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw);
+        m = m > e ? m : e;
+    }
     // the bf16 forward takes its fastest form when the workspace also holds a channels-last copy of x
     if (xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad)) {
         size_t d = xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad);
@@ -115,10 +124,10 @@ int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w, float *dx, 
     const bool beside = async || tiles <= xsmi::cu_count();
     int rc = beside ? xsmi::side_begin() : xsmi::side_join();    // in main-stream order: after any earlier async work
     if (rc) return rc;
-    rc = xsmi_conv2d_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, beta_dw, kflags, workspace_dw, weight_need);
+    rc = xsmi_conv2d_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, beta_dw, kflags, workspace_dw, workspace_dw_bytes);
     if (beside) xsmi::side_end();
     if (rc == XSMI_OK)
-        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, kflags, workspace, data_need);
+        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, kflags, workspace, workspace_bytes);
     const int rj = (beside && !async) || rc ? xsmi::side_join() : XSMI_OK;
     return rc ? rc : rj;
 }

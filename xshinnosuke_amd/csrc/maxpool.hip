@@ -58,24 +58,24 @@ __global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restri
 
 // 3x3 window, stride 2, pad 1, W % 4 == 0 (so OW = W/2): one thread produces two
 // adjacent outputs of one row from float4 loads of columns [4j, 4j+3] of the
-// three input rows, so a wavefront's loads are contiguous.  Column 4j-1 comes
-// from the previous lane (or one scalar load at a wavefront edge, or the zero
-// border at j == 0).  All loads are issued before the first comparison so that
-// their latencies overlap.  x is fetched once per window row; the row shared by
+// three input rows, so a wavefront's loads are contiguous.  Column 4j-1 is one
+// more dword load per row (the previous lane's cache line; the zero border at
+// j == 0): taking it from the previous lane's registers instead needs a
+// divergent extra load at every wavefront edge, a second memory round trip that
+// the whole wave waits for (measured 4 us of 33 in the backward kernel).  All
+// loads are issued before the first comparison so that their latencies overlap.  x is fetched once per window row; the row shared by
 // vertically adjacent windows is re-read from cache.
 __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restrict__ x, float *__restrict__ y,
                                                             uint8_t *__restrict__ idx, PoolGeom g,
                                                             xsmi::FastDiv dQ, uint32_t total_pairs) {
     uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    const bool live = t < total_pairs;
-    if (!live) t = total_pairs - 1;          // keep the lane for the shuffles below
+    if (t >= total_pairs) return;
     const int Q = g.OW >> 1;                 // output pairs per row == float4 per input row
     uint32_t row = xsmi::fdiv(t, dQ);        // (nc, oh)
     const int j = (int)(t - row * Q);
     uint32_t nc = xsmi::fdiv(row, g.dOH);
     const int oh = (int)(row - nc * g.OH);
     const float *plane = x + (size_t)nc * g.H * g.W;
-    const int lane = threadIdx.x & 63;
 
     float4 v[3];
     float lf[3];
@@ -84,22 +84,16 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         const int ih = 2 * oh - 1 + r;
         v[r] = make_float4(0.f, 0.f, 0.f, 0.f);   // border row
         lf[r] = 0.f;
-        if ((unsigned)ih < (unsigned)g.H) v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
-    }
-    if (lane == 0 && j > 0) {
-#pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const int ih = 2 * oh - 1 + r;
-            if ((unsigned)ih < (unsigned)g.H) lf[r] = plane[(size_t)ih * g.W + 4 * j - 1];
+        if ((unsigned)ih < (unsigned)g.H) {
+            v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
+            if (j > 0) lf[r] = plane[(size_t)ih * g.W + 4 * j - 1];
         }
     }
     float b0 = 0.f, b1 = 0.f;
     int w0 = 0, w1 = 0;
 #pragma unroll
     for (int r = 0; r < 3; ++r) {
-        float left = __shfl_up(v[r].w, 1);
-        if (j == 0) left = 0.f;                                       // zero border
-        else if (lane == 0) left = lf[r];
+        const float left = lf[r];                                     // 0 at the border
         // output 2j: columns 4j-1, 4j, 4j+1 ; output 2j+1: columns 4j+1, 4j+2, 4j+3
         if (r == 0 || left > b0) { b0 = left; w0 = r * 3 + 0; }
         if (v[r].x > b0) { b0 = v[r].x; w0 = r * 3 + 1; }
@@ -108,7 +102,6 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         if (v[r].z > b1) { b1 = v[r].z; w1 = r * 3 + 1; }
         if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
     }
-    if (!live) return;
     size_t o = (size_t)row * g.OW + 2 * j;
     *reinterpret_cast<float2 *>(y + o) = make_float2(b0, b1);
     if (idx) *reinterpret_cast<uchar2 *>(idx + o) = make_uchar2((unsigned char)w0, (unsigned char)w1);
@@ -148,8 +141,8 @@ __global__ void __launch_bounds__(256) maxpool_bwd_gather(const float *__restric
 // 3x3 window, stride 2, pad 1, W % 4 == 0, H % 2 == 0: one thread produces dx
 // columns 4j .. 4j+3 of the two input rows 2a and 2a+1 with one float4 store per
 // row, contiguous across the wavefront.  It reads output columns 2j, 2j+1 of the
-// output rows a and a+1 (dy and index) and takes column 2j+2 from the next lane
-// (one scalar load at a wavefront edge, nothing at the row end).
+// output rows a and a+1 (dy and index) and column 2j+2 with one more dword / byte
+// load (nothing at the row end; see the forward kernel for why not a shuffle).
 //   even row, even column: one contributor  (window row 1, kx 1)
 //   even row, odd column:  two              (kx 0 of the output column to the right, kx 2 of this one)
 //   odd row,  even column: two              (window row 0 of output row a+1, window row 2 of row a)
@@ -162,15 +155,13 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restri
                                                             float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ4,
                                                             xsmi::FastDiv dG, uint32_t total) {
     uint32_t t = blockIdx.x * 256u + threadIdx.x;
-    const bool live = t < total;
-    if (!live) t = total - 1;                // keep the lane for the shuffles below
+    if (t >= total) return;
     const int Q4 = g.W >> 2, G = g.H >> 1;
     uint32_t rowg = xsmi::fdiv(t, dQ4);      // (nc, a)
     const int j = (int)(t - rowg * Q4);
     uint32_t nc = xsmi::fdiv(rowg, dG);
     const int a = (int)(rowg - nc * G);
     const size_t obase = (size_t)nc * g.OH * g.OW;
-    const bool edge = (threadIdx.x & 63) == 63;
     float gv[2][3];
     int iv[2][3];
 #pragma unroll
@@ -185,18 +176,12 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restri
             gg = *reinterpret_cast<const float2 *>(dy + ro);
             uchar2 ii = *reinterpret_cast<const uchar2 *>(idx + ro);
             i0 = ii.x; i1 = ii.y;
-        }
-        float sg = __shfl_down(gg.x, 1);
-        int si = __shfl_down(i0, 1);
-        if (2 * j + 2 < g.OW && oh < g.OH) {
-            if (edge) { sg = dy[ro + 2]; si = idx[ro + 2]; }
-            gn = sg; in = si;
+            if (2 * j + 2 < g.OW) { gn = dy[ro + 2]; in = idx[ro + 2]; }
         }
         // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
         gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gn + 0.f;
         iv[q][0] = i0; iv[q][1] = i1; iv[q][2] = in;
     }
-    if (!live) return;
     const int h = 2 * a;
     float4 *pe = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h) * g.W + 4 * j);
     float4 *po = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h + 1) * g.W + 4 * j);
@@ -225,6 +210,74 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restri
     }
     *pe = make_float4(e[0], e[1], e[2], e[3]);
     *po = make_float4(o[0], o[1], o[2], o[3]);
+}
+
+// The same gather with eight dx columns per thread (W % 8 == 0): columns 8j .. 8j+7 of the input rows 2a and 2a+1
+// from output columns 4j .. 4j+3 (one 128-bit load of dy and one 32-bit load of the indices per output row) and
+// column 4j+4 (a dword and a byte): half as many memory instructions per byte as the four-column form.
+template <bool ACC>
+__global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
+                                                               float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ8,
+                                                               xsmi::FastDiv dG, uint32_t total) {
+    uint32_t t = blockIdx.x * 256u + threadIdx.x;
+    if (t >= total) return;
+    const int Q8 = g.W >> 3, G = g.H >> 1;
+    uint32_t rowg = xsmi::fdiv(t, dQ8);      // (nc, a)
+    const int j = (int)(t - rowg * Q8);
+    uint32_t nc = xsmi::fdiv(rowg, dG);
+    const int a = (int)(rowg - nc * G);
+    const size_t obase = (size_t)nc * g.OH * g.OW;
+    float gv[2][5];
+    int iv[2][5];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int oh = a + q;                 // a + 1 == OH: below the last output row
+        float4 gg = make_float4(0.f, 0.f, 0.f, 0.f);
+        int i0 = -1, i1 = -1, i2 = -1, i3 = -1;
+        float gn = 0.f;
+        int in = -1;
+        const size_t ro = obase + (size_t)oh * g.OW + 4 * j;
+        if (oh < g.OH) {
+            gg = *reinterpret_cast<const float4 *>(dy + ro);
+            uchar4 ii = *reinterpret_cast<const uchar4 *>(idx + ro);
+            i0 = ii.x; i1 = ii.y; i2 = ii.z; i3 = ii.w;
+            if (4 * j + 4 < g.OW) { gn = dy[ro + 4]; in = idx[ro + 4]; }
+        }
+        // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
+        gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gg.z + 0.f; gv[q][3] = gg.w + 0.f; gv[q][4] = gn + 0.f;
+        iv[q][0] = i0; iv[q][1] = i1; iv[q][2] = i2; iv[q][3] = i3; iv[q][4] = in;
+    }
+    const int h = 2 * a;
+    float4 *pe = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h) * g.W + 8 * j);
+    float4 *po = reinterpret_cast<float4 *>(dx + ((size_t)nc * g.H + h + 1) * g.W + 8 * j);
+    float e[8], o[8];
+    auto pick = [&](int q, int m, int tap) { return iv[q][m] == tap ? gv[q][m] : 0.f; };
+    if (ACC) {
+        const float4 ev0 = pe[0], ev1 = pe[1], ov0 = po[0], ov1 = po[1];
+        const float pe8[8] = {ev0.x, ev0.y, ev0.z, ev0.w, ev1.x, ev1.y, ev1.z, ev1.w};
+        const float po8[8] = {ov0.x, ov0.y, ov0.z, ov0.w, ov1.x, ov1.y, ov1.z, ov1.w};
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            e[2 * m] = (float)((double)pick(0, m, 4) + (double)pe8[2 * m]);
+            e[2 * m + 1] = (float)(((double)pick(0, m + 1, 3) + (double)pick(0, m, 5)) + (double)pe8[2 * m + 1]);
+            o[2 * m] = (float)(((double)pick(1, m, 1) + (double)pick(0, m, 7)) + (double)po8[2 * m]);
+            o[2 * m + 1] = (float)(((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                    (double)pick(0, m, 8)) + (double)po8[2 * m + 1]);
+        }
+    } else {
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            e[2 * m] = pick(0, m, 4);
+            e[2 * m + 1] = pick(0, m + 1, 3) + pick(0, m, 5);
+            o[2 * m] = pick(1, m, 1) + pick(0, m, 7);
+            o[2 * m + 1] = (float)((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                   (double)pick(0, m, 8));
+        }
+    }
+    pe[0] = make_float4(e[0], e[1], e[2], e[3]);
+    pe[1] = make_float4(e[4], e[5], e[6], e[7]);
+    po[0] = make_float4(o[0], o[1], o[2], o[3]);
+    po[1] = make_float4(o[4], o[5], o[6], o[7]);
 }
 
 int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw, int pad, PoolGeom *g) {
@@ -295,6 +348,16 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
     hipStream_t st = xsmi::stream();
     int acc = beta == 1.f ? 1 : 0;
     xsmi::prof_begin();
+    if (fast_3x3s2p1(g) && (W % 8) == 0 && (((uintptr_t)dy | (uintptr_t)dx) & 15) == 0 && ((uintptr_t)idx & 3) == 0) {
+        uint32_t threads = total / 16;       // eight columns of two rows each
+        xsmi::FastDiv dQ8 = xsmi::make_fastdiv(W / 8), dG = xsmi::make_fastdiv(H / 2);
+        dim3 grid((threads + 255) / 256);
+        if (acc) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<true>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        else hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<false>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        xsmi::prof_end();
+        XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_w8");
+        return XSMI_OK;
+    }
     if (fast_3x3s2p1(g)) {
         uint32_t threads = total / 8;        // four columns of two rows each
         xsmi::FastDiv dQ4 = xsmi::make_fastdiv(W / 4), dG = xsmi::make_fastdiv(H / 2);

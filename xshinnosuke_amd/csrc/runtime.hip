@@ -59,10 +59,12 @@ void prof_end() {
 }
 }  // namespace xsmi
 
+// One float4 per thread: of the forms tried on the box (grid-stride loops over 8 to 64 workgroups per CU, four loads
+// in flight per thread, the runtime's own device-to-device copy) this one moved the most bytes per second when source
+// and destination come from HBM (5.9 TB/s against 5.2-5.7 for the loops and 5.3 for hipMemcpyAsync).
 __global__ void __launch_bounds__(256) xsmi_copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4) {
-    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
-    size_t stride = (size_t)gridDim.x * blockDim.x;
-    for (; i < n4; i += stride) dst[i] = src[i];
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i < n4) dst[i] = src[i];
 }
 
 extern "C" {
@@ -274,8 +276,7 @@ int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
     size_t n4 = bytes / 16;
     if (n4 == 0) return XSMI_OK;
     size_t blocks = (n4 + 255) / 256;
-    size_t cap = (size_t)g_cus * 32;
-    if (blocks > cap) blocks = cap;
+    XSMI_CHECK_ARG(blocks < 2147483648ull, "xsmi_copy_kernel: more than 2^31 workgroups");
     xsmi::prof_begin();
     hipLaunchKernelGGL(xsmi_copy_f4, dim3((unsigned)blocks), dim3(256), 0, g_stream,
                        (const float4 *)src, (float4 *)dst, n4);

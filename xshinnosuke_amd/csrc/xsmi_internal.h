@@ -104,6 +104,19 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
 int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
                       int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace);
 
+// second-generation fp32 tap kernel (conv_tap_sk.hip): 64 x 64 outputs per wave, work split evenly over the resident
+// workgroups; needs its own, larger workspace (packed filter + partial tiles)
+bool sk_path_ok(int reduce_channels, int rows);
+bool sk_bwd_data_ok(int C, int K, int R, int S, int sh, int sw);
+bool sk_fwd_pays(int M, int rows, int R, int S, int sh, int sw);          // M = output pixels of the pass
+bool sk_bwd_data_pays(int M, int rows, int R, int S, int sh, int sw);
+size_t sk_fwd_ws_bytes(int C, int K, int R, int S);
+size_t sk_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw);
+int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace);
+int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
+                     int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace);
+
 // bf16 forward on a channels-last bf16 copy of the activations (conv_tap.hip): channels a multiple of 32, or
 // at most 8 (a stem); the workspace holds the packed filter followed by the copy
 bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad);
