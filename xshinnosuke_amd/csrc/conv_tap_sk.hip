@@ -139,6 +139,7 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     uint32_t i_plane = 0;
     int iyb = 0, ixb = 0, nbase = 0;
     bool live = false;
+    bool prep_stale = true;                            // the pixel offset must be formed again (new segment)
     uint32_t ld_asoff = 0, ld_stage = lds0, ld_voff = 0, ld_soff = 0;
     const uint32_t a_lane = (uint32_t)lane * 16u;
 
@@ -154,6 +155,7 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
         uint32_t n_seg = c.iters - ch;
         if (n_seg > u1 - iu) n_seg = u1 - iu;
         i_left = n_seg;
+        prep_stale = true;
         i_nch = c.nch; i_TS = c.TS; i_dstep = c.dstep; i_IH = c.IH; i_IW = c.IW; i_plane = c.plane_bytes;
         const uint32_t tap = ch / (uint32_t)c.nch;
         cc = (int)(ch - tap * (uint32_t)c.nch);
@@ -174,10 +176,12 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
         }
     };
     auto issue_prep = [&]() {
+        ld_soff = (uint32_t)(cc * KC + chan0) * i_plane;
+        if (cc != 0 && !prep_stale) return;            // same tap as the previous chunk: same pixel offset
+        prep_stale = false;
         int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
         bool ok = live && (unsigned)iy < (unsigned)i_IH && (unsigned)ix < (unsigned)i_IW;
         ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
-        ld_soff = (uint32_t)(cc * KC + chan0) * i_plane;
     };
     auto issue_b = [&](int e) {                        // channel chan0 + e of the chunk, this wave's 64 pixels
         xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((A_FLOATS + (chan0 + e) * PIX + pb * 64) * 4), ld_voff,
@@ -203,7 +207,7 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
             } else {
                 // Past the range every chunk still runs the full loop body; its loads are given no live pixel
                 // (they touch no memory and fill the stage with zeros) and re-read the first filter block.
-                live = false; ld_asoff = 0; r = 0; s = 0; cc = 0;
+                live = false; ld_asoff = 0; r = 0; s = 0; cc = 0; prep_stale = true;
             }
         }
     };
