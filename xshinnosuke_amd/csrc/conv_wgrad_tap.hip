@@ -47,6 +47,9 @@ struct WgradTapParams {
     int N, C, K, H, W, OH, OW, OHW, R, S, sh, sw, pad;
     int OHWa;           // plane length of the dy operand as stored (OHW rounded up to a multiple of 4)
     int cpi;            // chunks per image
+    int flat;           // the dy operand is a [K][N*OHW] copy and chunks run over the pixels of the whole batch
+    int Mtot;           // flat: N*OHW
+    xsmi::FastDiv dOHW; // flat: pixel index -> image
     int total_chunks, cps, ctiles;
     uint32_t xplane_bytes, yplane_bytes;
     xsmi::FastDiv dOW, dCT, dS;
@@ -109,12 +112,19 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
         ld_va1 = a_ok ? a_v1 : 0x80000000u;
         ld_sa = (uint32_t)((in_img * p.K + k0) * p.OHWa + ml0) * 4u;
         // B: the shifted input position of this lane's pixel
-        const int ml = ml0 + b_m;
+        int ml = ml0 + b_m;
+        int img = 0;                                  // flat: this lane's image (the scalar part then has none)
+        bool inside = ml < p.OHW;
+        if (p.flat) {
+            inside = ml < p.Mtot;
+            img = (int)xsmi::fdiv((uint32_t)ml, p.dOHW);
+            ml -= img * p.OHW;
+        }
         const int oh = (int)xsmi::fdiv((uint32_t)ml, p.dOW);
         const int ow = ml - oh * p.OW;
         const int ih = oh * p.sh + tr - p.pad, iw = ow * p.sw + ts - p.pad;
-        const bool b_ok = ml < p.OHW && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-        ld_vb = b_ok ? (uint32_t)((ih * p.W + iw) * 4) + (uint32_t)b_chl * p.xplane_bytes : 0x80000000u;
+        const bool b_ok = inside && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+        ld_vb = b_ok ? (uint32_t)((ih * p.W + iw) * 4) + (uint32_t)(img * p.C + b_chl) * p.xplane_bytes : 0x80000000u;
         ld_sb = (uint32_t)(in_img * p.C + c0) * p.xplane_bytes;
     };
     auto issue_a = [&](int j) {
@@ -297,20 +307,58 @@ __global__ void __launch_bounds__(256) pad_planes_kernel(const float *__restrict
     }
 }
 
+// dst[k][0 .. Ma) = the pixels of filter plane k of every image, image after image (N*OHW values), then zeros:
+// the reduction index of the weight gradient as one dense run per filter.
+__global__ void __launch_bounds__(256) gather_filter_rows_kernel(const float *__restrict__ src, float *__restrict__ dst, int K,
+                                                                 int OHW, int M, int Ma, xsmi::FastDiv dMa, xsmi::FastDiv dOHW,
+                                                                 uint32_t total) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < total; i += gridDim.x * 256u) {
+        const uint32_t k = xsmi::fdiv(i, dMa), m = i - k * (uint32_t)Ma;
+        float v = 0.f;
+        if (m < (uint32_t)M) {
+            const uint32_t n = xsmi::fdiv(m, dOHW), pl = m - n * (uint32_t)OHW;
+            v = src[((size_t)n * K + k) * OHW + pl];
+        }
+        dst[i] = v;
+    }
+}
+
+// Small feature maps waste chunk slots when chunks may not straddle images (49 pixels fill 64 slots to 77 %, 196
+// fill 224 to 88 %): they take the dense form.
+bool use_flat(int OHW) { return OHW * 20 < xsmi::ceil_div(OHW, MC) * MC * 19; }
+
 void plan(int N, int C, int K, int R, int S, int OHW, int *cpi, int *total, int *cps, int *splits) {
+    if (use_flat(OHW)) {                              // one "image" holding the pixels of the whole batch
+        OHW = N * OHW;
+        N = 1;
+    }
     const int tiles = R * S * (C / TC) * (K / TK);
     *cpi = xsmi::ceil_div(OHW, MC);
     *total = N * *cpi;
-    int want = xsmi::ceil_div(TARGET_BLOCKS, tiles);
-    int c = xsmi::ceil_div(*total, want);
-    if (c < 8) c = 8;
-    // Long pixel ranges let the R*S workgroups that share a range drift apart until each fetches dy and x from
-    // HBM on its own; at most 64 chunks (2048 pixels) per range keeps them within reach of one L2
-    // (measured at N=256, 64->64, 56x56: 631 -> 516 us).
-    if (c > 64) c = 64;
-    if (c > *total) c = *total;
-    *cps = c;
-    *splits = xsmi::ceil_div(*total, c);
+    // The number of pixel ranges is chosen by a cost model of the launch: workgroups spread evenly over the compute
+    // units (four resident per CU) and the units' matrix pipes are shared by their workgroups, so the launch takes
+    // about ceil(workgroups / CUs) * (chunks per range).  A few workgroups beyond a multiple of the CU count cost a
+    // whole extra share (128 -> 128 at 28 x 28: 29 ranges x 36 tiles = 1044 workgroups took 88 us, 28 x 36 = 1008
+    // take 74; 512 -> 512 at 7 x 7 is better off with 2 x 576 than with 1 x 576).  The CU count is the MI355X's, as a
+    // constant: the workspace query must plan the same split before a device is initialised.
+    constexpr int CUS = 256;
+    const int want = TARGET_BLOCKS / tiles > 1 ? TARGET_BLOCKS / tiles : 1;
+    long best_cost = -1;
+    int best_c = 0;
+    for (int sgl = want > 3 ? want - 2 : 1; sgl <= want + 2; ++sgl) {
+        int c = xsmi::ceil_div(*total, sgl);
+        if (c < 8) c = 8;
+        // Long pixel ranges let the R*S workgroups that share a range drift apart until each fetches dy and x from
+        // HBM on its own; at most 64 chunks (2048 pixels) per range keeps them within reach of one L2
+        // (measured at N=256, 64->64, 56x56: 631 -> 516 us).
+        if (c > 64) c = 64;
+        if (c > *total) c = *total;
+        const long wgs = (long)tiles * xsmi::ceil_div(*total, c);
+        const long cost = ((wgs + CUS - 1) / CUS) * c;
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best_c = c; }
+    }
+    *cps = best_c;
+    *splits = xsmi::ceil_div(*total, best_c);
 }
 
 }  // namespace
@@ -325,7 +373,8 @@ size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW) {
     int cpi, total, cps, splits;
     plan(N, C, K, R, S, OH * OW, &cpi, &total, &cps, &splits);
     const int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
-    const size_t padded = OHWa != OHW ? align_up((size_t)N * K * OHWa * sizeof(float), 256) : 0;
+    size_t padded = OHWa != OHW ? align_up((size_t)N * K * OHWa * sizeof(float), 256) : 0;
+    if (use_flat(OHW)) padded = align_up((size_t)K * ((N * OHW + 3) & ~3) * sizeof(float), 256);
     return align_up((size_t)splits * R * S * K * C * sizeof(float), 256) + align_up((size_t)splits * K * sizeof(float), 256) + padded;
 }
 
@@ -338,8 +387,23 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     p.part = (float *)workspace;
     float *dbpart = (float *)((char *)workspace + align_up((size_t)splits * R * S * K * C * sizeof(float), 256));
     hipStream_t st = stream();
-    const int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
-    if (OHWa != OHW) {
+    int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
+    const bool flat = use_flat(OHW);
+    p.flat = flat ? 1 : 0;
+    p.Mtot = N * OHW;
+    p.dOHW = make_fastdiv(OHW);
+    if (flat) {
+        float *dyp = (float *)((char *)dbpart + align_up((size_t)splits * K * sizeof(float), 256));
+        const int Ma = (p.Mtot + 3) & ~3;
+        const uint32_t total = (uint32_t)((size_t)K * Ma);
+        uint32_t blocks = (total + 255) / 256;
+        if (blocks > 4096) blocks = 4096;
+        hipLaunchKernelGGL(gather_filter_rows_kernel, dim3(blocks), dim3(256), 0, st, dy, dyp, K, OHW, p.Mtot, Ma, make_fastdiv(Ma),
+                           p.dOHW, total);
+        XSMI_LAUNCH_CHECK("gather_filter_rows_kernel");
+        p.dy = dyp;
+        OHWa = Ma;                                   // the "plane" of the dy operand is now a filter's whole row
+    } else if (OHWa != OHW) {
         float *dyp = (float *)((char *)dbpart + align_up((size_t)splits * K * sizeof(float), 256));
         const uint32_t total = (uint32_t)((size_t)N * K * OHWa);
         uint32_t blocks = (total + 255) / 256;
@@ -350,7 +414,7 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     }
     p.dbpart = db ? dbpart : nullptr;
     p.x_bytes = (uint32_t)((size_t)N * C * H * W * 4);
-    p.dy_bytes = (uint32_t)((size_t)N * K * OHWa * 4);
+    p.dy_bytes = flat ? (uint32_t)((size_t)K * OHWa * 4) : (uint32_t)((size_t)N * K * OHWa * 4);
     p.N = N; p.C = C; p.K = K; p.H = H; p.W = W; p.OH = OH; p.OW = OW; p.OHW = OHW; p.OHWa = OHWa; p.R = R; p.S = S;
     p.sh = sh; p.sw = sw; p.pad = pad;
     p.ctiles = C / TC;
