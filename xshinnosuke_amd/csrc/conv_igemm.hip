@@ -344,6 +344,10 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
         workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
         return xsmi::nhwc_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
                                    (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
+    if (!(flags & XSMI_CONV_BF16) && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad) &&
+        workspace_bytes >= xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
+        return xsmi::stem_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
+                                   (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
     if (!(flags & XSMI_CONV_BF16) && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * g.OH * g.OW, K, R, S, sh, sw) &&
         workspace_bytes >= xsmi::sk_fwd_ws_bytes(C, K, R, S))
         return xsmi::sk_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,

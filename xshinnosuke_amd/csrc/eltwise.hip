@@ -74,6 +74,10 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
     size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
     size_t m = a > b ? a : b;
     m = m > c ? m : c;
+    if (xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad)) {
+        size_t e = xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad);
+        m = m > e ? m : e;
+    }
     // the second-generation fp32 kernels are chosen when the workspace also has room for their partial tiles
     if (xsmi::sk_path_ok(C, K)) {
         size_t e = xsmi::sk_fwd_ws_bytes(C, K, R, S);

@@ -117,6 +117,13 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
 int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S, int sh,
                      int sw, int pad, int OH, int OW, int accumulate, int opts, void *workspace);
 
+// forward for very few input channels (conv_stem.hip): 1 or 3 channels, square filter of 3, 5 or 7, horizontal stride 2;
+// the workspace holds the packed filter followed by a zero-bordered copy of the input
+bool stem_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
+size_t stem_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
+int stem_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
+                  int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace);
+
 // bf16 forward on a channels-last bf16 copy of the activations (conv_tap.hip): channels a multiple of 32, or
 // at most 8 (a stem); the workspace holds the packed filter followed by the copy
 bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad);
