@@ -550,6 +550,55 @@ __global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ 
     }
 }
 
+// The 3x3, stride-1 case of sk_pack_kernel with wide accesses: a thread takes one row and one quad of channels, i.e.
+// 36 floats of w (mode 0: one contiguous run, read as nine float4; mode 1: four runs of nine), and stores one float4 per
+// tap; the lanes of a wavefront are consecutive rows, so a store instruction writes 1 KB of one tap's block and every
+// byte of w is requested once.
+__global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restrict__ w, float *__restrict__ apk,
+                                                           uint32_t *__restrict__ flags, int nflags, int mode, int rows, int CH,
+                                                           int rowtiles, int ROWS, int KC) {
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < nflags; i += gridDim.x * 256) flags[i] = 0;
+    const int nch = CH / KC, quads = KC / 4;
+    const uint32_t total = (uint32_t)rowtiles * (uint32_t)nch * (uint32_t)quads * (uint32_t)ROWS;
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= total) return;
+    const int rr = (int)(i % (uint32_t)ROWS);
+    uint32_t rest = i / (uint32_t)ROWS;
+    const int q = (int)(rest % (uint32_t)quads);
+    rest /= (uint32_t)quads;
+    const int cc = (int)(rest % (uint32_t)nch), rt = (int)(rest / (uint32_t)nch);
+    const int ch0 = cc * KC + q * 4, row = rt * ROWS + rr;
+    float v[4][9];
+    if (row < rows) {
+        if (mode == 0) {
+            const float4 *src = reinterpret_cast<const float4 *>(w + ((size_t)row * CH + ch0) * 9);
+            float buf[36];
+#pragma unroll
+            for (int u = 0; u < 9; ++u) *reinterpret_cast<float4 *>(buf + 4 * u) = src[u];
+#pragma unroll
+            for (int e = 0; e < 4; ++e)
+#pragma unroll
+                for (int t = 0; t < 9; ++t) v[e][t] = buf[e * 9 + t];
+        } else {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const float *src = w + ((size_t)(ch0 + e) * rows + row) * 9;
+#pragma unroll
+                for (int t = 0; t < 9; ++t) v[e][t] = src[t];
+            }
+        }
+    } else {
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int t = 0; t < 9; ++t) v[e][t] = 0.f;
+    }
+    // float4 index ((rt * iters + tap * nch + cc) * quads + q) * ROWS + rr with iters = 9 * nch
+    float4 *dst = reinterpret_cast<float4 *>(apk) + (((size_t)rt * 9 * nch + cc) * quads + q) * ROWS + rr;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) dst[(size_t)t * nch * quads * ROWS] = make_float4(v[0][t], v[1][t], v[2][t], v[3][t]);
+}
+
 struct SkShape { int rows_tile, pix_tile, kc, blk; };
 int sk_env() {
     static int v = -1;
@@ -669,7 +718,12 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     float *apk = (float *)workspace;
     uint32_t *flags = (uint32_t *)((char *)workspace + pack);
     float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
-    if (!(opts & 2)) {
+    if (!(opts & 2) && R == 3 && S == 3 && (((uintptr_t)w) & 15) == 0) {
+        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(C / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
+        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, apk, flags, SK_MAX_GRID, 0, K, C,
+                           rowtiles, shp.rows_tile, shp.kc);
+        XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
+    } else if (!(opts & 2)) {
         SkPackMulti pm;
         pm.njobs = 1;
         pm.job[0] = SkPackJob{apk, R, S, 0, 0};
@@ -748,7 +802,12 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
     const size_t pack = off;
     uint32_t *flags = (uint32_t *)((char *)workspace + pack);
     float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
-    if (!(opts & 2)) {
+    if (!(opts & 2) && R == 3 && S == 3 && sh == 1 && sw == 1 && nplans == 1) {
+        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(K / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
+        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, jobs[0].apk, flags, SK_MAX_GRID, 1, C,
+                           K, rowtiles, shp.rows_tile, shp.kc);
+        XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
+    } else if (!(opts & 2)) {
         SkPackMulti pm;
         pm.njobs = nplans;
         uint32_t blocks = 0;

@@ -298,6 +298,37 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__re
     }
 }
 
+// The same reduction for large 3x3 filters (K*C >= 65536) with few splits: a thread owns one (k, c) and all nine taps,
+// adds the splits in ascending order in float64 and writes nine consecutive floats of dw, so that a wavefront reads
+// 256 contiguous bytes per (split, tap) and fills 2304 contiguous bytes of dw.  Bias blocks as above.
+__global__ void __launch_bounds__(256) wgrad_tap_reduce9_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                                 const float *__restrict__ dbpart, float *__restrict__ db,
+                                                                 int K, int C, int splits, int dw_blocks, int accumulate) {
+    if ((int)blockIdx.x >= dw_blocks) {
+        if (threadIdx.x >= 64) return;
+        const int k = ((int)blockIdx.x - dw_blocks) * 64 + (int)threadIdx.x;
+        double s = 0.0;
+        for (int sp = 0; sp < splits; ++sp) s += (double)dbpart[(size_t)sp * K + k];
+        if (accumulate) s += (double)db[k];
+        db[k] = (float)s;
+        return;
+    }
+    const size_t kc = (size_t)blockIdx.x * 256 + threadIdx.x;      // k * C + c
+    const size_t KC = (size_t)K * C;
+    if (kc >= KC) return;
+    double s[9];
+#pragma unroll
+    for (int t = 0; t < 9; ++t) s[t] = 0.0;
+    for (int sp = 0; sp < splits; ++sp) {
+        const float *src = part + (size_t)sp * 9 * KC + kc;
+#pragma unroll
+        for (int t = 0; t < 9; ++t) s[t] += (double)src[(size_t)t * KC];
+    }
+    float *dst = dw + kc * 9;
+#pragma unroll
+    for (int t = 0; t < 9; ++t) dst[t] = (float)(accumulate ? s[t] + (double)dst[t] : s[t]);
+}
+
 // dst[plane][0 .. OHWa) = src[plane][0 .. OHW) followed by zeros
 __global__ void __launch_bounds__(256) pad_planes_kernel(const float *__restrict__ src, float *__restrict__ dst, int OHW,
                                                           int OHWa, uint32_t total) {
@@ -426,6 +457,13 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     hipLaunchKernelGGL(wgrad_tap_f32_kernel, grid, dim3(256), 0, st, p);
     prof_end();
     XSMI_LAUNCH_CHECK("wgrad_tap_f32_kernel");
+    if (R * S == 9 && (size_t)K * C >= 65536 && splits <= 16) {
+        const int blocks9 = (int)(((size_t)K * C + 255) / 256);
+        hipLaunchKernelGGL(wgrad_tap_reduce9_kernel, dim3(blocks9 + (db ? K / 64 : 0)), dim3(256), 0, st, p.part, dw, dbpart, db,
+                           K, C, splits, blocks9, accumulate);
+        XSMI_LAUNCH_CHECK("wgrad_tap_reduce9_kernel");
+        return XSMI_OK;
+    }
     const int dw_blocks = R * S * K * p.ctiles;
     hipLaunchKernelGGL(wgrad_tap_reduce_kernel, dim3(dw_blocks + (db ? K / 64 : 0)), dim3(256), 0, st, p.part, dw, dbpart, db,
                        K, C, R * S, splits, dw_blocks, accumulate);
