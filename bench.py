@@ -419,8 +419,10 @@ def bench_resnet18_infer(be, steps, warmup, with_oracle=True):
             out["resnet18_infer_%s_logits_rel_l2_vs_oracle" % mode] = float(
                 np.linalg.norm(logits[mode][pick] - r64) / np.linalg.norm(r64))
     out["resnet18_infer_workload"] = ("N=256x3x224x224, forward only, moving-statistics BN (fresh: mean 0, var 1), "
-                                      "fp32 tensors in HBM, batch norm folded into the convolutions; bf16 = each conv rewrites "
-                                      "its input as a channels-last bf16 copy and multiplies bf16 operands with fp32 accumulation")
+                                      "batch norm folded into the convolutions; fp32 = float32 NCHW tensors and fp32 MFMA; bf16 = "
+                                      "bf16 MFMA operands with fp32 accumulation, activations between the stem and the "
+                                      "average pool kept as channels-last bf16 tensors (conv, add+ReLU, max-pool read and write "
+                                      "them directly)")
     return out
 
 

@@ -127,6 +127,38 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
                     int sh, int sw, int pad, unsigned flags,
                     void *workspace, size_t workspace_bytes);
 
+/* ---- channels-last bf16 activations (inference) ----------------------------
+ * An extension of the forward above for chains of layers evaluated without gradients
+ * (Model.predict / evaluate, xs/nn/models.py:98-116, under bf16 conv precision): the
+ * reference keeps every activation as float32 NCHW; here a tensor may instead live as
+ * bf16 [N][H + 2 b][W + 2 b][C] with a zero border of b pixels ("channels-last"),
+ * which is the operand layout of the bf16 MFMA kernel, so that conv -> add/ReLU ->
+ * max-pool -> conv chains neither rewrite nor convert their activations.
+ *
+ * xsmi_conv2d_fwd_cl: conv2d (+bias, +ReLU with XSMI_CONV_RELU) with bf16 operands and
+ * fp32 accumulation.  Exactly one of x (fp32 NCHW) / x_cl (channels-last, C % 32 == 0,
+ * border x_border >= pad) and exactly one of y (fp32 NCHW) / y_cl (channels-last,
+ * K % 8 == 0, border y_border; only the interior is written: the caller zeroes the
+ * buffer once) is given.  flags: XSMI_CONV_RELU, XSMI_CONV_WS_PACKED.  Workspace:
+ * xsmi_conv2d_workspace_bytes of the geometry is always enough. */
+int xsmi_conv2d_fwd_cl(const float *x, const void *x_cl, int x_border, const float *w, const float *bias,
+                       float *y, void *y_cl, int y_border,
+                       int N, int C, int H, int W, int K, int R, int S,
+                       int sh, int sw, int pad, unsigned flags,
+                       void *workspace, size_t workspace_bytes);
+/* out = a + b (relu = 0) or max(0, a + b) over `count` bf16 elements (a multiple of 8) of
+ * equally shaped channels-last tensors, borders included: add (xs/nn/functional.py:41-52)
+ * followed by relu (xs/nn/functional.py:156-163); out may be a or b. */
+int xsmi_cl_add(const void *a, const void *b, void *out, size_t count, int relu);
+/* max_pool2d (xs/nn/functional.py:445-491) on channels-last tensors: the input's zero
+ * border (x_border >= pad) is the reference's zero-valued padding that takes part in
+ * the max; writes the interior of y_cl (border y_border).  No argmax: inference only. */
+int xsmi_cl_maxpool2d(const void *x_cl, int x_border, void *y_cl, int y_border,
+                      int N, int C, int H, int W, int k, int sh, int sw, int pad);
+/* y (fp32, N,C,H,W) = the interior of a channels-last tensor: for every consumer that
+ * reads float32 NCHW. */
+int xsmi_cl_to_nchw(const void *x_cl, int border, float *y, int N, int C, int H, int W);
+
 /* The forward for callers that cannot allocate device memory or pass a workspace: code under HIP graph
  * capture, tight serving loops, harnesses that forbid hipMalloc.  No counterpart in the reference.  Same kernels,
  * arguments and results as xsmi_conv2d_fwd (flags: XSMI_CONV_RELU, XSMI_CONV_BF16); the scratch memory is a static

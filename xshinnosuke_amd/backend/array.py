@@ -10,6 +10,8 @@ from .capi import lib, ensure_init, XsmiError
 _DTYPE_CLASS = np.dtype(np.float32).__class__
 
 _POOL = {}            # rounded size -> list of free device pointers
+_CL_POOL = {}         # (n, c, h, w, border) -> ChannelsLast forms of released arrays (their borders are zero)
+_CL_POOL_DEPTH = 4
 _POOL_BYTES = [0]
 _POOL_LIMIT = 64 << 30
 
@@ -23,6 +25,7 @@ def _round_size(nbytes):
 
 def release_cached_memory():
     """Return every cached block to the driver."""
+    _CL_POOL.clear()                      # their buffers return to _POOL first
     for ptrs in _POOL.values():
         for ptr in ptrs:
             lib.call("xsmi_free", ctypes.c_void_p(ptr))
@@ -36,12 +39,13 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl")
 
     def __init__(self, nbytes):
         ensure_init()
         self.logical = int(nbytes)
         self.lazy_zero = False
+        self.cl = None                       # ChannelsLast form of the array that fills this block, if it has one
         self.version = 0                     # counts every hand-out of the address and every pending clear
         size = _round_size(nbytes)
         free = _POOL.get(size)
@@ -64,6 +68,13 @@ class _Block:
 
     def __del__(self):
         try:
+            cl = self.cl
+            if cl is not None:               # keep the zero-bordered buffer for the next array of this geometry
+                self.cl = None
+                cl.valid = False
+                kept = _CL_POOL.setdefault((cl.n, cl.c, cl.h, cl.w, cl.border), [])
+                if len(kept) < _CL_POOL_DEPTH:
+                    kept.append(cl)
             if self.ptr:
                 if _POOL_BYTES[0] + self.nbytes <= _POOL_LIMIT:
                     _POOL.setdefault(self.nbytes, []).append(self.ptr)
@@ -73,6 +84,24 @@ class _Block:
                 self.ptr = None
         except Exception:
             pass
+
+
+class ChannelsLast:
+    """A float32 NCHW array's contents held as bf16 [N][H + 2 border][W + 2 border][C] with a zero border (the operand
+    layout of the bf16 convolution kernel; csrc/cl_ops.hip).  While ``valid`` the float32 memory of the owning
+    block is stale: ``DeviceArray.ptr`` converts back before it hands the address out, so only the operations that
+    ask for this form (conv, add + ReLU and max-pool without gradients under bf16 precision) ever see it."""
+
+    __slots__ = ("buf", "n", "c", "h", "w", "border", "valid")
+
+    def __init__(self, n, c, h, w, border):
+        self.n, self.c, self.h, self.w, self.border = n, c, h, w, border
+        # zeroed once: the kernels write the interior only, the border stays zero
+        self.buf = DeviceArray((n, h + 2 * border, w + 2 * border, c), np.uint16).fill_zero()
+        self.valid = False
+
+    def same_layout(self, other):
+        return (self.n, self.c, self.h, self.w, self.border) == (other.n, other.c, other.h, other.w, other.border)
 
 
 def _rebuild_array(host):
@@ -112,6 +141,10 @@ class DeviceArray:
         if blk.lazy_zero:                    # logically zero, memory not cleared yet: clear it on first use
             blk.lazy_zero = False
             lib.call("xsmi_memset", ctypes.c_void_p(blk.ptr), 0, blk.nbytes)
+        cl = blk.cl
+        if cl is not None and cl.valid:      # the contents live in channels-last form: convert back first
+            cl.valid = False
+            lib.call("xsmi_cl_to_nchw", cl.buf.cptr, cl.border, ctypes.c_void_p(blk.ptr), cl.n, cl.c, cl.h, cl.w)
         return blk.ptr + self._offset
 
     def state(self):
@@ -124,6 +157,37 @@ class DeviceArray:
         """The device address as an integer; unlike ``ptr`` it leaves a pending clear pending (for alignment and
         aliasing checks)."""
         return self._block.ptr + self._offset
+
+    def channels_last(self):
+        """The ChannelsLast form if that is where this array's contents currently live, else None (never converts)."""
+        cl = self._block.cl
+        if cl is not None and cl.valid and self._offset == 0 and self.shape == (cl.n, cl.c, cl.h, cl.w):
+            return cl
+        return None
+
+    def channels_last_out(self, border=1):
+        """Declare that this array (float32 NCHW, a whole allocation, channels a multiple of 8) is about to be
+        produced in channels-last form: returns the ChannelsLast whose ``buf`` interior the producer writes, marked
+        valid, or None if the array does not qualify.  A pending clear is dropped (everything is overwritten)."""
+        blk = self._block
+        if (len(self.shape) != 4 or self.dtype != np.float32 or self._offset != 0 or self.nbytes < blk.logical
+                or self.shape[1] % 8 or self.size == 0):
+            return None
+        n, c, h, w = self.shape
+        cl = blk.cl
+        if cl is None or (cl.n, cl.c, cl.h, cl.w, cl.border) != (n, c, h, w, border):
+            kept = _CL_POOL.get((n, c, h, w, border))
+            cl = blk.cl = kept.pop() if kept else ChannelsLast(n, c, h, w, border)
+        blk.lazy_zero = False
+        blk.version += 1
+        cl.valid = True
+        return cl
+
+    def _overwritten(self):
+        """Called before the whole array is overwritten: a channels-last form need not be converted back."""
+        cl = self._block.cl
+        if cl is not None and cl.valid and self._offset == 0 and self.nbytes >= self._block.logical:
+            cl.valid = False
 
     def is_fresh(self):
         """True if the array is a whole allocation whose clear is still pending."""
@@ -170,6 +234,7 @@ class DeviceArray:
         if host.shape != self.shape:
             host = np.ascontiguousarray(np.broadcast_to(host, self.shape))
         self.take_fresh()                     # everything is overwritten: a pending clear is moot
+        self._overwritten()
         if self.nbytes:
             lib.call("xsmi_memcpy_h2d", self.cptr, host.ctypes.data_as(ctypes.c_void_p), self.nbytes)
         return self
@@ -191,6 +256,7 @@ class DeviceArray:
         if other.nbytes != self.nbytes:
             raise ValueError("size mismatch in device copy: %s vs %s" % (other.shape, self.shape))
         self.take_fresh()
+        self._overwritten()
         if self.nbytes:
             lib.call("xsmi_memcpy_d2d", self.cptr, other.cptr, self.nbytes)
         return self
@@ -202,6 +268,7 @@ class DeviceArray:
         """Clear the array.  ``lazy=True`` only marks a whole allocation as zero: the memset happens on
         the first ordinary use, and not at all if the first use overwrites everything (take_fresh)."""
         blk = self._block
+        self._overwritten()
         if lazy and self._offset == 0 and self.nbytes >= blk.logical:
             blk.lazy_zero = True
             blk.version += 1

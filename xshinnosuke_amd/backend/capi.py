@@ -76,6 +76,10 @@ SIGNATURES = {
     "xsmi_relu_fwd": (_i, [_vp, _vp, _sz]),
     "xsmi_relu_fwd_mask": (_i, [_vp, _vp, _vp, _sz]),
     "xsmi_relu_bwd": (_i, [_vp, _vp, _vp, _sz]),
+    "xsmi_conv2d_fwd_cl": (_i, [_vp, _vp, _i, _vp, _vp, _vp, _vp, _i] + [_i] * 10 + [_u, _vp, _sz]),
+    "xsmi_cl_add": (_i, [_vp, _vp, _vp, _sz, _i]),
+    "xsmi_cl_maxpool2d": (_i, [_vp, _i, _vp, _i] + [_i] * 8),
+    "xsmi_cl_to_nchw": (_i, [_vp, _i, _vp] + [_i] * 4),
     "xsmi_act_fwd": (_i, [_vp, _vp, _sz, _i]),
     "xsmi_act_bwd": (_i, [_vp, _vp, _vp, _sz, _i]),
     "xsmi_lerp": (_i, [_vp, _vp, _f, _sz]),

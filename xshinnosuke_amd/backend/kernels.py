@@ -47,10 +47,13 @@ def _f32(a, what):
 
 
 def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False, packed=False,
-               workspace=None):
+               workspace=None, channels_last=False):
     """``packed=True`` promises that the previous conv call on this workspace was this same forward with the same
     geometry and filter values (the workspace still holds the filter's packed form), so it is not laid out again.
-    ``workspace``: a ``Workspace`` of the caller's instead of the shared one (a layer that keeps its packed filter)."""
+    ``workspace``: a ``Workspace`` of the caller's instead of the shared one (a layer that keeps its packed filter).
+    ``channels_last=True`` (with ``bf16``, no mask): the result may be left in channels-last bf16 form, and an input
+    that lives in that form is read as it is (``DeviceArray.channels_last``); results equal the plain bf16 path's up
+    to the bf16 rounding of the stored activations."""
     _f32(x, "x"); _f32(w, "w")
     dims = _dims(x.shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -69,6 +72,18 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
         raise ValueError("conv2d: neg_mask must be uint8 with one byte per output element")
     flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0)
     ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(lib.raw("xsmi_conv2d_workspace_bytes")(*dims))
+    if channels_last and bf16 and neg_mask is None:
+        xcl = x.channels_last()
+        if xcl is not None and not (c % 32 == 0 and xcl.border >= pad):
+            xcl = None                                # read through the float32 form (x.cptr converts)
+        if xcl is not None or c % 32 == 0 or c <= 8:
+            ycl = out.channels_last_out(1) if k % 8 == 0 else None
+            lib.call("xsmi_conv2d_fwd_cl", None if xcl is not None else x.cptr, xcl.buf.cptr if xcl is not None else None,
+                     xcl.border if xcl is not None else 0, w.cptr, bias.cptr if bias is not None else None,
+                     None if ycl is not None else out.cptr, ycl.buf.cptr if ycl is not None else None, 1, *dims,
+                     flags & ~CONV_BF16, ws, ws_bytes)
+            return out
+    out._overwritten()
     lib.call("xsmi_conv2d_fwd", x.cptr, w.cptr, bias.cptr if bias is not None else None, out.cptr,
              neg_mask.cptr if neg_mask is not None else None, *dims, flags, ws, ws_bytes)
     return out
@@ -177,6 +192,13 @@ def maxpool2d_fwd(x, k, stride, pad=0, out=None, idx=None, want_idx=True):
         raise ValueError("max_pool2d: out has shape %s, expected %s" % (out.shape, (n, c, oh, ow)))
     if idx is None and want_idx:
         idx = empty((n, c, oh, ow), np.uint8)
+    xcl = x.channels_last() if idx is None else None
+    if xcl is not None and xcl.border >= pad:         # no argmax wanted and the input lives in channels-last form
+        ycl = out.channels_last_out(1)
+        if ycl is not None:
+            lib.call("xsmi_cl_maxpool2d", xcl.buf.cptr, xcl.border, ycl.buf.cptr, ycl.border, n, c, h, w, int(k),
+                     int(stride[0]), int(stride[1]), int(pad))
+            return out, None
     lib.call("xsmi_maxpool2d_fwd", x.cptr, out.cptr, idx.cptr if idx is not None else None,
              n, c, h, w, int(k), int(stride[0]), int(stride[1]), int(pad))
     return out, idx
@@ -267,7 +289,9 @@ def add(a, b, out=None, defer=False):
     _f32(a, "a"); _f32(b, "b")
     if defer and out is None and a.size == b.size:
         out = empty(a.shape)
-        a.ptr; b.ptr                                  # operands with a pending clear are cleared now
+        acl, bcl = a.channels_last(), b.channels_last()
+        if acl is None or bcl is None or not acl.same_layout(bcl):
+            a.ptr; b.ptr                              # operands with a pending clear are cleared now
         capi.defer_add(a, b, out)
         return out
     out = _like(a, out)
@@ -291,6 +315,12 @@ def relu_fwd(x, out=None):
     if out is x:                                      # in place: a held-back add that produced x joins this pass
         ops = capi.take_deferred_add(x)
         if ops is not None:
+            acl, bcl = ops[0].channels_last(), ops[1].channels_last()
+            if acl is not None and bcl is not None and acl.same_layout(bcl):
+                xcl = x.channels_last_out(acl.border)     # both operands live in channels-last form: so does the sum
+                if xcl is not None:
+                    lib.call("xsmi_cl_add", acl.buf.cptr, bcl.buf.cptr, xcl.buf.cptr, xcl.buf.size, 1)
+                    return x
             lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, None, x.size)
             return x
     out = _like(x, out)

@@ -1,0 +1,146 @@
+// Neighbours of the bf16 convolution on channels-last bf16 activations.
+//
+// A channels-last tensor is bf16 [N][H + 2 b][W + 2 b][C] with a zero border of b pixels and C a multiple of 8: eight
+// consecutive channels of a pixel are one 16-byte vector, which is what the bf16 convolution kernel loads as an MFMA
+// operand, so a chain conv -> add/ReLU -> pool -> conv never rewrites its activations as fp32 NCHW.  All three
+// kernels here move 16-byte vectors and are bound by memory bandwidth:
+//   cl_add_relu   out = max(0, a + b) (or a + b) over whole buffers, borders included (0 + 0 = 0 keeps them zero)
+//   cl_maxpool    k x k / stride max pooling; the zero border of the input IS the reference's zero-valued padding
+//                 that takes part in the max (xs/nn/functional.py:445-491), so no bounds tests in the window loop
+//   cl_to_nchw    the fp32 NCHW form of a channels-last tensor, for every consumer that does not read channels-last
+#include "xsmi_internal.h"
+
+namespace {
+
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+
+__global__ void __launch_bounds__(256) cl_add_kernel(const bf16x8 *__restrict__ a, const bf16x8 *__restrict__ b,
+                                                      bf16x8 *__restrict__ out, size_t vecs, int relu) {
+    const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    if (i >= vecs) return;
+    const bf16x8 va = a[i], vb = b[i];
+    bf16x8 r;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) {
+        float s = (float)va[e] + (float)vb[e];
+        if (relu) s = s > 0.f ? s : 0.f;
+        r[e] = (__bf16)s;
+    }
+    out[i] = r;
+}
+
+// one thread = one output pixel x eight channels; consecutive threads = consecutive channel octets, then pixels
+__global__ void __launch_bounds__(256) cl_maxpool_kernel(const bf16x8 *__restrict__ x, bf16x8 *__restrict__ y, int C8, int Wpi,
+                                                          int Hpi, int off, int k, int sh, int sw, int OH, int OW, int Wpo,
+                                                          int Hpo, int ob, uint32_t total, xsmi::FastDiv dC8,
+                                                          xsmi::FastDiv dOW, xsmi::FastDiv dOH) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= total) return;
+    const uint32_t pq = xsmi::fdiv(i, dC8), c8 = i - pq * (uint32_t)C8;
+    const uint32_t rq = xsmi::fdiv(pq, dOW), ox = pq - rq * (uint32_t)OW;
+    const uint32_t n = xsmi::fdiv(rq, dOH), oy = rq - n * (uint32_t)OH;
+    // window origin inside the padded input: (border - pad) + stride * o
+    const bf16x8 *src = x + (((size_t)n * Hpi + (size_t)(off + (int)oy * sh)) * Wpi + (size_t)(off + (int)ox * sw)) * C8 + c8;
+    float m[8];
+#pragma unroll
+    for (int e = 0; e < 8; ++e) m[e] = -INFINITY;
+    for (int r = 0; r < k; ++r)
+        for (int s = 0; s < k; ++s) {
+            const bf16x8 v = src[((size_t)r * Wpi + s) * C8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) {
+                const float f = (float)v[e];
+                m[e] = f > m[e] ? f : m[e];
+            }
+        }
+    bf16x8 o;
+#pragma unroll
+    for (int e = 0; e < 8; ++e) o[e] = (__bf16)m[e];
+    y[(((size_t)n * Hpo + oy + ob) * Wpo + ox + ob) * C8 + c8] = o;
+}
+
+// A workgroup converts one image row (W pixels) of 64 channels through an LDS tile [64][W | 1] of floats: reading,
+// eight threads cover a pixel's 64 channels (128 contiguous bytes); writing, a wave writes runs of one channel's row.
+__global__ void __launch_bounds__(256) cl_to_nchw_kernel(const bf16x8 *__restrict__ x, float *__restrict__ y, int C, int H, int W,
+                                                          int b, int cgroups) {
+    extern __shared__ float tile[];                   // [64][W | 1]
+    const int ldw = W | 1;
+    const int t = threadIdx.x;
+    const int cg = (int)(blockIdx.x % (uint32_t)cgroups);
+    const int rowid = (int)(blockIdx.x / (uint32_t)cgroups);       // n * H + h
+    const int h = rowid % H, n = rowid / H;
+    const int Wp = W + 2 * b, Hp = H + 2 * b, C8 = C / 8;
+    const int c0 = cg * 64;
+    const int oct = t & 7;                             // octet of the 64-channel group
+    const bool oct_ok = c0 + oct * 8 < C;
+    const bf16x8 *row = x + (((size_t)n * Hp + h + b) * Wp + b) * C8 + (c0 >> 3) + oct;
+    for (int px = t >> 3; px < W; px += 32) {
+        if (oct_ok) {
+            const bf16x8 v = row[(size_t)px * C8];
+#pragma unroll
+            for (int e = 0; e < 8; ++e) tile[(oct * 8 + e) * ldw + px] = (float)v[e];
+        }
+    }
+    __syncthreads();
+    const int nch = C - c0 < 64 ? C - c0 : 64;
+    float *dst = y + (((size_t)n * C + c0) * H + h) * W;
+    for (int i = t; i < nch * W; i += 256) {
+        const int c = i / W, px = i - c * W;
+        dst[(size_t)c * H * W + px] = tile[c * ldw + px];
+    }
+}
+
+}  // namespace
+
+int xsmi_cl_add(const void *a, const void *b, void *out, size_t count, int relu) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(a && b && out, "xsmi_cl_add: null pointer");
+    XSMI_CHECK_ARG(count % 8 == 0 && (((uintptr_t)a | (uintptr_t)b | (uintptr_t)out) & 15) == 0,
+                   "xsmi_cl_add: count must be a multiple of 8 and the buffers 16-byte aligned");
+    const size_t vecs = count / 8;
+    if (vecs == 0) return XSMI_OK;
+    XSMI_CHECK_ARG((vecs + 255) / 256 < ((size_t)1 << 31), "xsmi_cl_add: too many elements");
+    hipLaunchKernelGGL(cl_add_kernel, dim3((unsigned)((vecs + 255) / 256)), dim3(256), 0, xsmi::stream(), (const bf16x8 *)a,
+                       (const bf16x8 *)b, (bf16x8 *)out, vecs, relu);
+    XSMI_LAUNCH_CHECK("cl_add_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_cl_maxpool2d(const void *x_cl, int x_border, void *y_cl, int y_border, int N, int C, int H, int W, int k, int sh,
+                      int sw, int pad) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(x_cl && y_cl, "xsmi_cl_maxpool2d: null pointer");
+    XSMI_CHECK_ARG(N > 0 && C > 0 && C % 8 == 0 && H > 0 && W > 0, "xsmi_cl_maxpool2d: needs C %% 8 == 0 (N=%d C=%d H=%d W=%d)", N,
+                   C, H, W);
+    XSMI_CHECK_ARG(k >= 1 && sh >= 1 && sw >= 1 && pad >= 0 && x_border >= pad && y_border >= 0,
+                   "xsmi_cl_maxpool2d: window %d stride %dx%d pad %d needs an input border >= pad (%d)", k, sh, sw, pad, x_border);
+    XSMI_CHECK_ARG(H + 2 * pad >= k && W + 2 * pad >= k, "xsmi_cl_maxpool2d: window larger than the padded input");
+    XSMI_CHECK_ARG((((uintptr_t)x_cl | (uintptr_t)y_cl) & 15) == 0, "xsmi_cl_maxpool2d: buffers must be 16-byte aligned");
+    const int OH = (H + 2 * pad - k) / sh + 1, OW = (W + 2 * pad - k) / sw + 1;
+    const int C8 = C / 8;
+    const size_t total = (size_t)N * OH * OW * C8;
+    XSMI_CHECK_ARG(total < ((size_t)1 << 32), "xsmi_cl_maxpool2d: too many outputs");
+    hipLaunchKernelGGL(cl_maxpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, xsmi::stream(),
+                       (const bf16x8 *)x_cl, (bf16x8 *)y_cl, C8, W + 2 * x_border, H + 2 * x_border, x_border - pad, k, sh, sw, OH,
+                       OW, OW + 2 * y_border, OH + 2 * y_border, y_border, (uint32_t)total, xsmi::make_fastdiv(C8),
+                       xsmi::make_fastdiv(OW), xsmi::make_fastdiv(OH));
+    XSMI_LAUNCH_CHECK("cl_maxpool_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_cl_to_nchw(const void *x_cl, int border, float *y, int N, int C, int H, int W) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(x_cl && y, "xsmi_cl_to_nchw: null pointer");
+    XSMI_CHECK_ARG(N > 0 && C > 0 && C % 8 == 0 && H > 0 && W > 0 && border >= 0,
+                   "xsmi_cl_to_nchw: needs C %% 8 == 0 (N=%d C=%d H=%d W=%d border=%d)", N, C, H, W, border);
+    XSMI_CHECK_ARG(((uintptr_t)x_cl & 15) == 0, "xsmi_cl_to_nchw: x_cl must be 16-byte aligned");
+    const size_t lds = (size_t)64 * (W | 1) * sizeof(float);
+    XSMI_CHECK_ARG(lds <= 64 * 1024, "xsmi_cl_to_nchw: rows of more than 255 pixels are not supported (W=%d)", W);
+    const int cgroups = xsmi::ceil_div(C, 64);
+    const size_t blocks = (size_t)N * H * cgroups;
+    XSMI_CHECK_ARG(blocks < ((size_t)1 << 31), "xsmi_cl_to_nchw: too many rows");
+    hipLaunchKernelGGL(cl_to_nchw_kernel, dim3((unsigned)blocks), dim3(256), lds, xsmi::stream(), (const bf16x8 *)x_cl, y, C, H, W,
+                       border, cgroups);
+    XSMI_LAUNCH_CHECK("cl_to_nchw_kernel");
+    return XSMI_OK;
+}

@@ -342,7 +342,7 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
                    workspace_bytes);
     if ((flags & XSMI_CONV_BF16) && xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad) &&
         workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
-        return xsmi::nhwc_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
+        return xsmi::nhwc_conv_fwd(x, nullptr, 0, w, bias, y, nullptr, 0, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
                                    (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
     if (!(flags & XSMI_CONV_BF16) && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad) &&
         workspace_bytes >= xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
@@ -388,6 +388,38 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     xsmi::prof_end();
     XSMI_LAUNCH_CHECK("igemm_f32_kernel");
     return XSMI_OK;
+}
+
+
+int xsmi_conv2d_fwd_cl(const float *x, const void *x_cl, int x_border, const float *w, const float *bias, float *y, void *y_cl,
+                       int y_border, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, unsigned flags,
+                       void *workspace, size_t workspace_bytes) {
+    XSMI_REQUIRE_INIT();
+    ConvGeom g;
+    int rc = check_conv("xsmi_conv2d_fwd_cl", N, C, H, W, K, R, S, sh, sw, pad, &g);
+    if (rc) return rc;
+    XSMI_CHECK_ARG(w && ((x != nullptr) != (x_cl != nullptr)) && ((y != nullptr) != (y_cl != nullptr)),
+                   "xsmi_conv2d_fwd_cl: exactly one of x / x_cl and one of y / y_cl must be given");
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_fwd_cl: unknown flags 0x%x", flags);
+    if (x_cl) {
+        XSMI_CHECK_ARG(C % 32 == 0 && x_border >= pad && x_border <= 8,
+                       "xsmi_conv2d_fwd_cl: a channels-last input needs C %% 32 == 0 and pad <= border <= 8 (C=%d pad=%d border=%d)",
+                       C, pad, x_border);
+        XSMI_CHECK_ARG(((uintptr_t)x_cl & 15) == 0, "xsmi_conv2d_fwd_cl: x_cl must be 16-byte aligned");
+    }
+    if (y_cl) {
+        XSMI_CHECK_ARG(K % 8 == 0 && y_border >= 0 && y_border <= 8,
+                       "xsmi_conv2d_fwd_cl: a channels-last output needs K %% 8 == 0 and 0 <= border <= 8 (K=%d border=%d)", K,
+                       y_border);
+        XSMI_CHECK_ARG(((uintptr_t)y_cl & 15) == 0, "xsmi_conv2d_fwd_cl: y_cl must be 16-byte aligned");
+    }
+    const int b = x_cl ? x_border : pad;
+    XSMI_CHECK_ARG(xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, b), "xsmi_conv2d_fwd_cl: geometry outside the channels-last kernel's range");
+    const size_t need = x_cl ? xsmi::nhwc_filter_ws_bytes(C, K, R, S) : xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad);
+    XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd_cl: workspace of %zu bytes needed, %zu given", need,
+                   workspace_bytes);
+    return xsmi::nhwc_conv_fwd(x, x_cl, x_border, w, bias, y, y_cl, y_border, nullptr, N, C, H, W, K, R, S, sh, sw, pad, g.OH,
+                               g.OW, (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
 }
 
 int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int C, int H, int W, int K, int R, int S,

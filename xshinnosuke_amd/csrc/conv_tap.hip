@@ -548,6 +548,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
 }
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
 
 // bf16 tile kernel: operands are rounded to bf16 on their way INTO the LDS, so a stage holds bf16 in the
 // layout the matrix instruction consumes and every fragment is one 128-bit LDS read.
@@ -778,6 +779,9 @@ struct NhwcParams {
     int relu;
     int rowtiles;
     uint32_t tiles;       // pixel tiles x row tiles
+    // channels-last bf16 output instead of `out`: [N][OY + 2 ob][OX + 2 ob][ocp], only the interior is written
+    __bf16 *out_cl;
+    int ob, ocp;
 };
 
 // x fp32 [N][C][H][W] -> xp bf16 [N][Hp][Wp][CP]; a workgroup converts WS pixels of one padded row through an
@@ -879,7 +883,6 @@ __global__ void __launch_bounds__(256) nhwc_pad_c4_kernel(const float *__restric
         for (int c = 0; c < 4; ++c)
             if (c < C) v[c] = src[(size_t)c * H * W];
     }
-    typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
     bf16x4 pk;
 #pragma unroll
     for (int c = 0; c < 4; ++c) pk[c] = (__bf16)v[c];
@@ -1057,6 +1060,40 @@ __global__ void __launch_bounds__(256, WR == 2 ? 3 : 2) tap_nhwc_bf16_kernel(Nhw
             __syncthreads();
         }
         const int lrow = wr * 64 + 4 * h;
+        if (p.out_cl) {
+            // A lane holds four consecutive filters (v % 4) of a pixel: one 8-byte store of four bf16.  The two lane
+            // halves and the four register groups of a block cover 32 consecutive channels, 64 contiguous bytes.
+#pragma unroll
+            for (int j = 0; j < 2; ++j) {
+                const int m = m0 + wc * 64 + 32 * j + l31;
+                if (m >= p.M) continue;
+                uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
+                int x = m - (int)q * p.OX;
+                uint32_t n = xsmi::fdiv(q, p.dOY);
+                int y = (int)q - (int)n * p.OY;
+                const size_t pix = ((size_t)((int)n * (p.OY + 2 * p.ob) + y + p.ob) * (size_t)(p.OX + 2 * p.ob) + (size_t)(x + p.ob)) *
+                                   (size_t)p.ocp;
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int gq = 0; gq < 4; ++gq) {
+                        const int row = rbase + 32 * i + 8 * gq;
+                        if (row >= p.rows) continue;                 // rows is a multiple of 4 on this path
+                        float v4[4];
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) {
+                            float val = acc[i][j][4 * gq + e];
+                            if (p.bias) val += s_bias[lrow + 32 * i + 8 * gq + e];
+                            if (p.relu) val = val > 0.f ? val : 0.f;
+                            v4[e] = val;
+                        }
+                        bf16x4 o4;
+                        o4[0] = (__bf16)v4[0]; o4[1] = (__bf16)v4[1]; o4[2] = (__bf16)v4[2]; o4[3] = (__bf16)v4[3];
+                        *reinterpret_cast<bf16x4 *>(p.out_cl + pix + row) = o4;
+                    }
+            }
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < 2; ++j) {
             const int m = m0 + wc * 64 + 32 * j + l31;
@@ -1457,16 +1494,23 @@ bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad) {
     return nhwc_xp_bytes(N, C, H, W, S, pad) < ((size_t)1 << 31) && nhwc_apk_bytes(C, K, R, S) < ((size_t)1 << 32);
 }
 
+size_t nhwc_filter_ws_bytes(int C, int K, int R, int S) { return nhwc_apk_bytes(C, K, R, S); }
+
 size_t nhwc_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int pad) {
     return nhwc_apk_bytes(C, K, R, S) + nhwc_xp_bytes(N, C, H, W, S, pad);
 }
 
-int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
-                  int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace) {
+// x_cl: the input as a channels-last bf16 tensor [N][H + 2 xb][W + 2 xb][C] with a zero border xb >= pad (C a multiple
+// of 32), instead of x: no copy is made.  y_cl: the output goes to a channels-last bf16 tensor with border yb
+// (K a multiple of 8; only its interior is written) instead of y.
+int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, const float *bias, float *y, void *y_cl, int yb,
+                  uint8_t *mask, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OH, int OW,
+                  int relu, int opts, void *workspace) {
     hipStream_t st = stream();
     const bool pair = nhwc_pair(C, S);
     const int CP = nhwc_cp(C, S), C8 = pair ? 4 : CP / 8, ROWS = nhwc_rows(K);
-    const int Hp = H + 2 * pad, Wp = W + 2 * pad;
+    const int border = x_cl ? xb : pad;
+    const int Hp = H + 2 * border, Wp = W + 2 * border;
     const int nchunks = nhwc_chunks(C, R, S), rowtiles = ceil_div(K, ROWS);
     __bf16 *apk = (__bf16 *)workspace;
     __bf16 *xp = (__bf16 *)((char *)workspace + nhwc_apk_bytes(C, K, R, S));
@@ -1479,7 +1523,10 @@ int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
         XSMI_LAUNCH_CHECK("tap_pack_oct_kernel");
     }
     prof_begin();
-    if (CP == 4) {
+    if (x_cl) {
+        // the window of output (0, 0) starts (xb - pad) rows and columns inside the border
+        xp = (__bf16 *)x_cl + ((size_t)(xb - pad) * Wp + (size_t)(xb - pad)) * CP;
+    } else if (CP == 4) {
         const int nwb = ceil_div(Wp, 256);
         hipLaunchKernelGGL(nhwc_pad_c4_kernel, dim3((unsigned)nwb * (unsigned)(N * Hp)), dim3(256), 0, st, x, xp, C, H,
                            W, pad, Hp, Wp, nwb);
@@ -1501,6 +1548,8 @@ int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
     NhwcParams p;
     p.xp = xp; p.apk = (const float *)apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
     p.xp_bytes = (uint32_t)((size_t)N * Hp * Wp * CP * 2);
+    if (x_cl) p.xp_bytes -= (uint32_t)(((size_t)(xb - pad) * Wp + (size_t)(xb - pad)) * CP * 2);
+    p.out_cl = (__bf16 *)y_cl; p.ob = yb; p.ocp = K;
     p.apk_bytes = (uint32_t)nhwc_apk_bytes(C, K, R, S);
     p.M = N * OH * OW; p.rows = K; p.nchunks = nchunks;
     p.R = R; p.S = pair ? 1 : S; p.C8 = C8; p.Hp = Hp; p.Wp = Wp; p.sy = sh; p.sx = sw;

@@ -128,8 +128,11 @@ int stem_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
 // at most 8 (a stem); the workspace holds the packed filter followed by the copy
 bool nhwc_fwd_ok(int N, int C, int H, int W, int K, int R, int S, int pad);
 size_t nhwc_fwd_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int pad);
-int nhwc_conv_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *mask, int N, int C, int H, int W,
-                  int K, int R, int S, int sh, int sw, int pad, int OH, int OW, int relu, int opts, void *workspace);
+size_t nhwc_filter_ws_bytes(int C, int K, int R, int S);    // the packed filter alone (input already channels-last)
+// x_cl / y_cl: channels-last bf16 tensors [N][H + 2 b][W + 2 b][C] with a zero border b, used instead of x / y when given
+int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, const float *bias, float *y, void *y_cl, int yb,
+                  uint8_t *mask, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OH, int OW,
+                  int relu, int opts, void *workspace);
 
 // tap-major backward-weight (conv_wgrad_tap.hip)
 bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW);

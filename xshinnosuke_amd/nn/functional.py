@@ -86,13 +86,17 @@ def conv2d(inputs, weight, bias=None, stride=(1, 1), padding=0, out=None, activa
     neg_mask = dev.empty((n, k, oh, ow), np.uint8) if (activation == 'relu' and track) else None
     bf16 = bool(GLOBAL.CONV_BF16)
 
+    # without gradients a bf16 result may stay in channels-last form for the next bf16 consumer (DeviceArray.channels_last)
+    cl = bf16 and not track and on_device
     if out is None:
-        y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16)
+        y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16,
+                             channels_last=cl)
         out = Tensor(y_dev if on_device else y_dev.numpy().astype(x.dtype, copy=False))
     else:
         dst = out.eval
         if is_device(dst):
-            K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask, bf16=bf16)
+            K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask, bf16=bf16,
+                         channels_last=cl)
         else:
             y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16)
             out.eval = y_dev.numpy()              # cast to the buffer's dtype on store
@@ -140,13 +144,13 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
         need = K.conv2d_workspace_bytes(x.shape, weight.shape, stride, padding)
         if kept is not None and kept['key'] == now and kept['ws'].holds(need):
             y = K.conv2d_fwd(x, kept['w'], kept['b'], stride, padding, relu=relu, out=dst, bf16=bf16, packed=True,
-                             workspace=kept['ws'])
+                             workspace=kept['ws'], channels_last=bf16)
         else:
             stats = [a.reshape(-1) for a in sources[-4:]]
             b_dev = None if bias is None else bias.eval.reshape(-1)
             w2, b2 = K.bn_fold(weight.eval, b_dev, *stats, epsilon)
             ws = kept['ws'] if kept is not None else K.Workspace()
-            y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, workspace=ws)
+            y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, workspace=ws, channels_last=bf16)
             # the fold has read the parameters: their state as of now is what the kept filter belongs to
             key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape))
             _FOLDED[weight] = {'key': key, 'w': w2, 'b': b2, 'ws': ws, 'of': sources}   # 'of' keeps the ids in the key alive
@@ -154,7 +158,7 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
         stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]
         b_dev = None if bias is None else _f32_device(bias.eval).reshape(-1)
         w2, b2 = K.bn_fold(_f32_device(weight.eval), b_dev, *stats, epsilon)
-        y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16)
+        y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, channels_last=bf16)
     if out is None:
         out = Tensor(y)
     elif y is not dst:
