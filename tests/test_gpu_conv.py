@@ -30,6 +30,9 @@ CASES = [  # n c h w k r s sh sw pad
     (1, 2, 6, 6, 3, 3, 3, 1, 1, 2),        # pad > (R-1)/2
     (5, 33, 10, 10, 65, 1, 1, 1, 1, 0),    # 1x1 == GEMM, odd sizes
     (1, 1, 3, 3, 1, 3, 3, 1, 1, 0),        # single output pixel
+    (3, 1, 20, 32, 64, 5, 5, 1, 2, 2),     # few-channel first layers (horizontal stride 2, output width % 8 == 0):
+    (2, 3, 17, 32, 128, 3, 3, 2, 2, 1),    #   one channel with vertical stride 1; two row tiles of filters;
+    (2, 4, 12, 30, 64, 3, 3, 2, 2, 2),     #   four channels, padding wider than the filter's reach
 ]
 
 

@@ -227,8 +227,178 @@ __global__ void __launch_bounds__(64 * WAVES) stem_fwd_f32_kernel(StemParams p) 
     else emit_mode(std::true_type{});
 }
 
+
+// ---- weight gradient of the same layers --------------------------------------------------------------------------
+// dw[k][j] = sum over pixels of dy[n][k][y][x] * xp[n][c][sh y + r][2 x + s], j = (c R + r) S + s, on the zero-bordered
+// copy xp.  MFMA rows are filters (64 per workgroup row tile), columns the filter positions j (JB blocks of 32), the
+// reduction runs over pixels.  Eight consecutive pixels of an output row are one unit: step t = 0..3 pairs pixel
+// 8g + t (lane half 0) with pixel 8g + 4 + t (half 1), so a lane's four A values are one aligned float4 of dy and its
+// four B values are xp[base + 2t]: both operands go straight from memory to registers (B as gathers of single floats
+// that hit the L1: the S columns of a filter row read the same 24 floats), nothing is staged, and the waves of a
+// workgroup never synchronise until the end.  Each wave takes an equal run of units; the four waves' accumulators
+// are added in wave order through the LDS and the workgroup writes one partial [64][32 JB]; a second kernel adds
+// the partials in float64 in ascending order.
+struct StemWgradParams {
+    const float *dy;       // [N][K][OH][OW]
+    const float *xp;       // [N][C][Hp][Wp]
+    float *part;           // [workgroups.x][K][32 JB]
+    float *dbpart;         // [workgroups.x][K] or nullptr
+    int K, C, R, S, J, Hp, Wp, OH, OW, sh;
+    uint32_t units;        // N * OH * (OW / 8)
+    xsmi::FastDiv dG8, dOH, dS, dR;
+};
+
+template <int JB>
+__global__ void __launch_bounds__(256, 1) stem_wgrad_f32_kernel(StemWgradParams p) {
+    extern __shared__ __attribute__((aligned(16))) float red[];       // [64][32 JB] (+ [4][64] for the bias sums)
+    const int t = threadIdx.x, lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const int kk = lane >> 5, l31 = lane & 31;
+    const int rowtile = blockIdx.y;
+    const int G8 = p.OW >> 3;
+
+    constexpr int LDJ = 32 * JB;
+    // this lane's column of each block: element offset of (c, r, s) inside an image of the copy
+    uint32_t coloff[JB];
+#pragma unroll
+    for (int jb = 0; jb < JB; ++jb) {
+        int j = 32 * jb + l31;
+        if (j > p.J - 1) j = p.J - 1;                       // columns past the filter repeat the last one; never stored
+        const uint32_t rc = xsmi::fdiv((uint32_t)j, p.dS), s_ = (uint32_t)j - rc * (uint32_t)p.S;
+        const uint32_t c = xsmi::fdiv(rc, p.dR), r = rc - c * (uint32_t)p.R;
+        coloff[jb] = ((c * (uint32_t)p.Hp + r) * (uint32_t)p.Wp + s_ + 8u * (uint32_t)kk);
+    }
+    const uint32_t nw = gridDim.x * 4u, wv = blockIdx.x * 4u + (uint32_t)wave;
+    const uint32_t u0 = (uint32_t)(((uint64_t)wv * p.units) / nw), u1 = (uint32_t)(((uint64_t)(wv + 1) * p.units) / nw);
+    const size_t img_in = (size_t)p.C * p.Hp * p.Wp, plane_out = (size_t)p.OH * p.OW;
+    const float *dy_row = p.dy + ((size_t)rowtile * 64 + l31) * plane_out + 4 * kk;   // + n K plane + y OW + 8 g
+
+    floatx16 acc[2][JB];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int jb = 0; jb < JB; ++jb)
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[i][jb][v] = 0.f;
+    float dbs[2] = {0.f, 0.f};
+
+    // Two register buffers: a unit's operands are requested while the previous unit multiplies (a third buffer,
+    // i.e. requests two units ahead, measured slower: the loop is bound by the gathers' address work, not by latency).
+    float4 a[2][2];
+    float b[2][JB][4];
+    auto load_unit = [&](int buf, uint32_t u) {
+        const uint32_t q = xsmi::fdiv(u, p.dG8), g = u - q * (uint32_t)G8;
+        const uint32_t n = xsmi::fdiv(q, p.dOH), y = q - n * (uint32_t)p.OH;
+        const float *ap = dy_row + (size_t)n * p.K * plane_out + (size_t)y * p.OW + 8 * g;
+        a[buf][0] = *reinterpret_cast<const float4 *>(ap);
+        a[buf][1] = *reinterpret_cast<const float4 *>(ap + 32 * plane_out);
+        const float *bp = p.xp + (size_t)n * img_in + (size_t)(y * (uint32_t)p.sh) * p.Wp + 16 * g;
+#pragma unroll
+        for (int jb = 0; jb < JB; ++jb)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) b[buf][jb][e] = bp[coloff[jb] + 2 * e];
+    };
+    auto multiply = [&](int buf) {
+        dbs[0] += (a[buf][0].x + a[buf][0].y) + (a[buf][0].z + a[buf][0].w);
+        dbs[1] += (a[buf][1].x + a[buf][1].y) + (a[buf][1].z + a[buf][1].w);
+#pragma unroll
+        for (int e = 0; e < 4; ++e)
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float av = e == 0 ? a[buf][i].x : e == 1 ? a[buf][i].y : e == 2 ? a[buf][i].z : a[buf][i].w;
+#pragma unroll
+                for (int jb = 0; jb < JB; ++jb)
+                    acc[i][jb] = __builtin_amdgcn_mfma_f32_32x32x2f32(av, b[buf][jb][e], acc[i][jb], 0, 0, 0);
+            }
+    };
+    if (u0 < u1) {
+        load_unit(0, u0);
+        uint32_t u = u0;
+        for (; u + 2 < u1; u += 2) {                        // two units per trip: the buffers alternate statically
+            load_unit(1, u + 1);
+            multiply(0);
+            load_unit(0, u + 2);
+            multiply(1);
+        }
+        if (u + 1 < u1) {
+            load_unit(1, u + 1);
+            multiply(0);
+            multiply(1);
+        } else {
+            multiply(0);
+        }
+    }
+
+    // the four waves' accumulators, added in wave order: register v of lane l in block (i, jb) is
+    // row 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, column 32 jb + l % 32
+    float *dbred = red + 64 * LDJ;
+    for (int w = 0; w < 4; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int jb = 0; jb < JB; ++jb)
+#pragma unroll
+                    for (int v = 0; v < 16; ++v) {
+                        const int idx = (32 * i + 8 * (v >> 2) + 4 * kk + (v & 3)) * LDJ + 32 * jb + l31;
+                        red[idx] = w == 0 ? acc[i][jb][v] : red[idx] + acc[i][jb][v];
+                    }
+            // bias sums: the two lane halves hold different pixels of the same filter row
+#pragma unroll
+            for (int i = 0; i < 2; ++i) {
+                const float both = dbs[i] + __shfl_xor(dbs[i], 32);
+                if (kk == 0) dbred[w * 64 + 32 * i + l31] = both;
+            }
+        }
+        __syncthreads();
+    }
+    float *dst = p.part + ((size_t)blockIdx.x * p.K + (size_t)rowtile * 64) * LDJ;
+    for (int i = t; i < 64 * LDJ; i += 256) dst[i] = red[i];
+    if (p.dbpart && t < 64)
+        p.dbpart[(size_t)blockIdx.x * p.K + rowtile * 64 + t] = ((dbred[t] + dbred[64 + t]) + dbred[128 + t]) + dbred[192 + t];
+}
+
+// dw[k][j] = (accumulate ? dw : 0) + sum over the workgroups' partials, db likewise: 16 threads per output, each adds
+// every 16th partial in ascending order in float64, then the 16 sums are added in a fixed order.
+__global__ void __launch_bounds__(256) stem_wgrad_reduce_kernel(const float *__restrict__ part, float *__restrict__ dw,
+                                                                 const float *__restrict__ dbpart, float *__restrict__ db, int K,
+                                                                 int J, int LDJ, int splits, int accumulate) {
+    __shared__ double sm[16][17];
+    const int col = threadIdx.x & 15, grp = threadIdx.x >> 4;
+    const int o = blockIdx.x * 16 + col;                    // output index: [0, K J) weights, then K biases
+    const int nw = K * J;
+    const float *src = nullptr;
+    float *dst = nullptr;
+    size_t stride = 0;
+    if (o < nw) {
+        const int k = o / J, j = o - k * J;
+        src = part + (size_t)k * LDJ + j; stride = (size_t)K * LDJ; dst = dw + o;
+    } else if (db && o < nw + K) {
+        src = dbpart + (o - nw); stride = (size_t)K; dst = db + (o - nw);
+    }
+    double s = 0.0;
+    if (src) {
+        int sp = grp;
+        for (; sp + 48 < splits; sp += 64) {
+            const float v0 = src[(size_t)sp * stride], v1 = src[(size_t)(sp + 16) * stride];
+            const float v2 = src[(size_t)(sp + 32) * stride], v3 = src[(size_t)(sp + 48) * stride];
+            s += (double)v0; s += (double)v1; s += (double)v2; s += (double)v3;
+        }
+        for (; sp < splits; sp += 16) s += (double)src[(size_t)sp * stride];
+    }
+    sm[grp][col] = s;
+    __syncthreads();
+    if (grp == 0 && dst) {
+        double tot = 0.0;
+#pragma unroll
+        for (int g = 0; g < 16; ++g) tot += sm[g][col];
+        if (accumulate) tot += (double)*dst;
+        *dst = (float)tot;
+    }
+}
+
 int stem_Wp(int W, int S, int sw, int pad, int OW) {
-    int need = sw * (OW - 1) + 8;                        // the last pixel's run of eight
+    int need = sw * OW + 8;                              // the last pixel's run of eight; 24 floats from the last unit of eight pixels
     int wp = W + 2 * pad > need ? W + 2 * pad : need;
     return (wp + 3) & ~3;                                // runs start on 8-byte boundaries; the copy writes 16 bytes per thread
 }
@@ -305,6 +475,72 @@ int stem_conv_fwd(const float *x, const float *w, const float *bias, float *y, u
     }
     prof_end();
     XSMI_LAUNCH_CHECK("stem_fwd_f32_kernel");
+    return XSMI_OK;
+}
+
+
+// ---- weight gradient ----
+static int stem_wgrad_groups() { return cu_count(); }        // workgroups per row tile = partial sums to reduce
+
+bool stem_wgrad_ok(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad) {
+    if (C > 4 || C * R * S > 160 || R > 8 || S > 8 || sw != 2 || sh < 1 || K % 64 != 0) return false;
+    const int OW = (W + 2 * pad - S) / sw + 1;
+    if (OW % 8 != 0) return false;
+    const size_t xp = (size_t)N * C * (H + 2 * pad) * stem_Wp(W, S, sw, pad, OW) * 4;
+    return xp < ((size_t)1 << 31);
+}
+
+size_t stem_wgrad_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad) {
+    const int OW = (W + 2 * pad - S) / sw + 1;
+    const int JB = ceil_div(C * R * S, 32);
+    const size_t xp = align_up((size_t)N * C * (H + 2 * pad) * stem_Wp(W, S, sw, pad, OW) * sizeof(float), 256);
+    const size_t part = align_up((size_t)stem_wgrad_groups() * K * 32 * JB * sizeof(float), 256);
+    const size_t dbp = align_up((size_t)stem_wgrad_groups() * K * sizeof(float), 256);
+    return xp + part + dbp;
+}
+
+template <int JB>
+static void stem_wgrad_launch(hipStream_t st, dim3 grid, const StemWgradParams &p) {
+    const size_t lds = ((size_t)64 * 32 * JB + 256) * sizeof(float);
+    hipLaunchKernelGGL((stem_wgrad_f32_kernel<JB>), grid, dim3(256), lds, st, p);
+}
+
+int stem_conv_bwd_weight(const float *dy, const float *x, float *dw, float *db, int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int pad, int OH, int OW, int accumulate, void *workspace) {
+    hipStream_t st = stream();
+    const int Hp = H + 2 * pad, Wp = stem_Wp(W, S, sw, pad, OW);
+    const int J = C * R * S, JB = ceil_div(J, 32);
+    const int groups = stem_wgrad_groups();
+    const size_t xp_bytes = align_up((size_t)N * C * Hp * Wp * sizeof(float), 256);
+    const size_t part_bytes = align_up((size_t)groups * K * 32 * JB * sizeof(float), 256);
+    float *xp = (float *)workspace;
+    float *part = (float *)((char *)workspace + xp_bytes);
+    float *dbpart = (float *)((char *)workspace + xp_bytes + part_bytes);
+    const uint32_t quads = (uint32_t)((size_t)N * C * Hp * Wp / 4);
+    const uint32_t pad_blocks = (quads + 255) / 256;
+    hipLaunchKernelGGL(stem_prepare_kernel, dim3(pad_blocks), dim3(256), 0, st, x, xp, H, W, pad, Hp, Wp / 4, make_fastdiv(Wp / 4),
+                       make_fastdiv(Hp), quads, pad_blocks, (const float *)nullptr, (float *)nullptr, K, C, R, S, 0);
+    XSMI_LAUNCH_CHECK("stem_prepare_kernel");
+    StemWgradParams p;
+    p.dy = dy; p.xp = xp; p.part = part; p.dbpart = db ? dbpart : nullptr;
+    p.K = K; p.C = C; p.R = R; p.S = S; p.J = J; p.Hp = Hp; p.Wp = Wp; p.OH = OH; p.OW = OW; p.sh = sh;
+    p.units = (uint32_t)((size_t)N * OH * (OW / 8));
+    p.dG8 = make_fastdiv(OW / 8); p.dOH = make_fastdiv(OH); p.dS = make_fastdiv(S); p.dR = make_fastdiv(R);
+    const dim3 grid((unsigned)groups, (unsigned)(K / 64));
+    prof_begin();
+    switch (JB) {
+        case 1: stem_wgrad_launch<1>(st, grid, p); break;
+        case 2: stem_wgrad_launch<2>(st, grid, p); break;
+        case 3: stem_wgrad_launch<3>(st, grid, p); break;
+        case 4: stem_wgrad_launch<4>(st, grid, p); break;
+        default: stem_wgrad_launch<5>(st, grid, p); break;
+    }
+    prof_end();
+    XSMI_LAUNCH_CHECK("stem_wgrad_f32_kernel");
+    const int outputs = K * J + (db ? K : 0);
+    hipLaunchKernelGGL(stem_wgrad_reduce_kernel, dim3((unsigned)ceil_div(outputs, 16)), dim3(256), 0, st, part, dw,
+                       db ? dbpart : nullptr, db, K, J, 32 * JB, groups, accumulate);
+    XSMI_LAUNCH_CHECK("stem_wgrad_reduce_kernel");
     return XSMI_OK;
 }
 

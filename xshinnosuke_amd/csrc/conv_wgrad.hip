@@ -240,6 +240,15 @@ size_t conv_bwd_weight_ws_bytes(int N, int C, int K, int R, int S, int OH, int O
     }
     return generic;
 }
+
+int wgrad_reduce_partials(const float *part, float *dw, const float *dbpart, float *db, int K, int J, int Kp, int Jp, int splits,
+                          int accumulate) {
+    const int dw_blocks = K * ceil_div(J, 64);
+    hipLaunchKernelGGL(wgrad_reduce_kernel, dim3(dw_blocks + (db ? ceil_div(K, 64) : 0)), dim3(256), 0, stream(), part, dw, dbpart,
+                       db, K, J, Kp, Jp, splits, dw_blocks, accumulate);
+    XSMI_LAUNCH_CHECK("wgrad_reduce_kernel");
+    return XSMI_OK;
+}
 }  // namespace xsmi
 
 extern "C" {
@@ -270,6 +279,9 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
         if (rj) return rj;
     }
 
+    if (xsmi::stem_wgrad_ok(N, C, H, W, K, R, S, sh, sw, pad) && ((uintptr_t)dy & 15) == 0 &&
+        workspace_bytes >= xsmi::stem_wgrad_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
+        return xsmi::stem_conv_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, OH, OW, beta == 1.f ? 1 : 0, workspace);
     if (xsmi::wgrad_tap_ok(dy, x, C, K, OH, OW))
         return xsmi::wgrad_tap(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, OH, OW, beta == 1.f ? 1 : 0, workspace);
 

@@ -78,6 +78,10 @@ size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int
         size_t e = xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad);
         m = m > e ? m : e;
     }
+    if (xsmi::stem_wgrad_ok(N, C, H, W, K, R, S, sh, sw, pad)) {
+        size_t e = xsmi::stem_wgrad_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad);
+        m = m > e ? m : e;
+    }
     // the second-generation fp32 kernels are chosen when the workspace also has room for their partial tiles
     if (xsmi::sk_path_ok(C, K)) {
         size_t e = xsmi::sk_fwd_ws_bytes(C, K, R, S);

@@ -134,6 +134,17 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
                   uint8_t *mask, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OH, int OW,
                   int relu, int opts, void *workspace);
 
+// weight gradient for the same few-channel layers (conv_stem.hip): horizontal stride 2, output width a multiple of 8,
+// filters a multiple of 64, at most 160 filter positions; the workspace holds the copy and the workgroups' partial sums
+bool stem_wgrad_ok(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
+size_t stem_wgrad_ws_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
+int stem_conv_bwd_weight(const float *dy, const float *x, float *dw, float *db, int N, int C, int H, int W, int K, int R, int S,
+                         int sh, int sw, int pad, int OH, int OW, int accumulate, void *workspace);
+// dw[k][j] = (accumulate ? dw : 0) + sum over splits of part[split][k][j] (float64, ascending), db likewise from
+// dbpart[split][k] when given (conv_wgrad.hip)
+int wgrad_reduce_partials(const float *part, float *dw, const float *dbpart, float *db, int K, int J, int Kp, int Jp, int splits,
+                          int accumulate);
+
 // tap-major backward-weight (conv_wgrad_tap.hip)
 bool wgrad_tap_ok(const float *dy, const float *x, int C, int K, int OH, int OW);
 size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW);
