@@ -129,7 +129,7 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
 
 /* ---- channels-last bf16 activations (inference) ----------------------------
  * An extension of the forward above for chains of layers evaluated without gradients
- * (Model.predict / evaluate, xs/nn/models.py:98-116, under bf16 conv precision): the
+ * (Model.predict / evaluate, xs/nn/models.py:146-186, under bf16 conv precision): the
  * reference keeps every activation as float32 NCHW; here a tensor may instead live as
  * bf16 [N][H + 2 b][W + 2 b][C] with a zero border of b pixels ("channels-last"),
  * which is the operand layout of the bf16 MFMA kernel, so that conv -> add/ReLU ->
@@ -147,8 +147,8 @@ int xsmi_conv2d_fwd_cl(const float *x, const void *x_cl, int x_border, const flo
                        int sh, int sw, int pad, unsigned flags,
                        void *workspace, size_t workspace_bytes);
 /* out = a + b (relu = 0) or max(0, a + b) over `count` bf16 elements (a multiple of 8) of
- * equally shaped channels-last tensors, borders included: add (xs/nn/functional.py:41-52)
- * followed by relu (xs/nn/functional.py:156-163); out may be a or b. */
+ * equally shaped channels-last tensors, borders included: add (xs/nn/functional.py:6-21)
+ * followed by relu (xs/nn/functional.py:297-313); out may be a or b. */
 int xsmi_cl_add(const void *a, const void *b, void *out, size_t count, int relu);
 /* max_pool2d (xs/nn/functional.py:445-491) on channels-last tensors: the input's zero
  * border (x_border >= pad) is the reference's zero-valued padding that takes part in
