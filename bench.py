@@ -229,9 +229,13 @@ def bench_pool(be, steps, warmup):
 def bench_per_layer(be, reps):
     """Every distinct ResNet-18 convolution at N=32, pass by pass (forward incl. bias, backward-data,
     backward-weight incl. bias gradient): whole ops as the training step issues them (filter layout kernels and split
-    reductions included), `reps` launches back to back between two events after a clock ramp."""
+    reductions included), `reps` launches back to back between two events after a clock ramp.
+
+    Each (layer, pass) is preceded by one fill launch of 1024 * (index + 1) floats, so that a kernel trace of this mode
+    can be cut into its rows: that launch shows up as `ew_kernel<FillF>` with a grid of 256 * (index + 1) threads."""
     K = be.kernels
     rows = []
+    marker = be.empty((1024 * 3 * len(RESNET18_CONVS),))
     rng = np.random.default_rng(11)
     for name, count, c, k, h, r, st, pad in RESNET18_CONVS:
         oh = (h + 2 * pad - r) // st + 1
@@ -249,6 +253,7 @@ def bench_per_layer(be, reps):
         for pname, fn in passes.items():
             if pname == "bwd_data" and c == 3:
                 continue                                  # the network input needs no gradient
+            be.lib.call("xsmi_fill", marker.cptr, 0.0, 1024 * (len(rows) + 1))
             preheat(be, fn, seconds=0.25)
             ms = batch_ms(be, fn, reps)
             tf = flops / (ms * 1e-3) / 1e12
