@@ -168,12 +168,12 @@ def make_pool_inputs(p):
     return x, dy
 
 
-POOL_SETS = 5        # disjoint buffer sets the memory-bound kernels rotate over
+POOL_SETS = 10       # disjoint buffer sets the memory-bound kernels rotate over
 
 
 def bench_pool(be, steps, warmup):
     """Max-pool forward / backward and the plain copy kernel, HBM-true: consecutive launches work on POOL_SETS
-    disjoint buffer sets (5 x 135 MB per direction and kernel, far beyond the 256 MB of last-level cache), so no
+    disjoint buffer sets (10 x 135 MB per direction and kernel; even the 32 MB a backward launch reads come to 320 MB over a round, beyond the 256 MB of last-level cache), so no
     launch finds its operands cached by the previous one.  The "warm" figures repeat one set and are cache-assisted;
     they are reported for comparison only."""
     K = be.kernels

@@ -8,8 +8,12 @@
 // window whose recorded index points at that cell, in ascending (ky,kx) order in
 // float64, and rounds once.
 #include "xsmi_internal.h"
+#include <stdlib.h>
 
 namespace {
+
+typedef float f4v __attribute__((ext_vector_type(4)));
+typedef float f2v __attribute__((ext_vector_type(2)));
 
 struct PoolGeom {
     int N, C, H, W, OH, OW, k, sh, sw, pad;
@@ -65,6 +69,7 @@ __global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restri
 // the whole wave waits for (measured 4 us of 33 in the backward kernel).  All
 // loads are issued before the first comparison so that their latencies overlap.  x is fetched once per window row; the row shared by
 // vertically adjacent windows is re-read from cache.
+template <int NT>
 __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restrict__ x, float *__restrict__ y,
                                                             uint8_t *__restrict__ idx, PoolGeom g,
                                                             xsmi::FastDiv dQ, uint32_t total_pairs) {
@@ -85,7 +90,9 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         v[r] = make_float4(0.f, 0.f, 0.f, 0.f);   // border row
         lf[r] = 0.f;
         if ((unsigned)ih < (unsigned)g.H) {
-            v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
+            const f4v *src = reinterpret_cast<const f4v *>(plane + (size_t)ih * g.W + 4 * j);
+            const f4v q = NT >= 2 ? __builtin_nontemporal_load(src) : *src;
+            v[r] = make_float4(q.x, q.y, q.z, q.w);
             if (j > 0) lf[r] = plane[(size_t)ih * g.W + 4 * j - 1];
         }
     }
@@ -103,8 +110,14 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
     }
     size_t o = (size_t)row * g.OW + 2 * j;
-    *reinterpret_cast<float2 *>(y + o) = make_float2(b0, b1);
-    if (idx) *reinterpret_cast<uchar2 *>(idx + o) = make_uchar2((unsigned char)w0, (unsigned char)w1);
+    if (NT >= 1) {
+        f2v yv; yv.x = b0; yv.y = b1;
+        __builtin_nontemporal_store(yv, reinterpret_cast<f2v *>(y + o));
+        if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + o));
+    } else {
+        *reinterpret_cast<float2 *>(y + o) = make_float2(b0, b1);
+        if (idx) *reinterpret_cast<uchar2 *>(idx + o) = make_uchar2((unsigned char)w0, (unsigned char)w1);
+    }
 }
 
 // One thread per input-gradient element.
@@ -215,7 +228,7 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restri
 // The same gather with eight dx columns per thread (W % 8 == 0): columns 8j .. 8j+7 of the input rows 2a and 2a+1
 // from output columns 4j .. 4j+3 (one 128-bit load of dy and one 32-bit load of the indices per output row) and
 // column 4j+4 (a dword and a byte): half as many memory instructions per byte as the four-column form.
-template <bool ACC>
+template <bool ACC, int NT>
 __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
                                                                float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ8,
                                                                xsmi::FastDiv dG, uint32_t total) {
@@ -238,9 +251,12 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__res
         int in = -1;
         const size_t ro = obase + (size_t)oh * g.OW + 4 * j;
         if (oh < g.OH) {
-            gg = *reinterpret_cast<const float4 *>(dy + ro);
-            uchar4 ii = *reinterpret_cast<const uchar4 *>(idx + ro);
-            i0 = ii.x; i1 = ii.y; i2 = ii.z; i3 = ii.w;
+            const f4v *gp = reinterpret_cast<const f4v *>(dy + ro);
+            const f4v gq = NT >= 2 ? __builtin_nontemporal_load(gp) : *gp;
+            gg = make_float4(gq.x, gq.y, gq.z, gq.w);
+            const uint32_t ii = NT >= 2 ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(idx + ro))
+                                        : *reinterpret_cast<const uint32_t *>(idx + ro);
+            i0 = ii & 255; i1 = (ii >> 8) & 255; i2 = (ii >> 16) & 255; i3 = ii >> 24;
             if (4 * j + 4 < g.OW) { gn = dy[ro + 4]; in = idx[ro + 4]; }
         }
         // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
@@ -274,10 +290,102 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__res
                                    (double)pick(0, m, 8));
         }
     }
-    pe[0] = make_float4(e[0], e[1], e[2], e[3]);
-    pe[1] = make_float4(e[4], e[5], e[6], e[7]);
-    po[0] = make_float4(o[0], o[1], o[2], o[3]);
-    po[1] = make_float4(o[4], o[5], o[6], o[7]);
+    if (NT >= 1) {
+        f4v *qe = reinterpret_cast<f4v *>(pe), *qo = reinterpret_cast<f4v *>(po);
+        __builtin_nontemporal_store(f4v{e[0], e[1], e[2], e[3]}, qe);
+        __builtin_nontemporal_store(f4v{e[4], e[5], e[6], e[7]}, qe + 1);
+        __builtin_nontemporal_store(f4v{o[0], o[1], o[2], o[3]}, qo);
+        __builtin_nontemporal_store(f4v{o[4], o[5], o[6], o[7]}, qo + 1);
+    } else {
+        pe[0] = make_float4(e[0], e[1], e[2], e[3]);
+        pe[1] = make_float4(e[4], e[5], e[6], e[7]);
+        po[0] = make_float4(o[0], o[1], o[2], o[3]);
+        po[1] = make_float4(o[4], o[5], o[6], o[7]);
+    }
+}
+
+// The eight-column gather with the stores laid out by the workgroup instead of the thread (beta == 0 only).  In the
+// kernel above a lane's two float4 of a row sit side by side, so each store instruction of a wavefront covers every
+// other 16 bytes of its lines; measured on the box with the kernel's exact loads, that pattern writes 102.8 MB in
+// 32 us, stores whose lanes are contiguous in 26.6 us and the same as non-temporal stores in 18.6 us.  A workgroup
+// therefore takes whole row pairs (RG = 256 / (W/8) of them: a contiguous piece of dx, since planes and row pairs
+// follow each other in memory), every thread puts its four float4 into the LDS image of that piece, and the image is
+// written out with lane-contiguous non-temporal float4 stores.
+__global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_lds(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
+                                                                float *__restrict__ dx, PoolGeom g, int RG,
+                                                                uint32_t total_rowg) {
+    // With OH == H / 2 the row pair (nc, a) has the same linear number as the dy row (nc, a), and it needs that row
+    // and the next one: the workgroup's rows_here + 1 rows of dy and idx are one contiguous piece, fetched once.
+    __shared__ f4v img[1024];
+    __shared__ f4v s_dy[512];                         // (RG + 1) * W/8 float4, with RG * W/8 <= 256 and W/8 <= 256
+    __shared__ uint32_t s_ix[512];
+    const int Q8 = g.W >> 3, G = g.H >> 1;
+    const int lt = (int)threadIdx.x;
+    const int lrow = lt / Q8, j = lt - lrow * Q8;
+    const uint32_t rowg0 = blockIdx.x * (uint32_t)RG;
+    const uint32_t rows_here = total_rowg - rowg0 < (uint32_t)RG ? total_rowg - rowg0 : (uint32_t)RG;
+    {
+        const uint32_t q_total = total_rowg * (uint32_t)Q8;                  // float4 (or index words) of all of dy
+        const uint32_t q0 = rowg0 * (uint32_t)Q8;
+        const uint32_t want = (rows_here + 1u) * (uint32_t)Q8;
+        const f4v *gsrc = reinterpret_cast<const f4v *>(dy) + q0;
+        const uint32_t *isrc = reinterpret_cast<const uint32_t *>(idx) + q0;
+        for (uint32_t q = (uint32_t)lt; q < want; q += 256u) {
+            const bool ok = q0 + q < q_total;
+            s_dy[q] = ok ? gsrc[q] : f4v{0.f, 0.f, 0.f, 0.f};
+            s_ix[q] = ok ? isrc[q] : 0xffffffffu;
+        }
+    }
+    __syncthreads();
+    if ((uint32_t)lrow < rows_here) {
+        const uint32_t rowg = rowg0 + (uint32_t)lrow;       // (nc, a)
+        const uint32_t nc = rowg / (uint32_t)G;
+        const int a = (int)(rowg - nc * (uint32_t)G);
+        float gv[2][5];
+        int iv[2][5];
+        const float *fdy = reinterpret_cast<const float *>(s_dy);
+        const uint8_t *bix = reinterpret_cast<const uint8_t *>(s_ix);
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            const int oh = a + q;                 // a + 1 == OH: below the last output row
+            f4v gg = f4v{0.f, 0.f, 0.f, 0.f};
+            uint32_t ii = 0xffffffffu;
+            float gn = 0.f;
+            int in = -1;
+            const int lq = (lrow + q) * Q8 + j;
+            if (oh < g.OH) {
+                gg = s_dy[lq];
+                ii = s_ix[lq];
+                if (j + 1 < Q8) { gn = fdy[4 * lq + 4]; in = bix[4 * lq + 4]; }
+            }
+            // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
+            gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gg.z + 0.f; gv[q][3] = gg.w + 0.f; gv[q][4] = gn + 0.f;
+            iv[q][0] = ii & 255; iv[q][1] = (ii >> 8) & 255; iv[q][2] = (ii >> 16) & 255; iv[q][3] = ii >> 24; iv[q][4] = in;
+        }
+        float e[8], o[8];
+        auto pick = [&](int q, int m, int tap) { return iv[q][m] == tap ? gv[q][m] : 0.f; };
+#pragma unroll
+        for (int m = 0; m < 4; ++m) {
+            e[2 * m] = pick(0, m, 4);
+            e[2 * m + 1] = pick(0, m + 1, 3) + pick(0, m, 5);
+            o[2 * m] = pick(1, m, 1) + pick(0, m, 7);
+            o[2 * m + 1] = (float)((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                   (double)pick(0, m, 8));
+        }
+        f4v *row_e = img + lrow * 4 * Q8 + 2 * j;      // row 2a of the pair, then row 2a + 1
+        row_e[0] = f4v{e[0], e[1], e[2], e[3]};
+        row_e[1] = f4v{e[4], e[5], e[6], e[7]};
+        row_e[2 * Q8] = f4v{o[0], o[1], o[2], o[3]};
+        row_e[2 * Q8 + 1] = f4v{o[4], o[5], o[6], o[7]};
+    }
+    __syncthreads();
+    const uint32_t quads = rows_here * 4u * (uint32_t)Q8;
+    f4v *out = reinterpret_cast<f4v *>(dx) + (size_t)rowg0 * 4u * (uint32_t)Q8;
+#pragma unroll
+    for (int k = 0; k < 4; ++k) {
+        const uint32_t q = (uint32_t)lt + 256u * k;
+        if (q < quads) __builtin_nontemporal_store(img[q], out + q);
+    }
 }
 
 int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw, int pad, PoolGeom *g) {
@@ -296,6 +404,12 @@ int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw
     g->dW = xsmi::make_fastdiv(W); g->dH = xsmi::make_fastdiv(H);
     g->dsh = xsmi::make_fastdiv(sh); g->dsw = xsmi::make_fastdiv(sw);
     return XSMI_OK;
+}
+
+int pool_nt() {
+    static int v = -1;
+    if (v < 0) { const char *e = getenv("XSMI_POOL_NT"); v = e ? atoi(e) : 1; }
+    return v;
 }
 
 bool fast_3x3s2p1(const PoolGeom &g) {
@@ -319,7 +433,11 @@ int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int
     if (fast_3x3s2p1(g)) {
         uint32_t pairs = total / 2;
         xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 2);
-        hipLaunchKernelGGL(maxpool_fwd_3x3s2p1, dim3((pairs + 255) / 256), dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        const dim3 grid((pairs + 255) / 256);
+        const int nt = pool_nt();
+        if (nt >= 2) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<2>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        else if (nt == 1) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<1>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        else hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<0>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
         xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_fwd_3x3s2p1");
         return XSMI_OK;
@@ -352,8 +470,20 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
         uint32_t threads = total / 16;       // eight columns of two rows each
         xsmi::FastDiv dQ8 = xsmi::make_fastdiv(W / 8), dG = xsmi::make_fastdiv(H / 2);
         dim3 grid((threads + 255) / 256);
-        if (acc) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<true>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
-        else hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<false>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        const int nt = pool_nt();
+        if (!acc && W / 8 <= 256 && nt != 9) {
+            const int RG = 256 / (W / 8);
+            const uint32_t total_rowg = (uint32_t)N * C * (H / 2);
+            hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_lds, dim3((total_rowg + RG - 1) / RG), dim3(256), 0, st, dy, idx, dx, g, RG,
+                               total_rowg);
+            xsmi::prof_end();
+            XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_lds");
+            return XSMI_OK;
+        }
+        if (acc) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<true, 0>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        else if (nt >= 2) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 2>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        else if (nt == 1) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 1>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        else hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 0>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
         xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_w8");
         return XSMI_OK;

@@ -61,10 +61,12 @@ void prof_end() {
 
 // One float4 per thread: of the forms tried on the box (grid-stride loops over 8 to 64 workgroups per CU, four loads
 // in flight per thread, the runtime's own device-to-device copy) this one moved the most bytes per second when source
-// and destination come from HBM (5.9 TB/s against 5.2-5.7 for the loops and 5.3 for hipMemcpyAsync).
-__global__ void __launch_bounds__(256) xsmi_copy_f4(const float4 *__restrict__ src, float4 *__restrict__ dst, size_t n4) {
+// and destination come from HBM (5.9 TB/s against 5.2-5.7 for the loops and 5.3 for hipMemcpyAsync); with
+// non-temporal loads and stores it moves 6.3 TB/s (a pure read of the same size 6.6, a pure fill 6.5).
+typedef float xsmi_f4v __attribute__((ext_vector_type(4)));
+__global__ void __launch_bounds__(256) xsmi_copy_f4(const xsmi_f4v *__restrict__ src, xsmi_f4v *__restrict__ dst, size_t n4) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    if (i < n4) dst[i] = src[i];
+    if (i < n4) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
 
 extern "C" {
@@ -279,7 +281,7 @@ int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
     XSMI_CHECK_ARG(blocks < 2147483648ull, "xsmi_copy_kernel: more than 2^31 workgroups");
     xsmi::prof_begin();
     hipLaunchKernelGGL(xsmi_copy_f4, dim3((unsigned)blocks), dim3(256), 0, g_stream,
-                       (const float4 *)src, (float4 *)dst, n4);
+                       (const xsmi_f4v *)src, (xsmi_f4v *)dst, n4);
     xsmi::prof_end();
     XSMI_LAUNCH_CHECK("xsmi_copy_f4");
     return XSMI_OK;
