@@ -183,6 +183,18 @@ __device__ __forceinline__ double block_sum(double v, double *sm) {   // 256 thr
     return sm[0] + sm[1] + sm[2] + sm[3];
 }
 
+template <int NT>
+__device__ __forceinline__ double block_sum_n(double v, double *sm) {   // NT threads, sm[NT / 64]; waves added in order
+    v = wave_sum(v);
+    __syncthreads();
+    if ((threadIdx.x & 63) == 0) sm[threadIdx.x >> 6] = v;
+    __syncthreads();
+    double r = sm[0];
+#pragma unroll
+    for (int w = 1; w < NT / 64; ++w) r += sm[w];
+    return r;
+}
+
 // channel of flat element i of an (N, C, HW) tensor (tensors stay below 2^29 elements)
 struct ChanIdx {
     xsmi::FastDiv dHW, dC;
@@ -434,28 +446,49 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
 // per channel.  The elements are read once, summed in float64 (fixed order: per thread in element order, then
 // block_sum), normalised from the registers and written; a launch and a read of the tensor less than the two-kernel
 // form, which matters where a launch costs as much as the data movement (14x14 and 7x7 feature maps).
-constexpr int BN_SMALL_PER = 32;                      // elements per thread kept in registers
-constexpr int BN_SMALL_MAX = 256 * BN_SMALL_PER;      // 8192 elements per channel
-__device__ __forceinline__ size_t bn_small_off(uint32_t e, int c, int C, int HW, const xsmi::FastDiv &dHW) {
-    const uint32_t j = xsmi::fdiv(e, dHW), i = e - j * (uint32_t)HW;
-    return ((size_t)j * C + c) * (size_t)HW + i;
-}
-__global__ void __launch_bounds__(256) bn_fwd_small_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+constexpr int BN_SMALL_PER = 8;                       // elements per thread, kept in registers
+constexpr int BN_SMALL_MAX = 1024 * BN_SMALL_PER;     // 8192 elements per channel
+// Element e = thread + NT u of channel c is (image j, position i) = (e / HW, e % HW); a thread forms the pair once
+// and steps it by (NT / HW, NT % HW) with one wrap, so the loop has no division.  A workgroup has 256 threads for
+// channels of up to 2048 elements (7 x 7 at N=32: 1568) and 1024 threads above (14 x 14 at N=32: 6272), eight
+// elements per thread either way: the loads of a channel are all in flight at once and the chains behind them short.
+struct BnSmallWalk {
+    uint32_t j, i, dj, di, HW;
+    __device__ __forceinline__ BnSmallWalk(uint32_t e, uint32_t nt, int HW_, const xsmi::FastDiv &dHW) : HW((uint32_t)HW_) {
+        j = xsmi::fdiv(e, dHW); i = e - j * HW;
+        dj = xsmi::fdiv(nt, dHW); di = nt - dj * HW;
+    }
+    __device__ __forceinline__ size_t off(int c, int C) const { return ((size_t)j * C + c) * (size_t)HW + i; }
+    __device__ __forceinline__ void step() {
+        j += dj; i += di;
+        if (i >= HW) { i -= HW; ++j; }
+    }
+};
+template <int NT>
+__global__ void __launch_bounds__(NT) bn_fwd_small_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
                                                             const float *__restrict__ beta, double m, float eps, float momentum,
                                                             BnFwdOut o, int C, int HW, xsmi::FastDiv dHW, uint32_t total) {
-    __shared__ double sm[4];
+    constexpr int PER = BN_SMALL_PER;
+    __shared__ double sm[NT / 64];
     const int c = blockIdx.x;
-    float v[BN_SMALL_PER];
+    float v[PER];
+    uint32_t offs[PER];
+    BnSmallWalk wk(threadIdx.x, NT, HW, dHW);
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t e = threadIdx.x + (uint32_t)NT * u;
+        offs[u] = (uint32_t)wk.off(c, C);             // tensors stay below 2^29 elements
+        v[u] = e < total ? x[offs[u]] : 0.f;
+        wk.step();
+    }
     double s0 = 0.0, s1 = 0.0;
 #pragma unroll
-    for (int u = 0; u < BN_SMALL_PER; ++u) {
-        const uint32_t e = threadIdx.x + 256u * u;
-        v[u] = e < total ? x[bn_small_off(e, c, C, HW, dHW)] : 0.f;
+    for (int u = 0; u < PER; ++u) {
         s0 += (double)v[u];
         s1 += (double)v[u] * (double)v[u];
     }
-    s0 = block_sum(s0, sm);
-    s1 = block_sum(s1, sm);
+    s0 = block_sum_n<NT>(s0, sm);
+    s1 = block_sum_n<NT>(s1, sm);
     const double mu_d = s0 / m;
     double var = s1 / m - mu_d * mu_d;
     if (var < 0.0) var = 0.0;
@@ -470,10 +503,10 @@ __global__ void __launch_bounds__(256) bn_fwd_small_kernel(const float *__restri
         }
     }
 #pragma unroll
-    for (int u = 0; u < BN_SMALL_PER; ++u) {
-        const uint32_t e = threadIdx.x + 256u * u;
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t e = threadIdx.x + (uint32_t)NT * u;
         if (e >= total) break;
-        const size_t off = bn_small_off(e, c, C, HW, dHW);
+        const size_t off = offs[u];
         const float hv = (v[u] - mu) / rs;
         const float pre = g * hv + bt;
         if (o.xhat) o.xhat[off] = hv;
@@ -481,41 +514,53 @@ __global__ void __launch_bounds__(256) bn_fwd_small_kernel(const float *__restri
         if (o.neg_mask) o.neg_mask[off] = pre < 0.f ? 1 : 0;
     }
 }
-__global__ void __launch_bounds__(256) bn_bwd_small_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
+template <int NT>
+__global__ void __launch_bounds__(NT) bn_bwd_small_kernel(const float *__restrict__ dy, const float *__restrict__ xhat,
                                                             const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
                                                             float *__restrict__ dgamma, float *__restrict__ dbeta,
                                                             const uint8_t *__restrict__ zero, float *__restrict__ dx, float m,
                                                             const float *__restrict__ mean, int C, int HW, xsmi::FastDiv dHW,
                                                             uint32_t total) {
-    __shared__ double sm[4];
+    constexpr int PER = BN_SMALL_PER;
+    __shared__ double sm[NT / 64];
     const int c = blockIdx.x;
     const float rs = sqrtvar[c], mu = mean ? mean[c] : 0.f, g = gamma[c], den = m * rs;
-    float d[BN_SMALL_PER], h[BN_SMALL_PER];
+    float d[PER], h[PER];
+    uint8_t z[PER];
+    uint32_t offs[PER];
+    BnSmallWalk wk(threadIdx.x, NT, HW, dHW);
+    // all loads first (the masked gradient is selected afterwards: a load that depends on the mask would wait for it)
+#pragma unroll
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t e = threadIdx.x + (uint32_t)NT * u;
+        offs[u] = (uint32_t)wk.off(c, C);
+        const bool ok = e < total;
+        d[u] = ok ? dy[offs[u]] : 0.f;
+        h[u] = ok ? xhat[offs[u]] : 0.f;
+        z[u] = (ok && zero) ? zero[offs[u]] : (uint8_t)0;
+        wk.step();
+    }
     double s0 = 0.0, s1 = 0.0;
 #pragma unroll
-    for (int u = 0; u < BN_SMALL_PER; ++u) {
-        const uint32_t e = threadIdx.x + 256u * u;
-        d[u] = 0.f; h[u] = 0.f;
-        if (e < total) {
-            const size_t off = bn_small_off(e, c, C, HW, dHW);
-            d[u] = (zero && zero[off]) ? 0.f : dy[off];
-            h[u] = mean ? (xhat[off] - mu) / rs : xhat[off];
-        }
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t e = threadIdx.x + (uint32_t)NT * u;
+        if (z[u]) d[u] = 0.f;
+        if (mean) h[u] = e < total ? (h[u] - mu) / rs : 0.f;
         s0 += (double)d[u];
         s1 += (double)d[u] * (double)h[u];
     }
-    s0 = block_sum(s0, sm);
-    s1 = block_sum(s1, sm);
+    s0 = block_sum_n<NT>(s0, sm);
+    s1 = block_sum_n<NT>(s1, sm);
     const float db = (float)s0, dg = (float)s1;
     if (threadIdx.x == 0) {
         dbeta[c] = db;
         dgamma[c] = dg;
     }
 #pragma unroll
-    for (int u = 0; u < BN_SMALL_PER; ++u) {
-        const uint32_t e = threadIdx.x + 256u * u;
+    for (int u = 0; u < PER; ++u) {
+        const uint32_t e = threadIdx.x + (uint32_t)NT * u;
         if (e >= total) break;
-        dx[bn_small_off(e, c, C, HW, dHW)] = g * (m * d[u] - db - h[u] * dg) / den;
+        dx[offs[u]] = g * (m * d[u] - db - h[u] * dg) / den;
     }
 }
 
@@ -842,8 +887,10 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     hipStream_t st = xsmi::stream();
     if ((size_t)N * HW <= (size_t)BN_SMALL_MAX) {
         const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask};
-        hipLaunchKernelGGL(bn_fwd_small_kernel, dim3(C), dim3(256), 0, st, x, gamma, beta, (double)N * HW, eps, momentum, o, C,
-                           HW, xsmi::make_fastdiv(HW), (uint32_t)(N * HW));
+        const uint32_t total = (uint32_t)(N * HW);
+        const xsmi::FastDiv dHW = xsmi::make_fastdiv(HW);
+        if (total <= 256u * BN_SMALL_PER) hipLaunchKernelGGL(bn_fwd_small_kernel<256>, dim3(C), dim3(256), 0, st, x, gamma, beta, (double)N * HW, eps, momentum, o, C, HW, dHW, total);
+        else hipLaunchKernelGGL(bn_fwd_small_kernel<1024>, dim3(C), dim3(1024), 0, st, x, gamma, beta, (double)N * HW, eps, momentum, o, C, HW, dHW, total);
         XSMI_LAUNCH_CHECK("bn_fwd_small_kernel");
         return XSMI_OK;
     }
@@ -903,8 +950,11 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd: workspace too small");
     hipStream_t st = xsmi::stream();
     if ((size_t)N * HW <= (size_t)BN_SMALL_MAX) {
-        hipLaunchKernelGGL(bn_bwd_small_kernel, dim3(C), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, neg_mask, dx,
-                           (float)((double)N * HW), mean, C, HW, xsmi::make_fastdiv(HW), (uint32_t)(N * HW));
+        const uint32_t total = (uint32_t)(N * HW);
+        const xsmi::FastDiv dHW = xsmi::make_fastdiv(HW);
+        const float mf = (float)((double)N * HW);
+        if (total <= 256u * BN_SMALL_PER) hipLaunchKernelGGL(bn_bwd_small_kernel<256>, dim3(C), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, neg_mask, dx, mf, mean, C, HW, dHW, total);
+        else hipLaunchKernelGGL(bn_bwd_small_kernel<1024>, dim3(C), dim3(1024), 0, st, dy, xhat, sqrtvar, gamma, dgamma, dbeta, neg_mask, dx, mf, mean, C, HW, dHW, total);
         XSMI_LAUNCH_CHECK("bn_bwd_small_kernel");
         return XSMI_OK;
     }
