@@ -1514,7 +1514,10 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
     const int nchunks = nhwc_chunks(C, R, S), rowtiles = ceil_div(K, ROWS);
     __bf16 *apk = (__bf16 *)workspace;
     __bf16 *xp = (__bf16 *)((char *)workspace + nhwc_apk_bytes(C, K, R, S));
-    if (!(opts & 2)) {                       // bit 1: the workspace still holds this filter's packed form
+    // 3 x 3 stride-1 layers on large feature maps: the kernel that stages the input once for all nine taps
+    const bool halo = !pair && (!y_cl || yb == 1) && halo_fwd_ok(C, H, W, K, R, S, sh, sw, pad, border) &&
+                      halo_apk_bytes(C, K) <= nhwc_apk_bytes(C, K, R, S);
+    if (!(opts & 2) && !halo) {              // bit 1: the workspace still holds this filter's packed form
         const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 2048) blocks = 2048;
@@ -1544,6 +1547,9 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
         hipLaunchKernelGGL(nhwc_pad_bf16_kernel, dim3((unsigned)(N * Hp * nseg)), dim3(256), lds, st, x, xp, C, H, W, CP, pad, Hp,
                            Wp, WS, nseg, wlog, clog);
         XSMI_LAUNCH_CHECK("nhwc_pad_bf16_kernel");
+    }
+    if (halo) {
+        return halo_conv_fwd(xp, (size_t)N * Hp * Wp * CP * 2, w, apk, bias, y, y_cl, mask, N, C, H, W, K, relu, (opts & 2) != 0);
     }
     NhwcParams p;
     p.xp = xp; p.apk = (const float *)apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;

@@ -134,6 +134,13 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
                   uint8_t *mask, int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OH, int OW,
                   int relu, int opts, void *workspace);
 
+// 3 x 3, stride-1, pad-1 bf16 forward that stages the bordered channels-last input once for all nine taps
+// (conv_cl_halo.hip); called by nhwc_conv_fwd, shares its workspace layout (packed filter, then the copy)
+bool halo_fwd_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int border);
+size_t halo_apk_bytes(int C, int K);
+int halo_conv_fwd(const void *xp, size_t xp_bytes, const float *w, void *apk, const float *bias, float *y, void *y_cl,
+                  uint8_t *mask, int N, int C, int H, int W, int K, int relu, bool packed);
+
 // weight gradient for the same few-channel layers (conv_stem.hip): horizontal stride 2, output width a multiple of 8,
 // filters a multiple of 64, at most 160 filter positions; the workspace holds the copy and the workgroups' partial sums
 bool stem_wgrad_ok(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
