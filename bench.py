@@ -62,11 +62,11 @@ RESNET18_CONVS = [
 
 
 # HBM bytes per launch of tap_sk_f32_kernel on the CONV workload, from two hardware-counter runs (FETCH_SIZE
-# 36 052 KiB scaled by 1.9996, the factor that makes the plain copy kernel's known read size come out right, plus
-# WRITE_SIZE 58 940 KiB at factor 1.0): 73.8 MB read + 60.4 MB written, against 25.7 MB each way for the operands
+# 33 452 KiB scaled by 1.9997, the factor that makes the plain copy kernel's known read size come out right, plus
+# WRITE_SIZE 50 220 KiB at factor 0.9999): 68.5 MB read + 51.4 MB written, against 25.7 MB each way for the operands
 # alone: the even-split schedule exchanges about a thousand 16 KB partial tiles per launch through memory
 # (written through, read back uncached) and keeps three times as many tiles in flight as the L2 slices hold.
-TAP_SK_TRAFFIC_BYTES = 134.2e6
+TAP_SK_TRAFFIC_BYTES = 119.9e6
 
 
 def conv_flops(c):
