@@ -10,7 +10,10 @@ pytestmark = pytest.mark.gpu
 
 # per channel up to 8192 elements: one kernel does both passes; beyond: partial sums + apply (float4 or scalar form)
 @pytest.mark.parametrize("shape", [(4, 8, 6, 6), (32, 64, 14, 14), (5, 3, 7, 7), (2, 130, 9, 5), (64, 16),
-                                   (8, 16, 40, 40), (6, 5, 37, 41), (32, 8, 16, 16), (33, 4, 16, 16)])
+                                   (8, 16, 40, 40), (6, 5, 37, 41), (32, 8, 16, 16), (33, 4, 16, 16),
+                                   # single-kernel form: 2048 elements per channel (256 threads) and one more (1024),
+                                   # its upper limit 8192 and one more (two-kernel form), planes wider than a workgroup
+                                   (8, 3, 16, 16), (3, 5, 683), (2, 3, 64, 64), (1, 2, 8193), (3, 7, 20, 15), (256, 5)])
 def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     """xs/nn/functional.py:676-707 and xs/nn/grad_fn.py:379-411."""
     K = gpu.kernels

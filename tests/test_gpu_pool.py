@@ -22,6 +22,10 @@ CASES = [  # n c h w k sh sw pad
     (2, 3, 14, 10, 3, 2, 2, 1),      # W % 4 != 0 -> generic path
     (3, 2, 6, 8, 3, 2, 2, 1),        # W % 8 == 0: eight gradient columns per thread, one thread per row pair
     (1, 3, 4, 136, 3, 2, 2, 1),      # ... rows longer than one wavefront's 64 x 8 columns... and a lane at the wave edge
+    (5, 7, 6, 8, 3, 2, 2, 1),        # one thread per row pair: 105 row pairs in a single workgroup of the gradient kernel
+    (3, 37, 10, 16, 3, 2, 2, 1),     # 555 row pairs for workgroups of 128: a partial last workgroup
+    (2, 3, 38, 112, 3, 2, 2, 1),     # 114 row pairs for workgroups of 18: planes change inside a workgroup
+    (1, 1, 2, 2056, 3, 2, 2, 1),     # 257 threads per row pair: wider than a workgroup, the per-thread form serves it
 ]
 
 
