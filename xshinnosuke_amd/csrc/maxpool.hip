@@ -8,7 +8,6 @@
 // window whose recorded index points at that cell, in ascending (ky,kx) order in
 // float64, and rounds once.
 #include "xsmi_internal.h"
-#include <stdlib.h>
 
 namespace {
 
@@ -69,7 +68,6 @@ __global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restri
 // the whole wave waits for (measured 4 us of 33 in the backward kernel).  All
 // loads are issued before the first comparison so that their latencies overlap.  x is fetched once per window row; the row shared by
 // vertically adjacent windows is re-read from cache.
-template <int NT>
 __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restrict__ x, float *__restrict__ y,
                                                             uint8_t *__restrict__ idx, PoolGeom g,
                                                             xsmi::FastDiv dQ, uint32_t total_pairs) {
@@ -90,9 +88,7 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         v[r] = make_float4(0.f, 0.f, 0.f, 0.f);   // border row
         lf[r] = 0.f;
         if ((unsigned)ih < (unsigned)g.H) {
-            const f4v *src = reinterpret_cast<const f4v *>(plane + (size_t)ih * g.W + 4 * j);
-            const f4v q = NT >= 2 ? __builtin_nontemporal_load(src) : *src;
-            v[r] = make_float4(q.x, q.y, q.z, q.w);
+            v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * g.W + 4 * j);
             if (j > 0) lf[r] = plane[(size_t)ih * g.W + 4 * j - 1];
         }
     }
@@ -110,14 +106,11 @@ __global__ void __launch_bounds__(256) maxpool_fwd_3x3s2p1(const float *__restri
         if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
     }
     size_t o = (size_t)row * g.OW + 2 * j;
-    if (NT >= 1) {
-        f2v yv; yv.x = b0; yv.y = b1;
-        __builtin_nontemporal_store(yv, reinterpret_cast<f2v *>(y + o));
-        if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + o));
-    } else {
-        *reinterpret_cast<float2 *>(y + o) = make_float2(b0, b1);
-        if (idx) *reinterpret_cast<uchar2 *>(idx + o) = make_uchar2((unsigned char)w0, (unsigned char)w1);
-    }
+    // the outputs are not read again by this kernel: non-temporal stores (measured +4 % over plain ones; non-temporal
+    // loads of x lose, its rows are shared between neighbouring windows)
+    f2v yv; yv.x = b0; yv.y = b1;
+    __builtin_nontemporal_store(yv, reinterpret_cast<f2v *>(y + o));
+    if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + o));
 }
 
 // One thread per input-gradient element.
@@ -228,7 +221,7 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1(const float *__restri
 // The same gather with eight dx columns per thread (W % 8 == 0): columns 8j .. 8j+7 of the input rows 2a and 2a+1
 // from output columns 4j .. 4j+3 (one 128-bit load of dy and one 32-bit load of the indices per output row) and
 // column 4j+4 (a dword and a byte): half as many memory instructions per byte as the four-column form.
-template <bool ACC, int NT>
+template <bool ACC>
 __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
                                                                float *__restrict__ dx, PoolGeom g, xsmi::FastDiv dQ8,
                                                                xsmi::FastDiv dG, uint32_t total) {
@@ -251,11 +244,8 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__res
         int in = -1;
         const size_t ro = obase + (size_t)oh * g.OW + 4 * j;
         if (oh < g.OH) {
-            const f4v *gp = reinterpret_cast<const f4v *>(dy + ro);
-            const f4v gq = NT >= 2 ? __builtin_nontemporal_load(gp) : *gp;
-            gg = make_float4(gq.x, gq.y, gq.z, gq.w);
-            const uint32_t ii = NT >= 2 ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(idx + ro))
-                                        : *reinterpret_cast<const uint32_t *>(idx + ro);
+            gg = *reinterpret_cast<const float4 *>(dy + ro);
+            const uint32_t ii = *reinterpret_cast<const uint32_t *>(idx + ro);
             i0 = ii & 255; i1 = (ii >> 8) & 255; i2 = (ii >> 16) & 255; i3 = ii >> 24;
             if (4 * j + 4 < g.OW) { gn = dy[ro + 4]; in = idx[ro + 4]; }
         }
@@ -290,18 +280,10 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_w8(const float *__res
                                    (double)pick(0, m, 8));
         }
     }
-    if (NT >= 1) {
-        f4v *qe = reinterpret_cast<f4v *>(pe), *qo = reinterpret_cast<f4v *>(po);
-        __builtin_nontemporal_store(f4v{e[0], e[1], e[2], e[3]}, qe);
-        __builtin_nontemporal_store(f4v{e[4], e[5], e[6], e[7]}, qe + 1);
-        __builtin_nontemporal_store(f4v{o[0], o[1], o[2], o[3]}, qo);
-        __builtin_nontemporal_store(f4v{o[4], o[5], o[6], o[7]}, qo + 1);
-    } else {
-        pe[0] = make_float4(e[0], e[1], e[2], e[3]);
-        pe[1] = make_float4(e[4], e[5], e[6], e[7]);
-        po[0] = make_float4(o[0], o[1], o[2], o[3]);
-        po[1] = make_float4(o[4], o[5], o[6], o[7]);
-    }
+    pe[0] = make_float4(e[0], e[1], e[2], e[3]);
+    pe[1] = make_float4(e[4], e[5], e[6], e[7]);
+    po[0] = make_float4(o[0], o[1], o[2], o[3]);
+    po[1] = make_float4(o[4], o[5], o[6], o[7]);
 }
 
 // The eight-column gather with the stores laid out by the workgroup instead of the thread (beta == 0 only).  In the
@@ -406,12 +388,6 @@ int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw
     return XSMI_OK;
 }
 
-int pool_nt() {
-    static int v = -1;
-    if (v < 0) { const char *e = getenv("XSMI_POOL_NT"); v = e ? atoi(e) : 1; }
-    return v;
-}
-
 bool fast_3x3s2p1(const PoolGeom &g) {
     return g.k == 3 && g.sh == 2 && g.sw == 2 && g.pad == 1 && (g.W % 4) == 0 && (g.H % 2) == 0;
 }
@@ -433,11 +409,7 @@ int xsmi_maxpool2d_fwd(const float *x, float *y, uint8_t *idx, int N, int C, int
     if (fast_3x3s2p1(g)) {
         uint32_t pairs = total / 2;
         xsmi::FastDiv dQ = xsmi::make_fastdiv(g.OW / 2);
-        const dim3 grid((pairs + 255) / 256);
-        const int nt = pool_nt();
-        if (nt >= 2) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<2>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
-        else if (nt == 1) hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<1>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
-        else hipLaunchKernelGGL(maxpool_fwd_3x3s2p1<0>, grid, dim3(256), 0, st, x, y, idx, g, dQ, pairs);
+        hipLaunchKernelGGL(maxpool_fwd_3x3s2p1, dim3((pairs + 255) / 256), dim3(256), 0, st, x, y, idx, g, dQ, pairs);
         xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_fwd_3x3s2p1");
         return XSMI_OK;
@@ -470,8 +442,7 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
         uint32_t threads = total / 16;       // eight columns of two rows each
         xsmi::FastDiv dQ8 = xsmi::make_fastdiv(W / 8), dG = xsmi::make_fastdiv(H / 2);
         dim3 grid((threads + 255) / 256);
-        const int nt = pool_nt();
-        if (!acc && W / 8 <= 256 && nt != 9) {
+        if (!acc && W / 8 <= 256) {
             const int RG = 256 / (W / 8);
             const uint32_t total_rowg = (uint32_t)N * C * (H / 2);
             hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_lds, dim3((total_rowg + RG - 1) / RG), dim3(256), 0, st, dy, idx, dx, g, RG,
@@ -480,10 +451,8 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
             XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_lds");
             return XSMI_OK;
         }
-        if (acc) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<true, 0>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
-        else if (nt >= 2) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 2>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
-        else if (nt == 1) hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 1>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
-        else hipLaunchKernelGGL((maxpool_bwd_3x3s2p1_w8<false, 0>), grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        if (acc) hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<true>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
+        else hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_w8<false>, grid, dim3(256), 0, st, dy, idx, dx, g, dQ8, dG, threads);
         xsmi::prof_end();
         XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_w8");
         return XSMI_OK;
