@@ -174,7 +174,7 @@ __global__ void __launch_bounds__(256, 2) cl_halo_bf16_kernel(HaloParams p) {
 #pragma unroll
                         for (int e = 0; e < 4; ++e) {
                             float val = acc[i][j][4 * gq + e] + bv[e];
-                            val = val > floor_ ? val : floor_;
+                            val = __builtin_fmaxf(val, floor_);
                             o4[e] = (__bf16)val;
                         }
                         if (inside && row < p.rows) *reinterpret_cast<bf16x4 *>(dst + row) = o4;   // rows is a multiple of 8 here
@@ -311,6 +311,196 @@ __global__ void __launch_bounds__(256) tap_pack_halo_kernel(const float *__restr
     }
 }
 
+
+// ---- first layer: at most 4 input channels, filter up to 7 x 8, stride 2, channels-last bf16 output ---------------
+// The input is the zero-bordered bf16 copy [N][Hp][Wp][4] (8 bytes per pixel, Wp even), read as PAIRS of horizontally
+// adjacent pixels: 16 bytes = two taps x 4 channels = one lane's MFMA operand.  With stride 2 the window of output
+// x starts at pair x, so tap pair o of filter row r for output (y, x) is pair (2 y + r) * Wp/2 + x + o: for the 32
+// consecutive outputs of an MFMA block that is 32 consecutive pairs, whatever r and o are.  A work item is two output
+// rows (all of their columns, at most 128): its input is nine consecutive padded rows, one contiguous piece of memory,
+// copied to the LDS as it is; the filter (R rows x 4 tap pairs x 64 filters x 16 bytes = 28 KB) stays in the LDS for the
+// workgroup's whole life.  A persistent workgroup (two per CU) walks its items with the next item's rows requested
+// while the current item multiplies, and needs ONE barrier per item (56 MFMAs per wave): nothing inside an item is
+// produced by another wave.  The general channels-last kernel spends 21 other instructions per MFMA on this layer
+// (per-lane tap bookkeeping for every load) and takes 245 us at N=256.
+constexpr int STEM_ROWS_IN = 9;               // input rows of an item: 2 output rows x stride 2 + 7 - 2
+constexpr int STEM_B_PAIRS = 1088;            // pixel pairs of an item's LDS image: 17 wave-loads of 64 pairs
+struct StemParams {
+    const __bf16 *xp;      // [N][Hp][Wp][4]
+    const __bf16 *apk;     // [R][4 tap pairs][64 filters][8]
+    const float *bias;
+    __bf16 *out_cl;        // [N][OH + 2][OW + 2][K]
+    uint32_t xp_bytes;
+    int N, Hp, pitch;      // pitch = Wp / 2 pairs per padded row
+    int OH, OW, K, relu;
+    uint32_t items;        // N * ceil(OH / 2)
+    xsmi::FastDiv dYP;     // by ceil(OH / 2)
+};
+
+template <int R>
+__global__ void __launch_bounds__(256, 2) cl_stem_bf16_kernel(StemParams p) {
+    constexpr int NLOADS = STEM_B_PAIRS / 64;        // B wave-loads (64 pairs each) per item, dealt round-robin to the waves
+    constexpr int B_STAGE = STEM_B_PAIRS * 16;       // 9 rows x at most 115 pairs + the reach of the last block's junk columns
+    constexpr int NIMG = 3;                          // images in flight: an item's rows are requested two items ahead
+    __shared__ __attribute__((aligned(16))) unsigned char s_b[NIMG * B_STAGE];
+    __shared__ __attribute__((aligned(16))) float s_bias[64];
+
+    const int t = threadIdx.x;
+    const int lane = t & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
+    const uint32_t wg = blockIdx.x, grid = gridDim.x;
+    if (wg >= p.items) return;
+    const int n_items = (int)((p.items - wg + grid - 1) / grid);
+    const int pitch = p.pitch;
+    const uint32_t ypairs = p.dYP.d;
+
+    const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(p.xp, p.xp_bytes);
+    const uint32_t lds_b = (uint32_t)(uintptr_t)&s_b[0];
+
+    // an item's nine input rows: STEM_ROWS_IN * pitch * 16 contiguous bytes from row 2 * y0 of image n
+    auto issue_b = [&](uint32_t item, int image) {
+        const uint32_t n = xsmi::fdiv(item, p.dYP), yp = item - n * ypairs;
+        const uint32_t base = ((n * (uint32_t)p.Hp + 2u * 2u * yp) * (uint32_t)pitch) * 16u;
+        const uint32_t want = (uint32_t)(STEM_ROWS_IN * pitch) * 16u;
+#pragma unroll
+        for (int q0 = 0; q0 < NLOADS; q0 += 4) {
+            const int q = q0 + wave;
+            if (q >= NLOADS) break;
+            const uint32_t off = (uint32_t)(q * 1024 + lane * 16);
+            // bytes past the nine rows (or past the tensor) are junk columns' operands: zeros
+            const uint32_t voff = (off < want && base + off < p.xp_bytes) ? base + off : 0x80000000u;
+            xsmi::load_lds_b128(rin, lds_b + (uint32_t)(image * B_STAGE + q * 1024), voff, 0u);
+        }
+    };
+    issue_b(wg, 0);
+    if (n_items > 1) issue_b(wg + grid, 1);
+    if (t < 64) s_bias[t] = (p.bias && t < p.K) ? p.bias[t] : 0.f;
+
+    const int h = lane >> 5, l31 = lane & 31;
+    const int q_row = wave >> 1, xh = wave & 1;       // this wave's output row of the pair and 64-column half
+    // lane half h takes tap pair 2 u + h of k-step u
+    const int b_base = ((2 * q_row) * pitch + 64 * xh + l31 + h) * 16;
+    const int pitch16 = pitch * 16;
+    const float floor_ = p.relu ? 0.f : -__builtin_inff();
+    floatx16 acc[2][2];
+    // The filter never changes: this lane's A operands of all 2 R k-steps (its row of both 32-row blocks, tap pair
+    // 2 u + h of filter row r) stay in registers for the workgroup's whole life, 8 R registers, and the LDS serves
+    // only the B fragments: two 128-bit reads per four MFMAs instead of four (a 64 x 64 wave tile that reads both
+    // operands asks the LDS for 128 bytes per clock at full matrix rate, all it has).
+    bf16x8 fa[2 * R][2];
+#pragma unroll
+    for (int ks = 0; ks < 2 * R; ++ks)
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+            fa[ks][i] = *reinterpret_cast<const bf16x8 *>(p.apk + ((((ks >> 1) * 4 + 2 * (ks & 1) + h) * 64 + 32 * i + l31) * 8));
+    bf16x8 fb[2][2];                                 // [buffer][block]
+    auto read_frags = [&](auto buf_tag, auto ks_tag, int img_off) {
+        constexpr int bf = decltype(buf_tag)::value, ks = decltype(ks_tag)::value, r = ks >> 1, u = ks & 1;
+#pragma unroll
+        for (int j = 0; j < 2; ++j)
+            fb[bf][j] = *reinterpret_cast<const bf16x8 *>(s_b + img_off + b_base + r * pitch16 + (32 * j + 2 * u) * 16);
+    };
+
+    if (n_items > 1) xsmi::wait_vmcnt<(NLOADS + 3) / 4>(); else xsmi::wait_vmcnt<0>();    // the filter and the first item's rows
+    uint32_t item = wg;
+    int image = 0;
+    for (int it = 0; it < n_items; ++it, item += grid) {
+        const int img_off = image * B_STAGE;
+        // this item's rows have landed (waited for before the previous epilogue, or before the loop); everybody is done
+        // with the other image
+        __syncthreads();
+        // the image two ahead is the one the previous item used: free since the barrier above
+        if (it + 2 < n_items) issue_b(item + 2 * grid, image == 0 ? 2 : image - 1);
+        read_frags(IC<0>{}, IC<0>{}, img_off);
+        static_for<2 * R>([&](auto ks_c) {
+            constexpr int ks = decltype(ks_c)::value;
+            if constexpr (ks + 1 < 2 * R) read_frags(IC<(ks + 1) & 1>{}, IC<ks + 1>{}, img_off);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int i = 0; i < 2; ++i)
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    if constexpr (ks == 0) {
+                        floatx16 z;
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) z[v] = 0.f;
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks & 1][j], z, 0, 0, 0);
+                    } else {
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[ks][i], fb[ks & 1][j], acc[i][j], 0, 0, 0);
+                    }
+                }
+            __builtin_amdgcn_sched_barrier(0);
+        });
+        // The next item's rows were requested a whole item ago; waiting for them here, before this item's stores are
+        // issued, keeps those stores out of the wait (they drain behind the next item's MFMAs).  Only the rows
+        // requested at the top of this item (at most (NLOADS + 3) / 4 loads of this wave, a whole number less for the
+        // waves that got one load fewer: the wait is then a little stricter than needed) may still be in flight.
+        if (it + 2 < n_items) xsmi::wait_vmcnt<NLOADS / 4>(); else xsmi::wait_vmcnt<0>();
+        // Epilogue through the LDS.  A lane holds four consecutive filters of one column, its neighbours hold columns a
+        // whole 128-byte record apart: stored directly, every 8-byte store instruction touches 64 lines, and the
+        // address unit needs as long for an item's 64 such stores as the matrix pipes for its MFMAs.  The item's own
+        // input image is free now, and one output row (128 columns x 136 bytes: 8 bytes of padding spread the lanes'
+        // 8-byte writes over all banks) fits it exactly; the row then leaves as 16-byte pieces in memory order.
+        // register v of lane l in block (i, j) = filter 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, column 32 j + l % 32
+        const uint32_t n = xsmi::fdiv(item, p.dYP), yp = item - n * ypairs;
+        constexpr int O_PITCH = 136;
+        static_assert(128 * O_PITCH <= B_STAGE, "an output row fits an input image");
+        unsigned char *const o_img = s_b + img_off;
+        const int pieces = p.K >> 3;                   // 16-byte pieces of a column's record
+        const int piece_shift = 31 - __builtin_clz(pieces);
+        __syncthreads();                               // every wave has read this item's last fragments
+#pragma unroll
+        for (int q = 0; q < 2; ++q) {
+            if (q_row == q) {
+#pragma unroll
+                for (int j = 0; j < 2; ++j) {
+                    const int x = 64 * xh + 32 * j + l31;
+#pragma unroll
+                    for (int i = 0; i < 2; ++i)
+#pragma unroll
+                        for (int gq = 0; gq < 4; ++gq) {
+                            const int row = 32 * i + 8 * gq + 4 * h;
+                            const float4 b4 = *reinterpret_cast<const float4 *>(&s_bias[row]);
+                            const float bv[4] = {b4.x, b4.y, b4.z, b4.w};
+                            bf16x4 o4;
+#pragma unroll
+                            for (int e = 0; e < 4; ++e) {
+                                float val = acc[i][j][4 * gq + e] + bv[e];
+                                val = __builtin_fmaxf(val, floor_);
+                                o4[e] = (__bf16)val;
+                            }
+                            *reinterpret_cast<bf16x4 *>(o_img + x * O_PITCH + row * 2) = o4;
+                        }
+                }
+            }
+            __syncthreads();
+            const int y = 2 * (int)yp + q;
+            if (y < p.OH) {
+                __bf16 *dst = p.out_cl + (((size_t)n * (size_t)(p.OH + 2) + (size_t)(y + 1)) * (size_t)(p.OW + 2) + 1) * (size_t)p.K;
+                const int total = p.OW * pieces;
+                for (int pc = t; pc < total; pc += 256) {
+                    const int x = pc >> piece_shift, o8 = pc & (pieces - 1);     // K / 8 is a power of two (host check)
+                    const uint4 v = *reinterpret_cast<const uint4 *>(o_img + x * O_PITCH + o8 * 16);
+                    *reinterpret_cast<uint4 *>(dst + (size_t)pc * 8) = v;
+                }
+            }
+            __syncthreads();                           // the image is rewritten by the other row, then by new input rows
+        }
+        image = image == NIMG - 1 ? 0 : image + 1;
+    }
+}
+
+// A for the kernel above: element (((r * 4 + o) * 64 + k) * 8 + e) = w[k][e % 4][r][2 o + e / 4], zero past K, C or S.
+__global__ void __launch_bounds__(256) tap_pack_stem_kernel(const float *__restrict__ w, __bf16 *__restrict__ apk, int K, int C,
+                                                             int R, int S) {
+    const int total = R * 4 * 64 * 8;
+    for (int i = blockIdx.x * 256 + threadIdx.x; i < total; i += gridDim.x * 256) {
+        const int e = i & 7, k = (i >> 3) & 63, o = (i >> 9) & 3, r = i >> 11;
+        const int c = e & 3, sx = 2 * o + (e >> 2);
+        apk[i] = (__bf16)((k < K && c < C && sx < S) ? w[(((size_t)k * C + c) * R + r) * S + sx] : 0.f);
+    }
+}
+
 }  // namespace
 
 namespace xsmi {
@@ -325,6 +515,43 @@ bool halo_fwd_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int p
     if (C % 32 != 0 || K % 8 != 0) return false;
     if (HALO_PIX + 2 * (W + 2) + 2 > HALO_PITCH) return false;
     return env >= 2 || (H >= 14 && W >= 14);
+}
+
+// First layer through cl_stem_bf16_kernel: at most 4 channels copied with a border of `pad` pixels (Wp even), filter
+// 7 rows and at most 8 columns, stride 2 both ways, 8, 16, 32 or 64 filters, at most 128 output columns
+// and an input row of at most 115 pixel pairs, channels-last output with a border of one.
+bool stem_cl_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OW, int y_border) {
+    static int env = -1;
+    if (env < 0) { const char *e = getenv("XSMI_CL_STEM"); env = e ? atoi(e) : 1; }
+    if (!env) return false;
+    const int Wp = W + 2 * pad;
+    return C <= 4 && R == 7 && S <= 8 && sh == 2 && sw == 2 && (K == 8 || K == 16 || K == 32 || K == 64) && y_border == 1 &&
+           Wp % 2 == 0 &&
+           OW <= 128 && (STEM_ROWS_IN - 1) * (Wp / 2) + 131 <= STEM_B_PAIRS && H + 2 * pad >= R;
+}
+size_t stem_cl_apk_bytes() { return 7 * 4 * 64 * 16; }
+
+int stem_cl_conv_fwd(const void *xp, size_t xp_bytes, const float *w, void *apk, const float *bias, void *y_cl, int N, int C,
+                     int H, int W, int K, int R, int S, int pad, int OH, int OW, int relu, bool packed) {
+    hipStream_t st = stream();
+    if (!packed) {
+        hipLaunchKernelGGL(tap_pack_stem_kernel, dim3(14), dim3(256), 0, st, w, (__bf16 *)apk, K, C, R, S);
+        XSMI_LAUNCH_CHECK("tap_pack_stem_kernel");
+    }
+    StemParams p;
+    p.xp = (const __bf16 *)xp; p.apk = (const __bf16 *)apk; p.bias = bias; p.out_cl = (__bf16 *)y_cl;
+    p.xp_bytes = (uint32_t)xp_bytes;
+    p.N = N; p.Hp = H + 2 * pad; p.pitch = (W + 2 * pad) / 2;
+    p.OH = OH; p.OW = OW; p.K = K; p.relu = relu;
+    const int ypairs = ceil_div(OH, 2);
+    p.items = (uint32_t)N * (uint32_t)ypairs;
+    p.dYP = make_fastdiv(ypairs);
+    unsigned grid = 2u * (unsigned)(cu_count() > 0 ? cu_count() : 256);
+    if (grid > p.items) grid = p.items;
+    hipLaunchKernelGGL(cl_stem_bf16_kernel<7>, dim3(grid), dim3(256), 0, st, p);
+    prof_end();
+    XSMI_LAUNCH_CHECK("cl_stem_bf16_kernel");
+    return XSMI_OK;
 }
 
 size_t halo_apk_bytes(int C, int K) {

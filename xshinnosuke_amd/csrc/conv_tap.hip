@@ -1515,9 +1515,12 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
     __bf16 *apk = (__bf16 *)workspace;
     __bf16 *xp = (__bf16 *)((char *)workspace + nhwc_apk_bytes(C, K, R, S));
     // 3 x 3 stride-1 layers on large feature maps: the kernel that stages the input once for all nine taps
+    // the first layer with channels-last output: its own kernel, filter resident in the LDS
+    const bool stem_cl = pair && !x_cl && y_cl && stem_cl_ok(C, H, W, K, R, S, sh, sw, pad, OW, yb) &&
+                         stem_cl_apk_bytes() <= nhwc_apk_bytes(C, K, R, S);
     const bool halo = !pair && (!y_cl || yb == 1) && halo_fwd_ok(C, H, W, K, R, S, sh, sw, pad, border) &&
                       halo_apk_bytes(C, K) <= nhwc_apk_bytes(C, K, R, S);
-    if (!(opts & 2) && !halo) {              // bit 1: the workspace still holds this filter's packed form
+    if (!(opts & 2) && !halo && !stem_cl) {  // bit 1: the workspace still holds this filter's packed form
         const size_t total = (size_t)rowtiles * nchunks * ROWS * 32;
         int blocks = (int)((total + 255) / 256);
         if (blocks > 2048) blocks = 2048;
@@ -1548,6 +1551,9 @@ int nhwc_conv_fwd(const float *x, const void *x_cl, int xb, const float *w, cons
                            Wp, WS, nseg, wlog, clog);
         XSMI_LAUNCH_CHECK("nhwc_pad_bf16_kernel");
     }
+    if (stem_cl)
+        return stem_cl_conv_fwd(xp, ((size_t)N * Hp * Wp + 1) * CP * 2, w, apk, bias, y_cl, N, C, H, W, K, R, S, pad, OH, OW, relu,
+                                (opts & 2) != 0);
     if (halo) {
         return halo_conv_fwd(xp, (size_t)N * Hp * Wp * CP * 2, w, apk, bias, y, y_cl, mask, N, C, H, W, K, relu, (opts & 2) != 0);
     }

@@ -141,6 +141,13 @@ size_t halo_apk_bytes(int C, int K);
 int halo_conv_fwd(const void *xp, size_t xp_bytes, const float *w, void *apk, const float *bias, float *y, void *y_cl,
                   uint8_t *mask, int N, int C, int H, int W, int K, int relu, bool packed);
 
+// first layer (at most 4 channels, 7-row filter, stride 2) with channels-last bf16 output (conv_cl_halo.hip); called by
+// nhwc_conv_fwd after it has made the bordered 4-channel copy
+bool stem_cl_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OW, int y_border);
+size_t stem_cl_apk_bytes();
+int stem_cl_conv_fwd(const void *xp, size_t xp_bytes, const float *w, void *apk, const float *bias, void *y_cl, int N, int C,
+                     int H, int W, int K, int R, int S, int pad, int OH, int OW, int relu, bool packed);
+
 // weight gradient for the same few-channel layers (conv_stem.hip): horizontal stride 2, output width a multiple of 8,
 // filters a multiple of 64, at most 160 filter positions; the workspace holds the copy and the workgroups' partial sums
 bool stem_wgrad_ok(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad);
