@@ -121,15 +121,6 @@ __global__ void __launch_bounds__(256, 2) cl_halo_bf16_kernel(HaloParams p) {
 
     // ---- multiply side ----
     floatx16 acc[2][NBJ];
-    auto zero_acc = [&]() {
-#pragma unroll
-        for (int i = 0; i < 2; ++i)
-#pragma unroll
-            for (int j = 0; j < NBJ; ++j)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) acc[i][j][v] = 0.f;
-    };
-    zero_acc();
     const int h = lane >> 5, l31 = lane & 31;
     const int wr = wave / WC, wc = wave % WC;
     // lane half h takes octet 2 u + h of k-step u
@@ -230,11 +221,23 @@ __global__ void __launch_bounds__(256, 2) cl_halo_bf16_kernel(HaloParams p) {
             constexpr int tap = decltype(tap_c)::value, r = tap / 3, s = tap % 3;
             read_frags(IC<1>{}, IC<1>{}, (tap % 3) * A_STAGE, img_off + r * wp16 + s * 16);
             __builtin_amdgcn_sched_barrier(0);
+            if (tap == 0 && group == 0) {
+                // a tile's first MFMAs start from the constant zero: no pass over the accumulators between tiles
+                floatx16 z;
 #pragma unroll
-            for (int i = 0; i < 2; ++i)
+                for (int v = 0; v < 16; ++v) z[v] = 0.f;
 #pragma unroll
-                for (int j = 0; j < NBJ; ++j)
-                    acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < NBJ; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], z, 0, 0, 0);
+            } else {
+#pragma unroll
+                for (int i = 0; i < 2; ++i)
+#pragma unroll
+                    for (int j = 0; j < NBJ; ++j)
+                        acc[i][j] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(fa[0][i], fb[0][j], acc[i][j], 0, 0, 0);
+            }
             __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
             for (int j = 0; j < NBJ; ++j)
@@ -281,7 +284,6 @@ __global__ void __launch_bounds__(256, 2) cl_halo_bf16_kernel(HaloParams p) {
         if (!in_item) {
             xsmi::wait_vmcnt<0>();                    // the two A blocks in flight have landed (see the wait above)
             epilogue(tile);
-            zero_acc();
             tile += tile_step;
             group = 0;
             after_epilogue = p.out_cl != nullptr;
