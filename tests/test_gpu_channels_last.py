@@ -33,6 +33,13 @@ def _inputs(rng, n, c, h, k, r):
     (3, 32, 9, 128, 3, 2, 1, False),         # 128-row tiles, stride 2, ragged pixel tile
     (2, 3, 20, 64, 7, 2, 3, True),           # a stem: float32 input only, channels-last output
     (2, 64, 8, 72, 1, 1, 0, False),          # 1x1, K a multiple of 8 but not of 64
+    (2, 96, 30, 200, 3, 1, 1, True),         # input staged once for nine taps: three channel groups, two row tiles (one partial)
+    (3, 64, 14, 64, 3, 1, 1, False),         # ... on the smallest feature map that takes that kernel, 64-row tiles
+    (1, 32, 61, 64, 3, 1, 1, True),          # ... at its widest row (63 bordered pixels) ...
+    (1, 32, 62, 64, 3, 1, 1, True),          # ... and one pixel wider: the tap-major kernel serves it
+    (3, 3, 37, 32, 7, 2, 3, False),          # first-layer kernel: odd output height (a last item of one row), 32 filters
+    (1, 1, 224, 64, 7, 2, 3, True),          # ... one channel, the full 112-column row
+    (2, 4, 30, 8, 7, 2, 3, True),            # ... four channels, eight filters
 ])
 def test_channels_last_output_is_the_plain_result_rounded_to_bf16(gpu, n, c, h, k, r, stride, pad, relu):
     K = gpu.kernels
