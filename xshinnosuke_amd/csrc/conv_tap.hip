@@ -1628,6 +1628,22 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             plans[nplans++] = p;
         }
     }
+    // Residue classes no tap can reach (a stride larger than the filter: the 1 x 1 / 2 shortcuts leave three of four
+    // classes empty) receive no gradient.  Accumulating, they are left alone; overwriting, all of dx is cleared by one
+    // contiguous fill and only the classes with taps are computed, instead of tiles whose whole work is a strided
+    // store of zeros (64 -> 128 at 56 x 56, N=32: 25.8 -> 13 us).
+    {
+        int kept = 0;
+        for (int i = 0; i < nplans; ++i)
+            if (plans[i].TR * plans[i].TS > 0) { plans[kept] = plans[i]; specs[kept] = specs[i]; ++kept; }
+        if (kept < nplans) {
+            if (!accumulate) {
+                int rc = xsmi_fill(dx, 0.f, (size_t)N * C * H * W);
+                if (rc) return rc;
+            }
+            nplans = kept;
+        }
+    }
     // the residue classes of a pass run as one launch per TAP_MAX_CLASSES classes (stride 2: one launch)
     if (!(opts & 2)) {
         for (int i = 0; i < nplans; i += TAP_MAX_CLASSES) {
