@@ -314,10 +314,12 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
                 const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws,
                 size_t ws_bytes);
 
-/* Mean over non-overlapping k x k blocks of an NCHW tensor and its gradient
- * (the live mode of avg_pool2d, xs/nn/functional.py:539-583, xs/nn/grad_fn.py:284-309). */
-int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k);
-int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k);
+/* Mean over k x k windows at stride (sh, sw) of an NCHW tensor, no padding: y is (N, C, (H-k)/sh+1, (W-k)/sw+1),
+ * float64 sum, one rounding; and its gradient, overwritten into dx: every window hands dy / k^2 (a float32 quotient)
+ * to its cells, overlapping windows add up in float64 (avg_pool2d, xs/nn/functional.py:539-583,
+ * xs/nn/grad_fn.py:284-309; the reference's padded mode miscounts its output size and is not offered). */
+int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k, int sh, int sw);
+int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k, int sh, int sw);
 
 /* C[M,N] = op(A) . op(B) (+ bias[N] broadcast over rows); row-major, float32.  op is a transpose when
  * trans_a / trans_b is non-zero: A is stored (K,M) resp. B is stored (N,K).

@@ -204,6 +204,39 @@ def test_masked_gradient_into_two_tensors(gpu):
         np.testing.assert_array_equal(d1.numpy(), (o1 if acc else 0) + np.where(mask != 0, np.float32(0), dy))
 
 
+@pytest.mark.parametrize("n,c,h,w,k,sh,sw", [(2, 3, 9, 11, 3, 2, 2), (1, 5, 8, 8, 2, 1, 1), (3, 2, 12, 10, 3, 4, 5),
+                                             (2, 4, 7, 7, 5, 1, 2)])
+def test_average_pool_with_overlapping_or_sparse_windows(gpu, n, c, h, w, k, sh, sw):
+    """The im2col mode of avg_pool2d with stride != window (xs/nn/functional.py:563-571) and its gradient through the
+    float64 col2im (xs/nn/grad_fn.py:296-307): per-window share dy / k^2 in float32, sums in float64, one rounding."""
+    K = gpu.kernels
+    rng = np.random.default_rng(11 * h + w + k + sh)
+    x = rng.standard_normal((n, c, h, w)).astype(np.float32)
+    oh, ow = (h - k) // sh + 1, (w - k) // sw + 1
+    ref = np.zeros((n, c, oh, ow))
+    for i in range(oh):
+        for j in range(ow):
+            ref[:, :, i, j] = x[:, :, i * sh:i * sh + k, j * sw:j * sw + k].astype(np.float64).mean(axis=(2, 3))
+    y = K.avgpool_fwd(gpu.to_device(x), k, (sh, sw)).numpy()
+    assert y.shape == (n, c, oh, ow)
+    np.testing.assert_allclose(y, ref, rtol=1e-6, atol=1e-7)
+    dy = rng.standard_normal((n, c, oh, ow)).astype(np.float32)
+    share = (dy / np.float32(k * k)).astype(np.float64)
+    dref = np.zeros(x.shape)
+    for i in range(oh):
+        for j in range(ow):
+            dref[:, :, i * sh:i * sh + k, j * sw:j * sw + k] += share[:, :, i:i + 1, j:j + 1]
+    dx = K.avgpool_bwd(gpu.to_device(dy), x.shape, k, (sh, sw)).numpy()
+    np.testing.assert_allclose(dx, dref.astype(np.float32), rtol=1e-6, atol=1e-7)
+    # the host path of the functional op agrees with the device path
+    import xshinnosuke_amd as xs
+    t = xs.tensor(x, requires_grad=True)
+    out = xs.nn.functional.avg_pool2d(t, k, (sh, sw))
+    np.testing.assert_allclose(out.eval, ref, rtol=1e-6, atol=1e-7)
+    out.backward(xs.tensor(dy))
+    np.testing.assert_allclose(t.grad.eval, dref.astype(np.float32), rtol=1e-6, atol=1e-7)
+
+
 @pytest.mark.parametrize("n,c,h,w,k", [(3, 5, 6, 6, 2), (4, 70, 7, 7, 7), (2, 3, 7, 8, 3), (1, 2, 13, 13, 13)])
 def test_average_pool_blocks(gpu, n, c, h, w, k):
     """Mean over non-overlapping k x k blocks and its gradient (xs/nn/functional.py:539-583,

@@ -88,8 +88,8 @@ SIGNATURES = {
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f, _i]),
     "xsmi_bn_fold": (_i, [_vp] * 8 + [_i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 9 + [_i, _i, _i, _vp, _sz]),
-    "xsmi_avgpool_fwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
-    "xsmi_avgpool_bwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i]),
+    "xsmi_avgpool_fwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i]),
+    "xsmi_avgpool_bwd": (_i, [_vp, _vp, _i, _i, _i, _i, _i, _i, _i]),
     "xsmi_gemm": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _sz]),
     "xsmi_colsum": (_i, [_vp, _vp, _i, _i]),
     "xsmi_sum_all": (_i, [_vp, _vp, _sz]),

@@ -450,17 +450,23 @@ def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=
     return dx, dgamma, dbeta
 
 
-def avgpool_fwd(x, k):
+def avgpool_fwd(x, k, stride=None):
     n, c, h, w = x.shape
-    y = empty((n, c, h // k, w // k))
-    lib.call("xsmi_avgpool_fwd", x.cptr, y.cptr, n, c, h, w, int(k))
+    sh, sw = (int(k), int(k)) if stride is None else (int(stride[0]), int(stride[1]))
+    if k > h or k > w or sh < 1 or sw < 1:
+        raise ValueError("avg_pool2d: window %d does not fit the input %dx%d" % (k, h, w))
+    y = empty((n, c, (h - k) // sh + 1, (w - k) // sw + 1))
+    lib.call("xsmi_avgpool_fwd", x.cptr, y.cptr, n, c, h, w, int(k), sh, sw)
     return y
 
 
-def avgpool_bwd(dy, x_shape, k):
+def avgpool_bwd(dy, x_shape, k, stride=None):
     n, c, h, w = x_shape
+    sh, sw = (int(k), int(k)) if stride is None else (int(stride[0]), int(stride[1]))
+    if dy.shape != (n, c, (h - k) // sh + 1, (w - k) // sw + 1):
+        raise ValueError("avg_pool2d backward: dy %s does not match the pooled shape of %s" % (dy.shape, tuple(x_shape)))
     dx = empty(x_shape)
-    lib.call("xsmi_avgpool_bwd", dy.cptr, dx.cptr, n, c, h, w, int(k))
+    lib.call("xsmi_avgpool_bwd", dy.cptr, dx.cptr, n, c, h, w, int(k), sh, sw)
     return dx
 
 

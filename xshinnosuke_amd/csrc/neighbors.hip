@@ -603,13 +603,13 @@ __global__ void __launch_bounds__(256) bn_fold_kernel(const float *__restrict__ 
 
 // ---- average pool over k x k blocks --------------------------------------------
 __global__ void __launch_bounds__(256) avgpool_fwd_kernel(const float *__restrict__ x, float *__restrict__ y, int H, int W,
-                                                           int OH, int OW, int k, size_t total) {
+                                                           int OH, int OW, int k, int sh, int sw, size_t total) {
     for (size_t o = (size_t)blockIdx.x * 256 + threadIdx.x; o < total; o += (size_t)gridDim.x * 256) {
         int ow = (int)(o % OW);
         size_t t = o / OW;
         int oh = (int)(t % OH);
         size_t nc = t / OH;
-        const float *p = x + (nc * H + (size_t)oh * k) * W + (size_t)ow * k;
+        const float *p = x + (nc * H + (size_t)oh * sh) * W + (size_t)ow * sw;
         double s = 0.0;
         for (int r = 0; r < k; ++r)
             for (int q = 0; q < k; ++q) s += (double)p[(size_t)r * W + q];
@@ -637,6 +637,30 @@ __global__ void __launch_bounds__(256) avgpool_bwd_kernel(const float *__restric
         size_t nc = t / H;
         int oh = h / k, ow = w / k;
         dx[e] = (oh < OH && ow < OW) ? dy[(nc * OH + oh) * OW + ow] / (float)(k * k) : 0.f;
+    }
+}
+// Windows that overlap or leave gaps (stride != k): an input cell gathers dy / k^2 (rounded to float32 per window, as
+// the reference forms it) from every window that covers it, in ascending (ky, kx) order of its position in the window,
+// in float64, rounded once: the reference's float64 col2im (xs/nn/grad_fn.py:296-307).
+__global__ void __launch_bounds__(256) avgpool_bwd_strided_kernel(const float *__restrict__ dy, float *__restrict__ dx, int H,
+                                                                   int W, int OH, int OW, int k, int sh, int sw, size_t total) {
+    const float kk = (float)(k * k);
+    for (size_t e = (size_t)blockIdx.x * 256 + threadIdx.x; e < total; e += (size_t)gridDim.x * 256) {
+        int w = (int)(e % W);
+        size_t t = e / W;
+        int h = (int)(t % H);
+        size_t nc = t / H;
+        double s = 0.0;
+        for (int ky = 0; ky < k; ++ky) {
+            const int top = h - ky;
+            if (top < 0 || top % sh != 0 || top / sh >= OH) continue;
+            for (int kx = 0; kx < k; ++kx) {
+                const int left = w - kx;
+                if (left < 0 || left % sw != 0 || left / sw >= OW) continue;
+                s += (double)(dy[(nc * OH + top / sh) * OW + left / sw] / kk);
+            }
+        }
+        dx[e] = (float)s;
     }
 }
 
@@ -976,28 +1000,34 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
     return XSMI_OK;
 }
 
-int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k) {
+int xsmi_avgpool_fwd(const float *x, float *y, int N, int C, int H, int W, int k, int sh, int sw) {
     XSMI_REQUIRE_INIT();
-    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W, "xsmi_avgpool_fwd: bad geometry");
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W && sh >= 1 && sw >= 1,
+                   "xsmi_avgpool_fwd: bad geometry");
     XSMI_CHECK_ARG(x && y, "xsmi_avgpool_fwd: null pointer");
-    int OH = H / k, OW = W / k;
+    int OH = (H - k) / sh + 1, OW = (W - k) / sw + 1;
     size_t total = (size_t)N * C * OH * OW;
     if (k == H && k == W && total < 0x7fffffffu)
         hipLaunchKernelGGL(avgpool_plane_kernel, dim3((unsigned)((total + 3) / 4)), dim3(256), 0, xsmi::stream(), x, y, H * W,
                            (uint32_t)total);
     else
-        hipLaunchKernelGGL(avgpool_fwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, y, H, W, OH, OW, k, total);
+        hipLaunchKernelGGL(avgpool_fwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), x, y, H, W, OH, OW, k, sh, sw, total);
     XSMI_LAUNCH_CHECK("avgpool_fwd_kernel");
     return XSMI_OK;
 }
 
-int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k) {
+int xsmi_avgpool_bwd(const float *dy, float *dx, int N, int C, int H, int W, int k, int sh, int sw) {
     XSMI_REQUIRE_INIT();
-    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W, "xsmi_avgpool_bwd: bad geometry");
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0 && k >= 1 && k <= H && k <= W && sh >= 1 && sw >= 1,
+                   "xsmi_avgpool_bwd: bad geometry");
     XSMI_CHECK_ARG(dy && dx, "xsmi_avgpool_bwd: null pointer");
-    int OH = H / k, OW = W / k;
+    int OH = (H - k) / sh + 1, OW = (W - k) / sw + 1;
     size_t total = (size_t)N * C * H * W;
-    hipLaunchKernelGGL(avgpool_bwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), dy, dx, H, W, OH, OW, k, total);
+    if (sh == k && sw == k)
+        hipLaunchKernelGGL(avgpool_bwd_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), dy, dx, H, W, OH, OW, k, total);
+    else
+        hipLaunchKernelGGL(avgpool_bwd_strided_kernel, grid_for(total), dim3(256), 0, xsmi::stream(), dy, dx, H, W, OH, OW, k, sh,
+                           sw, total);
     XSMI_LAUNCH_CHECK("avgpool_bwd_kernel");
     return XSMI_OK;
 }

@@ -196,23 +196,35 @@ def batch_norm_backward(dy, xhat, sqrtvar, gamma):
     return dx, dgamma, dbeta
 
 
-def avg_pool_blocks(x, k):
-    """Non-overlapping k x k mean (the only live mode of the reference's avg_pool2d for stride == kernel)."""
+def avg_pool_blocks(x, k, stride=None):
+    """Mean over k x k windows at the given stride (default k: non-overlapping blocks), no padding: the im2col
+    mode of the reference's avg_pool2d, float64 sum and one rounding."""
+    sh, sw = (k, k) if stride is None else stride
     if is_device(x):
-        return K.avgpool_fwd(x, k)
+        return K.avgpool_fwd(x, k, (sh, sw))
     n, c, h, w = x.shape
-    oh, ow = h // k, w // k
-    return x[:, :, :oh * k, :ow * k].reshape(n, c, oh, k, ow, k).mean(axis=(3, 5)).astype(x.dtype, copy=False)
+    oh, ow = (h - k) // sh + 1, (w - k) // sw + 1
+    acc = np.zeros((n, c, oh, ow), dtype=np.float64)
+    for ky in range(k):
+        for kx in range(k):
+            acc += x[:, :, ky:ky + sh * oh:sh, kx:kx + sw * ow:sw]
+    return (acc / (k * k)).astype(x.dtype, copy=False)
 
 
-def avg_pool_blocks_grad(dy, x_shape, k):
+def avg_pool_blocks_grad(dy, x_shape, k, stride=None):
+    """Every window hands dy / k^2 (rounded to dy's dtype, as the reference forms it) to its cells; overlapping
+    windows add up in float64 in (ky, kx) order (the reference's col2im), rounded once."""
+    sh, sw = (k, k) if stride is None else stride
     if is_device(dy):
-        return K.avgpool_bwd(dy, x_shape, k)
+        return K.avgpool_bwd(dy, x_shape, k, (sh, sw))
     n, c, h, w = x_shape
     oh, ow = dy.shape[2], dy.shape[3]
-    g = np.zeros(x_shape, dtype=dy.dtype)
-    g[:, :, :oh * k, :ow * k] = np.repeat(np.repeat(dy, k, axis=2), k, axis=3) / (k * k)
-    return g
+    share = (dy / dy.dtype.type(k * k)).astype(np.float64)
+    g = np.zeros(x_shape, dtype=np.float64)
+    for ky in range(k):
+        for kx in range(k):
+            g[:, :, ky:ky + sh * oh:sh, kx:kx + sw * ow:sw] += share
+    return g.astype(dy.dtype, copy=False)
 
 
 def softmax_cross_entropy(logits, labels, reduction):

@@ -420,15 +420,15 @@ def mean(inputs, axis=None, keepdims=False):
 
 
 def avg_pool2d(inputs, kernel_size, stride=None, padding=0, out=None):
-    """Mean over non-overlapping k x k blocks.  The reference's overlapping and padded modes
-    (xs/nn/functional.py:539-583) are not reproduced: its padding arithmetic is wrong for
-    padding != 0 and every caller uses stride == kernel_size, padding == 0."""
+    """Mean over k x k windows at ``stride`` (default: the window size), reference xs/nn/functional.py:539-583 in
+    its im2col mode, which is the only live one there (it compares the int window with the stride pair).  The
+    reference's padded mode counts the padding twice in the output size and is not reproduced: padding must be 0."""
     _mark_input(inputs)
     k = int(kernel_size[0] if isinstance(kernel_size, (tuple, list)) else kernel_size)
     st = (k, k) if stride is None else _pair(stride)
-    if st != (k, k) or padding != 0:
-        raise NotImplementedError('avg_pool2d supports stride == kernel_size and padding == 0 only')
-    res = A.avg_pool_blocks(inputs.eval, k)
+    if padding != 0:
+        raise NotImplementedError('avg_pool2d supports padding == 0 only')
+    res = A.avg_pool_blocks(inputs.eval, k, st)
     if out is None:
         out = Tensor(res)
     else:
@@ -437,7 +437,7 @@ def avg_pool2d(inputs, kernel_size, stride=None, padding=0, out=None):
     _wire(out, inputs)
     if GLOBAL.COMPUTE_GRAD and out.requires_grad:
         out.cache['kernel_size'] = k
-        out.cache['mode'] = 'reshape'
+        out.cache['mode'] = 'im2col'
         out.cache['stride'] = st
         out.cache['padding'] = padding
         out.grad_fn = Avgpool2DBackward

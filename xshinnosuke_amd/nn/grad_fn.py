@@ -257,7 +257,8 @@ def MeanBackward(outputs):
 def Avgpool2DBackward(outputs):
     inputs, = outputs.in_bounds
     if inputs.requires_grad:
-        _accumulate(inputs, A.avg_pool_blocks_grad(outputs.grad.eval, inputs.shape, outputs.cache['kernel_size']))
+        _accumulate(inputs, A.avg_pool_blocks_grad(outputs.grad.eval, inputs.shape, outputs.cache['kernel_size'],
+                                                    outputs.cache['stride']))
 
 
 def _fresh_grad(t):
