@@ -40,9 +40,9 @@ sys.path.insert(1, os.path.join(ROOT, "tests"))      # the ResNet-18 workload (t
 FP32_MFMA_PEAK_TFLOPS = 157.3
 HBM_PEAK_GBPS = 8000.0
 
-# BASELINE conv config: N, C, H, W, K, R, S, stride, pad
+# the benchmark conv configuration: N, C, H, W, K, R, S, stride, pad
 CONV = dict(N=32, C=64, H=56, W=56, K=64, R=3, S=3, stride=(1, 1), pad=1)
-# BASELINE max-pool config
+# the benchmark max-pool configuration
 POOL = dict(N=32, C=64, H=112, W=112, k=3, stride=(2, 2), pad=1)
 
 # The 11 distinct convolutions of ResNet-18 at N=32, 224x224 input: name, count, Cin, Cout, H_in, k, stride, pad

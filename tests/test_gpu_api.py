@@ -132,7 +132,7 @@ def _readme_net_oracle(x, wc, bc, wd, bd, labels, lr):
 
 @pytest.mark.parametrize("kind", ["sequential", "functional"])
 def test_readme_network_one_training_step(kind):
-    """BASELINE config 0: N=256x1x28x28, Conv2D(8, 2x2, relu) -> MaxPool 2x2 -> Flatten -> Dense(10), CE, SGD lr 0.01."""
+    """The README network of the reference at its benchmark size: N=256x1x28x28, Conv2D(8, 2x2, relu) -> MaxPool 2x2 -> Flatten -> Dense(10), CE, SGD lr 0.01."""
     rng = np.random.default_rng(0)
     n = 256
     x = rng.standard_normal((n, 1, 28, 28)).astype(np.float32)

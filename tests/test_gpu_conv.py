@@ -19,7 +19,7 @@ CASES = [  # n c h w k r s sh sw pad
     (2, 3, 7, 6, 4, 3, 3, 1, 1, 1),
     (1, 3, 5, 5, 1, 3, 3, 1, 1, 0),        # tests/gradient_check/check_cnn.py shapes
     (4, 1, 28, 28, 8, 2, 2, 1, 1, 0),      # README net conv
-    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),    # BASELINE conv geometry, fewer images
+    (2, 64, 56, 56, 64, 3, 3, 1, 1, 1),    # the benchmark conv geometry, fewer images
     (2, 3, 32, 32, 64, 7, 7, 2, 2, 3),     # ResNet stem geometry (small image)
     (2, 64, 28, 28, 128, 3, 3, 2, 2, 1),   # layer2.0 conv_a
     (2, 64, 28, 28, 128, 1, 1, 2, 2, 0),   # 1x1 / 2 shortcut
@@ -291,7 +291,7 @@ def test_conv_golden_fixture(gpu):
 
 
 def test_conv_full_size_adjoint_and_slice(gpu):
-    """BASELINE conv config at full size (N=32, 64->64, 56x56, 3x3/1/1): bilinear identities in float64 on
+    """The benchmark conv configuration at full size (N=32, 64->64, 56x56, 3x3/1/1): bilinear identities in float64 on
     the device results plus oracle parity on a slice of images."""
     K = gpu.kernels
     x = np.random.default_rng(1).standard_normal((32, 64, 56, 56), dtype=np.float32)

@@ -10,7 +10,7 @@ pytestmark = pytest.mark.gpu
 CASES = [  # n c h w k sh sw pad
     (2, 3, 7, 7, 3, 2, 2, 1),
     (3, 5, 16, 12, 3, 2, 2, 1),      # vectorised 3x3/2/1 path (W % 4 == 0, H even)
-    (2, 4, 112, 112, 3, 2, 2, 1),    # BASELINE max-pool geometry, fewer images
+    (2, 4, 112, 112, 3, 2, 2, 1),    # the benchmark max-pool geometry, fewer images
     (1, 2, 8, 8, 2, 2, 2, 0),
     (4, 8, 27, 27, 2, 2, 2, 0),      # README net: last row/column dropped
     (1, 2, 9, 7, 3, 1, 1, 1),
@@ -72,7 +72,7 @@ def test_pool_golden_fixture(gpu):
 
 
 def test_pool_full_size_properties(gpu):
-    """BASELINE max-pool config at full size (32x64x112x112), checked through size-independent properties
+    """The benchmark max-pool configuration at full size (32x64x112x112), checked through size-independent properties
     plus an exact comparison on a slice of images."""
     rng = np.random.default_rng(4)
     n, c, h, w = 32, 64, 112, 112
