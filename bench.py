@@ -322,10 +322,27 @@ def bench_readme_net(be, steps, warmup):
         ms = e0.elapsed_ms(e1)
         be.synchronize()
         wall = (time.perf_counter() - t0) * 1e3
-        return {"readme_net_ms_per_step": ms / steps, "readme_net_wall_ms_per_step": wall / steps,
-                "readme_net_images_per_sec": README_N * steps / (ms * 1e-3), "readme_net_last_loss": loss.item(),
-                "readme_net_workload": "N=256x1x28x28, Conv2D(8, 2x2, relu) + MaxPool 2x2 + Flatten + Dense(10), cross-entropy, "
-                                       "SGD lr 0.01; fwd+bwd+step through the layer API, device-resident"}
+        out = {"readme_net_ms_per_step": ms / steps, "readme_net_wall_ms_per_step": wall / steps,
+               "readme_net_images_per_sec": README_N * steps / (ms * 1e-3), "readme_net_last_loss": loss.item(),
+               "readme_net_workload": "N=256x1x28x28, Conv2D(8, 2x2, relu) + MaxPool 2x2 + Flatten + Dense(10), cross-entropy, "
+                                      "SGD lr 0.01; fwd+bwd+step through the layer API, device-resident"}
+        # this step is bound by the host issuing its launches: recorded once and replayed it is bound by the device
+        graph = be.StepGraph()
+        with graph.capture():
+            loss = step()
+        for _ in range(warmup + 5):
+            graph.replay()
+        be.synchronize()
+        e0.record()
+        for _ in range(steps):
+            graph.replay()
+        e1.record()
+        ms = e0.elapsed_ms(e1)
+        be.synchronize()
+        out.update({"readme_net_graph_ms_per_step": ms / steps, "readme_net_graph_images_per_sec": README_N * steps / (ms * 1e-3),
+                    "readme_net_graph_last_loss": loss.item()})
+        graph.close()
+        return out
     finally:
         xs.GLOBAL.USE_CUDA = False
         xs.GLOBAL.INPUTS = None
@@ -363,14 +380,35 @@ def bench_resnet18(be, steps, warmup):
     e0.record()
     for _ in range(steps):
         loss = step()
+    enqueue = (time.perf_counter() - t0) * 1e3       # the host has issued every launch; the device is still running
     e1.record()
     ms = e0.elapsed_ms(e1)
     be.synchronize()
     wall = (time.perf_counter() - t0) * 1e3
+    out = {"resnet18_train_images_per_sec": 32 * steps / (ms * 1e-3), "resnet18_ms_per_step": ms / steps,
+           "resnet18_wall_ms_per_step": wall / steps, "resnet18_host_enqueue_ms_per_step": enqueue / steps,
+           "resnet18_last_loss": loss.item(),
+           "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
+    # the same step recorded once as a step graph and replayed: one call per step instead of ~230
+    graph = be.StepGraph()
+    with graph.capture():
+        loss = step()
+    for _ in range(warmup):
+        graph.replay()
+    be.synchronize()
+    t0 = time.perf_counter()
+    e0.record()
+    for _ in range(steps):
+        graph.replay()
+    enqueue = (time.perf_counter() - t0) * 1e3
+    e1.record()
+    ms = e0.elapsed_ms(e1)
+    be.synchronize()
+    out.update({"resnet18_graph_images_per_sec": 32 * steps / (ms * 1e-3), "resnet18_graph_ms_per_step": ms / steps,
+                "resnet18_graph_host_enqueue_ms_per_step": enqueue / steps, "resnet18_graph_last_loss": loss.item()})
+    graph.close()
     xs.GLOBAL.USE_CUDA = False
-    return {"resnet18_train_images_per_sec": 32 * steps / (ms * 1e-3), "resnet18_ms_per_step": ms / steps,
-            "resnet18_wall_ms_per_step": wall / steps, "resnet18_last_loss": loss.item(),
-            "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
+    return out
 
 
 def bench_resnet18_infer(be, steps, warmup, with_oracle=True):

@@ -89,7 +89,7 @@ int xsmi_host_alloc(void **ptr, size_t bytes);
 int xsmi_host_free(void *ptr);
 int xsmi_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes);   /* async on the stream */
-int xsmi_memset(void *dst, int byte_value, size_t bytes);        /* async on the stream */
+int xsmi_memset(void *dst, int byte_value, size_t bytes);        /* async on the stream (a fill kernel) */
 int xsmi_sync(void);
 int xsmi_event_create(void **event);
 int xsmi_event_record(void *event);                               /* on the library stream */
@@ -105,6 +105,27 @@ int xsmi_last_kernel_ms(float *ms);
 /* plain float4 copy kernel of `bytes` bytes (multiple of 16); used to
  * calibrate HBM counters and to quote the achievable copy bandwidth. */
 int xsmi_copy_kernel(void *dst, const void *src, size_t bytes);
+
+/* ---- step graphs ----------------------------------------------------------
+ * No counterpart in the reference, whose steps are NumPy calls.  A training or inference step here is a
+ * few hundred short launches, and the host needs about as long to issue them as the device needs to run
+ * them; a step whose launches do not change from one iteration to the next (same entry points, same
+ * pointers, same sizes, same scalars) can be recorded once and re-issued with one call.
+ *
+ * xsmi_graph_begin() opens the recording: until xsmi_graph_end() every entry point records its launches
+ * (both streams, with the fork and join of xsmi_conv2d_bwd) instead of running them, so nothing recorded has
+ * happened yet when the recording ends.  Entry points that wait for the device (xsmi_sync, xsmi_memcpy_h2d,
+ * xsmi_memcpy_d2h, the event calls, xsmi_last_kernel_ms) fail with XSMI_ERR_STATE while it is open, xsmi_malloc
+ * stays legal, xsmi_free takes effect when it closes.  xsmi_graph_end(&graph, keep) closes it and, with
+ * keep != 0, hands back an executable graph (keep == 0 discards what was recorded, e.g. after an error).
+ * xsmi_graph_launch() enqueues one replay on the library stream, in order with everything else;
+ * xsmi_graph_destroy() waits for the stream and releases the graph.  Every buffer the recorded launches
+ * touch must stay allocated, and unused by anything that expects its contents to survive a replay, for as
+ * long as the graph is replayed. */
+int xsmi_graph_begin(void);
+int xsmi_graph_end(void **graph, int keep);
+int xsmi_graph_launch(void *graph);
+int xsmi_graph_destroy(void *graph);
 
 /* ---- convolution ---------------------------------------------------------
  * x (N,C,H,W), w (K,C,R,S), bias (K) or NULL, y (N,K,OH,OW).

@@ -67,6 +67,25 @@ class ResNet18(Module):
         return self.fc(x)
 
 
+def named_params(net):
+    """Parameters in a reproducible order: walk the modules the way forward() uses them."""
+    out = []
+
+    def seq(s):
+        for layer in s._graph:
+            if hasattr(layer, '_graph'):
+                seq(layer)
+            elif hasattr(layer, 'conv1'):
+                seq(layer.conv1); seq(layer.shortcut)
+            else:
+                out.extend(p for p in layer.parameters() if p is not None)
+    seq(net.conv1)
+    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
+        seq(stage)
+    out.extend(net.fc.parameters())
+    return out
+
+
 def oracle_forward(net, x):
     """ResNet-18 inference (moving-statistics batch norm) in NumPy: convolutions and the max-pool through the
     oracle (float64 GEMM, one rounding), the rest in float64 rounded to float32 per op."""

@@ -4,7 +4,7 @@ import numpy as np
 import pytest
 
 import xshinnosuke_amd as xs
-from resnet18 import ResNet18, oracle_forward as _oracle_forward
+from resnet18 import ResNet18, oracle_forward as _oracle_forward, named_params as _named_params
 from xshinnosuke_amd.optim import SGD
 from util import rel_l2
 
@@ -19,25 +19,6 @@ def _fresh_state(gpu):
     yield
     xs.GLOBAL.INPUTS = None
     xs.GLOBAL.USE_CUDA = False
-
-
-def _named_params(net):
-    """Parameters in a reproducible order: walk the modules the way forward() uses them."""
-    out = []
-
-    def seq(s):
-        for layer in s._graph:
-            if hasattr(layer, '_graph'):
-                seq(layer)
-            elif hasattr(layer, 'conv1'):
-                seq(layer.conv1); seq(layer.shortcut)
-            else:
-                out.extend(p for p in layer.parameters() if p is not None)
-    seq(net.conv1)
-    for stage in (net.layer1, net.layer2, net.layer3, net.layer4):
-        seq(stage)
-    out.extend(net.fc.parameters())
-    return out
 
 
 def test_resnet18_device_path_matches_host_path():

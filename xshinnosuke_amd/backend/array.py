@@ -14,6 +14,8 @@ _CL_POOL = {}         # (n, c, h, w, border) -> ChannelsLast forms of released a
 _CL_POOL_DEPTH = 4
 _POOL_BYTES = [0]
 _POOL_LIMIT = 64 << 30
+_CAPTURE = [None]     # the StepGraph whose step is being recorded (backend/graph.py), else None
+_EPOCH = [0]          # moves whenever recorded work may have changed device memory behind Python's back
 
 
 def _round_size(nbytes):
@@ -39,7 +41,7 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl", "owner")
 
     def __init__(self, nbytes):
         ensure_init()
@@ -48,6 +50,15 @@ class _Block:
         self.cl = None                       # ChannelsLast form of the array that fills this block, if it has one
         self.version = 0                     # counts every hand-out of the address and every pending clear
         size = _round_size(nbytes)
+        # Memory handed out while a step is recorded belongs to that graph from then on: released blocks go to
+        # the graph's own pool (later allocations of the same recording may take them, which a replay repeats
+        # in the same order), never to code that runs between replays.
+        graph = self.owner = _CAPTURE[0]
+        free = graph._pool.get(size) if graph is not None else None
+        if free:
+            self.ptr = free.pop()
+            self.nbytes = size
+            return
         free = _POOL.get(size)
         if free:
             self.ptr = free.pop()
@@ -72,11 +83,15 @@ class _Block:
             if cl is not None:               # keep the zero-bordered buffer for the next array of this geometry
                 self.cl = None
                 cl.valid = False
-                kept = _CL_POOL.setdefault((cl.n, cl.c, cl.h, cl.w, cl.border), [])
-                if len(kept) < _CL_POOL_DEPTH:
-                    kept.append(cl)
+                if cl.buf._block.owner is None and _CAPTURE[0] is None:
+                    kept = _CL_POOL.setdefault((cl.n, cl.c, cl.h, cl.w, cl.border), [])
+                    if len(kept) < _CL_POOL_DEPTH:
+                        kept.append(cl)
             if self.ptr:
-                if _POOL_BYTES[0] + self.nbytes <= _POOL_LIMIT:
+                graph = self.owner
+                if graph is not None and not graph._closed:
+                    graph._pool.setdefault(self.nbytes, []).append(self.ptr)
+                elif _POOL_BYTES[0] + self.nbytes <= _POOL_LIMIT:
                     _POOL.setdefault(self.nbytes, []).append(self.ptr)
                     _POOL_BYTES[0] += self.nbytes
                 else:
@@ -138,6 +153,9 @@ class DeviceArray:
     def ptr(self):
         blk = self._block
         blk.version += 1                     # whoever takes the address may write through it
+        graph = _CAPTURE[0]
+        if graph is not None and blk.owner is not graph:
+            graph._refs[id(blk)] = blk       # recorded launches use this memory: it lives as long as the graph
         if blk.lazy_zero:                    # logically zero, memory not cleared yet: clear it on first use
             blk.lazy_zero = False
             lib.call("xsmi_memset", ctypes.c_void_p(blk.ptr), 0, blk.nbytes)
@@ -220,6 +238,9 @@ class DeviceArray:
         return len(self.shape)
 
     def numpy(self):
+        if _CAPTURE[0] is not None:
+            raise XsmiError("a device array cannot be read on the host while a step graph is being captured: "
+                            "nothing recorded has run yet")
         out = np.empty(self.shape, dtype=self.dtype)
         if self.nbytes:
             lib.call("xsmi_memcpy_d2h", out.ctypes.data_as(ctypes.c_void_p), self.cptr, self.nbytes)
@@ -230,6 +251,9 @@ class DeviceArray:
         return a if dtype is None else a.astype(dtype, copy=False)
 
     def set(self, host):
+        if _CAPTURE[0] is not None:
+            raise XsmiError("a blocking upload cannot be part of a step graph: fill the array before the capture, "
+                            "or enqueue set_async from pinned memory")
         host = np.ascontiguousarray(host, dtype=self.dtype)
         if host.shape != self.shape:
             host = np.ascontiguousarray(np.broadcast_to(host, self.shape))
@@ -363,6 +387,9 @@ class Workspace:
         if self._block is None or self._block.nbytes < nbytes:
             self._block = None
             self._block = _Block(max(int(nbytes), 256))
+        graph = _CAPTURE[0]
+        if graph is not None and self._block.owner is not graph:
+            graph._refs[id(self._block)] = self._block
         return ctypes.c_void_p(self._block.ptr), self._block.nbytes
 
 

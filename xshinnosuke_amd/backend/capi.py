@@ -96,6 +96,10 @@ SIGNATURES = {
     "xsmi_softmax_ce_fwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i]),
     "xsmi_softmax_ce_bwd": (_i, [_vp, _vp, _vp, _vp, _i, _i, _f]),
     "xsmi_fill": (_i, [_vp, _f, _sz]),
+    "xsmi_graph_begin": (_i, []),
+    "xsmi_graph_end": (_i, [_c.POINTER(_vp), _i]),
+    "xsmi_graph_launch": (_i, [_vp]),
+    "xsmi_graph_destroy": (_i, [_vp]),
 }
 
 CONV_RELU = 0x1
@@ -208,6 +212,12 @@ def take_deferred_add(out):
         return a, b
     _flush_deferred()
     return None
+
+
+def drop_pending():
+    """Forget a held-back add and the arrays kept for the second stream (a recording that is being discarded)."""
+    del _deferred[:]
+    del _side_hold[:]
 
 
 def init(device=0):

@@ -13,6 +13,11 @@ USE_CUDA = False
 # Opt-in: convolutions may round their MFMA operands to bf16 (fp32 accumulate).  Off by
 # default; the reference has no counterpart (its GEMMs run in float64).
 CONV_BF16 = False
+# Opt-in (also XSMI_STEP_GRAPH=1 in the environment): fit() on device-resident data records its full-batch training
+# step once as a step graph and replays it for every later full batch (backend/graph.py); a shorter last batch
+# runs launch by launch as before.  No counterpart in the reference.
+import os as _os
+STEP_GRAPH = _os.environ.get("XSMI_STEP_GRAPH", "0") not in ("", "0")
 
 
 class no_grad:

@@ -2,6 +2,7 @@
 #include "xsmi_internal.h"
 #include <stdarg.h>
 #include <string.h>
+#include <vector>
 
 namespace {
 thread_local char g_err[512] = "";
@@ -16,6 +17,10 @@ bool g_ready = false;
 bool g_profiling = false;
 hipEvent_t g_prof0 = nullptr, g_prof1 = nullptr;
 bool g_prof_valid = false;
+// A step graph under capture: the launches of every entry point are recorded instead of run.  Calls that must
+// wait for the device are refused while it lasts, and hipFree (which waits too) is put off to its end.
+bool g_capturing = false;
+std::vector<void *> g_free_after_capture;
 }  // namespace
 
 namespace xsmi {
@@ -48,11 +53,12 @@ bool side_pending() { return g_side_pending; }
 bool on_side_stream() { return g_current == g_side; }
 bool ready() { return g_ready; }
 int cu_count() { return g_cus; }
+bool capturing() { return g_capturing; }
 void prof_begin() {
-    if (g_profiling && g_current == g_stream) (void)hipEventRecord(g_prof0, g_stream);
+    if (g_profiling && !g_capturing && g_current == g_stream) (void)hipEventRecord(g_prof0, g_stream);
 }
 void prof_end() {
-    if (g_profiling && g_current == g_stream) {
+    if (g_profiling && !g_capturing && g_current == g_stream) {
         (void)hipEventRecord(g_prof1, g_stream);
         g_prof_valid = true;
     }
@@ -68,6 +74,24 @@ __global__ void __launch_bounds__(256) xsmi_copy_f4(const xsmi_f4v *__restrict__
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     if (i < n4) __builtin_nontemporal_store(__builtin_nontemporal_load(src + i), dst + i);
 }
+
+// Byte fill as a kernel (a memset node in a captured graph is not dependable): 16-byte stores over the aligned
+// middle, single bytes over the unaligned head and tail.
+__global__ void __launch_bounds__(256) xsmi_memset_kernel(unsigned char *p, unsigned word, size_t head, size_t n16, size_t tail) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    typedef unsigned u4v __attribute__((ext_vector_type(4)));
+    if (i < n16) reinterpret_cast<u4v *>(p + head)[i] = u4v{word, word, word, word};
+    if (i < head) p[i] = (unsigned char)word;
+    if (i < tail) p[head + n16 * 16 + i] = (unsigned char)word;
+}
+
+#define XSMI_NOT_WHILE_CAPTURING()                                                              \
+    do {                                                                                        \
+        if (g_capturing) {                                                                      \
+            xsmi::set_error("%s waits for the device: not possible while a step graph is being captured", __func__); \
+            return XSMI_ERR_STATE;                                                              \
+        }                                                                                       \
+    } while (0)
 
 extern "C" {
 
@@ -136,6 +160,10 @@ int xsmi_malloc(void **ptr, size_t bytes) {
 int xsmi_free(void *ptr) {
     XSMI_REQUIRE_INIT();
     if (ptr == nullptr) return XSMI_OK;
+    if (g_capturing) {
+        g_free_after_capture.push_back(ptr);
+        return XSMI_OK;
+    }
     // hipFree waits for the device; work queued on the stream that still uses
     // `ptr` has completed when it returns.
     XSMI_HIP(hipFree(ptr));
@@ -144,6 +172,7 @@ int xsmi_free(void *ptr) {
 
 int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes) {
     XSMI_REQUIRE_INIT();
+    XSMI_NOT_WHILE_CAPTURING();
     if (bytes == 0) return XSMI_OK;
     XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_h2d: null pointer");
     XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyHostToDevice, g_stream));
@@ -177,6 +206,7 @@ int xsmi_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes) {
 
 int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     XSMI_REQUIRE_INIT();
+    XSMI_NOT_WHILE_CAPTURING();
     if (bytes == 0) return XSMI_OK;
     XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_d2h: null pointer");
     XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
@@ -196,7 +226,16 @@ int xsmi_memset(void *dst, int byte_value, size_t bytes) {
     XSMI_REQUIRE_INIT();
     if (bytes == 0) return XSMI_OK;
     XSMI_CHECK_ARG(dst != nullptr, "xsmi_memset: null pointer");
-    XSMI_HIP(hipMemsetAsync(dst, byte_value, bytes, g_stream));
+    size_t head = (size_t)(-(intptr_t)dst) & 15;
+    if (head > bytes) head = bytes;
+    size_t n16 = (bytes - head) / 16, tail = bytes - head - n16 * 16;
+    size_t threads = n16 > 16 ? n16 : 16;
+    size_t blocks = (threads + 255) / 256;
+    XSMI_CHECK_ARG(blocks < 2147483648ull, "xsmi_memset: more than 2^31 workgroups");
+    unsigned word = 0x01010101u * (unsigned)(byte_value & 0xff);
+    hipLaunchKernelGGL(xsmi_memset_kernel, dim3((unsigned)blocks), dim3(256), 0, xsmi::stream(),
+                       (unsigned char *)dst, word, head, n16, tail);
+    XSMI_LAUNCH_CHECK("xsmi_memset_kernel");
     return XSMI_OK;
 }
 
@@ -207,6 +246,7 @@ int xsmi_conv2d_bwd_join(void) {
 
 int xsmi_sync(void) {
     XSMI_REQUIRE_INIT();
+    XSMI_NOT_WHILE_CAPTURING();
     int rc = xsmi::side_join();                      // weight gradients still on the second stream
     if (rc) return rc;
     XSMI_HIP(hipStreamSynchronize(g_stream));
@@ -215,6 +255,7 @@ int xsmi_sync(void) {
 
 int xsmi_event_synchronize(void *event) {
     XSMI_REQUIRE_INIT();
+    XSMI_NOT_WHILE_CAPTURING();
     XSMI_CHECK_ARG(event != nullptr, "xsmi_event_synchronize: null event");
     XSMI_HIP(hipEventSynchronize((hipEvent_t)event));
     return XSMI_OK;
@@ -232,6 +273,7 @@ int xsmi_event_create(void **event) {
 int xsmi_event_record(void *event) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(event != nullptr, "xsmi_event_record: null event");
+    XSMI_CHECK_ARG(!g_capturing, "xsmi_event_record: a timing event cannot be recorded into a step graph");
     XSMI_HIP(hipEventRecord((hipEvent_t)event, g_stream));
     return XSMI_OK;
 }
@@ -239,6 +281,7 @@ int xsmi_event_record(void *event) {
 int xsmi_event_elapsed_ms(void *start, void *stop, float *ms) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(start && stop && ms, "xsmi_event_elapsed_ms: null argument");
+    XSMI_NOT_WHILE_CAPTURING();
     XSMI_HIP(hipEventSynchronize((hipEvent_t)stop));
     XSMI_HIP(hipEventElapsedTime(ms, (hipEvent_t)start, (hipEvent_t)stop));
     return XSMI_OK;
@@ -266,6 +309,7 @@ int xsmi_last_kernel_ms(float *ms) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(ms != nullptr, "xsmi_last_kernel_ms: null argument");
     XSMI_CHECK_ARG(g_prof_valid, "xsmi_last_kernel_ms: no op has run since xsmi_profiling(1)");
+    XSMI_NOT_WHILE_CAPTURING();
     XSMI_HIP(hipEventSynchronize(g_prof1));
     XSMI_HIP(hipEventElapsedTime(ms, g_prof0, g_prof1));
     return XSMI_OK;
@@ -284,6 +328,76 @@ int xsmi_copy_kernel(void *dst, const void *src, size_t bytes) {
                        (const xsmi_f4v *)src, (xsmi_f4v *)dst, n4);
     xsmi::prof_end();
     XSMI_LAUNCH_CHECK("xsmi_copy_f4");
+    return XSMI_OK;
+}
+
+int xsmi_graph_begin(void) {
+    XSMI_REQUIRE_INIT();
+    if (g_capturing) {
+        xsmi::set_error("xsmi_graph_begin: a capture is already open");
+        return XSMI_ERR_STATE;
+    }
+    int rc = xsmi::side_join();
+    if (rc) return rc;
+    // relaxed mode: the host may still call hipMalloc (a pool miss) while the stream records
+    XSMI_HIP(hipStreamBeginCapture(g_stream, hipStreamCaptureModeRelaxed));
+    g_capturing = true;
+    return XSMI_OK;
+}
+
+int xsmi_graph_end(void **graph, int keep) {
+    XSMI_REQUIRE_INIT();
+    if (graph) *graph = nullptr;
+    if (!g_capturing) {
+        xsmi::set_error("xsmi_graph_end: no capture is open");
+        return XSMI_ERR_STATE;
+    }
+    // the second stream joined the capture when it first waited for the main stream; it has to come back
+    // before the capture can end
+    int rc = xsmi::side_join();
+    g_current = g_stream;
+    hipGraph_t g = nullptr;
+    hipError_t e = hipStreamEndCapture(g_stream, &g);
+    g_capturing = false;
+    for (void *p : g_free_after_capture) (void)hipFree(p);
+    g_free_after_capture.clear();
+    if (e != hipSuccess) {
+        (void)hipGetLastError();
+        xsmi::set_error("hipStreamEndCapture failed: %s", hipGetErrorString(e));
+        return XSMI_ERR_RUNTIME;
+    }
+    if (rc || !keep || !graph) {
+        if (g) (void)hipGraphDestroy(g);
+        return rc;
+    }
+    hipGraphExec_t exec = nullptr;
+    e = hipGraphInstantiate(&exec, g, nullptr, nullptr, 0);
+    (void)hipGraphDestroy(g);
+    if (e != hipSuccess) {
+        xsmi::set_error("hipGraphInstantiate failed: %s", hipGetErrorString(e));
+        return XSMI_ERR_RUNTIME;
+    }
+    *graph = (void *)exec;
+    return XSMI_OK;
+}
+
+int xsmi_graph_launch(void *graph) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(graph != nullptr, "xsmi_graph_launch: null graph");
+    XSMI_CHECK_ARG(!g_capturing, "xsmi_graph_launch: a capture is open");
+    int rc = xsmi::side_join();
+    if (rc) return rc;
+    XSMI_HIP(hipGraphLaunch((hipGraphExec_t)graph, g_stream));
+    return XSMI_OK;
+}
+
+int xsmi_graph_destroy(void *graph) {
+    XSMI_REQUIRE_INIT();
+    if (graph == nullptr) return XSMI_OK;
+    XSMI_CHECK_ARG(!g_capturing, "xsmi_graph_destroy: a capture is open");
+    // replays still in flight read the executable graph: wait for them first
+    XSMI_HIP(hipStreamSynchronize(g_stream));
+    XSMI_HIP(hipGraphExecDestroy((hipGraphExec_t)graph));
     return XSMI_OK;
 }
 

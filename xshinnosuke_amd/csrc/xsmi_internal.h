@@ -20,6 +20,7 @@ void side_end();
 int side_join();              // no-op when the second stream holds nothing the main stream has not waited for
 bool side_pending();
 bool on_side_stream();
+bool capturing();            // a step graph is being recorded: nothing runs, nothing may wait for the device
 bool ready();
 int cu_count();
 // conv_noalloc.hip: resolves the device address of the static scratch array for `device` (the current device)

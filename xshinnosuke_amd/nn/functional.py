@@ -140,7 +140,8 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
         # Frozen parameters: the folded filter, its bias and its packed form (in a workspace of this filter's own) are
         # kept while nobody has taken the address of a parameter since they were made (DeviceArray.state).
         # (the batch size is part of the key: it decides which kernel, hence which packed layout, the library picks)
-        now = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape))
+        # (and so is the count of step-graph recordings and replays: those change parameters without taking addresses)
+        now = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape), dev._EPOCH[0])
         need = K.conv2d_workspace_bytes(x.shape, weight.shape, stride, padding)
         if kept is not None and kept['key'] == now and kept['ws'].holds(need):
             y = K.conv2d_fwd(x, kept['w'], kept['b'], stride, padding, relu=relu, out=dst, bf16=bf16, packed=True,
@@ -152,7 +153,7 @@ def conv2d_batch_norm_inference(inputs, weight, bias, stride, padding, gamma, be
             ws = kept['ws'] if kept is not None else K.Workspace()
             y = K.conv2d_fwd(x, w2, b2, stride, padding, relu=relu, out=dst, bf16=bf16, workspace=ws, channels_last=bf16)
             # the fold has read the parameters: their state as of now is what the kept filter belongs to
-            key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape))
+            key = (tuple(a.state() for a in sources), float(epsilon), bf16, stride, padding, tuple(x.shape), dev._EPOCH[0])
             _FOLDED[weight] = {'key': key, 'w': w2, 'b': b2, 'ws': ws, 'of': sources}   # 'of' keeps the ids in the key alive
     else:
         stats = [_f32_device(t.eval).reshape(-1) for t in (gamma, beta, moving_mean, moving_variance)]

@@ -5,6 +5,7 @@ path depends on: lazily created parameters, per-layer preallocated output tensor
 shorter last batch (written through ``out=``), ``layer.backward()`` in reverse order for static
 graphs, and parameter discovery by graph walk for ``Module``.
 """
+import contextlib
 import pickle
 import time
 
@@ -21,6 +22,7 @@ from ..optim import get_optimizer
 from ..utils.data import DataSet, DataLoader
 from .objectives import get_objective
 from . import functional as F
+from ..backend.graph import StepGraph
 
 
 class _Base:
@@ -83,6 +85,11 @@ class _Model(_Base):
         loader = DataLoader(DataSet(x, y), batch_size, shuffle, device=self._device)
         history = {'train_loss': [], 'train_acc': [], 'validation_loss': [], 'validation_acc': []}
         self.train()
+        # GLOBAL.STEP_GRAPH: the loader refills the same two device tensors for every batch and the static graph
+        # writes the same buffers every step, so the third full-batch step is recorded instead of run and every
+        # later full batch is one replay; `pred` and `loss` are then the recording's tensors.
+        graph, recorded, eager_steps = None, None, 0
+        want_graph = GLOBAL.STEP_GRAPH and self._device == 'cuda'
         for epoch in range(initial_epoch, epochs):
             t0 = time.time()
             losses, accs = [], []
@@ -90,11 +97,25 @@ class _Model(_Base):
                 bx, by = self._place(bx), self._place(by)
                 if idx == 0 or idx == len(loader) - 1:
                     self.init_graph_out_tensor(bx, by)
-                self.optimizer.zero_grad()
-                pred = self.forward(bx)
-                loss = self.loss.forward(pred, by)
-                self.backward(loss)
-                self.optimizer.step()
+                full = bx.shape[0] == loader.batch_size
+                record = want_graph and graph is None and full and eager_steps >= 2
+                if graph is not None and full:
+                    pred, loss = recorded
+                    graph.replay()
+                    self.optimizer.iterations += 1
+                else:
+                    if record:
+                        graph = StepGraph()
+                    with (graph.capture() if record else contextlib.nullcontext()):
+                        self.optimizer.zero_grad()
+                        pred = self.forward(bx)
+                        loss = self.loss.forward(pred, by)
+                        self.backward(loss)
+                        self.optimizer.step()
+                    if record:
+                        recorded = (pred, loss)
+                        graph.replay()
+                    eager_steps += 1
                 losses.append(loss.item())
                 accs.append(self.loss.calc_acc(pred, by))
             history['train_loss'].append(float(np.mean(losses)))
