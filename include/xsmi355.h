@@ -50,8 +50,11 @@ extern "C" {
                                     The weight gradient ignores the flag.                     */
 #define XSMI_CONV_WS_PACKED 0x4u /* the workspace still holds what the previous call of the same
                                     entry point with the same geometry and the same filter values
-                                    left there: the filter is not laid out again (inference loops).
-                                    Ignored where no reusable layout exists.                */
+                                    left there, or what xsmi_conv2d_pack left there for this pass,
+                                    geometry and filter values: the filter is not laid out again
+                                    (inference loops; training steps that lay all filters out right
+                                    after the optimizer step).  Ignored where no reusable layout
+                                    exists.  xsmi_conv2d_bwd applies it to the data gradient.  */
 
 #define XSMI_CONV_DW_ASYNC 0x8u  /* xsmi_conv2d_bwd only: the weight gradient stays on the library's
                                     second stream when the call returns; see xsmi_conv2d_bwd_join */
@@ -213,7 +216,8 @@ int xsmi_conv2d_bwd_weight(const float *dy, const float *x, float *dw, float *db
  * xsmi_conv2d_bwd_data compute, with the same results bit for bit (Conv2DBackward,
  * xs/nn/grad_fn.py:191-203, does the two one after the other).  The two share only
  * their inputs, so the weight gradient can run on a second stream of the library
- * beside the data gradient.  db may be NULL.  flags: XSMI_CONV_BF16, XSMI_CONV_DW_ASYNC.
+ * beside the data gradient.  db may be NULL.  flags: XSMI_CONV_BF16, XSMI_CONV_DW_ASYNC,
+ * XSMI_CONV_WS_PACKED (the data gradient's workspace holds the filter layout already).
  * workspace serves the data gradient, workspace_dw the weight gradient; each of
  * xsmi_conv2d_workspace_bytes() bytes is enough, and the two must not overlap.
  *
@@ -234,9 +238,30 @@ int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w,
                     int sh, int sw, int pad, float beta_dx, float beta_dw, unsigned flags,
                     void *workspace, size_t workspace_bytes,
                     void *workspace_dw, size_t workspace_dw_bytes);
-/* The main stream waits for every weight gradient that xsmi_conv2d_bwd left on the second
- * stream; a no-op when there is none. */
+/* The main stream waits for everything on the second stream (weight gradients that xsmi_conv2d_bwd
+ * left there, filter layouts of xsmi_conv2d_pack); a no-op when there is nothing. */
 int xsmi_conv2d_bwd_join(void);
+
+/* Lay filters out ahead of time.  Every conv call first rewrites w into the layout its kernel reads
+ * (a few microseconds of a tiny launch in front of each of the ~40 convolution passes of a ResNet-18
+ * step; the reference has no counterpart, its im2col GEMM reads w as it is, xs/nn/functional.py:428).
+ * This entry point runs only that step, for every job: pass 0 (xsmi_conv2d_fwd) or 1
+ * (xsmi_conv2d_bwd_data / the data gradient of xsmi_conv2d_bwd) of the given fp32 geometry, all on the
+ * library's second stream: ordered after everything enqueued so far, beside whatever the main stream is
+ * given next.  job.packed is set to 1 when the job's workspace now holds a layout that the later call
+ * accepts through XSMI_CONV_WS_PACKED (same geometry, same workspace size, w unchanged in between), and
+ * to 0 when this geometry's kernel has nothing to prepare ahead (first layers, the generic kernels);
+ * the later call must then not pass the flag.  The main stream has to wait for the second one
+ * (xsmi_conv2d_bwd_join) before the first call that uses a prepared workspace. */
+typedef struct xsmi_pack_job {
+    const float *w;
+    void *workspace;
+    size_t workspace_bytes;
+    int N, C, H, W, K, R, S, sh, sw, pad;
+    int pass;
+    int packed;                  /* out */
+} xsmi_pack_job_t;
+int xsmi_conv2d_pack(int count, xsmi_pack_job_t *jobs);
 
 /* ---- max pooling ---------------------------------------------------------
  * x (N,C,H,W) -> y (N,C,OH,OW), square window k, zero-valued padding that takes

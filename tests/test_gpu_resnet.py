@@ -118,6 +118,54 @@ def test_resnet18_steps_do_not_depend_on_the_weight_gradient_overlap(monkeypatch
         np.testing.assert_array_equal(u, v)
 
 
+def test_resnet18_steps_do_not_depend_on_filter_layouts_made_ahead(monkeypatch):
+    """After each optimizer step the backend lays every filter out again on its second stream and the next
+    step's convolutions skip their own layout launch.  Five SGD steps with that and five without end in the same
+    bits, also when a filter is overwritten from the host between two steps (its layout made ahead is then stale
+    and must not be used) and when the batch size changes for one step."""
+    from xshinnosuke_amd.backend import kernels as K, capi
+
+    def run(ahead):
+        monkeypatch.setattr(K, "_PREPACK", ahead)
+        np.random.seed(4)
+        X = np.random.randn(8, 3, 64, 64).astype(np.float32)
+        Y = np.random.randint(0, 10, (8,))
+        net = ResNet18(classes=10, pool=2).to('cuda')
+        x, y = xs.tensor(X).to('cuda'), xs.tensor(Y).to('cuda')
+        x6, y6 = xs.tensor(X[:6]).to('cuda'), xs.tensor(Y[:6]).to('cuda')
+        net(x)
+        xs.GLOBAL.INPUTS = None
+        opt = SGD(net.parameters(), lr=0.05)
+        crit = xs.nn.CrossEntropyLoss()
+        params = _named_params(net)
+        flags = []
+        real = capi.lib.call
+        monkeypatch.setattr(capi.lib, "call", lambda name, *a: (flags.append((name, a[15])) if name == "xsmi_conv2d_fwd" else None,
+                                                                real(name, *a))[1])
+        losses = []
+        for i in range(5):
+            if i == 2:                               # a filter changes behind the optimizer's back
+                w = [p for p in params if len(p.shape) == 4 and p.shape[1] == 64][1]     # a layer1 filter
+                w.eval = w.numpy() * np.float32(0.5)
+            bx, by = (x6, y6) if i == 3 else (x, y)
+            opt.zero_grad()
+            loss = crit(net(bx), by)
+            loss.backward()
+            opt.step()
+            losses.append(loss.item())
+        out = [p.numpy().copy() for p in params]
+        monkeypatch.undo()
+        xs.GLOBAL.INPUTS = None
+        return losses, out, sum(1 for _, f in flags if f & capi.CONV_WS_PACKED)
+
+    la, pa, skipped_a = run(True)
+    lb, pb, skipped_b = run(False)
+    assert skipped_b == 0 and skipped_a >= 19 * 2        # steps 2 and 5 at least find every layout in place
+    assert la == lb
+    for u, v in zip(pa, pb):
+        np.testing.assert_array_equal(u, v)
+
+
 def test_resnet18_bf16_inference_against_oracle():
     """Inference configuration: moving-statistics batch norm, forward only, convolutions allowed to use bf16
     MFMA operands.  Logits against the NumPy/oracle forward: rel-L2 <= 1e-2 for bf16, <= 1e-4 for fp32."""

@@ -41,7 +41,7 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl", "owner")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl", "owner", "__weakref__")
 
     def __init__(self, nbytes):
         ensure_init()
@@ -378,6 +378,10 @@ class Workspace:
 
     def __reduce__(self):
         raise TypeError("a device workspace cannot be pickled")
+
+    def address(self):
+        """The present block's device address (0 before the first ``get``)."""
+        return self._block.ptr if self._block is not None else 0
 
     def holds(self, nbytes):
         """True if ``get(nbytes)`` would hand out the present block (no reallocation)."""

@@ -29,6 +29,12 @@ class DeviceInfo(ctypes.Structure):
     ]
 
 
+class PackJob(ctypes.Structure):
+    """xsmi_pack_job_t"""
+    _fields_ = [("w", ctypes.c_void_p), ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t)] + \
+               [(n, ctypes.c_int) for n in ("N", "C", "H", "W", "K", "R", "S", "sh", "sw", "pad", "pass_", "packed")]
+
+
 _c = ctypes
 _vp, _i, _sz, _f, _u = _c.c_void_p, _c.c_int, _c.c_size_t, _c.c_float, _c.c_uint
 _CONV_DIMS = [_i] * 10   # N C H W K R S sh sw pad
@@ -64,6 +70,7 @@ SIGNATURES = {
     "xsmi_conv2d_bwd_weight": (_i, [_vp, _vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
     "xsmi_conv2d_bwd": (_i, [_vp] * 6 + _CONV_DIMS + [_f, _f, _u, _vp, _sz, _vp, _sz]),
     "xsmi_conv2d_bwd_join": (_i, []),
+    "xsmi_conv2d_pack": (_i, [_i, _vp]),
     "xsmi_maxpool2d_fwd": (_i, [_vp, _vp, _vp] + [_i] * 8),
     "xsmi_maxpool2d_bwd": (_i, [_vp, _vp, _vp] + [_i] * 8 + [_f]),
     "xsmi_relu_mask_bwd": (_i, [_vp, _vp, _vp, _sz, _f]),
@@ -178,12 +185,27 @@ def side_pending():
 
 
 def join_side():
-    """The main stream waits for the weight gradients on the second stream; their operands are released."""
-    if _side_hold:
+    """The main stream waits for the second stream (weight gradients, filter layouts made ahead); the operands
+    held for it are released."""
+    if _side_hold or _layouts_pending[0]:
         try:
             lib.call("xsmi_conv2d_bwd_join")
         finally:
             del _side_hold[:]
+            del _layouts_hold[:]
+            _layouts_pending[0] = False
+
+
+# Filter layouts that xsmi_conv2d_pack put on the second stream (kernels.refresh_layouts).  Unlike a weight
+# gradient they do not force the next call into the library to join: only a convolution that is about to read
+# one of those workspaces does (kernels._layout_for), so that the layouts run beside whatever comes first.
+_layouts_pending = [False]
+_layouts_hold = []          # the filters being read and the workspaces being written there stay allocated until the join
+
+
+def layouts_enqueued(*held):
+    _layouts_pending[0] = True
+    _layouts_hold.extend(held)
 
 
 # One element-wise add may be held back until the next call into the library: if that call is the in-place ReLU
@@ -218,6 +240,8 @@ def drop_pending():
     """Forget a held-back add and the arrays kept for the second stream (a recording that is being discarded)."""
     del _deferred[:]
     del _side_hold[:]
+    del _layouts_hold[:]
+    _layouts_pending[0] = False
 
 
 def init(device=0):

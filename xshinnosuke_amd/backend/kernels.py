@@ -5,11 +5,14 @@ the host before anything is launched, and raises ``ValueError`` for geometry
 the reference would also reject.
 """
 import ctypes
+import os
+import weakref
 
 import numpy as np
 
 from . import capi
 from .capi import lib, CONV_RELU, CONV_BF16, CONV_WS_PACKED, CONV_DW_ASYNC
+from . import array as _array
 from .array import DeviceArray, Workspace, empty
 
 _ws = Workspace()
@@ -30,14 +33,111 @@ def _dims(x_shape, w_shape, stride, pad):
     return [int(v) for v in (n, c, h, w, k, r, s, stride[0], stride[1], pad)]
 
 
+_NEED = {}                  # geometry -> xsmi_conv2d_workspace_bytes (a pure function of the ten numbers)
+
+
+def _need(dims):
+    key = tuple(dims)
+    need = _NEED.get(key)
+    if need is None:
+        need = _NEED[key] = lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
+    return need
+
+
 def conv2d_workspace_bytes(x_shape, w_shape, stride, pad):
     """Bytes of workspace the conv entry points want for this geometry."""
-    return lib.raw("xsmi_conv2d_workspace_bytes")(*_dims(x_shape, w_shape, stride, pad))
+    return _need(_dims(x_shape, w_shape, stride, pad))
 
 
 def _workspace(dims):
-    need = lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
-    return _ws.get(need)
+    return _ws.get(_need(dims))
+
+
+# ---- filter layouts made ahead of time -----------------------------------------------------------------------
+# Every conv call first rewrites its filter into the layout its kernel reads: a launch of a few microseconds in
+# front of each of the ~40 convolution passes of a ResNet-18 training step, on the critical path although the
+# filters only change once per step.  A training forward / backward therefore works in a workspace of its own per
+# (filter, pass, geometry), and right after an optimizer step `refresh_layouts` lays all filters used since the
+# previous one out again on the library's second stream (xsmi_conv2d_pack), beside the start of the next step.  A
+# call that finds its workspace's layout still belonging to the filter's current contents (DeviceArray.state)
+# skips the layout launch (XSMI_CONV_WS_PACKED).  XSMI_PREPACK=0 switches this off.
+_PREPACK = os.environ.get("XSMI_PREPACK", "1") not in ("", "0")
+_LAYOUTS = weakref.WeakKeyDictionary()        # filter's memory block -> {(pass, dims): _Layout}
+
+
+class _Layout:
+    __slots__ = ("ws", "key", "used", "ahead")
+
+    def __init__(self):
+        self.ws = Workspace()
+        self.key = None       # DeviceArray.state() of the filter when the workspace's layout was made
+        self.used = False     # a convolution ran in this workspace since the last refresh
+        self.ahead = True     # False once xsmi_conv2d_pack reported that this geometry has nothing to lay out ahead
+
+
+def _layout_for(w, pass_, dims):
+    """(entry, current): the layout workspace of this filter, pass and geometry, and whether it already holds the
+    layout of the filter's present contents.  Waits for layouts still on the second stream."""
+    blk = w._block
+    if w._offset or blk.lazy_zero or (blk.cl is not None and blk.cl.valid):
+        return None, False
+    entries = _LAYOUTS.get(blk)
+    if entries is None:
+        entries = _LAYOUTS[blk] = {}
+    key = (pass_,) + tuple(dims)
+    entry = entries.get(key)
+    if entry is None:
+        entry = entries[key] = _Layout()
+    entry.used = True
+    if capi._layouts_pending[0]:                  # the workspace may still be written on the second stream
+        capi.join_side()
+    return entry, entry.key is not None and entry.key == w.state()
+
+
+_plan = {"sig": None, "jobs": None}
+
+
+def refresh_layouts(arrays):
+    """After an update of ``arrays`` (an optimizer step): every filter among them whose layouts were used since the
+    last refresh gets them made again, on the second stream, in one call; layouts that were not used are dropped."""
+    if not _LAYOUTS:
+        return
+    todo = []
+    for v in arrays:
+        entries = _LAYOUTS.get(v._block)
+        if not entries:
+            continue
+        for key in [k for k, e in entries.items() if not e.used]:
+            del entries[key]
+        for key, e in entries.items():
+            e.used = False
+            e.key = None
+            if e.ahead:
+                todo.append((v, e, key))
+    if not todo:
+        return
+    # the job table is rebuilt only when the set of layouts changes (and while a step graph records, which must see
+    # every buffer's address being taken)
+    sig = tuple((v.address(), e.ws.address(), key) for v, e, key in todo)
+    if sig != _plan["sig"] or _array._CAPTURE[0] is not None:
+        jobs = (capi.PackJob * len(todo))()
+        for job, (v, e, (pass_, *dims)) in zip(jobs, todo):
+            ws, ws_bytes = e.ws.get(_need(dims))
+            job.w, job.workspace, job.workspace_bytes = v.ptr, ws.value, ws_bytes
+            job.N, job.C, job.H, job.W, job.K, job.R, job.S, job.sh, job.sw, job.pad = dims
+            job.pass_ = pass_
+        _plan["sig"], _plan["jobs"] = sig, jobs
+    jobs = _plan["jobs"]
+    lib.call("xsmi_conv2d_pack", len(todo), ctypes.cast(jobs, ctypes.c_void_p))
+    held = []
+    for job, (v, e, _) in zip(jobs, todo):
+        if job.packed:
+            e.key = v.state()
+            held.append((v, e.ws))
+        else:
+            e.ahead = False
+    if held:
+        capi.layouts_enqueued(*held)
 
 
 def _f32(a, what):
@@ -47,8 +147,10 @@ def _f32(a, what):
 
 
 def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_mask=None, bf16=False, packed=False,
-               workspace=None, channels_last=False):
-    """``packed=True`` promises that the previous conv call on this workspace was this same forward with the same
+               workspace=None, channels_last=False, keep_layout=False):
+    """``keep_layout=True`` (training steps; fp32, the shared workspace): the call works in a workspace that belongs
+    to this filter, pass and geometry, whose layout ``refresh_layouts`` renews after each update of the filter.
+    ``packed=True`` promises that the previous conv call on this workspace was this same forward with the same
     geometry and filter values (the workspace still holds the filter's packed form), so it is not laid out again.
     ``workspace``: a ``Workspace`` of the caller's instead of the shared one (a layer that keeps its packed filter).
     ``channels_last=True`` (with ``bf16``, no mask): the result may be left in channels-last bf16 form, and an input
@@ -70,8 +172,13 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
         raise ValueError("conv2d: out has shape %s, expected %s" % (out.shape, (n, k, oh, ow)))
     if neg_mask is not None and (neg_mask.dtype != np.uint8 or neg_mask.size != out.size):
         raise ValueError("conv2d: neg_mask must be uint8 with one byte per output element")
+    layout = None
+    if keep_layout and _PREPACK and not bf16 and not packed and workspace is None:
+        layout, packed = _layout_for(w, 0, dims)
+        if layout is not None:
+            workspace = layout.ws
     flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0)
-    ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(lib.raw("xsmi_conv2d_workspace_bytes")(*dims))
+    ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(_need(dims))
     if channels_last and bf16 and neg_mask is None:
         xcl = x.channels_last()
         if xcl is not None and not (c % 32 == 0 and xcl.border >= pad):
@@ -84,8 +191,12 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
                      flags & ~CONV_BF16, ws, ws_bytes)
             return out
     out._overwritten()
-    lib.call("xsmi_conv2d_fwd", x.cptr, w.cptr, bias.cptr if bias is not None else None, out.cptr,
+    # a filter whose layout is in place is not read: its address goes along without counting as handed out
+    wptr = ctypes.c_void_p(w.address()) if layout is not None and packed else w.cptr
+    lib.call("xsmi_conv2d_fwd", x.cptr, wptr, bias.cptr if bias is not None else None, out.cptr,
              neg_mask.cptr if neg_mask is not None else None, *dims, flags, ws, ws_bytes)
+    if layout is not None and not packed:
+        layout.key = w.state()                    # the call has laid the present filter out in this workspace
     return out
 
 
@@ -101,7 +212,8 @@ def _beta(accumulate, *outs):
     return 0.0
 
 
-def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=False, bf16=False, packed=False):
+def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=False, bf16=False, packed=False,
+                    keep_layout=False):
     _f32(dy, "dy"); _f32(w, "w")
     dims = _dims(x_shape, w.shape, stride, pad)
     n, c, h, wd, k, r, s = dims[:7]
@@ -113,10 +225,16 @@ def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=Fa
         accumulate = False
     elif dx.shape != tuple(x_shape):
         raise ValueError("conv2d backward: dx has shape %s, expected %s" % (dx.shape, tuple(x_shape)))
-    ws, ws_bytes = _workspace(dims)
+    layout = None
+    if keep_layout and _PREPACK and not bf16 and not packed:
+        layout, packed = _layout_for(w, 1, dims)
+    ws, ws_bytes = _workspace(dims) if layout is None else layout.ws.get(_need(dims))
     beta = _beta(accumulate, dx)
-    lib.call("xsmi_conv2d_bwd_data", dy.cptr, w.cptr, dx.cptr, *dims, beta,
+    wptr = ctypes.c_void_p(w.address()) if layout is not None and packed else w.cptr
+    lib.call("xsmi_conv2d_bwd_data", dy.cptr, wptr, dx.cptr, *dims, beta,
              (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0), ws, ws_bytes)
+    if layout is not None and not packed:
+        layout.key = w.state()
     return dx
 
 
@@ -144,7 +262,8 @@ def conv2d_bwd_weight(dy, x, w_shape, stride=(1, 1), pad=0, dw=None, db=None, ac
     return dw, db
 
 
-def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False, bf16=False, async_dw=False):
+def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False, bf16=False, async_dw=False,
+               keep_layout=False):
     """Both gradients of one layer in one call, into existing device buffers.  Same results as ``conv2d_bwd_weight``
     followed by ``conv2d_bwd_data``.  ``async_dw=True`` leaves the weight gradient running on the library's second
     stream beside whatever is enqueued next; dw and db are complete after ``capi.join_side()``, which every call into
@@ -159,16 +278,22 @@ def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False
         raise ValueError("conv2d backward: dx %s / dw %s do not match x %s / w %s" % (dx.shape, dw.shape, x.shape, w.shape))
     if db is not None and db.size != k:
         raise ValueError("conv2d backward: db has %d elements for %d filters" % (db.size, k))
-    need = lib.raw("xsmi_conv2d_workspace_bytes")(*dims)
+    need = _need(dims)
     if capi.side_pending() and not _ws_dw.holds(need):
         capi.join_side()                        # the block about to be replaced may still be in use
-    ws, ws_bytes = _ws.get(need)
+    layout, packed = None, False
+    if keep_layout and _PREPACK and not bf16:
+        layout, packed = _layout_for(w, 1, dims)          # the data gradient's filter layout
+    ws, ws_bytes = _ws.get(need) if layout is None else layout.ws.get(need)
     ws_dw, ws_dw_bytes = _ws_dw.get(need)
     beta_dw = _beta(accumulate, dw, db)
     beta_dx = _beta(accumulate, dx)
-    flags = (CONV_BF16 if bf16 else 0) | (CONV_DW_ASYNC if async_dw else 0)
-    lib.call("xsmi_conv2d_bwd", dy.cptr, x.cptr, w.cptr, dx.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
+    flags = (CONV_BF16 if bf16 else 0) | (CONV_DW_ASYNC if async_dw else 0) | (CONV_WS_PACKED if packed else 0)
+    wptr = ctypes.c_void_p(w.address()) if layout is not None and packed else w.cptr
+    lib.call("xsmi_conv2d_bwd", dy.cptr, x.cptr, wptr, dx.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
              beta_dx, beta_dw, flags, ws, ws_bytes, ws_dw, ws_dw_bytes)
+    if layout is not None and not packed:
+        layout.key = w.state()
     if async_dw:
         capi.hold_side(dy, x, dw, db)
     return dx, dw, db

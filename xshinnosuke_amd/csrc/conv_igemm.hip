@@ -325,6 +325,35 @@ size_t conv_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
 }
 }  // namespace xsmi
 
+// Which forward / backward-data kernel family serves a geometry with the given flags and workspace size: one place,
+// so that xsmi_conv2d_pack lays a filter out for exactly the kernel that the later call will pick.
+enum class FwdPath { ChannelsLast, FirstLayer, EvenSplit, Tap, Generic };
+enum class BwdDataPath { EvenSplit, Tap, Generic };
+
+static FwdPath fwd_path(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OH, int OW, unsigned flags,
+                        size_t workspace_bytes) {
+    const bool bf16 = (flags & XSMI_CONV_BF16) != 0;
+    if (bf16 && xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad) && workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
+        return FwdPath::ChannelsLast;
+    if (!bf16 && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad) &&
+        workspace_bytes >= xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
+        return FwdPath::FirstLayer;
+    if (!bf16 && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * OH * OW, K, R, S, sh, sw) &&
+        workspace_bytes >= xsmi::sk_fwd_ws_bytes(C, K, R, S))
+        return FwdPath::EvenSplit;
+    if (xsmi::tap_path_ok(C)) return FwdPath::Tap;
+    return FwdPath::Generic;
+}
+
+static BwdDataPath bwd_data_path(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, unsigned flags,
+                                 size_t workspace_bytes) {
+    if (!(flags & XSMI_CONV_BF16) && xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw) && xsmi::sk_bwd_data_pays(N * H * W, C, R, S, sh, sw) &&
+        workspace_bytes >= xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw))
+        return BwdDataPath::EvenSplit;
+    if (xsmi::tap_path_ok(K)) return BwdDataPath::Tap;
+    return BwdDataPath::Generic;
+}
+
 extern "C" {
 
 int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y, uint8_t *neg_mask, int N, int C, int H,
@@ -335,27 +364,29 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     int rc = check_conv("xsmi_conv2d_fwd", N, C, H, W, K, R, S, sh, sw, pad, &g);
     if (rc) return rc;
     XSMI_CHECK_ARG(x && w && y, "xsmi_conv2d_fwd: null tensor pointer");
-    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED | XSMI_CONV_PACK_ONLY)) == 0,
+                   "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
     const int J = C * R * S;
     const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_fwd: workspace of %zu bytes needed, %zu given", need,
                    workspace_bytes);
-    if ((flags & XSMI_CONV_BF16) && xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad) &&
-        workspace_bytes >= xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad))
+    const int relu = (flags & XSMI_CONV_RELU) ? 1 : 0;
+    const int opts = ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0) | ((flags & XSMI_CONV_PACK_ONLY) ? 4 : 0);
+    switch (fwd_path(N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, flags, workspace_bytes)) {
+    case FwdPath::ChannelsLast:
         return xsmi::nhwc_conv_fwd(x, nullptr, 0, w, bias, y, nullptr, 0, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
-                                   (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
-    if (!(flags & XSMI_CONV_BF16) && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad) &&
-        workspace_bytes >= xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
-        return xsmi::stem_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
-                                   (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
-    if (!(flags & XSMI_CONV_BF16) && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * g.OH * g.OW, K, R, S, sh, sw) &&
-        workspace_bytes >= xsmi::sk_fwd_ws_bytes(C, K, R, S))
-        return xsmi::sk_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
-                                 (flags & XSMI_CONV_RELU) ? 1 : 0, (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
-    if (xsmi::tap_path_ok(C))
-        return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW,
-                                  (flags & XSMI_CONV_RELU) ? 1 : 0,
-                                  ((flags & XSMI_CONV_BF16) ? 1 : 0) | ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0), workspace);
+                                   relu, opts, workspace);
+    case FwdPath::FirstLayer:
+        return xsmi::stem_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, relu, opts, workspace);
+    case FwdPath::EvenSplit:
+        return xsmi::sk_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, relu, opts, workspace);
+    case FwdPath::Tap:
+        return xsmi::tap_conv_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, relu,
+                                  ((flags & XSMI_CONV_BF16) ? 1 : 0) | opts, workspace);
+    case FwdPath::Generic:
+        break;
+    }
+    if (flags & XSMI_CONV_PACK_ONLY) return XSMI_OK;     // the generic kernel's table is cheap and rebuilt per call
     const int rowtiles = xsmi::ceil_div(K, TM);
     const int nchunks = xsmi::ceil_div(J, KC);
     float *apk = (float *)workspace;
@@ -430,17 +461,22 @@ int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int 
     if (rc) return rc;
     XSMI_CHECK_ARG(dy && w && dx, "xsmi_conv2d_bwd_data: null tensor pointer");
     XSMI_CHECK_ARG(beta == 0.f || beta == 1.f, "xsmi_conv2d_bwd_data: beta must be 0 or 1");
-    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED)) == 0, "xsmi_conv2d_bwd_data: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED | XSMI_CONV_PACK_ONLY)) == 0,
+                   "xsmi_conv2d_bwd_data: unknown flags 0x%x", flags);
     const size_t need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     XSMI_CHECK_ARG(workspace && workspace_bytes >= need, "xsmi_conv2d_bwd_data: workspace of %zu bytes needed, %zu given",
                    need, workspace_bytes);
-    if (!(flags & XSMI_CONV_BF16) && xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw) &&
-        xsmi::sk_bwd_data_pays(N * H * W, C, R, S, sh, sw) && workspace_bytes >= xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw))
-        return xsmi::sk_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
-                                      (flags & XSMI_CONV_WS_PACKED) ? 2 : 0, workspace);
-    if (xsmi::tap_path_ok(K))
+    const int opts = ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0) | ((flags & XSMI_CONV_PACK_ONLY) ? 4 : 0);
+    switch (bwd_data_path(N, C, H, W, K, R, S, sh, sw, flags, workspace_bytes)) {
+    case BwdDataPath::EvenSplit:
+        return xsmi::sk_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0, opts, workspace);
+    case BwdDataPath::Tap:
         return xsmi::tap_conv_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, g.OH, g.OW, beta == 1.f ? 1 : 0,
-                                       ((flags & XSMI_CONV_BF16) ? 1 : 0) | ((flags & XSMI_CONV_WS_PACKED) ? 2 : 0), workspace);
+                                       ((flags & XSMI_CONV_BF16) ? 1 : 0) | opts, workspace);
+    case BwdDataPath::Generic:
+        break;
+    }
+    if (flags & XSMI_CONV_PACK_ONLY) return XSMI_OK;
     hipStream_t st = xsmi::stream();
     char *ws = (char *)workspace;
     const int rowtiles = xsmi::ceil_div(C, TM);
@@ -500,6 +536,48 @@ int xsmi_conv2d_bwd_data(const float *dy, const float *w, float *dx, int N, int 
     }
     xsmi::prof_end();
     return XSMI_OK;
+}
+
+int xsmi_conv2d_pack(int count, xsmi_pack_job_t *jobs) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(count >= 0 && (count == 0 || jobs), "xsmi_conv2d_pack: bad argument");
+    bool forked = false;
+    int rc = XSMI_OK;
+    for (int i = 0; i < count && rc == XSMI_OK; ++i) {
+        xsmi_pack_job_t &j = jobs[i];
+        j.packed = 0;
+        ConvGeom g;
+        rc = check_conv("xsmi_conv2d_pack", j.N, j.C, j.H, j.W, j.K, j.R, j.S, j.sh, j.sw, j.pad, &g);
+        if (rc) break;
+        if (!j.w || (j.pass != 0 && j.pass != 1)) {
+            xsmi::set_error("xsmi_conv2d_pack: job %d has a null filter or an unknown pass %d", i, j.pass);
+            rc = XSMI_ERR_INVALID;
+            break;
+        }
+        // the first-layer kernels lay their filter out inside the launch that pads the input, the generic kernels
+        // rebuild a small table per call: nothing to do ahead of time for either
+        if (j.pass == 0) {
+            const FwdPath path = fwd_path(j.N, j.C, j.H, j.W, j.K, j.R, j.S, j.sh, j.sw, j.pad, g.OH, g.OW, 0, j.workspace_bytes);
+            if (path != FwdPath::EvenSplit && path != FwdPath::Tap) continue;
+        } else if (bwd_data_path(j.N, j.C, j.H, j.W, j.K, j.R, j.S, j.sh, j.sw, 0, j.workspace_bytes) == BwdDataPath::Generic) {
+            continue;
+        }
+        if (!forked) {
+            // the second stream, after everything the main stream holds so far (earlier users of these workspaces
+            // included); one fork serves all jobs, the second stream runs them in order
+            rc = xsmi::side_begin();
+            if (rc) break;
+            forked = true;
+        }
+        float *unused = const_cast<float *>(j.w);        // activations are not touched by a layout-only call
+        rc = j.pass == 0 ? xsmi_conv2d_fwd(unused, j.w, nullptr, unused, nullptr, j.N, j.C, j.H, j.W, j.K, j.R, j.S, j.sh, j.sw,
+                                           j.pad, XSMI_CONV_PACK_ONLY, j.workspace, j.workspace_bytes)
+                         : xsmi_conv2d_bwd_data(unused, j.w, unused, j.N, j.C, j.H, j.W, j.K, j.R, j.S, j.sh, j.sw, j.pad, 0.f,
+                                                XSMI_CONV_PACK_ONLY, j.workspace, j.workspace_bytes);
+        if (rc == XSMI_OK) j.packed = 1;
+    }
+    if (forked) xsmi::side_end();
+    return rc;
 }
 
 }  // extern "C"

@@ -1447,6 +1447,7 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
         int rc = launch_pack(st, w, &spec, 1, 0, K, C, R, S, 1, 1, opts);
         if (rc) return rc;
     }
+    if (opts & 4) return XSMI_OK;            // bit 2: lay the filter out and stop
     TapParams p;
     p.in = x; p.apk = apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
     p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
@@ -1637,7 +1638,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
         for (int i = 0; i < nplans; ++i)
             if (plans[i].TR * plans[i].TS > 0) { plans[kept] = plans[i]; specs[kept] = specs[i]; ++kept; }
         if (kept < nplans) {
-            if (!accumulate) {
+            if (!accumulate && !(opts & 4)) {
                 int rc = xsmi_fill(dx, 0.f, (size_t)N * C * H * W);
                 if (rc) return rc;
             }
@@ -1652,6 +1653,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             if (rc) return rc;
         }
     }
+    if (opts & 4) return XSMI_OK;            // bit 2: lay the filter out and stop
     prof_begin();
     for (int i = 0; i < nplans; i += TAP_MAX_CLASSES) {
         TapMulti mp;

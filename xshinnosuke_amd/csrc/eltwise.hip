@@ -108,7 +108,8 @@ int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w, float *dx, 
                    "xsmi_conv2d_bwd: bad geometry");
     XSMI_CHECK_ARG(dy && x && w && dx && dw, "xsmi_conv2d_bwd: null tensor pointer");
     XSMI_CHECK_ARG((beta_dx == 0.f || beta_dx == 1.f) && (beta_dw == 0.f || beta_dw == 1.f), "xsmi_conv2d_bwd: beta must be 0 or 1");
-    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_DW_ASYNC)) == 0, "xsmi_conv2d_bwd: unknown flags 0x%x", flags);
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_BF16 | XSMI_CONV_DW_ASYNC | XSMI_CONV_WS_PACKED)) == 0,
+                   "xsmi_conv2d_bwd: unknown flags 0x%x", flags);
     const int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
     const size_t data_need = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
     const size_t weight_need = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
@@ -135,7 +136,8 @@ int xsmi_conv2d_bwd(const float *dy, const float *x, const float *w, float *dx, 
     rc = xsmi_conv2d_bwd_weight(dy, x, dw, db, N, C, H, W, K, R, S, sh, sw, pad, beta_dw, kflags, workspace_dw, workspace_dw_bytes);
     if (beside) xsmi::side_end();
     if (rc == XSMI_OK)
-        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, kflags, workspace, workspace_bytes);
+        rc = xsmi_conv2d_bwd_data(dy, w, dx, N, C, H, W, K, R, S, sh, sw, pad, beta_dx, kflags | (flags & XSMI_CONV_WS_PACKED),
+                                  workspace, workspace_bytes);
     const int rj = (beside && !async) || rc ? xsmi::side_join() : XSMI_OK;
     return rc ? rc : rj;
 }

@@ -46,6 +46,9 @@ void prof_end();
         }                                          \
     } while (0)
 
+// internal flag of xsmi_conv2d_fwd / xsmi_conv2d_bwd_data (set by xsmi_conv2d_pack): lay the filter out and return
+#define XSMI_CONV_PACK_ONLY 0x40000000u
+
 #define XSMI_HIP(call)                                                          \
     do {                                                                        \
         hipError_t e_ = (call);                                                 \
@@ -96,7 +99,8 @@ __device__ __forceinline__ uint32_t xcd_contiguous_id(uint32_t lin, uint32_t tot
 }
 
 // tap-major fast path (conv_tap.hip): reduction channels must be a multiple of 32.
-// opts: bit 0 = bf16 MFMA operands, bit 1 = the workspace already holds the packed filter
+// opts: bit 0 = bf16 MFMA operands, bit 1 = the workspace already holds the packed filter, bit 2 = lay the filter
+// out in the workspace and return (no activation pointer is touched)
 bool tap_path_ok(int reduce_channels);
 size_t tap_fwd_ws_bytes(int C, int K, int R, int S);
 size_t tap_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw);

@@ -262,6 +262,7 @@ def sgd_step_all(pairs, lr):
         else:
             sgd_step(param, grad, lr)
     K.axpy_multi(dev_p, dev_g, -float(lr))
+    K.refresh_layouts(dev_p)                      # filters among them: their kernels' layouts, made beside what follows
 
 
 def sgd_step(param, grad, lr):

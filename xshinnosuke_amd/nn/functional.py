@@ -88,15 +88,17 @@ def conv2d(inputs, weight, bias=None, stride=(1, 1), padding=0, out=None, activa
 
     # without gradients a bf16 result may stay in channels-last form for the next bf16 consumer (DeviceArray.channels_last)
     cl = bf16 and not track and on_device
+    # a tracked forward on a device-resident filter is a training step's: the filter's layout is kept between calls
+    keep = track and w_dev is weight.eval
     if out is None:
         y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16,
-                             channels_last=cl)
+                             channels_last=cl, keep_layout=keep)
         out = Tensor(y_dev if on_device else y_dev.numpy().astype(x.dtype, copy=False))
     else:
         dst = out.eval
         if is_device(dst):
             K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', out=dst, neg_mask=neg_mask, bf16=bf16,
-                         channels_last=cl)
+                         channels_last=cl, keep_layout=keep)
         else:
             y_dev = K.conv2d_fwd(x_dev, w_dev, b_dev, stride, padding, relu=activation == 'relu', neg_mask=neg_mask, bf16=bf16)
             out.eval = y_dev.numpy()              # cast to the buffer's dtype on store

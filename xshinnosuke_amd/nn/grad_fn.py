@@ -65,7 +65,7 @@ def Conv2DBackward(outputs):
             # all gradients live on the device: one call; the weight gradient keeps running on the second
             # stream beside the rest of the sweep (the backend joins it before anything else can touch it)
             K.conv2d_bwd(dy, x_dev, w_dev, dx_buf, dw_buf, db_buf.reshape(-1) if want_db else None, stride, pad,
-                         accumulate=True, bf16=bf16, async_dw=True)
+                         accumulate=True, bf16=bf16, async_dw=True, keep_layout=w_dev is weight.eval)
             return
     if want_dw or want_db:
         dw_buf = weight.grad.eval if want_dw else None
@@ -82,7 +82,8 @@ def Conv2DBackward(outputs):
     if inputs.requires_grad:
         dx_buf = inputs.grad.eval
         if is_device(dx_buf):
-            K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, dx=dx_buf, accumulate=True, bf16=bf16)
+            K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, dx=dx_buf, accumulate=True, bf16=bf16,
+                              keep_layout=w_dev is weight.eval)
         else:
             _accumulate(inputs, K.conv2d_bwd_data(dy, w_dev, inputs.shape, stride, pad, bf16=bf16))
 
