@@ -665,19 +665,21 @@ __global__ void __launch_bounds__(256) avgpool_bwd_strided_kernel(const float *_
 }
 
 // ---- small GEMM (dense layer) ----------------------------------------------------
-// 32x32 output tile per 256 threads (each thread 2x2), K in chunks of 128 through LDS: the dense layer's
-// matrices are skinny (a batch of 32 rows), so few workgroups run and each must keep many loads in
-// flight; a chunk is 32 independent loads per thread.  Lanes always run along the contiguous axis of
-// the operand in memory, whichever way it is transposed.  The dense layer of the networks here is a
-// few tens of MFLOP, far below what would justify an MFMA kernel of its own.
+// 32x32 output tile per 256 threads, K in chunks of 128 through LDS: the dense layer's matrices are skinny (a
+// batch of 32 rows), so few workgroups run and each must keep many loads in flight; a chunk is 32 independent
+// loads per thread.  Lanes always run along the contiguous axis of the operand in memory, whichever way it is
+// transposed.  Each of the four waves multiplies a quarter of the chunk (32 values of k: sixteen
+// v_mfma_f32_32x32x2_f32) into its own 32x32 accumulator; the four are added in wave order at the end.
 constexpr int GEMM_KC = 128;
+typedef float gemm_f16v __attribute__((ext_vector_type(16)));
 __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, const float *__restrict__ B,
                                                     const float *__restrict__ bias, float *__restrict__ C, int M, int N,
                                                     int K, int ta, int tb, int chunks_per_split) {
     __shared__ float As[32][GEMM_KC + 1], Bs[GEMM_KC][33];
-    const int tx = threadIdx.x & 15, ty = threadIdx.x >> 4;
+    static_assert(sizeof(As) >= 4 * 1024 * sizeof(float), "the accumulators of four waves are exchanged through As");
+    const int lane = threadIdx.x & 63, wv = threadIdx.x >> 6, l31 = lane & 31, half = lane >> 5;
     const int m0 = blockIdx.y * 32, n0 = blockIdx.x * 32;
-    float acc[2][2] = {{0.f, 0.f}, {0.f, 0.f}};
+    gemm_f16v acc = {0};
     // split z multiplies K range [kbeg, kend) and writes its own M x N slab of C (C is then the partial buffer)
     const int kbeg = blockIdx.z * chunks_per_split * GEMM_KC;
     const int kend = min(K, kbeg + chunks_per_split * GEMM_KC);
@@ -710,19 +712,26 @@ __global__ void __launch_bounds__(256) gemm_kernel(const float *__restrict__ A, 
             if (tb) Bs[i % GEMM_KC][i / GEMM_KC] = rb[u]; else Bs[i >> 5][i & 31] = rb[u];
         }
         __syncthreads();
-#pragma unroll 8
-        for (int kk = 0; kk < GEMM_KC; ++kk) {
-            float a0 = As[ty * 2][kk], a1 = As[ty * 2 + 1][kk];
-            float b0 = Bs[kk][tx * 2], b1 = Bs[kk][tx * 2 + 1];
-            acc[0][0] += a0 * b0; acc[0][1] += a0 * b1; acc[1][0] += a1 * b0; acc[1][1] += a1 * b1;
+        // operand lane l of an MFMA holds row (column) l % 32 at k = l / 32
+#pragma unroll
+        for (int s = 0; s < GEMM_KC / 8; ++s) {
+            const int kk = wv * (GEMM_KC / 4) + 2 * s + half;
+            acc = __builtin_amdgcn_mfma_f32_32x32x2f32(As[l31][kk], Bs[kk][l31], acc, 0, 0, 0);
         }
         __syncthreads();
     }
-    for (int i = 0; i < 2; ++i)
-        for (int j = 0; j < 2; ++j) {
-            int m = m0 + ty * 2 + i, n = n0 + tx * 2 + j;
-            if (m < M && n < N) C[(size_t)m * N + n] = acc[i][j] + (bias ? bias[n] : 0.f);
-        }
+    // register v of lane l holds row 8 * (v / 4) + 4 * (l / 32) + v % 4, column l % 32 of the tile
+    float *red = &As[0][0];
+#pragma unroll
+    for (int v = 0; v < 16; ++v) red[wv * 1024 + v * 64 + lane] = acc[v];
+    __syncthreads();
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        const int e = (int)threadIdx.x + 256 * i, v = e >> 6, l = e & 63;
+        const float sum = ((red[e] + red[1024 + e]) + red[2048 + e]) + red[3072 + e];
+        const int m = m0 + 8 * (v >> 2) + 4 * (l >> 5) + (v & 3), n = n0 + (l & 31);
+        if (m < M && n < N) C[(size_t)m * N + n] = sum + (bias ? bias[n] : 0.f);
+    }
 }
 // C = bias + the K-split partial products, added in ascending split order
 __global__ void __launch_bounds__(256) gemm_reduce_kernel(const float *__restrict__ part, const float *__restrict__ bias,
@@ -1039,11 +1048,14 @@ int xsmi_gemm(const float *A, const float *B, const float *bias, float *C, int M
     XSMI_CHECK_ARG(A && B && C, "xsmi_gemm: null pointer");
     XSMI_CHECK_ARG((double)M * N < 2147483648.0, "xsmi_gemm: outputs of 2^31 elements or more are not supported");
     // A skinny product (a batch of 32 rows) has few 32 x 32 output tiles and a long K: with a workspace, K is
-    // split over enough workgroups to occupy the chip and the partial products are added in a second pass.
+    // split over enough workgroups to occupy the chip and the partial products are added in a second pass.  A
+    // workgroup spends most of a chunk waiting for its loads, so "occupy" means about four workgroups per CU
+    // (256 x 1000 x 512, the ResNet-18 classifier at N=256: one workgroup per CU 56 us, four 21 us).
     const int tiles = ((N + 31) / 32) * ((M + 31) / 32), chunks = (K + GEMM_KC - 1) / GEMM_KC;
+    const int want = 4 * xsmi::cu_count();
     int splits = 1;
-    if (ws && chunks > 1 && tiles < xsmi::cu_count()) {
-        splits = (xsmi::cu_count() + tiles - 1) / tiles;
+    if (ws && chunks > 1 && tiles < want) {
+        splits = (want + tiles - 1) / tiles;
         if (splits > chunks) splits = chunks;
         const size_t fit = ws_bytes / ((size_t)M * N * sizeof(float));
         if ((size_t)splits > fit) splits = (int)fit;
