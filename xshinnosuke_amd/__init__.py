@@ -11,6 +11,7 @@ reference's Tensor / layer / model interface that those ops plug into.
 import numpy as _np
 
 from . import backend  # noqa: F401
+from .backend.graph import StepGraph
 from .core import state as GLOBAL
 from .core.state import no_grad, conv_precision
 from .core.base import Tensor, Parameter
