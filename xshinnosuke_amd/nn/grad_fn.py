@@ -33,6 +33,23 @@ def _accumulate(t, g):
         np.add(dst, g.reshape(dst.shape), out=dst)
 
 
+def _product_into_fresh_grad(t, a, b, trans_a=False, trans_b=False):
+    """t.grad = op(a) @ op(b) written straight into a device gradient whose clear is still pending (nothing to add
+    to, so no temporary and no copy); False when that is not the situation."""
+    dst = t.grad.eval
+    if not (is_device(dst) and is_device(a) and is_device(b) and dst.is_fresh()):
+        return False
+    if any(v.dtype != np.float32 for v in (dst, a, b)) or len(a.shape) != 2 or len(b.shape) != 2:
+        return False
+    m = a.shape[1] if trans_a else a.shape[0]
+    n = b.shape[0] if trans_b else b.shape[1]
+    if dst.size != m * n:
+        return False
+    dst.take_fresh()
+    K.gemm(a, b, trans_a=trans_a, trans_b=trans_b, out=dst)
+    return True
+
+
 def _f32_device(a):
     """Device float32 copy of a host array (or the device array itself)."""
     if is_device(a):
@@ -201,9 +218,11 @@ def MMBackward(outputs):
     x1, x2 = outputs.in_bounds
     g = outputs.grad.eval
     if x1.requires_grad:
-        _accumulate(x1, A.mm_nt(g, x2.eval))
+        if not _product_into_fresh_grad(x1, g, x2.eval, trans_b=True):
+            _accumulate(x1, A.mm_nt(g, x2.eval))
     if x2.requires_grad:
-        _accumulate(x2, A.mm_tn(x1.eval, g))
+        if not _product_into_fresh_grad(x2, x1.eval, g, trans_a=True):
+            _accumulate(x2, A.mm_tn(x1.eval, g))
 
 
 def AddmmBackward(outputs):
@@ -213,9 +232,11 @@ def AddmmBackward(outputs):
     if b is not None and b.requires_grad:
         _accumulate(b, A.sum_leading(g) if b.eval.size != g.size else g)
     if x1.requires_grad:
-        _accumulate(x1, A.mm_nt(g, x2.eval))
+        if not _product_into_fresh_grad(x1, g, x2.eval, trans_b=True):
+            _accumulate(x1, A.mm_nt(g, x2.eval))
     if x2.requires_grad:
-        _accumulate(x2, A.mm_tn(x1.eval, g))
+        if not _product_into_fresh_grad(x2, x1.eval, g, trans_a=True):
+            _accumulate(x2, A.mm_tn(x1.eval, g))
 
 
 def FlattenBackward(outputs):
