@@ -29,9 +29,12 @@ __global__ void __launch_bounds__(256) cl_add_kernel(const bf16x8 *__restrict__ 
     out[i] = r;
 }
 
-// one thread = one output pixel x eight channels; consecutive threads = consecutive channel octets, then pixels
+// one thread = one output pixel x eight channels; consecutive threads = consecutive channel octets, then pixels.
+// K > 0: the window size at compile time, so that the K * K loads of a thread are all issued before the first
+// comparison (with a run-time window each load waits for the comparison loop in front of it).
+template <int K>
 __global__ void __launch_bounds__(256) cl_maxpool_kernel(const bf16x8 *__restrict__ x, bf16x8 *__restrict__ y, int C8, int Wpi,
-                                                          int Hpi, int off, int k, int sh, int sw, int OH, int OW, int Wpo,
+                                                          int Hpi, int off, int k_rt, int sh, int sw, int OH, int OW, int Wpo,
                                                           int Hpo, int ob, uint32_t total, xsmi::FastDiv dC8,
                                                           xsmi::FastDiv dOW, xsmi::FastDiv dOH) {
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -44,15 +47,30 @@ __global__ void __launch_bounds__(256) cl_maxpool_kernel(const bf16x8 *__restric
     float m[8];
 #pragma unroll
     for (int e = 0; e < 8; ++e) m[e] = -INFINITY;
-    for (int r = 0; r < k; ++r)
-        for (int s = 0; s < k; ++s) {
-            const bf16x8 v = src[((size_t)r * Wpi + s) * C8];
+    if (K > 0) {
+        bf16x8 v[K > 0 ? K * K : 1];
+#pragma unroll
+        for (int r = 0; r < K; ++r)
+#pragma unroll
+            for (int s = 0; s < K; ++s) v[r * K + s] = src[((size_t)r * Wpi + s) * C8];
+#pragma unroll
+        for (int t = 0; t < K * K; ++t)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const float f = (float)v[e];
+                const float f = (float)v[t][e];
                 m[e] = f > m[e] ? f : m[e];
             }
-        }
+    } else {
+        for (int r = 0; r < k_rt; ++r)
+            for (int s = 0; s < k_rt; ++s) {
+                const bf16x8 v = src[((size_t)r * Wpi + s) * C8];
+#pragma unroll
+                for (int e = 0; e < 8; ++e) {
+                    const float f = (float)v[e];
+                    m[e] = f > m[e] ? f : m[e];
+                }
+            }
+    }
     bf16x8 o;
 #pragma unroll
     for (int e = 0; e < 8; ++e) o[e] = (__bf16)m[e];
@@ -120,10 +138,16 @@ int xsmi_cl_maxpool2d(const void *x_cl, int x_border, void *y_cl, int y_border, 
     const int C8 = C / 8;
     const size_t total = (size_t)N * OH * OW * C8;
     XSMI_CHECK_ARG(total < ((size_t)1 << 32), "xsmi_cl_maxpool2d: too many outputs");
-    hipLaunchKernelGGL(cl_maxpool_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, xsmi::stream(),
-                       (const bf16x8 *)x_cl, (bf16x8 *)y_cl, C8, W + 2 * x_border, H + 2 * x_border, x_border - pad, k, sh, sw, OH,
-                       OW, OW + 2 * y_border, OH + 2 * y_border, y_border, (uint32_t)total, xsmi::make_fastdiv(C8),
-                       xsmi::make_fastdiv(OW), xsmi::make_fastdiv(OH));
+    const dim3 grid((unsigned)((total + 255) / 256));
+#define XSMI_CL_POOL(KK)                                                                                                     \
+    hipLaunchKernelGGL(cl_maxpool_kernel<KK>, grid, dim3(256), 0, xsmi::stream(), (const bf16x8 *)x_cl, (bf16x8 *)y_cl, C8,    \
+                       W + 2 * x_border, H + 2 * x_border, x_border - pad, k, sh, sw, OH, OW, OW + 2 * y_border,              \
+                       OH + 2 * y_border, y_border, (uint32_t)total, xsmi::make_fastdiv(C8), xsmi::make_fastdiv(OW),          \
+                       xsmi::make_fastdiv(OH))
+    if (k == 3) XSMI_CL_POOL(3);
+    else if (k == 2) XSMI_CL_POOL(2);
+    else XSMI_CL_POOL(0);
+#undef XSMI_CL_POOL
     XSMI_LAUNCH_CHECK("cl_maxpool_kernel");
     return XSMI_OK;
 }
