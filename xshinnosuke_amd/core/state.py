@@ -4,6 +4,8 @@ The reference switches devices by swapping a global array module (``np`` -> CuPy
 xs/core/__global.py:9).  Here ``USE_CUDA`` only records that new parameters
 should be created on the device; each Tensor knows where its own data lives.
 """
+import os as _os
+
 INPUTS = None
 OUTPUTS = None
 GRAPH = None
@@ -16,7 +18,6 @@ CONV_BF16 = False
 # Opt-in (also XSMI_STEP_GRAPH=1 in the environment): fit() on device-resident data records its full-batch training
 # step once as a step graph and replays it for every later full batch (backend/graph.py); a shorter last batch
 # runs launch by launch as before.  No counterpart in the reference.
-import os as _os
 STEP_GRAPH = _os.environ.get("XSMI_STEP_GRAPH", "0") not in ("", "0")
 
 
