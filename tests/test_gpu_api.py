@@ -309,6 +309,7 @@ def test_device_fit_allocates_nothing_in_the_steady_state():
     labels = rng.integers(0, 4, size=96)
     np.random.seed(5)
     xs.GLOBAL.USE_CUDA = True
+    graph_switch, xs.GLOBAL.STEP_GRAPH = xs.GLOBAL.STEP_GRAPH, False      # every step is to be issued launch by launch
     calls = []
     real = capi.lib.call
     try:
@@ -318,6 +319,7 @@ def test_device_fit_allocates_nothing_in_the_steady_state():
     finally:
         capi.lib.call = real
         xs.GLOBAL.USE_CUDA = False
+        xs.GLOBAL.STEP_GRAPH = graph_switch
     steps = [i for i, name in enumerate(calls) if name == "xsmi_axpy_multi"]       # one optimizer step each
     assert len(steps) == 6
     steady = calls[steps[1] + 1:steps[5] + 1]                                       # steps 3..6
