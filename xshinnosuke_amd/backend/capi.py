@@ -281,4 +281,7 @@ def last_kernel_ms():
 
 
 def synchronize():
-    lib.call("xsmi_sync")
+    lib.call("xsmi_sync")                  # joins the second stream and waits for both
+    del _side_hold[:]
+    del _layouts_hold[:]
+    _layouts_pending[0] = False
