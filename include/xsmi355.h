@@ -94,6 +94,16 @@ int xsmi_memcpy_h2d_async(void *dst, const void *pinned_src, size_t bytes);
 int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes);   /* async on the stream */
 int xsmi_memset(void *dst, int byte_value, size_t bytes);        /* async on the stream (a fill kernel) */
 int xsmi_sync(void);
+/* Tuning switches of the kernel selection, by name: "tap_sk" (0: one tile per workgroup only, 1: even split of
+ * the chunks where it pays, 3: even split wherever it applies), "sk_spin_limit" (polls before an even-split
+ * workgroup gives up waiting for a partial tile; the calls that wait for the device then fail with
+ * XSMI_ERR_RUNTIME), "sk_wide" (0: one-dword loads of the activations in the even-split kernel also where 16-byte
+ * loads apply), "tap_stages", "tap_persist",
+ * "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
+ * A caller that changes one must drop every workspace content it counted on (XSMI_CONV_WS_PACKED) and ask for
+ * workspace sizes again.  No counterpart in the reference. */
+int xsmi_set_option(const char *name, long value);
+int xsmi_get_option(const char *name, long *value);
 int xsmi_event_create(void **event);
 int xsmi_event_record(void *event);                               /* on the library stream */
 int xsmi_event_synchronize(void *event);                          /* host waits for the event */

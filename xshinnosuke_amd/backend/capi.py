@@ -55,6 +55,8 @@ SIGNATURES = {
     "xsmi_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "xsmi_memset": (_i, [_vp, _i, _sz]),
     "xsmi_sync": (_i, []),
+    "xsmi_set_option": (_i, [_c.c_char_p, _c.c_long]),
+    "xsmi_get_option": (_i, [_c.c_char_p, _c.POINTER(_c.c_long)]),
     "xsmi_event_create": (_i, [_c.POINTER(_vp)]),
     "xsmi_event_record": (_i, [_vp]),
     "xsmi_event_synchronize": (_i, [_vp]),
@@ -281,7 +283,30 @@ def last_kernel_ms():
 
 
 def synchronize():
-    lib.call("xsmi_sync")                  # joins the second stream and waits for both
-    del _side_hold[:]
-    del _layouts_hold[:]
-    _layouts_pending[0] = False
+    try:
+        lib.call("xsmi_sync")              # joins the second stream and waits for both
+    finally:
+        del _side_hold[:]
+        del _layouts_hold[:]
+        _layouts_pending[0] = False
+
+
+# Kernel-selection switches of the library ("tap_sk", "sk_spin_limit", "tap_persist", ...).  What the host keeps
+# that depends on them (workspace sizes, filter layouts made ahead) is dropped by the listeners.
+_option_listeners = []
+
+
+def set_option(name, value):
+    """Set a tuning switch of the library; returns the previous value."""
+    old = get_option(name)
+    synchronize()
+    lib.call("xsmi_set_option", name.encode(), int(value))
+    for fn in _option_listeners:
+        fn()
+    return old
+
+
+def get_option(name):
+    v = ctypes.c_long()
+    lib.call("xsmi_get_option", name.encode(), ctypes.byref(v))
+    return v.value

@@ -97,6 +97,17 @@ def _layout_for(w, pass_, dims):
 _plan = {"sig": None, "jobs": None}
 
 
+def _options_changed():
+    """A kernel-selection switch of the library changed: sizes and layouts made for the old selection are void."""
+    _NEED.clear()
+    for entries in list(_LAYOUTS.values()):
+        entries.clear()
+    _plan["sig"] = _plan["jobs"] = None
+
+
+capi._option_listeners.append(_options_changed)
+
+
 def refresh_layouts(arrays):
     """After an update of ``arrays`` (an optimizer step): every filter among them whose layouts were used since the
     last refresh gets them made again, on the second stream, in one call; layouts that were not used are dropped."""

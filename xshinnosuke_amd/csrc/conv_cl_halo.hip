@@ -510,8 +510,7 @@ namespace xsmi {
 // 3 x 3, stride 1, pad 1, channels a multiple of 32, a zero border of exactly one pixel, rows of at most 61 pixels,
 // and feature maps large enough that the border positions are a small part of the work.
 bool halo_fwd_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int border) {
-    static int env = -1;
-    if (env < 0) { const char *e = getenv("XSMI_CL_HALO"); env = e ? atoi(e) : 1; }
+    const int env = (int)xsmi::option(xsmi::OPT_CL_HALO);
     if (!env) return false;
     if (!(R == 3 && S == 3 && sh == 1 && sw == 1 && pad == 1 && border == 1)) return false;
     if (C % 32 != 0 || K % 8 != 0) return false;
@@ -523,9 +522,7 @@ bool halo_fwd_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int p
 // 7 rows and at most 8 columns, stride 2 both ways, 8, 16, 32 or 64 filters, at most 128 output columns
 // and an input row of at most 115 pixel pairs, channels-last output with a border of one.
 bool stem_cl_ok(int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int OW, int y_border) {
-    static int env = -1;
-    if (env < 0) { const char *e = getenv("XSMI_CL_STEM"); env = e ? atoi(e) : 1; }
-    if (!env) return false;
+    if (!xsmi::option(xsmi::OPT_CL_STEM)) return false;
     const int Wp = W + 2 * pad;
     return C <= 4 && R == 7 && S <= 8 && sh == 2 && sw == 2 && (K == 8 || K == 16 || K == 32 || K == 64) && y_border == 1 &&
            Wp % 2 == 0 &&

@@ -338,7 +338,7 @@ static FwdPath fwd_path(int N, int C, int H, int W, int K, int R, int S, int sh,
     if (!bf16 && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad) &&
         workspace_bytes >= xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad))
         return FwdPath::FirstLayer;
-    if (!bf16 && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * OH * OW, K, R, S, sh, sw) &&
+    if (!bf16 && !(flags & XSMI_CONV_WS_ONLY) && xsmi::sk_path_ok(C, K) && xsmi::sk_fwd_pays(N * OH * OW, K, R, S, sh, sw) &&
         workspace_bytes >= xsmi::sk_fwd_ws_bytes(C, K, R, S))
         return FwdPath::EvenSplit;
     if (xsmi::tap_path_ok(C)) return FwdPath::Tap;
@@ -364,7 +364,7 @@ int xsmi_conv2d_fwd(const float *x, const float *w, const float *bias, float *y,
     int rc = check_conv("xsmi_conv2d_fwd", N, C, H, W, K, R, S, sh, sw, pad, &g);
     if (rc) return rc;
     XSMI_CHECK_ARG(x && w && y, "xsmi_conv2d_fwd: null tensor pointer");
-    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED | XSMI_CONV_PACK_ONLY)) == 0,
+    XSMI_CHECK_ARG((flags & ~(XSMI_CONV_RELU | XSMI_CONV_BF16 | XSMI_CONV_WS_PACKED | XSMI_CONV_PACK_ONLY | XSMI_CONV_WS_ONLY)) == 0,
                    "xsmi_conv2d_fwd: unknown flags 0x%x", flags);
     const int J = C * R * S;
     const size_t need = xsmi::conv_fwd_ws_bytes(C, K, R, S);

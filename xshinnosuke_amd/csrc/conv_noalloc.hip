@@ -60,7 +60,8 @@ int xsmi_conv2d_fwd_noalloc(const float *x, const float *w, const float *bias, f
     XSMI_HIP(hipGetDevice(&device));
     XSMI_CHECK_ARG(device >= 0 && device < MAX_DEVICES && g_scratch[device] != nullptr,
                    "xsmi_conv2d_fwd_noalloc: the current device %d is not the one xsmi_init bound", device);
-    return xsmi_conv2d_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, flags, g_scratch[device], SCRATCH_BYTES);
+    return xsmi_conv2d_fwd(x, w, bias, y, neg_mask, N, C, H, W, K, R, S, sh, sw, pad, flags | XSMI_CONV_WS_ONLY, g_scratch[device],
+                           SCRATCH_BYTES);
 }
 
 }  // extern "C"

@@ -1345,13 +1345,7 @@ void launch_tap(hipStream_t st, TapMulti mp, int opts) {
         else hipLaunchKernelGGL((tap_bf16_tile_kernel<2, 2>), dim3(first), dim3(256), 0, st, m2);
         return;
     }
-    static int stages_env = -1, persist = -1;
-    if (stages_env < 0) {
-        const char *e = getenv("XSMI_TAP_STAGES");
-        stages_env = e ? atoi(e) : 0;
-        e = getenv("XSMI_TAP_PERSIST");
-        persist = e ? atoi(e) : 1;
-    }
+    const int stages_env = (int)xsmi::option(xsmi::OPT_TAP_STAGES), persist = (int)xsmi::option(xsmi::OPT_TAP_PERSIST);
     // With at most one tile per CU a workgroup runs alone and the two-stage pipeline waits a full load
     // latency per chunk; a third stage in flight covers it (measured 104 -> 91 us on 32x512x7x7, 3x3).
     const int stages = stages_env ? stages_env : (tiles <= (uint32_t)xsmi::cu_count() ? 3 : TAP_STAGES);

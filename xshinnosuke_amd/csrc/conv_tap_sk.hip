@@ -1,31 +1,22 @@
-// Tap-major implicit-GEMM convolution (forward and backward-data), fp32 MFMA, second generation:
-// 64 x 64 outputs per wave and an even split of the launch's work over the resident workgroups.
+// Tap-major implicit-GEMM convolution (forward and backward-data), fp32 MFMA, with an even split of the launch's
+// work over the resident workgroups.
 //
-// Same reduction order and data path as conv_tap.hip (reduction index = (tap, channel); global -> LDS
-// directly; zero border through the buffer range check), with two changes that the measurements of
-// that kernel asked for:
+// Same reduction order and data path as conv_tap.hip (reduction index = (tap, channel); global -> LDS directly; zero
+// border through the buffer range check; 64 x 64 outputs per workgroup, 32 x 32 per wave, 32-channel chunks), but
+// work is counted in chunks (one tap x 32 channels of one tile): the launch has exactly as many workgroups as fit on
+// the chip at once and workgroup g takes the contiguous range [g * U / G, (g + 1) * U / G) of the U chunks of all
+// tiles, walking it as one software-pipelined stream.  Every compute unit therefore gets the same amount of matrix
+// work whatever the tile count is (ResNet-18 at N=32 has 1.5 to 6.1 tiles per CU: up to a quarter of the machine
+// idled in the last round of tiles).  A tile whose chunks are split between workgroups is finished by the workgroup
+// that holds its first chunk: the others store their accumulators to the library's partial-tile area and raise a flag,
+// the owner adds them in ascending chunk order and runs the epilogue.  The summation order is a function of the
+// geometry and the grid size only: results are reproducible bit for bit, there are no float atomics.
 //
-//  * A wave owns 64 rows x 64 pixels = 2 x 2 blocks of v_mfma_f32_32x32x2_f32.  One reduction step
-//    feeds four MFMAs from two A and two B registers, so LDS reads, global -> LDS loads, address
-//    arithmetic and workgroup barriers per MFMA are half of what the 32 x 32 wave tile needs.
-//    Workgroup tile: 128 rows x 128 pixels (2 x 2 waves), or 64 rows x 256 pixels when the layer has
-//    at most 64 rows.
-//
-//  * Work is counted in chunks (one tap x KC channels of one tile).  The launch has exactly as many
-//    workgroups as fit on the chip at once and workgroup g takes the contiguous range
-//    [g * U / G, (g + 1) * U / G) of the U chunks of all tiles, walking it as one software-pipelined
-//    stream.  Every compute unit therefore gets the same amount of matrix work whatever the tile
-//    count is (ResNet-18 at N=32 has 1.5 to 6.1 tiles of the old size per CU: up to a quarter of the
-//    machine idled in the last round of tiles).  A tile whose chunks are split between workgroups is
-//    finished by the workgroup that holds its first chunk: the others store their 64 x 64 x 4
-//    accumulators to the workspace and raise a flag, the owner adds them in ascending chunk order and
-//    runs the epilogue.  The summation order is a function of the geometry and the grid size only:
-//    results are reproducible bit for bit, there are no float atomics.
-//
-// Forward progress: a workgroup waits only for workgroups with a higher logical id, and each of those
-// stores its partial tile right after its first (at most one tile long) segment, before it can wait
-// for anything itself.  Workgroups start in id order, so whatever is resident either finishes or
-// waits for something that has already started.  The wait is bounded all the same (spin_limit).
+// Forward progress: a workgroup waits only for workgroups with a higher logical id, and each of those stores its
+// partial tile right after its first (at most one tile long) segment, before it can wait for anything itself.
+// Workgroups start in id order, so whatever is resident either finishes or waits for something that has already
+// started.  The wait is bounded all the same (spin_limit); when it runs out the workgroup sets the library's device
+// error word and stores nothing more, and the host reports the launch as failed at its next check.
 #include "xsmi_internal.h"
 #include <stdlib.h>
 #include <string.h>
@@ -37,8 +28,8 @@ namespace {
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
 constexpr int SK_MAX_CLASSES = 4;
-constexpr int SK_MAX_GRID = 1024;           // upper bound of resident workgroups the workspace is sized for
-constexpr int SK_MAX_GRID_BIG = 768;        // ... of the kernels with 64 x 64 wave tiles (64 KB of partial tile each)
+constexpr int SK_MAX_GRID = 1024;           // upper bound of resident workgroups (flags and partial tiles are sized for it)
+constexpr int SK_ROWS = 64, SK_PIX = 64, SK_KC = 32;      // outputs per workgroup, reduction channels per chunk
 
 // One parameter set: the layer (forward) or one residue class of a strided backward-data pass.
 struct SkClass {
@@ -67,9 +58,10 @@ struct SkParams {
     uint8_t *mask;
     float *part;           // [grid][64 accumulator registers][256 threads]
     uint32_t *flags;       // [grid], zero between launches
-    uint32_t in_bytes, apk_bytes;
+    uint32_t *err;         // set (system scope) when a wait for a partial tile ran out
+    uint32_t in_bytes, apk_bytes, out_bytes, part_bytes;
     uint32_t units;        // chunks of all tiles of all classes
-    uint32_t spin_limit;
+    uint32_t spin_limit;   // polls of a flag before giving up; 0: every wait counts as run out (error-path tests)
     int ncls, rowtiles, accumulate, relu;
 };
 
@@ -87,33 +79,42 @@ __device__ __forceinline__ void static_for(F &&f) {
 
 __device__ __forceinline__ float comp4(const float4 &v, int t) { return t == 0 ? v.x : t == 1 ? v.y : t == 2 ? v.z : v.w; }
 
-__device__ __forceinline__ void agent_store(float *p, float v) {
-    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), __builtin_bit_cast(uint32_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// Buffer accesses with a wave-uniform part of the address in a scalar register.  AGENT: the sc1 bit, i.e. the
+// access goes past the caches that are not coherent across the chip's XCDs (partial tiles are written by one
+// compute unit and read by another).
+constexpr int AGENT = 16;
+template <int AUX = 0>
+__device__ __forceinline__ void buf_store(__amdgpu_buffer_rsrc_t r, float v, uint32_t voff, uint32_t soff) {
+    __builtin_amdgcn_raw_buffer_store_b32(__builtin_bit_cast(int, v), r, (int)voff, (int)soff, AUX);
 }
-__device__ __forceinline__ float agent_load(const float *p) {
-    return __builtin_bit_cast(float, __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+template <int AUX = 0>
+__device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t voff, uint32_t soff) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_raw_buffer_load_b32(r, (int)voff, (int)soff, AUX));
 }
 
-// ROWS x PIX outputs per 256-thread workgroup, KC reduction channels per chunk (a multiple of 16); a wave owns
-// BLK x BLK blocks of 32 x 32 (BLK = 2: the 64 x 64 wave tile described above; BLK = 1: the first-generation
-// kernel's 32 x 32 wave tile and loop body under the same even split of the work, for launches whose tiles are
-// so few that large partial tiles and the final burst of output stores would cost more than they save).
-template <int ROWS, int PIX, int KC, int BLK>
-__global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkParams sp) {
-    constexpr int WRn = ROWS / (32 * BLK), WCn = PIX / (32 * BLK);   // waves along rows / pixels
-    static_assert(WRn * WCn == 4, "four waves");
-    static_assert(BLK == 2 || KC == 32, "the 32 x 32 wave tile's loop body is written for 32-channel chunks");
+// VEC = 1: a B wave-load is one channel x 64 pixels, any geometry.  VEC = 4 (launches of one class only): a B wave-load is four channels x 64 pixels, a lane fetching
+// the 16 bytes of four consecutive pixels of one row (input walked with stride 1, rows a multiple of 4 pixels wide, taps
+// that reach at most one column past a row end: the host checks) -- a quarter of the vector-memory instructions of the
+// one-dword form.  A run that reaches one column past a row end is fetched as it lies, so the slot of the border
+// column holds the neighbouring row's last or first value; the lane overwrites that slot with zero once the load has
+// landed, between the wait for the loads and the workgroup barrier.
+template <int VEC>
+__global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
+    static_assert(VEC == 1 || VEC == 4, "B loads of one or four dwords per lane");
+    constexpr int ROWS = SK_ROWS, PIX = SK_PIX, KC = SK_KC;
+    constexpr int WCn = PIX / 32;                    // waves along pixels (2 x 2 waves of 32 x 32)
     constexpr int RT = ROWS / 64, PT = PIX / 64;     // 64-row / 64-pixel blocks of the tile (units of one wave-load)
     constexpr int QUADS = KC / 4;                    // 16-byte channel groups of a chunk
-    constexpr int GROUPS = KC / 8;                   // BLK = 2: a group = 4 reduction steps of both lane halves = 16 MFMAs per wave
+    constexpr int GROUPS = KC / 8;
     constexpr int A_FLOATS = ROWS * KC, B_FLOATS = PIX * KC, STAGE_FLOATS = A_FLOATS + B_FLOATS;
     constexpr int NA = QUADS * RT / 4;               // A wave-loads (64 rows x 16 bytes) per wave and chunk
     constexpr int NB = KC * PT / 4;                  // B wave-loads (64 pixels of one channel) per wave and chunk
-    constexpr int NI = NB + NA + 2;                  // issue items per chunk: prepare, B loads, A loads, advance
-    constexpr int NOUT = BLK * BLK;                  // accumulator blocks a lane holds of the output tile
-    static_assert(NA >= 1 && (BLK == 1 || NI <= 12 + 16 * (GROUPS - 1)), "the issue items must fit the slots of one chunk");
+    constexpr int NBW = NB / VEC;                    // ... as VEC-wide loads
+    constexpr int NI = NBW + NA + 2;                 // issue items per chunk: prepare, B loads, A loads, advance
+    static_assert(NB == 8 && NA == 2 && NI <= 12, "64 x 64 tile, 32-channel chunks: the issue items fit the slots of one chunk");
     __shared__ __attribute__((aligned(16))) float smem[2][STAGE_FLOATS];
-    __shared__ float s_bias[2][ROWS];
+    __shared__ __attribute__((aligned(16))) float s_bias[2][ROWS];
+    __shared__ uint32_t s_fail;                        // a wait of this workgroup ran out: its tiles are not stored
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -127,6 +128,7 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(sp.in, sp.in_bytes);
     const xsmi::xsmi_int32x4 rap = xsmi::make_rsrc(sp.apk, sp.apk_bytes);
     const uint32_t lds0 = (uint32_t)(uintptr_t)&smem[0][0];
+    if (t == 0) s_fail = 0;                            // published by the prologue's barrier
 
     // ------------------------------------------------------------------ issue side
     // position of the next chunk to load: unit iu; inside a tile (r, s, cc) and the packed-filter offset
@@ -140,12 +142,15 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     int iyb = 0, ixb = 0, nbase = 0;
     bool live = false;
     bool prep_stale = true;                            // the pixel offset must be formed again (new segment)
-    uint32_t ld_asoff = 0, ld_stage = lds0, ld_voff = 0, ld_soff = 0;
+    uint32_t ld_asoff = 0, ld_voff = 0, ld_soff = 0;
+    int ld_fix = 0;                                    // VEC = 4: what the lane does to its run once it has landed (issue_prep)
+    const int csub = VEC == 4 ? lane >> 4 : 0;         // VEC = 4: which of the wave-load's four channels the lane fetches
     const uint32_t a_lane = (uint32_t)lane * 16u;
 
     auto issue_segment = [&]() {                       // set up for the segment that starts at unit iu (iu < u1)
         int ci = 0;
-        while (ci + 1 < sp.ncls && iu >= sp.end_unit[ci]) ++ci;
+        if constexpr (VEC != 4)
+            while (ci + 1 < sp.ncls && iu >= sp.end_unit[ci]) ++ci;
         const SkClass &c = sp.cls[ci];
         const uint32_t ul = iu - c.first_unit;
         const uint32_t tile = xsmi::fdiv(ul, c.dIT);
@@ -162,7 +167,7 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
         r = (int)(tap / (uint32_t)c.TS);
         s = (int)(tap - (uint32_t)r * (uint32_t)c.TS);
         ld_asoff = c.apk_off + (rt * c.iters + ch) * (uint32_t)(ROWS * KC * 4);
-        const int m = (int)mt * PIX + pb * 64 + lane;
+        const int m = VEC == 4 ? (int)mt * PIX + 4 * (lane & 15) : (int)mt * PIX + pb * 64 + lane;
         live = m < c.M;
         iyb = 0; ixb = 0; nbase = 0;
         if (live) {
@@ -172,28 +177,71 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
             int y = (int)q - (int)n * c.OY;
             iyb = y * c.sy + c.dy0;
             ixb = x * c.sx + c.dx0;
-            nbase = (int)n * c.in_n_stride;
+            nbase = (int)n * c.in_n_stride + csub * (int)(c.plane_bytes >> 2);
         }
     };
     auto issue_prep = [&]() {
         ld_soff = (uint32_t)(cc * KC + chan0) * i_plane;
         if (cc != 0 && !prep_stale) return;            // same tap as the previous chunk: same pixel offset
         prep_stale = false;
-        int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
-        bool ok = live && (unsigned)iy < (unsigned)i_IH && (unsigned)ix < (unsigned)i_IW;
-        ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
+        const int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
+        if constexpr (VEC == 4) {
+            // The lane's run is columns ix .. ix + 3 of one input row; ix = -1 and ix + 3 = IW (one column past either
+            // end) are the cases the host admits.  The run is fetched as it lies and the border column's slot is
+            // cleared once it has landed (fix 1: first slot, 2: last slot), except where the run would leave the tensor
+            // at its very beginning or end: there the four columns inside the row are fetched and moved by one place
+            // afterwards (fix 3 / 4: a handful of lanes of the whole launch).
+            int off = nbase + iy * i_IW + ix;
+            int fix = ix < 0 ? 1 : (ix + 4 > i_IW ? 2 : 0);
+            if (fix == 1 && off < 0) { off += 1; fix = 3; }
+            if (fix == 2 && (uint32_t)(off + 4) * 4u > sp.in_bytes) { off -= 1; fix = 4; }
+            const bool ok = live && (unsigned)iy < (unsigned)i_IH;
+            ld_voff = ok ? (uint32_t)(off * 4) : 0x80000000u;
+            ld_fix = ok ? fix : 0;
+        } else {
+            bool ok = live && (unsigned)iy < (unsigned)i_IH && (unsigned)ix < (unsigned)i_IW;
+            ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
+        }
     };
-    auto issue_b = [&](int e) {                        // channel chan0 + e of the chunk, this wave's 64 pixels
-        xsmi::load_lds_b32(rin, ld_stage + (uint32_t)((A_FLOATS + (chan0 + e) * PIX + pb * 64) * 4), ld_voff,
-                           ld_soff + (uint32_t)e * i_plane);
+    // `stage`: byte address of the LDS stage the chunk goes to
+    auto issue_b = [&](int e, uint32_t stage) {
+        if constexpr (VEC == 4)                        // channels chan0 + 4 e .. + 3, the tile's 64 pixels
+            xsmi::load_lds_b128(rin, stage + (uint32_t)((A_FLOATS + (chan0 + 4 * e) * PIX) * 4), ld_voff,
+                                ld_soff + (uint32_t)(4 * e) * i_plane);
+        else                                           // channel chan0 + e of the chunk, this wave's 64 pixels
+            xsmi::load_lds_b32(rin, stage + (uint32_t)((A_FLOATS + (chan0 + e) * PIX + pb * 64) * 4), ld_voff,
+                               ld_soff + (uint32_t)e * i_plane);
     };
-    auto issue_a = [&](int e) {                        // 64 rows of one quad
+    auto issue_a = [&](int e, uint32_t stage) {        // 64 rows of one quad
         const int f = wave * NA + e, q = f / RT, rh = f % RT;
         const uint32_t off = (uint32_t)((q * ROWS + rh * 64) * 16);
-        xsmi::load_lds_b128(rap, ld_stage + off, a_lane + off, ld_asoff);
+        xsmi::load_lds_b128(rap, stage + off, a_lane + off, ld_asoff);
+    };
+    // VEC = 4, after the chunk's loads have landed and before the barrier that publishes them: border columns are
+    // overwritten with zero, moved runs are put in place.  `stage_floats`: float offset of that stage.
+    auto fix_borders = [&](int stage_floats, int fix) {
+        if constexpr (VEC == 4) {
+            asm volatile("" ::: "memory");
+            if (fix != 0) {
+                float *run = &smem[0][0] + stage_floats + A_FLOATS + chan0 * PIX + lane * 4;    // wave-load e: + 4 e PIX
+                if (fix <= 2) {
+                    float *z = run + (fix == 1 ? 0 : 3);
+#pragma unroll
+                    for (int e = 0; e < NBW; ++e) z[4 * e * PIX] = 0.f;
+                } else {
+#pragma unroll
+                    for (int e = 0; e < NBW; ++e) {
+                        float4 *q4 = reinterpret_cast<float4 *>(run + 4 * e * PIX);
+                        const float4 v = *q4;
+                        *q4 = fix == 3 ? make_float4(0.f, v.x, v.y, v.z) : make_float4(v.y, v.z, v.w, 0.f);
+                    }
+                }
+            }
+            xsmi::wait_lgkmcnt0();
+            asm volatile("" ::: "memory");
+        }
     };
     auto issue_advance = [&]() {
-        ld_stage = ld_stage == lds0 ? lds0 + (uint32_t)(STAGE_FLOATS * 4) : lds0;
         if (i_left == 0) return;                       // past the end of the range: dummy chunks, nothing to advance
         ++iu;
         ld_asoff += (uint32_t)(ROWS * KC * 4);
@@ -211,19 +259,21 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
             }
         }
     };
-    auto issue_item = [&](auto ic) {
+    // the stage a chunk is loaded into follows from where the call stands in the unrolled loop (`st_`: 0 or 1)
+    auto issue_item_at = [&](auto ic, auto st_) {
         constexpr int n = decltype(ic)::value;
+        const uint32_t stage = lds0 + (uint32_t)(decltype(st_)::value * STAGE_FLOATS * 4);
         if constexpr (n == 0) issue_prep();
-        else if constexpr (n >= 1 && n <= NB) issue_b(n - 1);
-        else if constexpr (n > NB && n <= NB + NA) issue_a(n - 1 - NB);
-        else if constexpr (n == NB + NA + 1) issue_advance();
+        else if constexpr (n >= 1 && n <= NBW) issue_b(n - 1, stage);
+        else if constexpr (n > NBW && n <= NBW + NA) issue_a(n - 1 - NBW, stage);
+        else if constexpr (n == NBW + NA + 1) issue_advance();
     };
-    auto issue_all = [&]() { static_for<NI>([&](auto ic) { issue_item(ic); }); };
+    auto issue_all_at = [&](auto st_) { static_for<NI>([&](auto ic) { issue_item_at(ic, st_); }); };
 
     // ------------------------------------------------------------------ multiply side
-    // BLK = 2: acc[2 i + j] is block (i, j).  BLK = 1: two accumulators take alternate reduction steps of the one
+    // two accumulators take alternate reduction steps of the wave's one
     // block and are added when a segment ends.
-    constexpr int NACC = BLK == 2 ? 4 : 2;
+    constexpr int NACC = 2;
     floatx16 acc[NACC];
     auto zero_acc = [&]() {
 #pragma unroll
@@ -235,23 +285,11 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     const int h = lane >> 5, l31 = lane & 31;
     const int wr = wave / WCn, wc = wave % WCn;
     // lane half h takes channels (KC/2) h .. of a chunk: quad (KC/8) h + group, channel (KC/2) h + 4 group + step
-    const int a_rd = ((GROUPS * h) * ROWS + wr * (32 * BLK) + l31) * 4;
-    const int b_rd = A_FLOATS + (KC / 2) * h * PIX + wc * (32 * BLK) + l31;
-    // BLK = 2: fragments of one group, two buffers.  BLK = 1: fragments of a whole chunk, two buffers.
-    float4 fa[2][BLK == 2 ? 2 : 4];                    // BLK = 2: [buffer][row block]; BLK = 1: [buffer][quad]
-    float fb[2][BLK == 2 ? 8 : 16];                    // BLK = 2: [buffer][2 step + pixel block]; BLK = 1: [buffer][channel]
-    int rd_off = 0;                                    // float offset of the stage the fragments are read from
-    auto read_item = [&](auto rt_, auto buf_, auto grp_) {          // BLK = 2 only
-        constexpr int n = decltype(rt_)::value, bf = decltype(buf_)::value, gn = decltype(grp_)::value;
-        const float *base = &smem[0][0] + rd_off;
-        if constexpr (n < 2) {
-            fa[bf][n] = *reinterpret_cast<const float4 *>(base + a_rd + (gn * ROWS + 32 * n) * 4);
-        } else {
-            constexpr int st = n - 2;
-            fb[bf][2 * st] = base[b_rd + (4 * gn + st) * PIX];
-            fb[bf][2 * st + 1] = base[b_rd + (4 * gn + st) * PIX + 32];
-        }
-    };
+    const int a_rd = ((GROUPS * h) * ROWS + wr * 32 + l31) * 4;
+    const int b_rd = A_FLOATS + (KC / 2) * h * PIX + wc * 32 + l31;
+    // fragments of a whole chunk, two buffers
+    float4 fa[2][4];                                   // [buffer][quad]
+    float fb[2][16];                                   // [buffer][channel]
 
     // compute-side cursor
     uint32_t cu = u0;
@@ -263,7 +301,8 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     bool flag_pending = false;                         // a partial tile has been stored, its flag not raised yet
     auto compute_segment = [&]() {
         int ci = 0;
-        while (ci + 1 < sp.ncls && cu >= sp.end_unit[ci]) ++ci;
+        if constexpr (VEC != 4)
+            while (ci + 1 < sp.ncls && cu >= sp.end_unit[ci]) ++ci;
         const SkClass &c = sp.cls[ci];
         const uint32_t ul = cu - c.first_unit;
         const uint32_t tile = xsmi::fdiv(ul, c.dIT);
@@ -283,47 +322,84 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     };
 
     // accumulator register v of lane l in block (i, j): row 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, pixel 32 j + l % 32
+    // Whole row tiles (all layers whose row count is a multiple of the tile): one byte offset per lane, the row's
+    // displacement in a scalar register, out-of-range pixels through the buffer range check; the bias, ReLU / mask
+    // and accumulate steps are passes over the lane's 16 registers, each behind one uniform branch.  Tensors hold
+    // fewer than 2^29 elements, so 32-bit byte offsets suffice.
     auto store_tile = [&]() {
         const SkClass &c = sp.cls[c_ci];
-        const int lrow = wr * (32 * BLK) + 4 * h;
-        const int rbase = c_rt * ROWS + lrow;
+        const int lrow = wr * 32 + 4 * h;
+        const int m = c_m0 + wc * 32 + l31;
+        const uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
+        const int x = m - (int)q * c.OX;
+        const uint32_t n = xsmi::fdiv(q, c.dOY);
+        const int y = (int)q - (int)n * c.OY;
+        if ((c_rt + 1) * ROWS <= c.rows) {
+            const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc((void *)sp.out, 0, (int)sp.out_bytes, 0x00020000);
+            const __amdgpu_buffer_rsrc_t rmask =
+                __builtin_amdgcn_make_buffer_rsrc((void *)sp.mask, 0, sp.mask ? (int)(sp.out_bytes >> 2) : 0, 0x00020000);
+            const uint32_t os_k4 = (uint32_t)c.os_k * 4u;
+            const uint32_t srow = (uint32_t)(c_rt * ROWS) * os_k4;
+            const uint32_t pix = (uint32_t)((int)n * (int)c.os_n + y * c.os_y + x * c.os_x + (int)c.o_base) * 4u + (uint32_t)lrow * os_k4;
+            const uint32_t voff = m < c.M ? pix : 0x80000000u;
+            auto row_off = [&](int v) { return srow + (uint32_t)(8 * (v >> 2) + (v & 3)) * os_k4; };
+            floatx16 r = acc[0];
+            if (sp.bias) {
 #pragma unroll
-        for (int j = 0; j < BLK; ++j) {
-            const int m = c_m0 + wc * (32 * BLK) + 32 * j + l31;
-            if (m >= c.M) continue;
-            uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
-            int x = m - (int)q * c.OX;
-            uint32_t n = xsmi::fdiv(q, c.dOY);
-            int y = (int)q - (int)n * c.OY;
-            const long long pix_off = (long long)n * c.os_n + (long long)y * c.os_y + (long long)x * c.os_x + c.o_base;
-#pragma unroll
-            for (int i = 0; i < BLK; ++i)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    const int ro = 32 * i + 8 * (v >> 2) + (v & 3);
-                    if (rbase + ro < c.rows) {
-                        float val = acc[i * BLK + j][v];
-                        if (sp.bias) val += s_bias[bias_buf][lrow + ro];
-                        long long o = pix_off + (long long)(rbase + ro) * c.os_k;
-                        if (sp.relu) {
-                            if (sp.mask) sp.mask[o] = val < 0.f ? 1 : 0;
-                            val = val > 0.f ? val : 0.f;
-                        }
-                        if (sp.accumulate) val += sp.out[o];
-                        sp.out[o] = val;
-                    }
+                for (int q4 = 0; q4 < 4; ++q4) {
+                    const float4 bz = *reinterpret_cast<const float4 *>(&s_bias[bias_buf][lrow + 8 * q4]);
+                    r[4 * q4] += bz.x; r[4 * q4 + 1] += bz.y; r[4 * q4 + 2] += bz.z; r[4 * q4 + 3] += bz.w;
                 }
+            }
+            if (sp.relu) {
+                if (sp.mask) {
+#pragma unroll
+                    for (int v = 0; v < 16; ++v)
+                        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)(r[v] < 0.f ? 1 : 0), rmask, (int)(voff >> 2), (int)(row_off(v) >> 2), 0);
+                }
+#pragma unroll
+                for (int v = 0; v < 16; ++v) r[v] = r[v] > 0.f ? r[v] : 0.f;
+            }
+            if (sp.accumulate) {
+                float old[16];
+#pragma unroll
+                for (int v = 0; v < 16; ++v) old[v] = buf_load(rout, voff, row_off(v));
+#pragma unroll
+                for (int v = 0; v < 16; ++v) r[v] += old[v];
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) buf_store(rout, r[v], voff, row_off(v));
+            return;
+        }
+        // ragged last row tile: every row is tested
+        if (m >= c.M) return;
+        const int rbase = c_rt * ROWS + lrow;
+        const long long pix_off = (long long)n * c.os_n + (long long)y * c.os_y + (long long)x * c.os_x + c.o_base;
+#pragma unroll
+        for (int v = 0; v < 16; ++v) {
+            const int ro = 8 * (v >> 2) + (v & 3);
+            if (rbase + ro < c.rows) {
+                float val = acc[0][v];
+                if (sp.bias) val += s_bias[bias_buf][lrow + ro];
+                long long o = pix_off + (long long)(rbase + ro) * c.os_k;
+                if (sp.relu) {
+                    if (sp.mask) sp.mask[o] = val < 0.f ? 1 : 0;
+                    val = val > 0.f ? val : 0.f;
+                }
+                if (sp.accumulate) val += sp.out[o];
+                sp.out[o] = val;
+            }
         }
     };
+    // the partial tile of workgroup j: register v of thread t at float (j * 16 + v) * 256 + t of the partial-tile area
+    constexpr uint32_t PART_BYTES = 16 * 256 * 4;
     auto end_segment = [&]() {
-        if constexpr (BLK == 1) acc[0] += acc[1];
+        const __amdgpu_buffer_rsrc_t rpart = __builtin_amdgcn_make_buffer_rsrc((void *)sp.part, 0, (int)sp.part_bytes, 0x00020000);
+        acc[0] += acc[1];
         if (!c_head) {
             // not this workgroup's tile: hand the accumulators to the workgroup that holds the tile's first chunk
-            float *dst = sp.part + (size_t)g * (NOUT * 16 * 256) + t;
 #pragma unroll
-            for (int a = 0; a < NOUT; ++a)
-#pragma unroll
-                for (int v = 0; v < 16; ++v) agent_store(dst + (a * 16 + v) * 256, acc[a][v]);
+            for (int v = 0; v < 16; ++v) buf_store<AGENT>(rpart, acc[0][v], (uint32_t)t * 4u, g * PART_BYTES + (uint32_t)v * 1024u);
             if (cu < u1) {
                 // More chunks follow: the next chunk's body waits for all outstanding memory operations of every wave
                 // (vmcnt(0), then the workgroup barrier) before it reads the next stage, which covers these stores;
@@ -342,21 +418,33 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
                 const uint32_t js = (uint32_t)(((uint64_t)j * sp.units) / G);
                 if (js >= c_tile_end) break;
                 if (t == 0) {
+                    // spin_limit 0: every wait counts as run out (the host's way to exercise this path)
                     uint32_t spins = 0;
-                    while (__hip_atomic_load(sp.flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == 0u &&
+                    bool there = false;
+                    while (sp.spin_limit != 0u &&
+                           !(there = __hip_atomic_load(sp.flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) &&
                            ++spins < sp.spin_limit)
                         __builtin_amdgcn_s_sleep(2);
+                    if (!there) {
+                        // Give up: the host finds the word at its next check and reports the launch as failed.  Neither
+                        // this tile nor any later one of the workgroup is stored, and the late partial's flag stays
+                        // raised for the host to clear.
+                        s_fail = 1u;
+                        __hip_atomic_store(sp.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    }
                 }
                 __syncthreads();
-                const float *src = sp.part + (size_t)j * (NOUT * 16 * 256) + t;
+                if (s_fail) return;
+                float part[16];
 #pragma unroll
-                for (int a = 0; a < NOUT; ++a)
+                for (int v = 0; v < 16; ++v) part[v] = buf_load<AGENT>(rpart, (uint32_t)t * 4u, j * PART_BYTES + (uint32_t)v * 1024u);
 #pragma unroll
-                    for (int v = 0; v < 16; ++v) acc[a][v] += agent_load(src + (a * 16 + v) * 256);
+                for (int v = 0; v < 16; ++v) acc[0][v] += part[v];
                 __syncthreads();                       // everybody has read the part before its flag is cleared
                 if (t == 0) __hip_atomic_store(sp.flags + j, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
+        if (s_fail) return;
         store_tile();
     };
     auto chunk_done = [&]() {
@@ -376,64 +464,22 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
     if (total == 0) return;
 #define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
 #define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
-    if constexpr (BLK == 2) {
-        // One group = 16 MFMAs on the fragments in buffer `g & 1`.  Each MFMA is followed in program order by at most
-        // one LDS fragment read of the next group and one issue item of the chunk after next, so that this work enters
-        // the pipes while the matrix unit is busy; sched_barrier pins the order.  In the chunk's last group the first
-        // four MFMAs are followed by the wait for the next chunk's loads and the workgroup barrier: after it every wave
-        // has all fragments of the current chunk in registers, so the current stage is free for the chunk after next,
-        // and the next chunk's first group can be read.
-        auto group = [&](auto gt) {
-            constexpr int gi = decltype(gt)::value;
-            constexpr int cur = gi & 1, nxt = cur ^ 1;
-            constexpr bool last = gi == GROUPS - 1;
-            static_for<16>([&](auto kt) {
-                constexpr int k = decltype(kt)::value;
-                constexpr int st = k >> 2, i = (k >> 1) & 1, j = k & 1;
-                XSMI_MFMA(acc[2 * i + j], comp4(fa[cur][i], st), fb[cur][2 * st + j]);
-                if constexpr (last && k == 3) {
-                    XSMI_PIN();
-                    xsmi::wait_vmcnt<0>();
-                    xsmi::wait_lgkmcnt0();             // this wave's fragment reads of the current stage have returned
-                    xsmi::block_barrier();
-                    rd_off = STAGE_FLOATS - rd_off;
-                    XSMI_PIN();
-                }
-                constexpr int rbase = last ? 4 : 0;
-                if constexpr (k >= rbase && k < rbase + 6) read_item(IC<k - rbase>{}, IC<nxt>{}, IC<(last ? 0 : gi + 1)>{});
-                constexpr int item = last ? k - 4 : 12 + 16 * gi + k;
-                if constexpr (item >= 0 && item < NI) issue_item(IC<item>{});
-                XSMI_PIN();
-            });
-        };
-        // prologue: chunk 0 of the range landed and its first group in registers; of chunk 1 the issue items that the
-        // last group of a loop iteration would have issued (the loop's first groups issue the rest)
-        issue_segment();
-        issue_all();
-        static_for<12>([&](auto ic) { issue_item(ic); });
-        compute_segment();
-        constexpr int EARLY_LOADS = NB + NA < 11 ? NB + NA : 11;     // loads among the items 1..11 of chunk 1
-        xsmi::wait_vmcnt<EARLY_LOADS>();
-        xsmi::block_barrier();
-        static_for<6>([&](auto n) { read_item(n, IC<0>{}, IC<0>{}); });
-        for (uint32_t k = 0; k < total; ++k) {
-            static_for<GROUPS>([&](auto gt) { group(gt); });
-            chunk_done();
-        }
-    } else {
-        // The first-generation loop body: the fragments of two consecutive chunks live in registers.  A chunk is 16
+    {
+        // The loop body: the fragments of two consecutive chunks live in registers.  A chunk is 16
         // MFMAs on the current fragments; after the first four it waits for the next chunk and crosses the barrier
         // (every wave then holds the current chunk in registers, so its stage is free), and every later MFMA is
         // followed by one slice of the remaining work: LDS fragment reads of the next chunk, LDS-direct loads of the
         // chunk after next.
-        static_assert(BLK == 2 || (NB == 8 && NA == 2), "32 x 32 wave tile: 64 x 64 workgroup tile, 32-channel chunks");
+                // Chunk 2 i of the workgroup's range lives in stage 0 and its fragments in register set 0, chunk 2 i + 1 in
+        // stage 1 and set 1: everything that depends on the stage is a constant of the unrolled loop body.
         auto read_chunk = [&](auto buf_) {
             constexpr int bf = decltype(buf_)::value;
-            const float *base = &smem[0][0] + rd_off;
+            const float *base = &smem[0][0] + bf * STAGE_FLOATS;
+            const float *bsrc = base + b_rd;
 #pragma unroll
             for (int q4 = 0; q4 < 4; ++q4) fa[bf][q4] = *reinterpret_cast<const float4 *>(base + a_rd + q4 * ROWS * 4);
 #pragma unroll
-            for (int jj = 0; jj < 16; ++jj) fb[bf][jj] = base[b_rd + jj * PIX];
+            for (int jj = 0; jj < 16; ++jj) fb[bf][jj] = bsrc[jj * PIX];
         };
         auto body = [&](auto buf_) {
             constexpr int cur = decltype(buf_)::value, nxt = cur ^ 1;
@@ -443,31 +489,32 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
             XSMI_MFMA(acc[1], fa[cur][0].w, fb[cur][3]);
             XSMI_PIN();
             xsmi::wait_vmcnt<0>();
+            fix_borders(nxt * STAGE_FLOATS, ld_fix);   // the chunk that has just landed is the one issued last
             xsmi::block_barrier();
-            rd_off = STAGE_FLOATS - rd_off;
             XSMI_PIN();
-            const float *base = &smem[0][0] + rd_off;
+            const float *base = &smem[0][0] + nxt * STAGE_FLOATS;
+            const float *bsrc = base + b_rd;
             XSMI_MFMA(acc[0], fa[cur][1].x, fb[cur][4]);
             fa[nxt][0] = *reinterpret_cast<const float4 *>(base + a_rd);
-            issue_item(IC<0>{});
+            issue_item_at(IC<0>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[1], fa[cur][1].y, fb[cur][5]);
             fa[nxt][1] = *reinterpret_cast<const float4 *>(base + a_rd + ROWS * 4);
-            issue_item(IC<1>{});
+            issue_item_at(IC<1>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[0], fa[cur][1].z, fb[cur][6]);
             fa[nxt][2] = *reinterpret_cast<const float4 *>(base + a_rd + 2 * ROWS * 4);
-            issue_item(IC<2>{});
+            issue_item_at(IC<2>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[1], fa[cur][1].w, fb[cur][7]);
             fa[nxt][3] = *reinterpret_cast<const float4 *>(base + a_rd + 3 * ROWS * 4);
-            issue_item(IC<3>{});
+            issue_item_at(IC<3>{}, buf_);
             XSMI_PIN();
 #define XSMI_SLOT(A, AV, J)                                           \
             XSMI_MFMA(acc[A], AV, fb[cur][J]);                       \
-            fb[nxt][2 * (J - 8)] = base[b_rd + (2 * (J - 8)) * PIX];     \
-            fb[nxt][2 * (J - 8) + 1] = base[b_rd + (2 * (J - 8) + 1) * PIX]; \
-            issue_item(IC<J - 4>{});                                 \
+            fb[nxt][2 * (J - 8)] = bsrc[(2 * (J - 8)) * PIX];            \
+            fb[nxt][2 * (J - 8) + 1] = bsrc[(2 * (J - 8) + 1) * PIX];    \
+            issue_item_at(IC<J - 4>{}, buf_);                        \
             XSMI_PIN();
             XSMI_SLOT(0, fa[cur][2].x, 8)
             XSMI_SLOT(1, fa[cur][2].y, 9)
@@ -481,12 +528,13 @@ __global__ void __launch_bounds__(256, BLK == 2 ? 2 : 4) tap_sk_f32_kernel(SkPar
         };
         // prologue: chunk 0 landed and in registers, chunk 1 in flight
         issue_segment();
-        issue_all();
+        issue_all_at(IC<0>{});
         compute_segment();
         xsmi::wait_vmcnt<0>();
+        fix_borders(0, ld_fix);
         xsmi::block_barrier();
         read_chunk(IC<0>{});
-        issue_all();
+        issue_all_at(IC<1>{});
         for (uint32_t k = 0; k < total; k += 2) {
             body(IC<0>{});
             chunk_done();
@@ -514,11 +562,8 @@ struct SkPackMulti {
     uint32_t first[SK_MAX_CLASSES + 1];
     int njobs;
 };
-__global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ w, SkPackMulti pm, uint32_t *__restrict__ flags,
-                                                       int nflags, int mode, int rows, int CH, int R, int S, int sh, int sw,
-                                                       int rowtiles, int ROWS, int KC) {
-    // the flags of the multiply kernel start at zero (it also leaves them at zero)
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < nflags; i += gridDim.x * 256) flags[i] = 0;
+__global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ w, SkPackMulti pm, int mode, int rows, int CH,
+                                                       int R, int S, int sh, int sw, int rowtiles, int ROWS, int KC) {
     int ji = 0;
     while (ji + 1 < pm.njobs && blockIdx.x >= pm.first[ji + 1]) ++ji;
     const SkPackJob &j = pm.job[ji];
@@ -554,10 +599,8 @@ __global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ 
 // 36 floats of w (mode 0: one contiguous run, read as nine float4; mode 1: four runs of nine), and stores one float4 per
 // tap; the lanes of a wavefront are consecutive rows, so a store instruction writes 1 KB of one tap's block and every
 // byte of w is requested once.
-__global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restrict__ w, float *__restrict__ apk,
-                                                           uint32_t *__restrict__ flags, int nflags, int mode, int rows, int CH,
-                                                           int rowtiles, int ROWS, int KC) {
-    for (int i = blockIdx.x * 256 + threadIdx.x; i < nflags; i += gridDim.x * 256) flags[i] = 0;
+__global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restrict__ w, float *__restrict__ apk, int mode,
+                                                           int rows, int CH, int rowtiles, int ROWS, int KC) {
     const int nch = CH / KC, quads = KC / 4;
     const uint32_t total = (uint32_t)rowtiles * (uint32_t)nch * (uint32_t)quads * (uint32_t)ROWS;
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -599,30 +642,15 @@ __global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restric
     for (int t = 0; t < 9; ++t) dst[(size_t)t * nch * quads * ROWS] = make_float4(v[0][t], v[1][t], v[2][t], v[3][t]);
 }
 
-struct SkShape { int rows_tile, pix_tile, kc, blk; };
-int sk_env() {
-    static int v = -1;
-    if (v < 0) {
-        const char *e = getenv("XSMI_TAP_SK");
-        v = e ? atoi(e) : 1;
-    }
-    return v;
-}
-// 64 x 64 tiles with 32 x 32 per wave by default; XSMI_TAP_SK=2 selects the 64 x 64 wave tile
-// (128 x 128 tiles, or 64 x 256 for layers of at most 64 rows)
-SkShape sk_shape(int rows) {
-    if (sk_env() == 2) {
-        if (rows <= 64) return SkShape{64, 256, 16, 2};
-        return SkShape{128, 128, 32, 2};
-    }
-    return SkShape{64, 64, 32, 1};
-}
+struct SkShape { int rows_tile, pix_tile, kc; };
+int sk_env() { return (int)xsmi::option(xsmi::OPT_TAP_SK); }
+SkShape sk_shape(int) { return SkShape{SK_ROWS, SK_PIX, SK_KC}; }
 
 size_t sk_pack_bytes(int rows, int CH, int taps, const SkShape &sh) {
     return xsmi::align_up((size_t)xsmi::ceil_div(rows, sh.rows_tile) * taps * (CH / sh.kc) * sh.rows_tile * sh.kc * sizeof(float), 256);
 }
-constexpr size_t SK_FLAG_BYTES = (size_t)SK_MAX_GRID * 4;
-constexpr size_t SK_PART_BYTES = (size_t)SK_MAX_GRID_BIG * 64 * 256 * sizeof(float);     // >= SK_MAX_GRID x 16 KB
+static_assert((size_t)SK_MAX_GRID * 4 <= xsmi::SK_SCRATCH_FLAG_BYTES, "one flag per workgroup");
+static_assert((size_t)SK_MAX_GRID * 16 * 256 * sizeof(float) <= xsmi::SK_SCRATCH_PART_BYTES, "one partial tile per workgroup");
 
 // resident workgroups of the kernel variant (occupancy x compute units), cached per variant
 template <typename K>
@@ -638,27 +666,40 @@ int sk_resident(K kernel, int *cache, int cap) {
     return *cache;
 }
 
-int sk_launch(hipStream_t st, SkParams &p, const SkShape &shp) {
-    static int res_a = 0, res_b = 0, res_c = 0;
-    int resident;
-    if (shp.blk == 1) resident = sk_resident(tap_sk_f32_kernel<64, 64, 32, 1>, &res_c, SK_MAX_GRID);
-    else if (shp.rows_tile == 64) resident = sk_resident(tap_sk_f32_kernel<64, 256, 16, 2>, &res_a, SK_MAX_GRID_BIG);
-    else resident = sk_resident(tap_sk_f32_kernel<128, 128, 32, 2>, &res_b, SK_MAX_GRID_BIG);
-    uint32_t gsz = (uint32_t)resident;
-    // Three workgroups per compute unit measured 1-4 % faster than four on the 32 x 32 wave-tile kernel (fewer partial
-    // tiles to exchange, same matrix-pipe occupancy).
-    if (shp.blk == 1 && gsz > 3u * (uint32_t)xsmi::cu_count()) gsz = 3u * (uint32_t)xsmi::cu_count();
+// Wide B loads: a launch of one class that walks its input with stride 1 over rows a multiple of four pixels wide,
+// with taps that reach at most one column past either end of a row.
+bool sk_wide_loads_ok(const SkParams &p) {
+    if (xsmi::option(xsmi::OPT_SK_WIDE) == 0 || p.ncls != 1) return false;
+    if ((((uintptr_t)p.in) & 3) != 0) return false;
+    for (int i = 0; i < p.ncls; ++i) {
+        const SkClass &c = p.cls[i];
+        if (c.sx != 1 || c.OX % 4 != 0 || c.IW < 4) return false;
+        for (int ts = 0; ts < c.TS; ++ts) {
+            const int shift = c.dx0 + ts * c.dstep;
+            if (shift < -1 || shift > c.IW - c.OX + 1) return false;
+        }
+    }
+    return true;
+}
+
+int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
+    static int res_narrow = 0, res_wide = 0;
+    const bool wide = sk_wide_loads_ok(p);
+    uint32_t gsz = (uint32_t)(wide ? sk_resident(tap_sk_f32_kernel<4>, &res_wide, SK_MAX_GRID)
+                                   : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
     if (gsz > p.units) gsz = p.units;                  // every workgroup gets at least one chunk
     if (gsz == 0) return XSMI_OK;
-    static long spin = -1;
-    if (spin < 0) {
-        const char *e = getenv("XSMI_SK_SPIN_LIMIT");
-        spin = e ? atol(e) : (1L << 22);
-    }
-    p.spin_limit = (uint32_t)spin;
-    if (shp.blk == 1) hipLaunchKernelGGL((tap_sk_f32_kernel<64, 64, 32, 1>), dim3(gsz), dim3(256), 0, st, p);
-    else if (shp.rows_tile == 64) hipLaunchKernelGGL((tap_sk_f32_kernel<64, 256, 16, 2>), dim3(gsz), dim3(256), 0, st, p);
-    else hipLaunchKernelGGL((tap_sk_f32_kernel<128, 128, 32, 2>), dim3(gsz), dim3(256), 0, st, p);
+    // the library's partial-tile area of this stream; a wait that ran out in an earlier launch is reported here
+    // (and by every call that waits for the device) instead of starting on flags that may be stale
+    int rc = xsmi::check_device_error("even-split convolution");
+    if (rc) return rc;
+    const xsmi::SkScratch scr = xsmi::sk_scratch();
+    p.part = scr.part; p.flags = scr.flags; p.err = xsmi::device_error_word();
+    p.part_bytes = (uint32_t)xsmi::SK_SCRATCH_PART_BYTES;
+    const long spin = xsmi::option(xsmi::OPT_SK_SPIN_LIMIT);
+    p.spin_limit = spin < 0 ? 0u : spin > 0x7fffffffL ? 0x7fffffffu : (uint32_t)spin;
+    if (wide) hipLaunchKernelGGL(tap_sk_f32_kernel<4>, dim3(gsz), dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(tap_sk_f32_kernel<1>, dim3(gsz), dim3(256), 0, st, p);
     XSMI_LAUNCH_CHECK("tap_sk_f32_kernel");
     return XSMI_OK;
 }
@@ -695,7 +736,7 @@ bool sk_bwd_data_pays(int M, int rows, int R, int S, int sh, int sw) {
 }
 
 size_t sk_fwd_ws_bytes(int C, int K, int R, int S) {
-    return sk_pack_bytes(K, C, R * S, sk_shape(K)) + SK_FLAG_BYTES + SK_PART_BYTES;
+    return sk_pack_bytes(K, C, R * S, sk_shape(K));
 }
 
 size_t sk_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
@@ -703,7 +744,7 @@ size_t sk_bwd_data_ws_bytes(int C, int K, int R, int S, int sh, int sw) {
     size_t total = 0;
     for (int ph = 0; ph < sh; ++ph)
         for (int pw = 0; pw < sw; ++pw) total += sk_pack_bytes(C, K, ceil_div(R, sh) * ceil_div(S, sw), s);
-    return total + SK_FLAG_BYTES + SK_PART_BYTES;
+    return total;
 }
 
 static void sk_fill_class(SkClass &c, const SkShape &shp, int rowtiles) {
@@ -719,12 +760,10 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     const int rowtiles = ceil_div(K, shp.rows_tile);
     const size_t pack = sk_pack_bytes(K, C, R * S, shp);
     float *apk = (float *)workspace;
-    uint32_t *flags = (uint32_t *)((char *)workspace + pack);
-    float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
     if (!(opts & 2) && R == 3 && S == 3 && (((uintptr_t)w) & 15) == 0) {
         const uint32_t total = (uint32_t)rowtiles * (uint32_t)(C / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
-        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, apk, flags, SK_MAX_GRID, 0, K, C,
-                           rowtiles, shp.rows_tile, shp.kc);
+        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, apk, 0, K, C, rowtiles,
+                           shp.rows_tile, shp.kc);
         XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
     } else if (!(opts & 2)) {
         SkPackMulti pm;
@@ -735,8 +774,8 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
         if (nb > 4096) nb = 4096;
         if (nb < 4) nb = 4;
         pm.first[0] = 0; pm.first[1] = nb;
-        hipLaunchKernelGGL(sk_pack_kernel, dim3(nb), dim3(256), 0, st, w, pm, flags, SK_MAX_GRID, 0, K, C, R, S, 1, 1, rowtiles,
-                           shp.rows_tile, shp.kc);
+        hipLaunchKernelGGL(sk_pack_kernel, dim3(nb), dim3(256), 0, st, w, pm, 0, K, C, R, S, 1, 1, rowtiles, shp.rows_tile,
+                           shp.kc);
         XSMI_LAUNCH_CHECK("sk_pack_kernel");
     }
     if (opts & 4) return XSMI_OK;            // bit 2: lay the filter out and stop
@@ -756,8 +795,8 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     p.units = tiles * c.iters;
     p.end_unit[0] = p.units;
     p.in = x; p.apk = apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
-    p.part = part; p.flags = flags;
     p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
+    p.out_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = 1; p.rowtiles = rowtiles; p.accumulate = 0; p.relu = relu;
     prof_begin();
@@ -804,12 +843,10 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
         }
     }
     const size_t pack = off;
-    uint32_t *flags = (uint32_t *)((char *)workspace + pack);
-    float *part = (float *)((char *)workspace + pack + SK_FLAG_BYTES);
     if (!(opts & 2) && R == 3 && S == 3 && sh == 1 && sw == 1 && nplans == 1) {
         const uint32_t total = (uint32_t)rowtiles * (uint32_t)(K / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
-        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, jobs[0].apk, flags, SK_MAX_GRID, 1, C,
-                           K, rowtiles, shp.rows_tile, shp.kc);
+        hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, jobs[0].apk, 1, C, K, rowtiles,
+                           shp.rows_tile, shp.kc);
         XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
     } else if (!(opts & 2)) {
         SkPackMulti pm;
@@ -825,8 +862,8 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
             blocks += nb;
         }
         pm.first[nplans] = blocks;
-        hipLaunchKernelGGL(sk_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, flags, SK_MAX_GRID, 1, C, K, R, S, sh, sw,
-                           rowtiles, shp.rows_tile, shp.kc);
+        hipLaunchKernelGGL(sk_pack_kernel, dim3(blocks), dim3(256), 0, st, w, pm, 1, C, K, R, S, sh, sw, rowtiles, shp.rows_tile,
+                           shp.kc);
         XSMI_LAUNCH_CHECK("sk_pack_kernel");
     }
     if (opts & 4) return XSMI_OK;            // bit 2: lay the filter out and stop
@@ -848,8 +885,8 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
     for (int i = ncls; i < SK_MAX_CLASSES; ++i) p.end_unit[i] = units;
     p.units = units;
     p.in = dy; p.apk = (const float *)workspace; p.bias = nullptr; p.out = dx; p.mask = nullptr;
-    p.part = part; p.flags = flags;
     p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
+    p.out_bytes = (uint32_t)((size_t)N * C * H * W * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = ncls; p.rowtiles = rowtiles; p.accumulate = accumulate; p.relu = 0;
     prof_begin();

@@ -1,6 +1,7 @@
 // Runtime part of the C ABI: device selection, memory, stream, events.
 #include "xsmi_internal.h"
 #include <stdarg.h>
+#include <stdlib.h>
 #include <string.h>
 #include <vector>
 
@@ -21,6 +22,30 @@ bool g_prof_valid = false;
 // wait for the device are refused while it lasts, and hipFree (which waits too) is put off to its end.
 bool g_capturing = false;
 std::vector<void *> g_free_after_capture;
+
+// Tuning switches: the value set through xsmi_set_option, else the environment variable read at first use, else
+// the default.  The order of the rows is xsmi::Option's.
+struct OptionRow {
+    const char *name, *env;
+    long value;
+    bool loaded;
+};
+OptionRow g_options[xsmi::OPT_COUNT] = {
+    {"tap_sk", "XSMI_TAP_SK", 1, false},
+    {"sk_spin_limit", "XSMI_SK_SPIN_LIMIT", 1L << 22, false},
+    {"tap_stages", "XSMI_TAP_STAGES", 0, false},
+    {"tap_persist", "XSMI_TAP_PERSIST", 1, false},
+    {"cl_halo", "XSMI_CL_HALO", 1, false},
+    {"cl_stem", "XSMI_CL_STEM", 1, false},
+    {"sk_wide", "XSMI_SK_WIDE", 1, false},
+};
+
+// Partial tiles and flags of the even-split convolution kernels: one area per stream, owned by the library (a
+// launch's partial tiles are dead when it ends, and launches of one stream run one after the other).
+xsmi::SkScratch g_sk_scratch[2] = {{nullptr, nullptr}, {nullptr, nullptr}};
+// A word in page-locked host memory that kernels write when a bounded wait ran out; the host reads it directly.
+volatile uint32_t *g_dev_error_host = nullptr;
+uint32_t *g_dev_error_dev = nullptr;
 }  // namespace
 
 namespace xsmi {
@@ -54,6 +79,35 @@ bool on_side_stream() { return g_current == g_side; }
 bool ready() { return g_ready; }
 int cu_count() { return g_cus; }
 bool capturing() { return g_capturing; }
+long option(Option o) {
+    OptionRow &r = g_options[o];
+    if (!r.loaded) {
+        const char *e = getenv(r.env);
+        if (e && *e) r.value = atol(e);
+        r.loaded = true;
+    }
+    return r.value;
+}
+SkScratch sk_scratch() { return g_sk_scratch[g_current == g_side ? 1 : 0]; }
+uint32_t *device_error_word() { return g_dev_error_dev; }
+// Non-zero when a kernel has reported a wait that ran out.  Outside a capture the streams are drained, the flags
+// of the even-split kernels are cleared (a late producer may have left one raised) and the word is reset, so the
+// library is usable again after the caller has seen the error.
+int check_device_error(const char *where) {
+    if (!g_dev_error_host || *g_dev_error_host == 0) return XSMI_OK;
+    const uint32_t code = *g_dev_error_host;
+    if (!g_capturing) {
+        (void)hipStreamSynchronize(g_side);
+        (void)hipStreamSynchronize(g_stream);
+        g_side_pending = false;
+        for (int i = 0; i < 2; ++i)
+            if (g_sk_scratch[i].flags) (void)hipMemset(g_sk_scratch[i].flags, 0, SK_SCRATCH_FLAG_BYTES);
+        *g_dev_error_host = 0;
+    }
+    set_error("%s: an even-split convolution kernel gave up waiting for a partial tile (code %u): the output of that "
+              "launch is incomplete; results since then are not valid", where, code);
+    return XSMI_ERR_RUNTIME;
+}
 void prof_begin() {
     if (g_profiling && !g_capturing && g_current == g_stream) (void)hipEventRecord(g_prof0, g_stream);
 }
@@ -123,6 +177,21 @@ int xsmi_init(int device) {
     XSMI_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
     XSMI_HIP(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));
     XSMI_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    for (int i = 0; i < 2; ++i) {
+        void *p = nullptr;
+        XSMI_HIP(hipMalloc(&p, xsmi::SK_SCRATCH_FLAG_BYTES + xsmi::SK_SCRATCH_PART_BYTES));
+        XSMI_HIP(hipMemset(p, 0, xsmi::SK_SCRATCH_FLAG_BYTES));
+        g_sk_scratch[i].flags = (uint32_t *)p;
+        g_sk_scratch[i].part = (float *)((char *)p + xsmi::SK_SCRATCH_FLAG_BYTES);
+    }
+    {
+        void *h = nullptr, *d = nullptr;
+        XSMI_HIP(hipHostMalloc(&h, 64, hipHostMallocMapped));
+        memset(h, 0, 64);
+        XSMI_HIP(hipHostGetDevicePointer(&d, h, 0));
+        g_dev_error_host = (volatile uint32_t *)h;
+        g_dev_error_dev = (uint32_t *)d;
+    }
     g_current = g_stream;
     g_device = device;
     g_cus = prop.multiProcessorCount;
@@ -211,7 +280,7 @@ int xsmi_memcpy_d2h(void *dst, const void *src, size_t bytes) {
     XSMI_CHECK_ARG(dst && src, "xsmi_memcpy_d2h: null pointer");
     XSMI_HIP(hipMemcpyAsync(dst, src, bytes, hipMemcpyDeviceToHost, g_stream));
     XSMI_HIP(hipStreamSynchronize(g_stream));
-    return XSMI_OK;
+    return xsmi::check_device_error("xsmi_memcpy_d2h");
 }
 
 int xsmi_memcpy_d2d(void *dst, const void *src, size_t bytes) {
@@ -241,7 +310,9 @@ int xsmi_memset(void *dst, int byte_value, size_t bytes) {
 
 int xsmi_conv2d_bwd_join(void) {
     XSMI_REQUIRE_INIT();
-    return xsmi::side_join();
+    int rc = xsmi::side_join();
+    if (rc) return rc;
+    return xsmi::check_device_error("xsmi_conv2d_bwd_join");
 }
 
 int xsmi_sync(void) {
@@ -250,7 +321,7 @@ int xsmi_sync(void) {
     int rc = xsmi::side_join();                      // weight gradients still on the second stream
     if (rc) return rc;
     XSMI_HIP(hipStreamSynchronize(g_stream));
-    return XSMI_OK;
+    return xsmi::check_device_error("xsmi_sync");
 }
 
 int xsmi_event_synchronize(void *event) {
@@ -258,7 +329,30 @@ int xsmi_event_synchronize(void *event) {
     XSMI_NOT_WHILE_CAPTURING();
     XSMI_CHECK_ARG(event != nullptr, "xsmi_event_synchronize: null event");
     XSMI_HIP(hipEventSynchronize((hipEvent_t)event));
-    return XSMI_OK;
+    return xsmi::check_device_error("xsmi_event_synchronize");
+}
+
+int xsmi_set_option(const char *name, long value) {
+    XSMI_CHECK_ARG(name != nullptr, "xsmi_set_option: null name");
+    for (int i = 0; i < xsmi::OPT_COUNT; ++i)
+        if (strcmp(name, g_options[i].name) == 0) {
+            g_options[i].value = value;
+            g_options[i].loaded = true;
+            return XSMI_OK;
+        }
+    xsmi::set_error("xsmi_set_option: no option named '%s'", name);
+    return XSMI_ERR_INVALID;
+}
+
+int xsmi_get_option(const char *name, long *value) {
+    XSMI_CHECK_ARG(name != nullptr && value != nullptr, "xsmi_get_option: null argument");
+    for (int i = 0; i < xsmi::OPT_COUNT; ++i)
+        if (strcmp(name, g_options[i].name) == 0) {
+            *value = xsmi::option((xsmi::Option)i);
+            return XSMI_OK;
+        }
+    xsmi::set_error("xsmi_get_option: no option named '%s'", name);
+    return XSMI_ERR_INVALID;
 }
 
 int xsmi_event_create(void **event) {

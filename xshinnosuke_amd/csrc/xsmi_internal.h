@@ -23,6 +23,22 @@ bool on_side_stream();
 bool capturing();            // a step graph is being recorded: nothing runs, nothing may wait for the device
 bool ready();
 int cu_count();
+// Tuning switches (xsmi_set_option / environment variable / default); the order is that of the table in runtime.hip.
+enum Option { OPT_TAP_SK, OPT_SK_SPIN_LIMIT, OPT_TAP_STAGES, OPT_TAP_PERSIST, OPT_CL_HALO, OPT_CL_STEM, OPT_SK_WIDE, OPT_COUNT };
+long option(Option o);
+// Partial tiles and flags of the even-split convolution kernels for the stream that stream() hands out; allocated
+// by xsmi_init, the flags are zero between launches.
+constexpr size_t SK_SCRATCH_FLAG_BYTES = 4096;                          // 1024 workgroups
+constexpr size_t SK_SCRATCH_PART_BYTES = (size_t)1024 * 16 * 256 * 4;   // 1024 workgroups x one 64 x 64 tile of floats
+struct SkScratch {
+    uint32_t *flags;
+    float *part;
+};
+SkScratch sk_scratch();
+// Device address of the word a kernel sets (system scope) when a bounded wait ran out, and the host-side check:
+// XSMI_OK, or XSMI_ERR_RUNTIME with the message set (and, outside a capture, the library reset for further use).
+uint32_t *device_error_word();
+int check_device_error(const char *where);
 // conv_noalloc.hip: resolves the device address of the static scratch array for `device` (the current device)
 int noalloc_setup(int device);
 // With xsmi_profiling(1) every op brackets its main kernel(s) with two events on
@@ -48,6 +64,9 @@ void prof_end();
 
 // internal flag of xsmi_conv2d_fwd / xsmi_conv2d_bwd_data (set by xsmi_conv2d_pack): lay the filter out and return
 #define XSMI_CONV_PACK_ONLY 0x40000000u
+// internal flag of xsmi_conv2d_fwd (set by xsmi_conv2d_fwd_noalloc): stay on the kernels whose scratch is the
+// workspace alone (the even-split kernels exchange partial tiles through memory that xsmi_init allocated)
+#define XSMI_CONV_WS_ONLY 0x20000000u
 
 #define XSMI_HIP(call)                                                          \
     do {                                                                        \
