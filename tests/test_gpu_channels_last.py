@@ -40,6 +40,8 @@ def _inputs(rng, n, c, h, k, r):
     (3, 3, 37, 32, 7, 2, 3, False),          # first-layer kernel: odd output height (a last item of one row), 32 filters
     (1, 1, 224, 64, 7, 2, 3, True),          # ... one channel, the full 112-column row
     (2, 4, 30, 8, 7, 2, 3, True),            # ... four channels, eight filters
+    (1, 3, 300, 16, 3, 1, 1, False),         # rows of 300 pixels: converted back to float32 in two segments
+    (1, 32, 256, 8, 1, 1, 0, True),          # ... 256 pixels, one more than a segment holds
 ])
 def test_channels_last_output_is_the_plain_result_rounded_to_bf16(gpu, n, c, h, k, r, stride, pad, relu):
     K = gpu.kernels

@@ -153,3 +153,39 @@ def test_refresh_reuses_its_job_table_and_drops_layouts_nobody_used(recorder):
     capi.join_side()
     gc.collect()
     assert len(K._LAYOUTS) == blocks - 1
+
+
+def test_a_replay_after_an_eager_filter_update_lays_the_recorded_filters_out_again(recorder):
+    """eager, eager, capture, replay, eager step on a short batch (other geometry), replay: the recording reads its
+    filters in layouts made at the previous step's end, and the eager step in between changed the filter without
+    renewing the full-batch layouts."""
+    w = dev.empty((64, 64, 3, 3))
+    full, short = [16, 64, 56, 56, 64, 3, 3, 1, 1, 1], [6, 64, 56, 56, 64, 3, 3, 1, 1, 1]
+
+    def step(dims):
+        entry, current = K._layout_for(w, 0, dims)    # what a training forward does
+        w.ptr                                         # the optimizer step writes the filter
+        K.refresh_layouts([w])
+        return current
+
+    assert step(full) is False                        # first step lays the filter out itself
+    assert step(full) is True                         # second finds the layout made ahead
+    graph = StepGraph()
+    with graph.capture():
+        assert step(full) is True                     # recorded as already laid out
+    packs = recorder.calls.count("xsmi_conv2d_pack")
+    graph.replay()
+    graph.replay()
+    assert recorder.calls.count("xsmi_conv2d_pack") == packs      # nothing touched the filter between replays
+    # a replay changes the filter without Python seeing it: no layout made before it counts as current for eager code
+    assert K._layout_for(w, 0, full)[1] is False
+    assert step(short) is False                       # the eager step on the short last batch
+    recorder.calls.clear()
+    graph.replay()
+    assert recorder.calls == ["xsmi_conv2d_pack", "xsmi_graph_launch"]          # laid out again, then launched
+    jobs = ctypes.cast(graph._layout_jobs[0], ctypes.POINTER(capi.PackJob))
+    assert graph._layout_jobs[1] == 1 and jobs[0].N == 16 and jobs[0].w == w.address()
+    recorder.calls.clear()
+    graph.replay()
+    assert recorder.calls == ["xsmi_graph_launch"]
+    graph.close()

@@ -16,6 +16,7 @@ _POOL_BYTES = [0]
 _POOL_LIMIT = 64 << 30
 _CAPTURE = [None]     # the StepGraph whose step is being recorded (backend/graph.py), else None
 _EPOCH = [0]          # moves whenever recorded work may have changed device memory behind Python's back
+_REPLAYS = [0]          # step-graph replays so far: each may have changed parameters without Python taking their address
 
 
 def _round_size(nbytes):

@@ -20,7 +20,11 @@ What the recording freezes, and what the caller therefore has to keep true:
     scalars, shapes) is part of the graph; state that only Python advances (an optimizer's iteration counter)
     does not move on a replay;
   * device memory handed out while recording stays with the graph, and arrays that existed before and were
-    used inside stay alive with it, until ``close()``.
+    used inside stay alive with it, until ``close()``;
+  * a recorded training step reads its convolution filters in the layouts that the previous step's end left in
+    per-filter workspaces, and renews them at its own end.  Code that changes a filter between two replays (an
+    eager step on a short last batch, a loaded checkpoint, a host write) would leave them stale: ``replay`` notices
+    that a filter's address has been handed out since and lays the filters out again before it launches.
 """
 import contextlib
 import ctypes
@@ -37,6 +41,8 @@ class StepGraph:
         self._refs = {}           # id -> pre-existing block that recorded launches read or write
         self._closed = False
         self.replays = 0
+        self._layout_jobs = None  # (job table, count, filters) of the layouts the recording reads as already made
+        self._filter_states = None
 
     @contextlib.contextmanager
     def capture(self):
@@ -72,13 +78,29 @@ class StepGraph:
             self._exec = handle if handle.value else None
             if self._exec is None:
                 self.close()
+            elif self._layout_jobs is not None:
+                self._filter_states = [v.state() for v in self._layout_jobs[2]]
+
+    def note_layout_jobs(self, jobs, count, filters):
+        """Called by the filter-layout bookkeeping while this graph records: the layouts made at the recorded step's
+        end are the ones its next replay starts from."""
+        self._layout_jobs = (jobs, count, list(filters))
 
     def replay(self):
         if self._exec is None:
             raise XsmiError("this step graph holds no recording")
+        if self._layout_jobs is not None:
+            jobs, count, filters = self._layout_jobs
+            if [v.state() for v in filters] != self._filter_states:
+                # a filter was touched outside the graph since the layouts were made: make them again (second
+                # stream; the launch below waits for it)
+                lib.call("xsmi_conv2d_pack", count, ctypes.cast(jobs, ctypes.c_void_p))
         lib.call("xsmi_graph_launch", self._exec)
         _array._EPOCH[0] += 1                # parameters may have changed without Python taking their address
+        _array._REPLAYS[0] += 1
         self.replays += 1
+        if self._layout_jobs is not None:
+            self._filter_states = [v.state() for v in self._layout_jobs[2]]
 
     def close(self):
         """Release the executable graph and return the graph's memory to the common pool."""
@@ -94,6 +116,7 @@ class StepGraph:
                 _array._POOL_BYTES[0] += size
         self._pool.clear()
         self._refs.clear()
+        self._layout_jobs = None
 
     def __del__(self):
         try:

@@ -65,12 +65,18 @@ _PREPACK = os.environ.get("XSMI_PREPACK", "1") not in ("", "0")
 _LAYOUTS = weakref.WeakKeyDictionary()        # filter's memory block -> {(pass, dims): _Layout}
 
 
+def _filter_key(w):
+    """What a layout of filter ``w`` is valid for: the filter's hand-out count, and the count of step-graph replays
+    (a replay changes parameters without Python taking their address)."""
+    return (w.state(), _array._REPLAYS[0])
+
+
 class _Layout:
     __slots__ = ("ws", "key", "used", "ahead")
 
     def __init__(self):
         self.ws = Workspace()
-        self.key = None       # DeviceArray.state() of the filter when the workspace's layout was made
+        self.key = None       # _filter_key of the filter when the workspace's layout was made
         self.used = False     # a convolution ran in this workspace since the last refresh
         self.ahead = True     # False once xsmi_conv2d_pack reported that this geometry has nothing to lay out ahead
 
@@ -91,7 +97,7 @@ def _layout_for(w, pass_, dims):
     entry.used = True
     if capi._layouts_pending[0]:                  # the workspace may still be written on the second stream
         capi.join_side()
-    return entry, entry.key is not None and entry.key == w.state()
+    return entry, entry.key is not None and entry.key == _filter_key(w)
 
 
 _plan = {"sig": None, "jobs": None}
@@ -140,10 +146,15 @@ def refresh_layouts(arrays):
         _plan["sig"], _plan["jobs"] = sig, jobs
     jobs = _plan["jobs"]
     lib.call("xsmi_conv2d_pack", len(todo), ctypes.cast(jobs, ctypes.c_void_p))
+    if _array._CAPTURE[0] is not None:
+        # The recorded step reads these workspaces as already laid out and lays them out again at its end; whoever
+        # changes a filter between two replays leaves them stale, so the graph keeps the jobs to redo them first.
+        _array._CAPTURE[0].note_layout_jobs(jobs, len(todo), [v for v, _, _ in todo])
+        _plan["sig"] = _plan["jobs"] = None       # the table now belongs to the graph
     held = []
     for job, (v, e, _) in zip(jobs, todo):
         if job.packed:
-            e.key = v.state()
+            e.key = _filter_key(v)
             held.append((v, e.ws))
         else:
             e.ahead = False
@@ -207,7 +218,7 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
     lib.call("xsmi_conv2d_fwd", x.cptr, wptr, bias.cptr if bias is not None else None, out.cptr,
              neg_mask.cptr if neg_mask is not None else None, *dims, flags, ws, ws_bytes)
     if layout is not None and not packed:
-        layout.key = w.state()                    # the call has laid the present filter out in this workspace
+        layout.key = _filter_key(w)               # the call has laid the present filter out in this workspace
     return out
 
 
@@ -245,7 +256,7 @@ def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=Fa
     lib.call("xsmi_conv2d_bwd_data", dy.cptr, wptr, dx.cptr, *dims, beta,
              (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0), ws, ws_bytes)
     if layout is not None and not packed:
-        layout.key = w.state()
+        layout.key = _filter_key(w)
     return dx
 
 
@@ -304,7 +315,7 @@ def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False
     lib.call("xsmi_conv2d_bwd", dy.cptr, x.cptr, wptr, dx.cptr, dw.cptr, db.cptr if db is not None else None, *dims,
              beta_dx, beta_dw, flags, ws, ws_bytes, ws_dw, ws_dw_bytes)
     if layout is not None and not packed:
-        layout.key = w.state()
+        layout.key = _filter_key(w)
     if async_dw:
         capi.hold_side(dy, x, dw, db)
     return dx, dw, db

@@ -77,21 +77,25 @@ __global__ void __launch_bounds__(256) cl_maxpool_kernel(const bf16x8 *__restric
     y[(((size_t)n * Hpo + oy + ob) * Wpo + ox + ob) * C8 + c8] = o;
 }
 
-// A workgroup converts one image row (W pixels) of 64 channels through an LDS tile [64][W | 1] of floats: reading,
-// eight threads cover a pixel's 64 channels (128 contiguous bytes); writing, a wave writes runs of one channel's row.
-__global__ void __launch_bounds__(256) cl_to_nchw_kernel(const bf16x8 *__restrict__ x, float *__restrict__ y, int C, int H, int W,
-                                                          int b, int cgroups) {
-    extern __shared__ float tile[];                   // [64][W | 1]
-    const int ldw = W | 1;
+// A workgroup converts one segment (at most 255 pixels) of an image row for 64 channels through an LDS tile
+// [64][seg | 1] of floats: reading, eight threads cover a pixel's 64 channels (128 contiguous bytes); writing, a wave
+// writes runs of one channel's row.
+__global__ void __launch_bounds__(256) cl_to_nchw_kernel(const bf16x8 *__restrict__ x, float *__restrict__ y, int C, int H, int Wfull,
+                                                          int b, int cgroups, int seg, int segs) {
+    extern __shared__ float tile[];                   // [64][seg | 1]
+    const int ldw = seg | 1;
     const int t = threadIdx.x;
     const int cg = (int)(blockIdx.x % (uint32_t)cgroups);
-    const int rowid = (int)(blockIdx.x / (uint32_t)cgroups);       // n * H + h
+    const int part = (int)((blockIdx.x / (uint32_t)cgroups) % (uint32_t)segs);
+    const int rowid = (int)(blockIdx.x / (uint32_t)(cgroups * segs));       // n * H + h
     const int h = rowid % H, n = rowid / H;
-    const int Wp = W + 2 * b, Hp = H + 2 * b, C8 = C / 8;
+    const int w0 = part * seg;
+    const int W = Wfull - w0 < seg ? Wfull - w0 : seg;            // pixels of this segment
+    const int Wp = Wfull + 2 * b, Hp = H + 2 * b, C8 = C / 8;
     const int c0 = cg * 64;
     const int oct = t & 7;                             // octet of the 64-channel group
     const bool oct_ok = c0 + oct * 8 < C;
-    const bf16x8 *row = x + (((size_t)n * Hp + h + b) * Wp + b) * C8 + (c0 >> 3) + oct;
+    const bf16x8 *row = x + (((size_t)n * Hp + h + b) * Wp + b + w0) * C8 + (c0 >> 3) + oct;
     for (int px = t >> 3; px < W; px += 32) {
         if (oct_ok) {
             const bf16x8 v = row[(size_t)px * C8];
@@ -101,10 +105,10 @@ __global__ void __launch_bounds__(256) cl_to_nchw_kernel(const bf16x8 *__restric
     }
     __syncthreads();
     const int nch = C - c0 < 64 ? C - c0 : 64;
-    float *dst = y + (((size_t)n * C + c0) * H + h) * W;
+    float *dst = y + (((size_t)n * C + c0) * H + h) * Wfull + w0;
     for (int i = t; i < nch * W; i += 256) {
         const int c = i / W, px = i - c * W;
-        dst[(size_t)c * H * W + px] = tile[c * ldw + px];
+        dst[(size_t)c * H * Wfull + px] = tile[c * ldw + px];
     }
 }
 
@@ -158,13 +162,14 @@ int xsmi_cl_to_nchw(const void *x_cl, int border, float *y, int N, int C, int H,
     XSMI_CHECK_ARG(N > 0 && C > 0 && C % 8 == 0 && H > 0 && W > 0 && border >= 0,
                    "xsmi_cl_to_nchw: needs C %% 8 == 0 (N=%d C=%d H=%d W=%d border=%d)", N, C, H, W, border);
     XSMI_CHECK_ARG(((uintptr_t)x_cl & 15) == 0, "xsmi_cl_to_nchw: x_cl must be 16-byte aligned");
-    const size_t lds = (size_t)64 * (W | 1) * sizeof(float);
-    XSMI_CHECK_ARG(lds <= 64 * 1024, "xsmi_cl_to_nchw: rows of more than 255 pixels are not supported (W=%d)", W);
+    // rows wider than 255 pixels are converted in equal segments (the tile of a segment must fit 64 KB of LDS)
+    const int segs = xsmi::ceil_div(W, 255), seg = xsmi::ceil_div(W, segs);
+    const size_t lds = (size_t)64 * (seg | 1) * sizeof(float);
     const int cgroups = xsmi::ceil_div(C, 64);
-    const size_t blocks = (size_t)N * H * cgroups;
+    const size_t blocks = (size_t)N * H * cgroups * segs;
     XSMI_CHECK_ARG(blocks < ((size_t)1 << 31), "xsmi_cl_to_nchw: too many rows");
     hipLaunchKernelGGL(cl_to_nchw_kernel, dim3((unsigned)blocks), dim3(256), lds, xsmi::stream(), (const bf16x8 *)x_cl, y, C, H, W,
-                       border, cgroups);
+                       border, cgroups, seg, segs);
     XSMI_LAUNCH_CHECK("cl_to_nchw_kernel");
     return XSMI_OK;
 }
