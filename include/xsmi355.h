@@ -98,7 +98,8 @@ int xsmi_sync(void);
  * the chunks where it pays, 3: even split wherever it applies), "sk_spin_limit" (polls before an even-split
  * workgroup gives up waiting for a partial tile; the calls that wait for the device then fail with
  * XSMI_ERR_RUNTIME), "sk_wide" (0: one-dword loads of the activations in the even-split kernel also where 16-byte
- * loads apply), "tap_stages", "tap_persist",
+ * loads apply), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
+ * several pieces; 0: one piece per workgroup), "tap_stages", "tap_persist",
  * "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
  * A caller that changes one must drop every workspace content it counted on (XSMI_CONV_WS_PACKED) and ask for
  * workspace sizes again.  No counterpart in the reference. */

@@ -39,11 +39,9 @@ __global__ void __launch_bounds__(256) maxpool_fwd_generic(const float *__restri
     float best = 0.f;
     int where = 0;
     bool first = true;
-#pragma unroll
-    for (int r = 0; r < k; ++r) {
+    for (int r = 0; r < k; ++r) {                            // (a compile-time k unrolls by itself)
         int ih = ih0 + r;
         bool rowok = (unsigned)ih < (unsigned)g.H;
-#pragma unroll
         for (int s = 0; s < k; ++s) {
             int iw = iw0 + s;
             float v = 0.f;                                   // border cell
@@ -370,6 +368,107 @@ __global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_lds(const float *__re
     }
 }
 
+// The same kernel with workgroups that stay: a workgroup takes the pieces p = id, id + grid, ... and has the next piece's
+// rows of dy and idx copied into a second staging area (global -> LDS directly, no registers) while it gathers and
+// writes out the current one.  The one-piece kernel above spends its life waiting, first for its loads and then for
+// its stores (without its stores it takes 14.7 us for the 32 MB of reads of a 32 x 64 x 112 x 112 tensor's gradient,
+// without its loads 18 us for the 103 MB of writes, with both 26 us); here the only wait is "at most four
+// vector-memory operations outstanding" after a piece's four stores, i.e. for the loads issued before them, never for
+// the stores themselves.  Two workgroups per compute unit measured best (24.8 us; three or four, or loads two pieces
+// ahead: 26 to 27 us).
+__global__ void __launch_bounds__(256) maxpool_bwd_3x3s2p1_stream(const float *__restrict__ dy, const uint8_t *__restrict__ idx,
+                                                                   float *__restrict__ dx, PoolGeom g, int RG,
+                                                                   uint32_t total_rowg, uint32_t pieces) {
+    __shared__ f4v img[1024];
+    __shared__ f4v s_dy[2][512];                      // (RG + 1) * W/8 float4, with RG * W/8 <= 256 and W/8 <= 256
+    __shared__ uint32_t s_ix[2][512];
+    const int Q8 = g.W >> 3, G = g.H >> 1;
+    const int lt = (int)threadIdx.x;
+    const int lane = lt & 63, wave = __builtin_amdgcn_readfirstlane(lt >> 6);
+    const int lrow = lt / Q8, j = lt - lrow * Q8;
+    const uint32_t q_total = total_rowg * (uint32_t)Q8;                      // float4 (or index words) of all of dy
+    auto fetch = [&](uint32_t piece, int buf) {        // the piece's rows of dy and idx as they lie, zeros past the end
+        const uint32_t rowg0 = piece * (uint32_t)RG;
+        const uint32_t rows_here = total_rowg - rowg0 < (uint32_t)RG ? total_rowg - rowg0 : (uint32_t)RG;
+        const uint32_t q0 = rowg0 * (uint32_t)Q8;
+        uint32_t want = (rows_here + 1u) * (uint32_t)Q8;
+        if (want > q_total - q0) want = q_total - q0;
+        const xsmi::xsmi_int32x4 rd = xsmi::make_rsrc(reinterpret_cast<const f4v *>(dy) + q0, want * 16u);
+        const xsmi::xsmi_int32x4 ri = xsmi::make_rsrc(reinterpret_cast<const uint32_t *>(idx) + q0, want * 4u);
+        const uint32_t ld = (uint32_t)(uintptr_t)&s_dy[buf][0], li = (uint32_t)(uintptr_t)&s_ix[buf][0];
+        for (uint32_t e = (uint32_t)wave; e * 64u < want; e += 4u) {        // want <= 512: e <= 7, inside the staging area
+            xsmi::load_lds_b128(rd, ld + e * 1024u, (e * 64u + (uint32_t)lane) * 16u, 0u);
+            xsmi::load_lds_b32(ri, li + e * 256u, (e * 64u + (uint32_t)lane) * 4u, 0u);
+        }
+    };
+    uint32_t piece = blockIdx.x;
+    if (piece >= pieces) return;
+    int cur = 0;
+    fetch(piece, 0);
+    xsmi::wait_vmcnt<0>();
+    for (; piece < pieces; piece += gridDim.x, cur ^= 1) {
+        const uint32_t rowg0 = piece * (uint32_t)RG;
+        const uint32_t rows_here = total_rowg - rowg0 < (uint32_t)RG ? total_rowg - rowg0 : (uint32_t)RG;
+        // this wave's loads of the piece have landed (first round: waited for above; later: at the end of the last round)
+        xsmi::block_barrier();                         // ... and everybody's; the other staging area and img are free
+        if (piece + gridDim.x < pieces) fetch(piece + gridDim.x, cur ^ 1);
+        if ((uint32_t)lrow < rows_here) {
+            const uint32_t rowg = rowg0 + (uint32_t)lrow;       // (nc, a)
+            const uint32_t nc = rowg / (uint32_t)G;
+            const int a = (int)(rowg - nc * (uint32_t)G);
+            float gv[2][5];
+            int iv[2][5];
+            const float *fdy = reinterpret_cast<const float *>(s_dy[cur]);
+            const uint8_t *bix = reinterpret_cast<const uint8_t *>(s_ix[cur]);
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int oh = a + q;                 // a + 1 == OH: below the last output row
+                f4v gg = f4v{0.f, 0.f, 0.f, 0.f};
+                uint32_t ii = 0xffffffffu;
+                float gn = 0.f;
+                int in = -1;
+                const int lq = (lrow + q) * Q8 + j;
+                if (oh < g.OH) {
+                    gg = s_dy[cur][lq];
+                    ii = s_ix[cur][lq];
+                    if (j + 1 < Q8) { gn = fdy[4 * lq + 4]; in = bix[4 * lq + 4]; }
+                }
+                // x + 0 turns -0 into +0 and changes nothing else: the reference's sums start at +0
+                gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gg.z + 0.f; gv[q][3] = gg.w + 0.f; gv[q][4] = gn + 0.f;
+                iv[q][0] = ii & 255; iv[q][1] = (ii >> 8) & 255; iv[q][2] = (ii >> 16) & 255; iv[q][3] = ii >> 24; iv[q][4] = in;
+            }
+            float e[8], o[8];
+            auto pick = [&](int q, int m, int tap) { return iv[q][m] == tap ? gv[q][m] : 0.f; };
+#pragma unroll
+            for (int m = 0; m < 4; ++m) {
+                e[2 * m] = pick(0, m, 4);
+                e[2 * m + 1] = pick(0, m + 1, 3) + pick(0, m, 5);
+                o[2 * m] = pick(1, m, 1) + pick(0, m, 7);
+                o[2 * m + 1] = (float)((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                       (double)pick(0, m, 8));
+            }
+            f4v *row_e = img + lrow * 4 * Q8 + 2 * j;      // row 2a of the pair, then row 2a + 1
+            row_e[0] = f4v{e[0], e[1], e[2], e[3]};
+            row_e[1] = f4v{e[4], e[5], e[6], e[7]};
+            row_e[2 * Q8] = f4v{o[0], o[1], o[2], o[3]};
+            row_e[2 * Q8 + 1] = f4v{o[4], o[5], o[6], o[7]};
+        }
+        __syncthreads();
+        // Always four stores per thread (those past the piece's end fall outside the buffer and are dropped), so that
+        // "four outstanding" below means exactly: the next piece's loads are done.
+        const uint32_t quads = rows_here * 4u * (uint32_t)Q8;
+        const __amdgpu_buffer_rsrc_t ro = __builtin_amdgcn_make_buffer_rsrc(
+            (void *)(reinterpret_cast<f4v *>(dx) + (size_t)rowg0 * 4u * (uint32_t)Q8), 0, (int)(quads * 16u), 0x00020000);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const uint32_t q = (uint32_t)lt + 256u * k;
+            __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(xsmi::xsmi_uint32x4, img[q]), ro, (int)(q * 16u), 0, 2 /* nt */);
+        }
+        asm volatile("" ::: "memory");
+        xsmi::wait_vmcnt<4>();                         // all but the four stores: the next piece's loads are done
+    }
+}
+
 int check_geom(const char *fn, int N, int C, int H, int W, int k, int sh, int sw, int pad, PoolGeom *g) {
     XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0, "%s: empty tensor (N=%d C=%d H=%d W=%d)", fn, N, C, H, W);
     XSMI_CHECK_ARG(k >= 1 && k <= 15, "%s: window %d outside 1..15 (index is stored in one byte)", fn, k);
@@ -445,7 +544,17 @@ int xsmi_maxpool2d_bwd(const float *dy, const uint8_t *idx, float *dx, int N, in
         if (!acc && W / 8 <= 256) {
             const int RG = 256 / (W / 8);
             const uint32_t total_rowg = (uint32_t)N * C * (H / 2);
-            hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_lds, dim3((total_rowg + RG - 1) / RG), dim3(256), 0, st, dy, idx, dx, g, RG,
+            const uint32_t pieces = (total_rowg + RG - 1) / RG;
+            const long mode = xsmi::option(xsmi::OPT_POOL_BWD);
+            if (mode > 0) {                               // workgroups per compute unit of the kernel whose workgroups stay
+                uint32_t grid_s = (uint32_t)xsmi::cu_count() * (uint32_t)(mode > 4 ? 4 : mode);
+                if (grid_s > pieces) grid_s = pieces;
+                hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_stream, dim3(grid_s), dim3(256), 0, st, dy, idx, dx, g, RG, total_rowg, pieces);
+                xsmi::prof_end();
+                XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_stream");
+                return XSMI_OK;
+            }
+            hipLaunchKernelGGL(maxpool_bwd_3x3s2p1_lds, dim3(pieces), dim3(256), 0, st, dy, idx, dx, g, RG,
                                total_rowg);
             xsmi::prof_end();
             XSMI_LAUNCH_CHECK("maxpool_bwd_3x3s2p1_lds");

@@ -38,6 +38,7 @@ OptionRow g_options[xsmi::OPT_COUNT] = {
     {"cl_halo", "XSMI_CL_HALO", 1, false},
     {"cl_stem", "XSMI_CL_STEM", 1, false},
     {"sk_wide", "XSMI_SK_WIDE", 1, false},
+    {"pool_bwd", "XSMI_POOL_BWD", 2, false},
 };
 
 // Partial tiles and flags of the even-split convolution kernels: one area per stream, owned by the library (a

@@ -24,7 +24,7 @@ bool capturing();            // a step graph is being recorded: nothing runs, no
 bool ready();
 int cu_count();
 // Tuning switches (xsmi_set_option / environment variable / default); the order is that of the table in runtime.hip.
-enum Option { OPT_TAP_SK, OPT_SK_SPIN_LIMIT, OPT_TAP_STAGES, OPT_TAP_PERSIST, OPT_CL_HALO, OPT_CL_STEM, OPT_SK_WIDE, OPT_COUNT };
+enum Option { OPT_TAP_SK, OPT_SK_SPIN_LIMIT, OPT_TAP_STAGES, OPT_TAP_PERSIST, OPT_CL_HALO, OPT_CL_STEM, OPT_SK_WIDE, OPT_POOL_BWD, OPT_COUNT };
 long option(Option o);
 // Partial tiles and flags of the even-split convolution kernels for the stream that stream() hands out; allocated
 // by xsmi_init, the flags are zero between launches.
@@ -196,6 +196,7 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
 // themselves (vmcnt + workgroup barrier) and contain no other instruction that
 // depends on M0.
 typedef int xsmi_int32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned xsmi_uint32x4 __attribute__((ext_vector_type(4)));
 
 __device__ __forceinline__ xsmi_int32x4 make_rsrc(const void *p, uint32_t bytes) {
     uint64_t a = (uint64_t)p;
