@@ -24,13 +24,13 @@
 // the MFMA (v_mfma_f32_32x32x2_f32), lanes 0-31 take channels 0..15 of the chunk
 // and lanes 32-63 channels 16..31: A comes as four 128-bit reads of consecutive
 // 16-byte slots (conflict-free), B as sixteen dword reads of 32 consecutive floats.
-#include "xsmi_internal.h"
+#include "conv_store.h"
 #include <stdlib.h>
 #include <type_traits>
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+using xsmi::floatx16;
 
 constexpr int TM = 64;
 constexpr int BP = 64;
@@ -47,6 +47,7 @@ struct TapParams {
     uint8_t *mask;
     uint32_t in_bytes;
     uint32_t apk_bytes;
+    uint32_t out_bytes;
     int M, rows;
     int nch;              // channel chunks per tap
     int TR, TS;           // taps
@@ -97,7 +98,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
     // The tile's bias goes through the LDS: one coalesced load here instead of a dependent global load per
     // output element in the epilogue.  Only the forward pass has a bias, and it has at least one chunk, so a
     // barrier of the main loop lies between this store and the epilogue's reads.
-    __shared__ float s_bias[TM];
+    __shared__ __attribute__((aligned(16))) float s_bias[TM];
     if (p.bias && t < TM) s_bias[t] = rowtile * TM + t < p.rows ? p.bias[rowtile * TM + t] : 0.f;
 
     // ---- gather role: pixel m0 + lane, channels 8*wave .. 8*wave+7 of each chunk ----
@@ -265,30 +266,9 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
 
     acc += acc2;
 
-    // ---- epilogue: register v of lane l = row 8*(v/4) + 4*(l/32) + v%4, pixel l%32 ----
-    const int m = m0 + wc * 32 + l31;
-    if (m >= p.M) return;
-    uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
-    int x = m - (int)q * p.OX;
-    uint32_t n = xsmi::fdiv(q, p.dOY);
-    int y = (int)q - (int)n * p.OY;
-    const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
-    const int rbase = rowtile * TM + wr * 32 + 4 * h;
-#pragma unroll
-    for (int v = 0; v < 16; ++v) {
-        int row = rbase + 8 * (v >> 2) + (v & 3);
-        if (row < p.rows) {
-            float val = acc[v];
-            if (p.bias) val += s_bias[row - rowtile * TM];
-            long long o = pix_off + (long long)row * p.os_k;
-            if (p.relu) {
-                if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
-                val = val > 0.f ? val : 0.f;
-            }
-            if (p.accumulate) val += p.out[o];
-            p.out[o] = val;
-        }
-    }
+    // ---- epilogue ----
+    xsmi::store_block_32x32(acc, p, p.out, p.out_bytes, p.mask, p.bias ? &s_bias[0] : nullptr, p.relu, p.accumulate, rowtile * TM, TM,
+                            wr * 32, m0 + wc * 32, lane);
 }
 
 // Persistent form of the kernel above (same tile, same loop body, 2 stages).  A launch has at most
@@ -303,7 +283,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
     constexpr int STAGES = 2;
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     __shared__ uint32_t s_next;
-    __shared__ float s_bias[2][TM];                   // bias of the current tile, alternating per tile
+    __shared__ __attribute__((aligned(16))) float s_bias[2][TM];    // bias of the current tile, alternating per tile
 
     const int t = threadIdx.x;
     const int lane = t & 63;
@@ -491,33 +471,9 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
         }
         acc += acc2;
 
-        // ---- epilogue: register v of lane l = row 8*(v/4) + 4*(l/32) + v%4, pixel l%32 ----
-        {
-            const int m = cur_m0 + wc * 32 + l31;
-            if (m < p.M) {
-                uint32_t q = xsmi::fdiv((uint32_t)m, p.dOX);
-                int x = m - (int)q * p.OX;
-                uint32_t n = xsmi::fdiv(q, p.dOY);
-                int y = (int)q - (int)n * p.OY;
-                const long long pix_off = (long long)n * p.os_n + (long long)y * p.os_y + (long long)x * p.os_x + p.o_base;
-                const int rbase = cur_rowtile * TM + wr * 32 + 4 * h;
-#pragma unroll
-                for (int v = 0; v < 16; ++v) {
-                    int row = rbase + 8 * (v >> 2) + (v & 3);
-                    if (row < p.rows) {
-                        float val = acc[v];
-                        if (p.bias) val += s_bias[bias_buf][row - cur_rowtile * TM];
-                        long long o = pix_off + (long long)row * p.os_k;
-                        if (p.relu) {
-                            if (p.mask) p.mask[o] = val < 0.f ? 1 : 0;
-                            val = val > 0.f ? val : 0.f;
-                        }
-                        if (p.accumulate) val += p.out[o];
-                        p.out[o] = val;
-                    }
-                }
-            }
-        }
+        // ---- epilogue ----
+        xsmi::store_block_32x32(acc, p, p.out, p.out_bytes, p.mask, p.bias ? &s_bias[bias_buf][0] : nullptr, p.relu, p.accumulate,
+                                cur_rowtile * TM, TM, wr * 32, cur_m0 + wc * 32, lane);
         if (last_tile) {
             xsmi::wait_vmcnt<0>();                            // the dummy chunk's loads target this workgroup's LDS
             break;
@@ -1445,6 +1401,7 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     TapParams p;
     p.in = x; p.apk = apk; p.bias = bias; p.out = y; p.mask = relu ? mask : nullptr;
     p.in_bytes = (uint32_t)((size_t)N * C * H * W * 4);
+    p.out_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
     p.M = N * OH * OW; p.rows = K; p.nch = C / KC; p.TR = R; p.TS = S;
     p.dy0 = -pad; p.dx0 = -pad; p.dstep = 1;
     p.IH = H; p.IW = W; p.sy = sh; p.sx = sw;
@@ -1612,6 +1569,7 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             p.counters = tap_counters(apk, apk_bytes);
             p.tiles = 0; p.rowtiles = 0;
             p.in_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
+            p.out_bytes = (uint32_t)((size_t)N * C * H * W * 4);
             p.M = N * OYc * OXc; p.rows = C; p.nch = K / KC; p.TR = T; p.TS = U;
             p.dy0 = cy; p.dx0 = cx; p.dstep = -1;
             p.IH = OH; p.IW = OW; p.sy = 1; p.sx = 1;

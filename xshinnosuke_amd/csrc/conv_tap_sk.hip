@@ -17,7 +17,7 @@
 // Workgroups start in id order, so whatever is resident either finishes or waits for something that has already
 // started.  The wait is bounded all the same (spin_limit); when it runs out the workgroup sets the library's device
 // error word and stores nothing more, and the host reports the launch as failed at its next check.
-#include "xsmi_internal.h"
+#include "conv_store.h"
 #include <stdlib.h>
 #include <string.h>
 #include <type_traits>
@@ -25,7 +25,7 @@
 
 namespace {
 
-typedef float floatx16 __attribute__((ext_vector_type(16)));
+using xsmi::floatx16;
 
 constexpr int SK_MAX_CLASSES = 4;
 constexpr int SK_MAX_GRID = 1024;           // upper bound of resident workgroups (flags and partial tiles are sized for it)
@@ -322,74 +322,9 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     };
 
     // accumulator register v of lane l in block (i, j): row 32 i + 8 (v / 4) + 4 (l / 32) + v % 4, pixel 32 j + l % 32
-    // Whole row tiles (all layers whose row count is a multiple of the tile): one byte offset per lane, the row's
-    // displacement in a scalar register, out-of-range pixels through the buffer range check; the bias, ReLU / mask
-    // and accumulate steps are passes over the lane's 16 registers, each behind one uniform branch.  Tensors hold
-    // fewer than 2^29 elements, so 32-bit byte offsets suffice.
     auto store_tile = [&]() {
-        const SkClass &c = sp.cls[c_ci];
-        const int lrow = wr * 32 + 4 * h;
-        const int m = c_m0 + wc * 32 + l31;
-        const uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
-        const int x = m - (int)q * c.OX;
-        const uint32_t n = xsmi::fdiv(q, c.dOY);
-        const int y = (int)q - (int)n * c.OY;
-        if ((c_rt + 1) * ROWS <= c.rows) {
-            const __amdgpu_buffer_rsrc_t rout = __builtin_amdgcn_make_buffer_rsrc((void *)sp.out, 0, (int)sp.out_bytes, 0x00020000);
-            const __amdgpu_buffer_rsrc_t rmask =
-                __builtin_amdgcn_make_buffer_rsrc((void *)sp.mask, 0, sp.mask ? (int)(sp.out_bytes >> 2) : 0, 0x00020000);
-            const uint32_t os_k4 = (uint32_t)c.os_k * 4u;
-            const uint32_t srow = (uint32_t)(c_rt * ROWS) * os_k4;
-            const uint32_t pix = (uint32_t)((int)n * (int)c.os_n + y * c.os_y + x * c.os_x + (int)c.o_base) * 4u + (uint32_t)lrow * os_k4;
-            const uint32_t voff = m < c.M ? pix : 0x80000000u;
-            auto row_off = [&](int v) { return srow + (uint32_t)(8 * (v >> 2) + (v & 3)) * os_k4; };
-            floatx16 r = acc[0];
-            if (sp.bias) {
-#pragma unroll
-                for (int q4 = 0; q4 < 4; ++q4) {
-                    const float4 bz = *reinterpret_cast<const float4 *>(&s_bias[bias_buf][lrow + 8 * q4]);
-                    r[4 * q4] += bz.x; r[4 * q4 + 1] += bz.y; r[4 * q4 + 2] += bz.z; r[4 * q4 + 3] += bz.w;
-                }
-            }
-            if (sp.relu) {
-                if (sp.mask) {
-#pragma unroll
-                    for (int v = 0; v < 16; ++v)
-                        __builtin_amdgcn_raw_buffer_store_b8((unsigned char)(r[v] < 0.f ? 1 : 0), rmask, (int)(voff >> 2), (int)(row_off(v) >> 2), 0);
-                }
-#pragma unroll
-                for (int v = 0; v < 16; ++v) r[v] = r[v] > 0.f ? r[v] : 0.f;
-            }
-            if (sp.accumulate) {
-                float old[16];
-#pragma unroll
-                for (int v = 0; v < 16; ++v) old[v] = buf_load(rout, voff, row_off(v));
-#pragma unroll
-                for (int v = 0; v < 16; ++v) r[v] += old[v];
-            }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) buf_store(rout, r[v], voff, row_off(v));
-            return;
-        }
-        // ragged last row tile: every row is tested
-        if (m >= c.M) return;
-        const int rbase = c_rt * ROWS + lrow;
-        const long long pix_off = (long long)n * c.os_n + (long long)y * c.os_y + (long long)x * c.os_x + c.o_base;
-#pragma unroll
-        for (int v = 0; v < 16; ++v) {
-            const int ro = 8 * (v >> 2) + (v & 3);
-            if (rbase + ro < c.rows) {
-                float val = acc[0][v];
-                if (sp.bias) val += s_bias[bias_buf][lrow + ro];
-                long long o = pix_off + (long long)(rbase + ro) * c.os_k;
-                if (sp.relu) {
-                    if (sp.mask) sp.mask[o] = val < 0.f ? 1 : 0;
-                    val = val > 0.f ? val : 0.f;
-                }
-                if (sp.accumulate) val += sp.out[o];
-                sp.out[o] = val;
-            }
-        }
+        xsmi::store_block_32x32(acc[0], sp.cls[c_ci], sp.out, sp.out_bytes, sp.mask, sp.bias ? &s_bias[bias_buf][0] : nullptr,
+                                sp.relu, sp.accumulate, c_rt * ROWS, ROWS, wr * 32, c_m0 + wc * 32, lane);
     };
     // the partial tile of workgroup j: register v of thread t at float (j * 16 + v) * 256 + t of the partial-tile area
     constexpr uint32_t PART_BYTES = 16 * 256 * 4;
