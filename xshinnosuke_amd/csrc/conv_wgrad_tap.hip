@@ -55,7 +55,7 @@ struct WgradTapParams {
     xsmi::FastDiv dOW, dCT, dS;
 };
 
-__global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
+__global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p) {
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     constexpr int D = STAGES - 1;
 
@@ -102,48 +102,87 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
         in_img = chunk_begin / p.cpi;
         ci = chunk_begin - in_img * p.cpi;
     }
-    uint32_t ld_stage = lds0;
-    uint32_t ld_va0 = 0, ld_va1 = 0, ld_vb = 0, ld_sa = 0, ld_sb = 0;
+    uint32_t ld_vb = 0, ld_sa = 0, ld_sb = 0;
+    int ld_ml0 = 0;
+    bool ld_tail = false;                                            // the chunk to load runs past the end of its image
+    // The input position of this lane's pixel is walked from chunk to chunk instead of being formed by two divisions per
+    // chunk (every vector instruction beside the MFMAs takes matrix-pipe time): the pixel advances by MC = q32 rows and
+    // r32 columns of the output, with at most one carry.  A pixel contributes when its output row lies in
+    // [ylo, ylo + ycnt) (input row inside the image, and the row exists at all: the last chunk of an image runs past its
+    // end) and its column in [xlo, xlo + xcnt).  Not used when the chunks run over the whole batch (p.flat).
+    const int q32 = MC / p.OW, r32 = MC - q32 * p.OW;
+    const int ylo = p.pad > tr ? (p.pad - tr + p.sh - 1) / p.sh : 0;
+    int yhi = (p.H - 1 + p.pad - tr) / p.sh;
+    if (yhi > p.OH - 1) yhi = p.OH - 1;
+    const uint32_t ycnt = yhi >= ylo ? (uint32_t)(yhi - ylo + 1) : 0u;
+    const int xlo = p.pad > ts ? (p.pad - ts + p.sw - 1) / p.sw : 0;
+    int xhi = (p.W - 1 + p.pad - ts) / p.sw;
+    if (xhi > p.OW - 1) xhi = p.OW - 1;
+    const uint32_t xcnt = xhi >= xlo ? (uint32_t)(xhi - xlo + 1) : 0u;
+    const int row_bytes = p.sh * p.W * 4, col_bytes = p.sw * 4;
+    const int step_bytes = q32 * row_bytes + r32 * col_bytes;        // no carry
+    const int carry_bytes = step_bytes + row_bytes - p.OW * col_bytes;
+    const int lane_bytes = ((tr - p.pad) * p.W + (ts - p.pad)) * 4 + b_chl * (int)p.xplane_bytes;
+    int w_oh, w_ow, w_addr;                                          // of the next chunk to load
+    {
+        const int ml = ci * MC + b_m;
+        w_oh = ml / p.OW;
+        w_ow = ml - w_oh * p.OW;
+        w_addr = w_oh * row_bytes + w_ow * col_bytes + lane_bytes;
+    }
     auto issue_prep = [&]() {
         const int ml0 = ci * MC;
-        // A: groups of 4 pixels are inside the (padded) plane or not as a whole
-        const bool a_ok = ml0 + 4 * a_q < p.OHWa;
-        ld_va0 = a_ok ? a_v0 : 0x80000000u;
-        ld_va1 = a_ok ? a_v1 : 0x80000000u;
         ld_sa = (uint32_t)((in_img * p.K + k0) * p.OHWa + ml0) * 4u;
-        // B: the shifted input position of this lane's pixel
-        int ml = ml0 + b_m;
-        int img = 0;                                  // flat: this lane's image (the scalar part then has none)
-        bool inside = ml < p.OHW;
-        if (p.flat) {
-            inside = ml < p.Mtot;
-            img = (int)xsmi::fdiv((uint32_t)ml, p.dOHW);
-            ml -= img * p.OHW;
-        }
-        const int oh = (int)xsmi::fdiv((uint32_t)ml, p.dOW);
-        const int ow = ml - oh * p.OW;
-        const int ih = oh * p.sh + tr - p.pad, iw = ow * p.sw + ts - p.pad;
-        const bool b_ok = inside && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
-        ld_vb = b_ok ? (uint32_t)((ih * p.W + iw) * 4) + (uint32_t)(img * p.C + b_chl) * p.xplane_bytes : 0x80000000u;
         ld_sb = (uint32_t)(in_img * p.C + c0) * p.xplane_bytes;
+        // A: groups of 4 pixels are inside the (padded) plane or not as a whole; only an image's last chunk can hold any outside
+        ld_ml0 = ml0;
+        ld_tail = ml0 + MC > p.OHWa;
+        if (p.flat) {
+            // B: the shifted input position of this lane's pixel, chunks running over the pixels of the whole batch
+            int ml = ml0 + b_m;
+            const bool inside = ml < p.Mtot;
+            const int img = (int)xsmi::fdiv((uint32_t)ml, p.dOHW);
+            ml -= img * p.OHW;
+            const int oh = (int)xsmi::fdiv((uint32_t)ml, p.dOW);
+            const int ow = ml - oh * p.OW;
+            const int ih = oh * p.sh + tr - p.pad, iw = ow * p.sw + ts - p.pad;
+            const bool b_ok = inside && (unsigned)ih < (unsigned)p.H && (unsigned)iw < (unsigned)p.W;
+            ld_vb = b_ok ? (uint32_t)((ih * p.W + iw) * 4) + (uint32_t)(img * p.C + b_chl) * p.xplane_bytes : 0x80000000u;
+            return;
+        }
+        const bool ok = (uint32_t)(w_oh - ylo) < ycnt && (uint32_t)(w_ow - xlo) < xcnt;
+        ld_vb = ok ? (uint32_t)w_addr : 0x80000000u;
     };
-    auto issue_a = [&](int j) {
-        xsmi::load_lds_b128(ry, ld_stage + (uint32_t)((wave + 4 * j) * 1024), j == 0 ? ld_va0 : ld_va1, ld_sa);
+    auto issue_a = [&](int j, uint32_t stage) {
+        uint32_t v = j == 0 ? a_v0 : a_v1;
+        if (ld_tail) v = ld_ml0 + 4 * a_q < p.OHWa ? v : 0x80000000u;
+        xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), v, ld_sa);
     };
-    auto issue_b = [&](int e) {
-        xsmi::load_lds_b32(rx, ld_stage + (uint32_t)(8192 + (wave + 4 * e) * 256), ld_vb, ld_sb + (uint32_t)(8 * e) * p.xplane_bytes);
+    auto issue_b = [&](int e, uint32_t stage) {
+        xsmi::load_lds_b32(rx, stage + (uint32_t)(8192 + (wave + 4 * e) * 256), ld_vb, ld_sb + (uint32_t)(8 * e) * p.xplane_bytes);
     };
     auto issue_advance = [&]() {
-        ld_stage += (uint32_t)(STAGE_FLOATS * 4);
-        if (ld_stage == lds0 + (uint32_t)(STAGES * STAGE_FLOATS * 4)) ld_stage = lds0;
-        if (++ci == p.cpi) { ci = 0; ++in_img; }
+        if (++ci == p.cpi) {
+            ci = 0; ++in_img;
+            w_oh = b_m / p.OW;                                       // the lane's pixel in an image's first chunk
+            w_ow = b_m - w_oh * p.OW;
+            w_addr = w_oh * row_bytes + w_ow * col_bytes + lane_bytes;
+        } else {
+            w_ow += r32;
+            const bool carry = w_ow >= p.OW;
+            w_ow -= carry ? p.OW : 0;
+            w_oh += q32 + (carry ? 1 : 0);
+            w_addr += carry ? carry_bytes : step_bytes;
+        }
     };
-    auto issue_all = [&]() {
+    // chunk i of the workgroup's range lives in stage i % 2 and its fragments in register set i % 2
+    auto issue_all = [&](int st) {
+        const uint32_t stage = lds0 + (uint32_t)(st * STAGE_FLOATS * 4);
         issue_prep();
-        issue_a(0);
-        issue_a(1);
+        issue_a(0, stage);
+        issue_a(1, stage);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) issue_b(e);
+        for (int e = 0; e < 8; ++e) issue_b(e, stage);
         issue_advance();
     };
 
@@ -160,11 +199,6 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
 
     floatx16 acc = {0}, acc2 = {0};
     float4 fa[2][4], fb[2][4];
-    const float *rd_stage = smem[0];
-    auto rd_advance = [&]() {
-        rd_stage += STAGE_FLOATS;
-        if (rd_stage == smem[0] + STAGES * STAGE_FLOATS) rd_stage = smem[0];
-    };
 #define XSMI_MFMA(ACC, AV, BV) ACC = __builtin_amdgcn_mfma_f32_32x32x2f32(AV, BV, ACC, 0, 0, 0)
 #define XSMI_PIN() __builtin_amdgcn_sched_barrier(0)
     auto body = [&](auto buf_tag, auto static_tag, int it) {
@@ -173,6 +207,8 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
         constexpr bool all = decltype(static_tag)::value;
         const bool has_next = all || it + 1 < nchunks;
         const bool has_load = all || it + 1 + D < nchunks;
+        const float *rd_stage = smem[nxt];                               // the next chunk's stage
+        const uint32_t ld_to = lds0 + (uint32_t)(cur * STAGE_FLOATS * 4);  // this chunk's stage is free after the barrier
         XSMI_MFMA(acc, fa[cur][0].x, fb[cur][0].x);
         XSMI_MFMA(acc2, fa[cur][0].y, fb[cur][0].y);
         XSMI_MFMA(acc, fa[cur][0].z, fb[cur][0].z);
@@ -190,39 +226,35 @@ __global__ void __launch_bounds__(256) wgrad_tap_f32_kernel(WgradTapParams p) {
         if (has_load) { STMT2; }                \
         XSMI_PIN();
         XSMI_SLOT(acc, fa[cur][1].x, fb[cur][1].x, fa[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[0]), issue_prep())
-        XSMI_SLOT(acc2, fa[cur][1].y, fb[cur][1].y, fb[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[0]), issue_a(0))
-        XSMI_SLOT(acc, fa[cur][1].z, fb[cur][1].z, fa[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[1]), issue_a(1))
-        XSMI_SLOT(acc2, fa[cur][1].w, fb[cur][1].w, fb[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[1]), issue_b(0))
-        XSMI_SLOT(acc, fa[cur][2].x, fb[cur][2].x, fa[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[2]), issue_b(1))
-        XSMI_SLOT(acc2, fa[cur][2].y, fb[cur][2].y, fb[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[2]), issue_b(2))
-        XSMI_SLOT(acc, fa[cur][2].z, fb[cur][2].z, fa[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[3]), issue_b(3))
-        XSMI_SLOT(acc2, fa[cur][2].w, fb[cur][2].w, fb[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[3]), issue_b(4))
-        XSMI_SLOT(acc, fa[cur][3].x, fb[cur][3].x, (void)0, issue_b(5))
-        XSMI_SLOT(acc2, fa[cur][3].y, fb[cur][3].y, (void)0, issue_b(6))
-        XSMI_SLOT(acc, fa[cur][3].z, fb[cur][3].z, (void)0, issue_b(7))
+        XSMI_SLOT(acc2, fa[cur][1].y, fb[cur][1].y, fb[nxt][0] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[0]), issue_a(0, ld_to))
+        XSMI_SLOT(acc, fa[cur][1].z, fb[cur][1].z, fa[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[1]), issue_a(1, ld_to))
+        XSMI_SLOT(acc2, fa[cur][1].w, fb[cur][1].w, fb[nxt][1] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[1]), issue_b(0, ld_to))
+        XSMI_SLOT(acc, fa[cur][2].x, fb[cur][2].x, fa[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[2]), issue_b(1, ld_to))
+        XSMI_SLOT(acc2, fa[cur][2].y, fb[cur][2].y, fb[nxt][2] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[2]), issue_b(2, ld_to))
+        XSMI_SLOT(acc, fa[cur][2].z, fb[cur][2].z, fa[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[3]), issue_b(3, ld_to))
+        XSMI_SLOT(acc2, fa[cur][2].w, fb[cur][2].w, fb[nxt][3] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[3]), issue_b(4, ld_to))
+        XSMI_SLOT(acc, fa[cur][3].x, fb[cur][3].x, (void)0, issue_b(5, ld_to))
+        XSMI_SLOT(acc2, fa[cur][3].y, fb[cur][3].y, (void)0, issue_b(6, ld_to))
+        XSMI_SLOT(acc, fa[cur][3].z, fb[cur][3].z, (void)0, issue_b(7, ld_to))
         XSMI_SLOT(acc2, fa[cur][3].w, fb[cur][3].w, (void)0, issue_advance())
 #undef XSMI_SLOT
         if (want_db) {
 #pragma unroll
             for (int g = 0; g < 4; ++g) dbacc += (fa[cur][g].x + fa[cur][g].y) + (fa[cur][g].z + fa[cur][g].w);
         }
-        if (has_next) rd_advance();
     };
 
-#pragma unroll
-    for (int d = 0; d < D; ++d)
-        if (d < nchunks) issue_all();
+    static_assert(STAGES == 2 && D == 1, "stage = chunk parity");
     if (nchunks > 0) {
-        if (D <= nchunks) xsmi::wait_vmcnt<(D - 1) * LOADS>();
-        else xsmi::wait_vmcnt<0>();
+        issue_all(0);
+        xsmi::wait_vmcnt<0>();
         xsmi::block_barrier();
 #pragma unroll
         for (int g = 0; g < 4; ++g) {
-            fa[0][g] = *reinterpret_cast<const float4 *>(rd_stage + a_rd[g]);
-            fb[0][g] = *reinterpret_cast<const float4 *>(rd_stage + b_rd[g]);
+            fa[0][g] = *reinterpret_cast<const float4 *>(smem[0] + a_rd[g]);
+            fb[0][g] = *reinterpret_cast<const float4 *>(smem[0] + b_rd[g]);
         }
-        rd_advance();
-        if (D < nchunks) issue_all();
+        if (1 < nchunks) issue_all(1);
     }
     {
         using T0 = std::integral_constant<int, 0>;
