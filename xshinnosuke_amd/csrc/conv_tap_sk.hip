@@ -650,18 +650,15 @@ bool sk_path_ok(int reduce_channels, int rows) {
     return reduce_channels % s.kc == 0 && reduce_channels % 32 == 0;
 }
 
-// Where the even split pays (measured on ResNet-18's layers at N=32 against the first-generation kernels, whose
-// workgroups take whole tiles): the exchange of partial tiles and the simultaneous end of all workgroups cost about
-// 5 us per launch, which is won back when whole tiles leave compute units idle (no more tiles than CUs: 512 -> 512
-// at 7 x 7, +17 %) or a last, mostly empty round (three or more tiles per CU: 64 -> 64 at 56 x 56, +6 %), and by
-// every strided backward-data pass, whose four residue classes of different lengths then share one balanced
-// launch (+20 to +26 %).  Strided forwards and 1 x 1 filters (a handful of chunks per tile) stay on whole tiles.
+// Where the even split pays (measured on ResNet-18's layers at N=32 against the kernels whose workgroups take whole
+// tiles): every stride-1 pass with at least four taps (+1 to +17 %: no idle compute units when there are fewer tiles
+// than CUs, no mostly empty last round of tiles otherwise), and every strided backward-data pass, whose four residue
+// classes of different lengths then share one balanced launch (+20 to +26 %).  Strided forwards (mixed: -13 to +5 %)
+// and 1 x 1 filters (a handful of chunks per tile) stay on whole tiles.
 bool sk_fwd_pays(int M, int rows, int R, int S, int sh, int sw) {
+    (void)M; (void)rows;
     if (sk_env() >= 3) return true;                    // forced, for tests and measurements
-    if (sh != 1 || sw != 1 || R * S < 4) return false;
-    const long long tiles = (long long)ceil_div(M, 64) * ceil_div(rows, 64);
-    const int cus = cu_count() > 0 ? cu_count() : 256;
-    return tiles <= cus || tiles >= 3LL * cus;
+    return sh == 1 && sw == 1 && R * S >= 4;
 }
 bool sk_bwd_data_pays(int M, int rows, int R, int S, int sh, int sw) {
     if (sk_env() >= 3) return true;
