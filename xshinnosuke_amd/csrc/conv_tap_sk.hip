@@ -141,7 +141,8 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     uint32_t i_plane = 0;
     int iyb = 0, ixb = 0, nbase = 0;
     bool live = false;
-    bool prep_stale = true;                            // the pixel offset must be formed again (new segment)
+    uint32_t prep_stale = 1;                           // the pixel offset must be formed again (new segment); the uniform
+                                                       // flags are integers so that they live in one scalar register each
     uint32_t ld_asoff = 0, ld_voff = 0, ld_soff = 0;
     int ld_fix = 0;                                    // VEC = 4: what the lane does to its run once it has landed (issue_prep)
     const int csub = VEC == 4 ? lane >> 4 : 0;         // VEC = 4: which of the wave-load's four channels the lane fetches
@@ -160,7 +161,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         uint32_t n_seg = c.iters - ch;
         if (n_seg > u1 - iu) n_seg = u1 - iu;
         i_left = n_seg;
-        prep_stale = true;
+        prep_stale = 1;
         i_nch = c.nch; i_TS = c.TS; i_dstep = c.dstep; i_IH = c.IH; i_IW = c.IW; i_plane = c.plane_bytes;
         const uint32_t tap = ch / (uint32_t)c.nch;
         cc = (int)(ch - tap * (uint32_t)c.nch);
@@ -183,7 +184,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     auto issue_prep = [&]() {
         ld_soff = (uint32_t)(cc * KC + chan0) * i_plane;
         if (cc != 0 && !prep_stale) return;            // same tap as the previous chunk: same pixel offset
-        prep_stale = false;
+        prep_stale = 0;
         const int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
         if constexpr (VEC == 4) {
             // The lane's run is columns ix .. ix + 3 of one input row; ix = -1 and ix + 3 = IW (one column past either
@@ -255,7 +256,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
             } else {
                 // Past the range every chunk still runs the full loop body; its loads are given no live pixel
                 // (they touch no memory and fill the stage with zeros) and re-read the first filter block.
-                live = false; ld_asoff = 0; r = 0; s = 0; cc = 0; prep_stale = true;
+                live = false; ld_asoff = 0; r = 0; s = 0; cc = 0; prep_stale = 1;
             }
         }
     };
@@ -295,10 +296,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     uint32_t cu = u0;
     uint32_t c_left = 0;                               // chunks left in the current segment
     int c_ci = 0, c_m0 = 0, c_rt = 0;
-    bool c_head = false, c_complete = false;           // segment holds the tile's first chunk / its last chunk
+    uint32_t c_head = 0, c_complete = 0;               // segment holds the tile's first chunk / its last chunk
     uint32_t c_tile_end = 0;                           // unit after the tile's last chunk
     int bias_buf = 0;
-    bool flag_pending = false;                         // a partial tile has been stored, its flag not raised yet
+    uint32_t flag_pending = 0;                         // a partial tile has been stored, its flag not raised yet
     auto compute_segment = [&]() {
         int ci = 0;
         if constexpr (VEC != 4)
@@ -313,8 +314,8 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if (n_seg > u1 - cu) n_seg = u1 - cu;
         c_left = n_seg;
         c_ci = ci; c_m0 = (int)mt * PIX; c_rt = (int)rt;
-        c_head = ch == 0;
-        c_complete = ch + n_seg == c.iters;
+        c_head = ch == 0 ? 1u : 0u;
+        c_complete = ch + n_seg == c.iters ? 1u : 0u;
         c_tile_end = cu + (c.iters - ch);
         // the tile's bias goes through the LDS (one coalesced load); the chunk loop's barriers publish it
         bias_buf ^= 1;
@@ -339,7 +340,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
                 // More chunks follow: the next chunk's body waits for all outstanding memory operations of every wave
                 // (vmcnt(0), then the workgroup barrier) before it reads the next stage, which covers these stores;
                 // the flag is raised after that body instead of stalling the workgroup for the write-through here.
-                flag_pending = true;
+                flag_pending = 1;
             } else {
                 xsmi::wait_vmcnt<0>();                 // this thread's stores have been written through
                 __syncthreads();                       // ... and everybody else's
@@ -384,7 +385,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     };
     auto chunk_done = [&]() {
         if (flag_pending) {                            // uniform: the partial tile stored before this chunk is complete
-            flag_pending = false;
+            flag_pending = 0;
             if (t == 0) __hip_atomic_store(sp.flags + g, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         ++cu;

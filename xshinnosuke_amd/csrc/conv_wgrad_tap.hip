@@ -314,14 +314,19 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce_kernel(const float *__re
         src = part + ((size_t)tap * K + k) * C + c;
         dst = dw; o = ((size_t)k * C + c) * taps + tap;
     }
-    double s0 = 0.0, s1 = 0.0;
+    // group g adds the splits g, g + 4, g + 8, ... in that order; eight loads are in flight before the first add (the
+    // loop is bound by memory latency: with two in flight it took 12 us for 113 splits of a 64 x 64 x 3 x 3 filter)
+    double sum = 0.0;
     int sp = g;
-    for (; sp + 4 < splits; sp += 8) {
-        s0 += (double)src[(size_t)sp * stride];
-        s1 += (double)src[(size_t)(sp + 4) * stride];
+    for (; sp + 28 < splits; sp += 32) {
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) v[i] = src[(size_t)(sp + 4 * i) * stride];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) sum += (double)v[i];
     }
-    if (sp < splits) s0 += (double)src[(size_t)sp * stride];
-    sm[g][cl] = s0 + s1;
+    for (; sp < splits; sp += 4) sum += (double)src[(size_t)sp * stride];
+    sm[g][cl] = sum;
     __syncthreads();
     if (g == 0) {
         double s = ((sm[0][cl] + sm[1][cl]) + sm[2][cl]) + sm[3][cl];
@@ -351,7 +356,16 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce9_kernel(const float *__r
     double s[9];
 #pragma unroll
     for (int t = 0; t < 9; ++t) s[t] = 0.0;
-    for (int sp = 0; sp < splits; ++sp) {
+    int sp = 0;
+    for (; sp + 1 < splits; sp += 2) {                 // 18 loads in flight
+        const float *src = part + (size_t)sp * 9 * KC + kc;
+        float v[18];
+#pragma unroll
+        for (int t = 0; t < 18; ++t) v[t] = src[(size_t)t * KC];
+#pragma unroll
+        for (int t = 0; t < 9; ++t) s[t] = (s[t] + (double)v[t]) + (double)v[9 + t];
+    }
+    if (sp < splits) {
         const float *src = part + (size_t)sp * 9 * KC + kc;
 #pragma unroll
         for (int t = 0; t < 9; ++t) s[t] += (double)src[(size_t)t * KC];
