@@ -104,7 +104,7 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
     }
     uint32_t ld_vb = 0, ld_sa = 0, ld_sb = 0;
     int ld_ml0 = 0;
-    bool ld_tail = false;                                            // the chunk to load runs past the end of its image
+    int ld_tail = 0;                                                 // the chunk to load runs past the end of its image
     // The input position of this lane's pixel is walked from chunk to chunk instead of being formed by two divisions per
     // chunk (every vector instruction beside the MFMAs takes matrix-pipe time): the pixel advances by MC = q32 rows and
     // r32 columns of the output, with at most one carry.  A pixel contributes when its output row lies in
@@ -136,7 +136,7 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
         ld_sb = (uint32_t)(in_img * p.C + c0) * p.xplane_bytes;
         // A: groups of 4 pixels are inside the (padded) plane or not as a whole; only an image's last chunk can hold any outside
         ld_ml0 = ml0;
-        ld_tail = ml0 + MC > p.OHWa;
+        ld_tail = ml0 + MC > p.OHWa ? 1 : 0;
         if (p.flat) {
             // B: the shifted input position of this lane's pixel, chunks running over the pixels of the whole batch
             int ml = ml0 + b_m;
@@ -154,9 +154,10 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
         ld_vb = ok ? (uint32_t)w_addr : 0x80000000u;
     };
     auto issue_a = [&](int j, uint32_t stage) {
-        uint32_t v = j == 0 ? a_v0 : a_v1;
-        if (ld_tail) v = ld_ml0 + 4 * a_q < p.OHWa ? v : 0x80000000u;
-        xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), v, ld_sa);
+        const uint32_t v = j == 0 ? a_v0 : a_v1;
+        // (a load in each branch keeps this a branch: as a select it would cost five vector instructions per chunk)
+        if (ld_tail) xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), ld_ml0 + 4 * a_q < p.OHWa ? v : 0x80000000u, ld_sa);
+        else xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), v, ld_sa);
     };
     auto issue_b = [&](int e, uint32_t stage) {
         xsmi::load_lds_b32(rx, stage + (uint32_t)(8192 + (wave + 4 * e) * 256), ld_vb, ld_sb + (uint32_t)(8 * e) * p.xplane_bytes);
@@ -194,7 +195,7 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
         a_rd[g] = (f_arow * 8 + ((4 * h + g) ^ (f_arow & 7))) * 4;
         b_rd[g] = 2048 + (f_bch * 8 + ((4 * h + g) ^ (f_bch & 7))) * 4;
     }
-    const bool want_db = p.dbpart != nullptr && lx == 0 && wc == 0;
+    const int want_db = __builtin_amdgcn_readfirstlane(p.dbpart != nullptr && lx == 0 && wc == 0 ? 1 : 0);
     float dbacc = 0.f;
 
     floatx16 acc = {0}, acc2 = {0};
