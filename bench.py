@@ -250,6 +250,12 @@ def bench_per_layer(be, reps):
             "bwd_data": lambda: K.conv2d_bwd_data(dy, w, x.shape, (st, st), pad, dx=gx),
             "bwd_weight": lambda: K.conv2d_bwd_weight(dy, x, w.shape, (st, st), pad, dw=gw, db=gb),
         }
+        # the same passes as a training step runs them: the filter's layout was made ahead (on the second stream,
+        # after the optimizer's update), so the pass itself is the convolution kernel alone
+        ahead = {
+            "fwd": lambda: K.conv2d_fwd(x, w, b, (st, st), pad, out=y, keep_layout=True),
+            "bwd_data": lambda: K.conv2d_bwd_data(dy, w, x.shape, (st, st), pad, dx=gx, keep_layout=True),
+        }
         for pname, fn in passes.items():
             if pname == "bwd_data" and c == 3:
                 continue                                  # the network input needs no gradient
@@ -257,13 +263,19 @@ def bench_per_layer(be, reps):
             preheat(be, fn, seconds=0.25)
             ms = batch_ms(be, fn, reps)
             tf = flops / (ms * 1e-3) / 1e12
-            rows.append({"layer": name, "count": count, "pass": pname, "ms": ms, "gflop": flops / 1e9, "tflops": tf,
-                         "frac_fp32_mfma_peak": tf / FP32_MFMA_PEAK_TFLOPS})
+            row = {"layer": name, "count": count, "pass": pname, "ms": ms, "gflop": flops / 1e9, "tflops": tf,
+                   "frac_fp32_mfma_peak": tf / FP32_MFMA_PEAK_TFLOPS}
+            if pname in ahead:
+                preheat(be, ahead[pname], seconds=0.1)
+                row["ms_layout_ahead"] = batch_ms(be, ahead[pname], reps)
+            rows.append(row)
         del x, w, b, dy, y, gx, gw, gb
     total_ms = sum(r_["ms"] * r_["count"] for r_ in rows)
+    ahead_ms = sum(r_.get("ms_layout_ahead", r_["ms"]) * r_["count"] for r_ in rows)
     total_gflop = sum(r_["gflop"] * r_["count"] for r_ in rows)
     return {"per_layer": rows, "conv_ms_per_training_step": total_ms, "conv_gflop_per_training_step": total_gflop,
             "conv_tflops_whole_network": total_gflop / total_ms, "reps": reps,
+            "conv_ms_per_training_step_layouts_ahead": ahead_ms,
             "frac_fp32_mfma_peak_whole_network": total_gflop / total_ms / FP32_MFMA_PEAK_TFLOPS}
 
 

@@ -65,6 +65,28 @@ def test_conv_fwd_bwd_parity(gpu, n, c, h, w, k, r, s, sh, sw, pad):
     assert rel_l2(gb.numpy(), db_ref) <= TOL
 
 
+@pytest.mark.parametrize("n,c,h,w,k", [(2, 64, 28, 28, 128), (3, 32, 8, 12, 40), (2, 64, 27, 28, 64), (1, 96, 6, 6, 32)])
+def test_shortcut_bwd_data_overwrites_every_element(gpu, n, c, h, w, k):
+    """1 x 1 / 2 backward-data into a tensor that holds other values: the three residue classes no tap reaches must
+    come out as exact zeros (even sizes: written by the kernel's own epilogue; odd sizes: by a fill), whole and ragged
+    row tiles alike."""
+    K = gpu.kernels
+    rng = np.random.default_rng(c + h)
+    wt = he_normal(rng, (k, c, 1, 1))
+    oh, ow = K.conv_out_hw(h, w, 1, 1, (2, 2), 0)
+    dy = rng.standard_normal((n, k, oh, ow)).astype(np.float32)
+    ref = np.zeros((n, c, h, w), np.float32)
+    ref[:, :, ::2, ::2] = np.einsum("nkyx,kc->ncyx", dy.astype(np.float64), wt[:, :, 0, 0].astype(np.float64))
+    dx = gpu.to_device(np.full((n, c, h, w), 7.0, np.float32))
+    got = K.conv2d_bwd_data(gpu.to_device(dy), gpu.to_device(wt), (n, c, h, w), (2, 2), 0, dx=dx).numpy()
+    lattice = np.zeros((h, w), bool); lattice[::2, ::2] = True
+    assert np.all(got[:, :, ~lattice] == 0.0)
+    assert rel_l2(got, ref) <= TOL
+    twice = K.conv2d_bwd_data(gpu.to_device(dy), gpu.to_device(wt), (n, c, h, w), (2, 2), 0, dx=dx, accumulate=True).numpy()
+    assert np.all(twice[:, :, ~lattice] == 0.0)
+    assert rel_l2(twice, 2 * ref) <= TOL
+
+
 def test_conv_accumulates_into_existing_gradients(gpu):
     K = gpu.kernels
     rng = np.random.default_rng(7)

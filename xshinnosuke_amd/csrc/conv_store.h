@@ -6,6 +6,7 @@
 namespace xsmi {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
+typedef uint32_t uint32x2_store __attribute__((ext_vector_type(2)));
 
 // Register v of lane l holds row 8 (v / 4) + 4 (l / 32) + v % 4 and pixel l % 32 of the block whose first row is
 // `row0` (a multiple of 32 inside the tile) and whose pixels are m0 .. m0 + 31 of the launch's pixel numbering.
@@ -17,10 +18,16 @@ typedef float floatx16 __attribute__((ext_vector_type(16)));
 // out-of-range pixels through the buffer range check, and the bias / ReLU and mask / accumulate steps as passes over
 // the 16 registers, each behind one uniform branch.  Tensors hold fewer than 2^29 elements, so 32-bit byte offsets
 // suffice.  A ragged last row tile tests every row.
+//
+// zfill (overwriting only, os_x == 2 and os_y == two tensor rows): the lattice is the (even row, even column) class of
+// a stride-2 backward-data pass whose other three classes no tap reaches.  Each value is then stored together with
+// its right-hand neighbour, and the same two places of the row below are cleared, so that one launch writes every
+// element of the tensor once, in runs of eight bytes per pixel, and no separate fill is needed.
 template <typename G>
 __device__ __forceinline__ void store_block_32x32(const floatx16 &acc, const G &c, float *out, uint32_t out_bytes,
                                                   uint8_t *mask, const float *bias_lds, int relu, int accumulate,
-                                                  int tile_row0, int tile_rows, int row0, int m0, int lane) {
+                                                  int tile_row0, int tile_rows, int row0, int m0, int lane,
+                                                  int zfill = 0) {
     const int h = lane >> 5, l31 = lane & 31;
     const int lrow = row0 + 4 * h;                     // inside the tile
     const int m = m0 + l31;
@@ -62,6 +69,17 @@ __device__ __forceinline__ void store_block_32x32(const floatx16 &acc, const G &
 #pragma unroll
             for (int v = 0; v < 16; ++v) r[v] += old[v];
         }
+        if (zfill) {
+            const uint32_t below = (uint32_t)c.os_y * 2u;     // one tensor row, in bytes
+#pragma unroll
+            for (int v = 0; v < 16; ++v) {
+                const float val = r[v];
+                const uint32x2_store pair = {__builtin_bit_cast(uint32_t, val), 0u}, zeros = {0u, 0u};
+                __builtin_amdgcn_raw_buffer_store_b64(pair, rout, (int)voff, (int)row_off(v), 0);
+                __builtin_amdgcn_raw_buffer_store_b64(zeros, rout, (int)voff, (int)(row_off(v) + below), 0);
+            }
+            return;
+        }
 #pragma unroll
         for (int v = 0; v < 16; ++v) {
             const float val = r[v];                    // (a bit_cast applied to the vector element itself reads element 0)
@@ -84,6 +102,7 @@ __device__ __forceinline__ void store_block_32x32(const floatx16 &acc, const G &
             }
             if (accumulate) val += out[o];
             out[o] = val;
+            if (zfill) { out[o + 1] = 0.f; out[o + c.os_y / 2] = 0.f; out[o + c.os_y / 2 + 1] = 0.f; }
         }
     }
 }

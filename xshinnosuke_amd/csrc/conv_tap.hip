@@ -60,6 +60,7 @@ struct TapParams {
     long long os_n, os_k, o_base;
     int os_y, os_x;
     int accumulate, relu;
+    int zfill;            // 1: the epilogue also clears the three neighbours of every stored value (see conv_store.h)
     // persistent kernel only
     uint32_t *counters;   // 8 tile counters (one per XCD), zeroed by the pack kernel
     uint32_t tiles;       // pixel tiles x row tiles
@@ -268,7 +269,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_kernel(TapMulti mp) {
 
     // ---- epilogue ----
     xsmi::store_block_32x32(acc, p, p.out, p.out_bytes, p.mask, p.bias ? &s_bias[0] : nullptr, p.relu, p.accumulate, rowtile * TM, TM,
-                            wr * 32, m0 + wc * 32, lane);
+                            wr * 32, m0 + wc * 32, lane, p.zfill);
 }
 
 // Persistent form of the kernel above (same tile, same loop body, 2 stages).  A launch has at most
@@ -473,7 +474,7 @@ __global__ void __launch_bounds__(256) tap_igemm_f32_persist_kernel(TapParams p)
 
         // ---- epilogue ----
         xsmi::store_block_32x32(acc, p, p.out, p.out_bytes, p.mask, p.bias ? &s_bias[bias_buf][0] : nullptr, p.relu, p.accumulate,
-                                cur_rowtile * TM, TM, wr * 32, cur_m0 + wc * 32, lane);
+                                cur_rowtile * TM, TM, wr * 32, cur_m0 + wc * 32, lane, p.zfill);
         if (last_tile) {
             xsmi::wait_vmcnt<0>();                            // the dummy chunk's loads target this workgroup's LDS
             break;
@@ -1408,7 +1409,7 @@ int tap_conv_fwd(const float *x, const float *w, const float *bias, float *y, ui
     p.in_n_stride = C * H * W; p.plane_bytes = (uint32_t)(H * W * 4);
     p.OY = OH; p.OX = OW; p.dOX = make_fastdiv(OW); p.dOY = make_fastdiv(OH);
     p.os_n = (long long)K * OH * OW; p.os_k = (long long)OH * OW; p.o_base = 0; p.os_y = OW; p.os_x = 1;
-    p.accumulate = 0; p.relu = relu;
+    p.accumulate = 0; p.relu = relu; p.zfill = 0;
     p.tiles = 0; p.rowtiles = 0;
     p.apk_bytes = (uint32_t)tap_pack_bytes(K, C, R * S);
     p.counters = tap_counters(apk, tap_pack_bytes(K, C, R * S));
@@ -1577,20 +1578,24 @@ int tap_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, 
             p.OY = OYc; p.OX = OXc; p.dOX = make_fastdiv(OXc); p.dOY = make_fastdiv(OYc);
             p.os_n = (long long)C * H * W; p.os_k = (long long)H * W; p.o_base = (long long)ph * W + pw;
             p.os_y = sh * W; p.os_x = sw;
-            p.accumulate = accumulate; p.relu = 0;
+            p.accumulate = accumulate; p.relu = 0; p.zfill = 0;
             plans[nplans++] = p;
         }
     }
     // Residue classes no tap can reach (a stride larger than the filter: the 1 x 1 / 2 shortcuts leave three of four
-    // classes empty) receive no gradient.  Accumulating, they are left alone; overwriting, all of dx is cleared by one
-    // contiguous fill and only the classes with taps are computed, instead of tiles whose whole work is a strided
-    // store of zeros (64 -> 128 at 56 x 56, N=32: 25.8 -> 13 us).
+    // classes empty) receive no gradient.  Accumulating, they are left alone.  Overwriting, the fp32 1 x 1 / 2 pass
+    // over an even-sized tensor clears them from its own epilogue (every value is stored with its three zero
+    // neighbours: one launch, every element written once); other geometries clear all of dx with one contiguous fill
+    // first.  Only the classes with taps are computed, instead of tiles whose whole work is a strided store of zeros.
     {
         int kept = 0;
         for (int i = 0; i < nplans; ++i)
             if (plans[i].TR * plans[i].TS > 0) { plans[kept] = plans[i]; specs[kept] = specs[i]; ++kept; }
         if (kept < nplans) {
-            if (!accumulate && !(opts & 4)) {
+            const bool own_zeros = !(opts & 1) && !accumulate && kept == 1 && sh == 2 && sw == 2 && R == 1 && S == 1 &&
+                                   pad == 0 && H % 2 == 0 && W % 2 == 0 && plans[0].o_base == 0;
+            if (own_zeros) plans[0].zfill = 1;
+            else if (!accumulate && !(opts & 4)) {
                 int rc = xsmi_fill(dx, 0.f, (size_t)N * C * H * W);
                 if (rc) return rc;
             }
