@@ -27,6 +27,7 @@ Everything goes through libxsmi355.so; there is no fallback path.
 import argparse
 import json
 import os
+import re
 import statistics
 import sys
 import time
@@ -61,12 +62,21 @@ RESNET18_CONVS = [
 ]
 
 
-# HBM bytes per launch of tap_sk_f32_kernel on the CONV workload, from two hardware-counter runs (FETCH_SIZE
-# 33 452 KiB scaled by 1.9997, the factor that makes the plain copy kernel's known read size come out right, plus
-# WRITE_SIZE 50 220 KiB at factor 0.9999): 68.5 MB read + 51.4 MB written, against 25.7 MB each way for the operands
-# alone: the even-split schedule exchanges about a thousand 16 KB partial tiles per launch through memory
-# (written through, read back uncached) and keeps three times as many tiles in flight as the L2 slices hold.
-TAP_SK_TRAFFIC_BYTES = 119.9e6
+def tap_sk_traffic_bytes():
+    """HBM bytes per launch of the headline kernel on the CONV workload: measured with hardware counters (FETCH_SIZE and
+    WRITE_SIZE runs of `bench.py --traffic-run`, each scaled by what the same counter reads for the plain copy kernel)
+    and kept with the measurement, in the line of profiles/conv_pool_hbm_traffic_pmc.md that starts with
+    `roofline.traffic`.  None when that file is not there."""
+    path = os.path.join(ROOT, "profiles", "conv_pool_hbm_traffic_pmc.md")
+    try:
+        with open(path) as f:
+            for line in f:
+                m = re.match(r"\s*`?roofline\.traffic`?\s*[:=]\s*([0-9.]+(?:e[0-9]+)?)\s*bytes", line)
+                if m:
+                    return float(m.group(1))
+    except OSError:
+        pass
+    return None
 
 
 def conv_flops(c):
@@ -398,6 +408,8 @@ def bench_resnet18(be, steps, warmup):
     be.synchronize()
     wall = (time.perf_counter() - t0) * 1e3
     out = {"resnet18_train_images_per_sec": 32 * steps / (ms * 1e-3), "resnet18_ms_per_step": ms / steps,
+           # device memory beside tensors: shared and per-filter workspaces plus the library's own scratch
+           "resnet18_workspace_MB": be.workspace_bytes() / 1e6,
            "resnet18_wall_ms_per_step": wall / steps, "resnet18_host_enqueue_ms_per_step": enqueue / steps,
            "resnet18_last_loss": loss.item(),
            "resnet18_workload": "N=32x3x224x224 fp32, fwd+bwd+SGD, batch-statistics BN, device-resident, layer API"}
@@ -714,8 +726,8 @@ def main():
                    "gflop_per_step": 3 * flops_pass / 1e9},
         "frac_fp32_mfma_peak": value / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
-                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": TAP_SK_TRAFFIC_BYTES,
-                     "kernel": "tap_sk_f32_kernel<64, 64, 32, 1>", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
+                     "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": tap_sk_traffic_bytes(),
+                     "kernel": "tap_sk_f32_kernel<4>", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
         "ops_ms": {"conv_fwd": per["fwd"], "conv_bwd_data": per["bwd_data"], "conv_bwd_weight": per["bwd_weight"]},
         "kernels_ms": {"tap_sk_fwd": per["fwd_kernel"], "tap_sk_bwd_data": per["bwd_data_kernel"]},
         "ops_tflops": {k: flops_pass / (per[k] * 1e-3) / 1e12 for k in ("fwd", "bwd_data", "bwd_weight")},

@@ -80,6 +80,11 @@ int xsmi_init(int device);
 int xsmi_is_initialized(void);
 const char *xsmi_last_error(void);
 int xsmi_device_info(xsmi_device_info_t *info);
+/* Device memory the library itself holds on a GPU once initialised there: the exchange
+ * buffers of the even-split fp32 convolution kernels (one per stream of the library) and
+ * the static array of xsmi_conv2d_fwd_noalloc.  Everything else is the caller's
+ * (tensors, workspaces).  No counterpart in the reference. */
+size_t xsmi_scratch_bytes(void);
 int xsmi_malloc(void **ptr, size_t bytes);
 int xsmi_free(void *ptr);
 int xsmi_memcpy_h2d(void *dst, const void *src, size_t bytes);   /* blocking */
@@ -149,6 +154,16 @@ int xsmi_graph_destroy(void *graph);
  * over fwd / bwd_data / bwd_weight / bwd and over flags). */
 size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S,
                                    int sh, int sw, int pad);
+
+/* The same for one pass alone (0 forward, 1 backward-data, 2 backward-weight) with the
+ * given flags (XSMI_CONV_BF16 or 0): the size with which that pass's entry point picks
+ * its fastest kernel.  For callers that keep one workspace per filter and pass (a filter
+ * layout made ahead, XSMI_CONV_WS_PACKED): a ResNet-18 training step at N=32 then holds
+ * tens of megabytes of layouts instead of a full-size workspace per filter and pass.
+ * No counterpart in the reference (its conv2d allocates the im2col matrix per call,
+ * xs/utils/common.py:35-46).  Returns 0 for a bad geometry or pass. */
+size_t xsmi_conv2d_pass_workspace_bytes(int N, int C, int H, int W, int K, int R, int S,
+                                        int sh, int sw, int pad, int pass, unsigned flags);
 
 /* Forward: replaces conv2d (xs/nn/functional.py:405-442) incl. im2col
  * (xs/utils/common.py:35-46); with XSMI_CONV_RELU also the ReLU that

@@ -38,15 +38,24 @@ def _fresh_state(gpu):
 
 
 def _head(a, n=SLICE):
-    return a[0:n].numpy()
+    """The first and the last `n` images of a batch (0, 1, 30, 31 of 32): the last ones sit in the tail of every
+    kernel's pixel range, where ragged tiles and the ends of split reductions are."""
+    total = a.shape[0]
+    return np.concatenate([a[0:n].numpy(), a[total - n:total].numpy()])
+
+
+def _ends(a, n=SLICE):
+    return np.concatenate([a[:n], a[-n:]])
 
 
 def _before(a, n=None):
     """Contents an accumulating kernel will add to: zeros while the buffer's clear is still pending."""
     if a is None:
         return None
-    view = a if n is None else a[0:n]
-    return np.zeros(view.shape, np.float32) if a.is_fresh() else view.numpy()
+    if a.is_fresh():
+        shape = a.shape if n is None else (2 * n,) + tuple(a.shape[1:])
+        return np.zeros(shape, np.float32)
+    return a.numpy() if n is None else _head(a, n)
 
 
 class _Recorder:
@@ -136,7 +145,7 @@ def test_resnet18_training_step_at_full_size_against_oracle(gpu, monkeypatch):
     opt.step()
     assert np.isfinite(loss.item())
 
-    # ---- forward: the 20 convolutions and the max-pool on the first two images ----
+    # ---- forward: the 20 convolutions and the max-pool on the first two and the last two images ----
     assert len(rec.fwd) == 20 and len(rec.bwd) == 20 and len(rec.pool_fwd) == 1 and len(rec.pool_bwd) == 1
     geoms = set()
     for f in rec.fwd:
@@ -175,7 +184,7 @@ def test_resnet18_training_step_at_full_size_against_oracle(gpu, monkeypatch):
             assert (c, w_shape[2]) == (3, 7)     # only the stem has an input without a gradient
             seen_stem = True
             continue
-        dx_ref, _, _ = oracle.conv2d_bwd(b['dy'][:SLICE], (SLICE, c, h, w), b['w'], None, b['stride'], b['pad'],
+        dx_ref, _, _ = oracle.conv2d_bwd(_ends(b['dy']), (2 * SLICE, c, h, w), b['w'], None, b['stride'], b['pad'],
                                          b['dx0'].copy(), None, None)
         assert rel_l2(b['dx'], dx_ref) <= TOL, (b['x'].shape, w_shape, rel_l2(b['dx'], dx_ref))
     assert seen_stem

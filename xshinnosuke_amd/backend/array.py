@@ -1,6 +1,7 @@
 """Device-resident arrays owned by Python, allocated through the C ABI."""
 import ctypes
 import math
+import weakref
 
 import numpy as np
 
@@ -371,11 +372,22 @@ class PinnedArray:
             pass
 
 
+_WORKSPACES = weakref.WeakSet()
+
+
+def workspace_bytes():
+    """Device bytes beside the tensors: all live workspaces (the shared ones and the per-filter layout workspaces)
+    plus what the library holds itself (``xsmi_scratch_bytes``)."""
+    ensure_init()
+    return sum(w._block.nbytes for w in _WORKSPACES if w._block is not None) + int(lib.raw("xsmi_scratch_bytes")())
+
+
 class Workspace:
     """Grow-only scratch buffer handed to the conv entry points."""
 
     def __init__(self):
         self._block = None
+        _WORKSPACES.add(self)
 
     def __reduce__(self):
         raise TypeError("a device workspace cannot be pickled")

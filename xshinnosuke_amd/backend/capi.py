@@ -45,6 +45,7 @@ SIGNATURES = {
     "xsmi_is_initialized": (_i, []),
     "xsmi_last_error": (_c.c_char_p, []),
     "xsmi_device_info": (_i, [_c.POINTER(DeviceInfo)]),
+    "xsmi_scratch_bytes": (_sz, []),
     "xsmi_malloc": (_i, [_c.POINTER(_vp), _sz]),
     "xsmi_free": (_i, [_vp]),
     "xsmi_memcpy_h2d": (_i, [_vp, _vp, _sz]),
@@ -66,6 +67,7 @@ SIGNATURES = {
     "xsmi_last_kernel_ms": (_i, [_c.POINTER(_f)]),
     "xsmi_copy_kernel": (_i, [_vp, _vp, _sz]),
     "xsmi_conv2d_workspace_bytes": (_sz, _CONV_DIMS),
+    "xsmi_conv2d_pass_workspace_bytes": (_sz, _CONV_DIMS + [_i, _u]),
     "xsmi_conv2d_fwd": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u, _vp, _sz]),
     "xsmi_conv2d_fwd_noalloc": (_i, [_vp, _vp, _vp, _vp, _vp] + _CONV_DIMS + [_u]),
     "xsmi_conv2d_bwd_data": (_i, [_vp, _vp, _vp] + _CONV_DIMS + [_f, _u, _vp, _sz]),
@@ -165,7 +167,7 @@ class _Lib:
             raise XsmiError(msg)
 
 
-_QUERIES = frozenset(("xsmi_conv2d_workspace_bytes", "xsmi_bn_workspace_bytes", "xsmi_is_initialized", "xsmi_last_error"))
+_QUERIES = frozenset(("xsmi_scratch_bytes", "xsmi_conv2d_workspace_bytes", "xsmi_conv2d_pass_workspace_bytes", "xsmi_bn_workspace_bytes", "xsmi_is_initialized", "xsmi_last_error"))
 
 lib = _Lib()
 

@@ -44,6 +44,15 @@ def _need(dims):
     return need
 
 
+def _need_pass(dims, pass_):
+    """Workspace of one fp32 pass alone (0 forward, 1 backward-data): what a filter's layout workspace holds."""
+    key = (pass_,) + tuple(dims)
+    need = _NEED.get(key)
+    if need is None:
+        need = _NEED[key] = lib.raw("xsmi_conv2d_pass_workspace_bytes")(*dims, pass_, 0)
+    return need
+
+
 def conv2d_workspace_bytes(x_shape, w_shape, stride, pad):
     """Bytes of workspace the conv entry points want for this geometry."""
     return _need(_dims(x_shape, w_shape, stride, pad))
@@ -139,7 +148,7 @@ def refresh_layouts(arrays):
     if sig != _plan["sig"] or _array._CAPTURE[0] is not None:
         jobs = (capi.PackJob * len(todo))()
         for job, (v, e, (pass_, *dims)) in zip(jobs, todo):
-            ws, ws_bytes = e.ws.get(_need(dims))
+            ws, ws_bytes = e.ws.get(_need_pass(dims, pass_))
             job.w, job.workspace, job.workspace_bytes = v.ptr, ws.value, ws_bytes
             job.N, job.C, job.H, job.W, job.K, job.R, job.S, job.sh, job.sw, job.pad = dims
             job.pass_ = pass_
@@ -200,7 +209,10 @@ def conv2d_fwd(x, w, bias=None, stride=(1, 1), pad=0, relu=False, out=None, neg_
         if layout is not None:
             workspace = layout.ws
     flags = (CONV_RELU if relu else 0) | (CONV_BF16 if bf16 else 0) | (CONV_WS_PACKED if packed else 0)
-    ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(_need(dims))
+    if layout is not None:
+        ws, ws_bytes = workspace.get(_need_pass(dims, 0))
+    else:
+        ws, ws_bytes = _workspace(dims) if workspace is None else workspace.get(_need(dims))
     if channels_last and bf16 and neg_mask is None:
         xcl = x.channels_last()
         if xcl is not None and not (c % 32 == 0 and xcl.border >= pad):
@@ -250,7 +262,7 @@ def conv2d_bwd_data(dy, w, x_shape, stride=(1, 1), pad=0, dx=None, accumulate=Fa
     layout = None
     if keep_layout and _PREPACK and not bf16 and not packed:
         layout, packed = _layout_for(w, 1, dims)
-    ws, ws_bytes = _workspace(dims) if layout is None else layout.ws.get(_need(dims))
+    ws, ws_bytes = _workspace(dims) if layout is None else layout.ws.get(_need_pass(dims, 1))
     beta = _beta(accumulate, dx)
     wptr = ctypes.c_void_p(w.address()) if layout is not None and packed else w.cptr
     lib.call("xsmi_conv2d_bwd_data", dy.cptr, wptr, dx.cptr, *dims, beta,
@@ -306,7 +318,7 @@ def conv2d_bwd(dy, x, w, dx, dw, db=None, stride=(1, 1), pad=0, accumulate=False
     layout, packed = None, False
     if keep_layout and _PREPACK and not bf16:
         layout, packed = _layout_for(w, 1, dims)          # the data gradient's filter layout
-    ws, ws_bytes = _ws.get(need) if layout is None else layout.ws.get(need)
+    ws, ws_bytes = _ws.get(need) if layout is None else layout.ws.get(_need_pass(dims, 1))
     ws_dw, ws_dw_bytes = _ws_dw.get(need)
     beta_dw = _beta(accumulate, dw, db)
     beta_dx = _beta(accumulate, dx)

@@ -65,37 +65,40 @@ __global__ void __launch_bounds__(256) relu_mask_bwd2_kernel(const float *__rest
 
 extern "C" {
 
-size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad) {
+size_t xsmi_conv2d_pass_workspace_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad, int pass,
+                                        unsigned flags) {
     if (N <= 0 || C <= 0 || H <= 0 || W <= 0 || K <= 0 || R <= 0 || S <= 0 || sh <= 0 || sw <= 0 || pad < 0) return 0;
     if (H + 2 * pad < R || W + 2 * pad < S) return 0;
-    int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
-    size_t a = xsmi::conv_fwd_ws_bytes(C, K, R, S);
-    size_t b = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
-    size_t c = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
-    size_t m = a > b ? a : b;
-    m = m > c ? m : c;
-    if (xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad)) {
-        size_t e = xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad);
-        m = m > e ? m : e;
+    const int OH = (H + 2 * pad - R) / sh + 1, OW = (W + 2 * pad - S) / sw + 1;
+    const bool bf16 = (flags & XSMI_CONV_BF16) != 0;
+    auto larger = [](size_t a, size_t b) { return a > b ? a : b; };
+    size_t m = 0;
+    if (pass == 0) {
+        m = xsmi::conv_fwd_ws_bytes(C, K, R, S);
+        if (!bf16 && xsmi::stem_fwd_ok(N, C, H, W, K, R, S, sh, sw, pad))
+            m = larger(m, xsmi::stem_fwd_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad));
+        // the even-split fp32 kernels read their own filter layout (their partial tiles live in the library)
+        if (!bf16 && xsmi::sk_path_ok(C, K)) m = larger(m, xsmi::sk_fwd_ws_bytes(C, K, R, S));
+        // the bf16 forward takes its fastest form when the workspace also holds a channels-last copy of x
+        if (bf16 && xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad)) m = larger(m, xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad));
+    } else if (pass == 1) {
+        m = xsmi::conv_bwd_data_ws_bytes(C, K, R, S, sh, sw);
+        if (!bf16 && xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw)) m = larger(m, xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw));
+    } else if (pass == 2) {
+        m = xsmi::conv_bwd_weight_ws_bytes(N, C, K, R, S, OH, OW);
+        if (!bf16 && xsmi::stem_wgrad_ok(N, C, H, W, K, R, S, sh, sw, pad))
+            m = larger(m, xsmi::stem_wgrad_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad));
     }
-    if (xsmi::stem_wgrad_ok(N, C, H, W, K, R, S, sh, sw, pad)) {
-        size_t e = xsmi::stem_wgrad_ws_bytes(N, C, H, W, K, R, S, sh, sw, pad);
-        m = m > e ? m : e;
-    }
-    // the second-generation fp32 kernels are chosen when the workspace also has room for their partial tiles
-    if (xsmi::sk_path_ok(C, K)) {
-        size_t e = xsmi::sk_fwd_ws_bytes(C, K, R, S);
-        m = m > e ? m : e;
-    }
-    if (xsmi::sk_bwd_data_ok(C, K, R, S, sh, sw)) {
-        size_t e = xsmi::sk_bwd_data_ws_bytes(C, K, R, S, sh, sw);
-        m = m > e ? m : e;
-    }
-    // the bf16 forward takes its fastest form when the workspace also holds a channels-last copy of x
-    if (xsmi::nhwc_fwd_ok(N, C, H, W, K, R, S, pad)) {
-        size_t d = xsmi::nhwc_fwd_ws_bytes(N, C, H, W, K, R, S, pad);
-        m = m > d ? m : d;
-    }
+    return m;
+}
+
+size_t xsmi_conv2d_workspace_bytes(int N, int C, int H, int W, int K, int R, int S, int sh, int sw, int pad) {
+    size_t m = 0;
+    for (int pass = 0; pass < 3; ++pass)
+        for (unsigned flags : {0u, (unsigned)XSMI_CONV_BF16}) {
+            const size_t e = xsmi_conv2d_pass_workspace_bytes(N, C, H, W, K, R, S, sh, sw, pad, pass, flags);
+            m = m > e ? m : e;
+        }
     return m;
 }
 

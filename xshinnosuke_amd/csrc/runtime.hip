@@ -316,6 +316,10 @@ int xsmi_conv2d_bwd_join(void) {
     return xsmi::check_device_error("xsmi_conv2d_bwd_join");
 }
 
+size_t xsmi_scratch_bytes(void) {
+    return 2 * (xsmi::SK_SCRATCH_FLAG_BYTES + xsmi::SK_SCRATCH_PART_BYTES) + (size_t)XSMI_NOALLOC_SCRATCH_BYTES;
+}
+
 int xsmi_sync(void) {
     XSMI_REQUIRE_INIT();
     XSMI_NOT_WHILE_CAPTURING();
