@@ -242,10 +242,12 @@ def bench_per_layer(be, reps):
     reductions included), `reps` launches back to back between two events after a clock ramp.
 
     Each (layer, pass) is preceded by one fill launch of 1024 * (index + 1) floats, so that a kernel trace of this mode
-    can be cut into its rows: that launch shows up as `ew_kernel<FillF>` with a grid of 256 * (index + 1) threads."""
+    can be cut into its rows: that launch shows up as `ew_kernel<FillF>` with a grid of 256 * (index + 1) threads.  The
+    second timing of a forward or backward-data row (`ms_layout_ahead`: the filter's layout made ahead of the pass, as
+    a training step has it) follows a fill of 1024 * (index + 129) floats."""
     K = be.kernels
     rows = []
-    marker = be.empty((1024 * 3 * len(RESNET18_CONVS),))
+    marker = be.empty((1024 * (3 * len(RESNET18_CONVS) + 129),))
     rng = np.random.default_rng(11)
     for name, count, c, k, h, r, st, pad in RESNET18_CONVS:
         oh = (h + 2 * pad - r) // st + 1
@@ -276,6 +278,7 @@ def bench_per_layer(be, reps):
             row = {"layer": name, "count": count, "pass": pname, "ms": ms, "gflop": flops / 1e9, "tflops": tf,
                    "frac_fp32_mfma_peak": tf / FP32_MFMA_PEAK_TFLOPS}
             if pname in ahead:
+                be.lib.call("xsmi_fill", marker.cptr, 0.0, 1024 * (len(rows) + 129))
                 preheat(be, ahead[pname], seconds=0.1)
                 row["ms_layout_ahead"] = batch_ms(be, ahead[pname], reps)
             rows.append(row)

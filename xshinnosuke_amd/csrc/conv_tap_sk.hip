@@ -61,6 +61,12 @@ struct SkParams {
     uint32_t *err;         // set (system scope) when a wait for a partial tile ran out
     uint32_t in_bytes, apk_bytes, out_bytes, part_bytes;
     uint32_t units;        // chunks of all tiles of all classes
+    // Workgroup j of a grid of G takes the units [j * units / G, (j + 1) * units / G).  With units = upg * G + urem that
+    // is j * upg + (j * urem) / G: 32-bit arithmetic with one multiply-high (j * urem < G * G), where the 64-bit
+    // quotient costs the scalar unit some 250 instructions, twice when a workgroup starts and once or twice more where
+    // its range ends, while every workgroup of the launch stands at its own end and the matrix pipes are idle.
+    uint32_t upg, urem;
+    xsmi::FastDiv dG;
     uint32_t spin_limit;   // polls of a flag before giving up; 0: every wait counts as run out (error-path tests)
     int ncls, rowtiles, accumulate, relu;
 };
@@ -121,8 +127,8 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     const int wave = __builtin_amdgcn_readfirstlane(t >> 6);
     const uint32_t G = gridDim.x;
     const uint32_t g = xsmi::xcd_contiguous_id(blockIdx.x, G);       // neighbours in chunk order share an L2
-    const uint32_t u0 = (uint32_t)(((uint64_t)g * sp.units) / G);
-    const uint32_t u1 = (uint32_t)(((uint64_t)(g + 1) * sp.units) / G);
+    auto range_start = [&](uint32_t j) { return j * sp.upg + xsmi::fdiv(j * sp.urem, sp.dG); };
+    const uint32_t u0 = range_start(g), u1 = range_start(g + 1);
     const int rowtiles = sp.rowtiles;
 
     const xsmi::xsmi_int32x4 rin = xsmi::make_rsrc(sp.in, sp.in_bytes);
@@ -351,7 +357,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if (!c_complete) {
             // the rest of the tile was multiplied by the workgroups that follow: add their parts in chunk order
             for (uint32_t j = g + 1; j < G; ++j) {
-                const uint32_t js = (uint32_t)(((uint64_t)j * sp.units) / G);
+                const uint32_t js = range_start(j);
                 if (js >= c_tile_end) break;
                 if (t == 0) {
                     // spin_limit 0: every wait counts as run out (the host's way to exercise this path)
@@ -625,6 +631,7 @@ int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
                                    : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
     if (gsz > p.units) gsz = p.units;                  // every workgroup gets at least one chunk
     if (gsz == 0) return XSMI_OK;
+    p.upg = p.units / gsz; p.urem = p.units % gsz; p.dG = xsmi::make_fastdiv(gsz);
     // the library's partial-tile area of this stream; a wait that ran out in an earlier launch is reported here
     // (and by every call that waits for the device) instead of starting on flags that may be stale
     int rc = xsmi::check_device_error("even-split convolution");
