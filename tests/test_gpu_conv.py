@@ -409,3 +409,33 @@ def test_conv_combined_backward_rejects_bad_arguments(gpu):
         K.relu_mask_bwd2(dy, gpu.zeros(dy.shape, np.uint8), dx, dx)               # one buffer given twice
     gpu.synchronize()
     assert not capi.side_pending()
+
+
+@pytest.mark.parametrize("n,c,h,w,k,r,s,sh,sw,pad", [CASES[4], CASES[5], CASES[6], CASES[7], CASES[9], CASES[10]])
+def test_each_pass_runs_in_a_workspace_of_its_own_size(gpu, n, c, h, w, k, r, s, sh, sw, pad):
+    """xsmi_conv2d_pass_workspace_bytes is enough for its pass and selects the same kernel as the full-size workspace:
+    the three passes through the C ABI with exactly that many bytes give the wrappers' bits."""
+    import ctypes
+    from xshinnosuke_amd.backend import capi
+    K = gpu.kernels
+    rng = np.random.default_rng(77 + c + k)
+    x = gpu.to_device(rng.standard_normal((n, c, h, w)).astype(np.float32))
+    wt = gpu.to_device(he_normal(rng, (k, c, r, s)))
+    oh, ow = K.conv_out_hw(h, w, r, s, (sh, sw), pad)
+    dy = gpu.to_device(rng.standard_normal((n, k, oh, ow)).astype(np.float32))
+    dims = [n, c, h, w, k, r, s, sh, sw, pad]
+    y_ref = K.conv2d_fwd(x, wt, None, (sh, sw), pad).numpy()
+    dx_ref = K.conv2d_bwd_data(dy, wt, x.shape, (sh, sw), pad).numpy()
+    dw_ref = K.conv2d_bwd_weight(dy, x, wt.shape, (sh, sw), pad)[0].numpy()
+    size = [capi.lib.raw("xsmi_conv2d_pass_workspace_bytes")(*dims, p, 0) for p in range(3)]
+    assert all(v > 0 for v in size)
+    y = gpu.empty(y_ref.shape); dx = gpu.empty(dx_ref.shape); dw = gpu.empty(dw_ref.shape)
+    ws = [gpu.empty(((v + 3) // 4,)) for v in size]
+    capi.lib.call("xsmi_conv2d_fwd", x.cptr, wt.cptr, None, y.cptr, None, *dims, 0, ws[0].cptr, size[0])
+    capi.lib.call("xsmi_conv2d_bwd_data", dy.cptr, wt.cptr, dx.cptr, *dims, 0.0, 0, ws[1].cptr, size[1])
+    capi.lib.call("xsmi_conv2d_bwd_weight", dy.cptr, x.cptr, dw.cptr, None, *dims, 0.0, 0, ws[2].cptr, size[2])
+    assert y.numpy().tobytes() == y_ref.tobytes()
+    assert dx.numpy().tobytes() == dx_ref.tobytes()
+    assert dw.numpy().tobytes() == dw_ref.tobytes()
+    with pytest.raises(ValueError, match="workspace"):
+        capi.lib.call("xsmi_conv2d_fwd", x.cptr, wt.cptr, None, y.cptr, None, *dims, 0, ws[0].cptr, 16)
