@@ -104,8 +104,8 @@ int xsmi_sync(void);
  * workgroup gives up waiting for a partial tile; the calls that wait for the device then fail with
  * XSMI_ERR_RUNTIME), "sk_wide" (0: one-dword loads of the activations in the even-split kernel also where 16-byte
  * loads apply), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
- * several pieces; 0: one piece per workgroup), "tap_stages", "tap_persist",
- * "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
+ * several pieces; 0: one piece per workgroup), "pack_lanes" (1 to 4: streams over which xsmi_conv2d_pack deals its
+ * layout launches), "tap_stages", "tap_persist", "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
  * A caller that changes one must drop every workspace content it counted on (XSMI_CONV_WS_PACKED) and ask for
  * workspace sizes again.  No counterpart in the reference. */
 int xsmi_set_option(const char *name, long value);

@@ -125,8 +125,10 @@ def test_resnet18_steps_do_not_depend_on_filter_layouts_made_ahead(monkeypatch):
     and must not be used) and when the batch size changes for one step."""
     from xshinnosuke_amd.backend import kernels as K, capi
 
-    def run(ahead):
+    def run(ahead, lanes=None):
         monkeypatch.setattr(K, "_PREPACK", ahead)
+        if lanes is not None:
+            be.set_option("pack_lanes", lanes)
         np.random.seed(4)
         X = np.random.randn(8, 3, 64, 64).astype(np.float32)
         Y = np.random.randint(0, 10, (8,))
@@ -158,12 +160,22 @@ def test_resnet18_steps_do_not_depend_on_filter_layouts_made_ahead(monkeypatch):
         xs.GLOBAL.INPUTS = None
         return losses, out, sum(1 for _, f in flags if f & capi.CONV_WS_PACKED)
 
-    la, pa, skipped_a = run(True)
-    lb, pb, skipped_b = run(False)
+    from xshinnosuke_amd import backend as be
+    lanes0 = be.get_option("pack_lanes")
+    try:
+        la, pa, skipped_a = run(True)
+        lb, pb, skipped_b = run(False)
+        lc, pc, skipped_c = run(True, 1)                 # the layout launches in a row on one stream ...
+        ld, pd, skipped_d = run(True, 4)                 # ... and dealt over four
+    finally:
+        be.set_option("pack_lanes", lanes0)
     assert skipped_b == 0 and skipped_a >= 19 * 2        # steps 2 and 5 at least find every layout in place
-    assert la == lb
-    for u, v in zip(pa, pb):
+    assert skipped_c == skipped_a and skipped_d == skipped_a
+    assert la == lb and la == lc and la == ld
+    for u, v, w1, w4 in zip(pa, pb, pc, pd):
         np.testing.assert_array_equal(u, v)
+        np.testing.assert_array_equal(u, w1)
+        np.testing.assert_array_equal(u, w4)
 
 
 def test_resnet18_bf16_inference_against_oracle():

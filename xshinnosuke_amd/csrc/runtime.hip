@@ -39,7 +39,13 @@ OptionRow g_options[xsmi::OPT_COUNT] = {
     {"cl_stem", "XSMI_CL_STEM", 1, false},
     {"sk_wide", "XSMI_SK_WIDE", 1, false},
     {"pool_bwd", "XSMI_POOL_BWD", 2, false},
+    {"pack_lanes", "XSMI_PACK_LANES", 2, false},
 };
+
+// Streams beside the second one for runs of short independent launches (filter layouts), see side_lane().
+hipStream_t g_lanes[xsmi::SIDE_LANES] = {nullptr, nullptr, nullptr, nullptr};
+hipEvent_t g_lane_done[xsmi::SIDE_LANES] = {nullptr, nullptr, nullptr, nullptr};
+bool g_lane_used[xsmi::SIDE_LANES] = {false, false, false, false};
 
 // Partial tiles and flags of the even-split convolution kernels: one area per stream, owned by the library (a
 // launch's partial tiles are dead when it ends, and launches of one stream run one after the other).
@@ -65,6 +71,28 @@ int side_begin() {
     XSMI_HIP(hipStreamWaitEvent(g_side, g_fork, 0));
     g_current = g_side;
     g_side_pending = true;
+    return XSMI_OK;
+}
+int side_lane(int lane) {
+    if (lane <= 0 || lane >= SIDE_LANES) {
+        g_current = g_side;
+        return XSMI_OK;
+    }
+    if (!g_lane_used[lane]) {                           // the lane starts where the second stream started
+        XSMI_HIP(hipStreamWaitEvent(g_lanes[lane], g_fork, 0));
+        g_lane_used[lane] = true;
+    }
+    g_current = g_lanes[lane];
+    return XSMI_OK;
+}
+int side_lanes_end() {
+    for (int l = 1; l < SIDE_LANES; ++l)
+        if (g_lane_used[l]) {
+            g_lane_used[l] = false;
+            XSMI_HIP(hipEventRecord(g_lane_done[l], g_lanes[l]));
+            XSMI_HIP(hipStreamWaitEvent(g_side, g_lane_done[l], 0));
+        }
+    g_current = g_side;
     return XSMI_OK;
 }
 void side_end() { g_current = g_stream; }
@@ -178,6 +206,10 @@ int xsmi_init(int device) {
     XSMI_HIP(hipStreamCreateWithFlags(&g_side, hipStreamNonBlocking));
     XSMI_HIP(hipEventCreateWithFlags(&g_fork, hipEventDisableTiming));
     XSMI_HIP(hipEventCreateWithFlags(&g_join, hipEventDisableTiming));
+    for (int l = 1; l < xsmi::SIDE_LANES; ++l) {
+        XSMI_HIP(hipStreamCreateWithFlags(&g_lanes[l], hipStreamNonBlocking));
+        XSMI_HIP(hipEventCreateWithFlags(&g_lane_done[l], hipEventDisableTiming));
+    }
     for (int i = 0; i < 2; ++i) {
         void *p = nullptr;
         XSMI_HIP(hipMalloc(&p, xsmi::SK_SCRATCH_FLAG_BYTES + xsmi::SK_SCRATCH_PART_BYTES));

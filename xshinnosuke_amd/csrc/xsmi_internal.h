@@ -19,12 +19,18 @@ int side_begin();
 void side_end();
 int side_join();              // no-op when the second stream holds nothing the main stream has not waited for
 bool side_pending();
+// Inside a side section: spread independent short launches over the second stream (lane 0) and three more streams
+// (lanes 1-3), which start after the same point of the main stream; side_lanes_end() makes the second stream wait
+// for the others, so that side_join() covers all of them.  Launches of one lane run in order.
+constexpr int SIDE_LANES = 4;
+int side_lane(int lane);
+int side_lanes_end();
 bool on_side_stream();
 bool capturing();            // a step graph is being recorded: nothing runs, nothing may wait for the device
 bool ready();
 int cu_count();
 // Tuning switches (xsmi_set_option / environment variable / default); the order is that of the table in runtime.hip.
-enum Option { OPT_TAP_SK, OPT_SK_SPIN_LIMIT, OPT_TAP_STAGES, OPT_TAP_PERSIST, OPT_CL_HALO, OPT_CL_STEM, OPT_SK_WIDE, OPT_POOL_BWD, OPT_COUNT };
+enum Option { OPT_TAP_SK, OPT_SK_SPIN_LIMIT, OPT_TAP_STAGES, OPT_TAP_PERSIST, OPT_CL_HALO, OPT_CL_STEM, OPT_SK_WIDE, OPT_POOL_BWD, OPT_PACK_LANES, OPT_COUNT };
 long option(Option o);
 // Partial tiles and flags of the even-split convolution kernels for the stream that stream() hands out; allocated
 // by xsmi_init, the flags are zero between launches.
