@@ -56,7 +56,7 @@ struct SkParams {
     const float *bias;
     float *out;
     uint8_t *mask;
-    float *part;           // [grid][64 accumulator registers][256 threads]
+    float *part;           // [grid][16 accumulator registers][256 threads]
     uint32_t *flags;       // [grid], zero between launches
     uint32_t *err;         // set (system scope) when a wait for a partial tile ran out
     uint32_t in_bytes, apk_bytes, out_bytes, part_bytes;
