@@ -22,6 +22,10 @@ and ResNet-18 inference configurations, each beside the GPU figure in `extra`.
 `--per-layer` times every distinct ResNet-18 convolution (N=32) pass by pass and
 prints one JSON line with a row per (layer, pass).
 
+The ResNet-18 workloads of `extra` are a caller of the package, not part of it: the model
+(and the NumPy forward used as their CPU leg) is tests/resnet18.py, so the test tree has
+to be present beside this file; `--no-extra` runs without it.
+
 Everything goes through libxsmi355.so; there is no fallback path.
 """
 import argparse
