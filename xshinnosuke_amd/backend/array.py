@@ -379,7 +379,7 @@ def workspace_bytes():
     """Device bytes beside the tensors: all live workspaces (the shared ones and the per-filter layout workspaces)
     plus what the library holds itself (``xsmi_scratch_bytes``)."""
     ensure_init()
-    return sum(w._block.nbytes for w in _WORKSPACES if w._block is not None) + int(lib.raw("xsmi_scratch_bytes")())
+    return sum(w._block.nbytes for w in list(_WORKSPACES) if w._block is not None) + int(lib.raw("xsmi_scratch_bytes")())
 
 
 class Workspace:
