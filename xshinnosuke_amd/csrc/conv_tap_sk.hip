@@ -210,19 +210,25 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
             ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
         }
     };
-    // `stage`: byte address of the LDS stage the chunk goes to
-    auto issue_b = [&](int e, uint32_t stage) {
+    // The LDS place of a load is a wave-uniform base (which of the chunk's channels / filter rows this wave fetches)
+    // plus a constant of the unrolled loop body (stage, which of the wave's loads): the constant rides in the load
+    // statement itself.
+    const uint32_t lds_b = lds0 + (uint32_t)((VEC == 4 ? chan0 * PIX : chan0 * PIX + pb * 64) * 4);
+    const uint32_t lds_a = lds0 + (uint32_t)(wave * NA * (ROWS / RT) * 16);
+    static_assert(RT == 1, "A wave-load f of a chunk is quad f");
+    auto issue_b = [&](auto e_, auto st_) {
+        constexpr int e = decltype(e_)::value, st = decltype(st_)::value;
         if constexpr (VEC == 4)                        // channels chan0 + 4 e .. + 3, the tile's 64 pixels
-            xsmi::load_lds_b128(rin, stage + (uint32_t)((A_FLOATS + (chan0 + 4 * e) * PIX) * 4), ld_voff,
-                                ld_soff + (uint32_t)(4 * e) * i_plane);
+            xsmi::load_lds_b128_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + 4 * e * PIX) * 4)>(rin, lds_b, ld_voff,
+                                                                                                  ld_soff + (uint32_t)(4 * e) * i_plane);
         else                                           // channel chan0 + e of the chunk, this wave's 64 pixels
-            xsmi::load_lds_b32(rin, stage + (uint32_t)((A_FLOATS + (chan0 + e) * PIX + pb * 64) * 4), ld_voff,
-                               ld_soff + (uint32_t)e * i_plane);
+            xsmi::load_lds_b32_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + e * PIX) * 4)>(rin, lds_b, ld_voff,
+                                                                                             ld_soff + (uint32_t)e * i_plane);
     };
-    auto issue_a = [&](int e, uint32_t stage) {        // 64 rows of one quad
-        const int f = wave * NA + e, q = f / RT, rh = f % RT;
-        const uint32_t off = (uint32_t)((q * ROWS + rh * 64) * 16);
-        xsmi::load_lds_b128(rap, stage + off, a_lane + off, ld_asoff);
+    auto issue_a = [&](auto e_, auto st_) {           // 64 rows of quad wave * NA + e
+        constexpr int e = decltype(e_)::value, st = decltype(st_)::value;
+        const uint32_t off = (uint32_t)((wave * NA + e) * ROWS * 16);
+        xsmi::load_lds_b128_at<(uint32_t)(st * STAGE_FLOATS * 4 + e * ROWS * 16)>(rap, lds_a, a_lane + off, ld_asoff);
     };
     // VEC = 4, after the chunk's loads have landed and before the barrier that publishes them: border columns are
     // overwritten with zero, moved runs are put in place.  `stage_floats`: float offset of that stage.
@@ -269,10 +275,9 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     // the stage a chunk is loaded into follows from where the call stands in the unrolled loop (`st_`: 0 or 1)
     auto issue_item_at = [&](auto ic, auto st_) {
         constexpr int n = decltype(ic)::value;
-        const uint32_t stage = lds0 + (uint32_t)(decltype(st_)::value * STAGE_FLOATS * 4);
         if constexpr (n == 0) issue_prep();
-        else if constexpr (n >= 1 && n <= NBW) issue_b(n - 1, stage);
-        else if constexpr (n > NBW && n <= NBW + NA) issue_a(n - 1 - NBW, stage);
+        else if constexpr (n >= 1 && n <= NBW) issue_b(IC<n - 1>{}, st_);
+        else if constexpr (n > NBW && n <= NBW + NA) issue_a(IC<n - 1 - NBW>{}, st_);
         else if constexpr (n == NBW + NA + 1) issue_advance();
     };
     auto issue_all_at = [&](auto st_) { static_for<NI>([&](auto ic) { issue_item_at(ic, st_); }); };

@@ -234,6 +234,30 @@ __device__ __forceinline__ void load_lds_b128(xsmi_int32x4 rsrc, uint32_t lds_ad
 #endif
 }
 
+// The same with the LDS address formed inside the statement as lds_base + IMM (IMM a compile-time constant): a loop
+// whose loads go to a few fixed places of each stage then keeps one wave-uniform base alive instead of one address per
+// load and stage.  (Addresses formed outside are loop invariants to the compiler, which keeps each in a scalar
+// register of its own and, when those run out, in a lane of a vector register: the reload between two MFMAs costs a
+// vector instruction and the wait states before a scalar register written by one may be used.)
+template <uint32_t IMM>
+__device__ __forceinline__ void load_lds_b32_at(xsmi_int32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    soff = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("s_add_u32 m0, %0, %4\n\tbuffer_load_dword %1, %2, %3 offen lds"
+                 :: "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory", "scc");
+#endif
+}
+template <uint32_t IMM>
+__device__ __forceinline__ void load_lds_b128_at(xsmi_int32x4 rsrc, uint32_t lds_base, uint32_t voff, uint32_t soff) {
+#if defined(__HIP_DEVICE_COMPILE__)
+    lds_base = __builtin_amdgcn_readfirstlane(lds_base);
+    soff = __builtin_amdgcn_readfirstlane(soff);
+    asm volatile("s_add_u32 m0, %0, %4\n\tbuffer_load_dwordx4 %1, %2, %3 offen lds"
+                 :: "s"(lds_base), "v"(voff), "s"(rsrc), "s"(soff), "n"(IMM) : "memory", "scc");
+#endif
+}
+
 // s_waitcnt that constrains only the vector-memory counter (gfx9 encoding:
 // vmcnt in bits 3:0 and 15:14, expcnt 6:4, lgkmcnt 11:8).
 template <int N>
