@@ -360,35 +360,51 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
             return;
         }
         if (!c_complete) {
-            // the rest of the tile was multiplied by the workgroups that follow: add their parts in chunk order
-            for (uint32_t j = g + 1; j < G; ++j) {
-                const uint32_t js = range_start(j);
-                if (js >= c_tile_end) break;
+            // The rest of the tile was multiplied by the workgroups that follow: add their parts in chunk order.  Up to
+            // three parts are fetched in one round trip (a tile of many chunks is shared by several workgroups, and
+            // every one of them stands at the end of its range when the owner asks); they are added one after the
+            // other, so the sum is the same as with one part at a time.
+            for (uint32_t j = g + 1; j < G; j += 3) {
+                if (range_start(j) >= c_tile_end) break;
+                const uint32_t n = j + 1 < G && range_start(j + 1) < c_tile_end
+                                       ? (j + 2 < G && range_start(j + 2) < c_tile_end ? 3u : 2u) : 1u;
                 if (t == 0) {
                     // spin_limit 0: every wait counts as run out (the host's way to exercise this path)
-                    uint32_t spins = 0;
-                    bool there = false;
-                    while (sp.spin_limit != 0u &&
-                           !(there = __hip_atomic_load(sp.flags + j, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) &&
-                           ++spins < sp.spin_limit)
-                        __builtin_amdgcn_s_sleep(2);
-                    if (!there) {
-                        // Give up: the host finds the word at its next check and reports the launch as failed.  Neither
-                        // this tile nor any later one of the workgroup is stored, and the late partial's flag stays
-                        // raised for the host to clear.
-                        s_fail = 1u;
-                        __hip_atomic_store(sp.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                    for (uint32_t i = 0; i < n; ++i) {
+                        uint32_t spins = 0;
+                        bool there = false;
+                        while (sp.spin_limit != 0u &&
+                               !(there = __hip_atomic_load(sp.flags + j + i, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0u) &&
+                               ++spins < sp.spin_limit)
+                            __builtin_amdgcn_s_sleep(2);
+                        if (!there) {
+                            // Give up: the host finds the word at its next check and reports the launch as failed.
+                            // Neither this tile nor any later one of the workgroup is stored, and the late partial's
+                            // flag stays raised for the host to clear.
+                            s_fail = 1u;
+                            __hip_atomic_store(sp.err, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+                            break;
+                        }
                     }
                 }
                 __syncthreads();
                 if (s_fail) return;
-                float part[16];
+                float part[3][16];
 #pragma unroll
-                for (int v = 0; v < 16; ++v) part[v] = buf_load<AGENT>(rpart, (uint32_t)t * 4u, j * PART_BYTES + (uint32_t)v * 1024u);
+                for (int i = 0; i < 3; ++i)
+                    if ((uint32_t)i < n) {
 #pragma unroll
-                for (int v = 0; v < 16; ++v) acc[0][v] += part[v];
-                __syncthreads();                       // everybody has read the part before its flag is cleared
-                if (t == 0) __hip_atomic_store(sp.flags + j, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+                        for (int v = 0; v < 16; ++v)
+                            part[i][v] = buf_load<AGENT>(rpart, (uint32_t)t * 4u, (j + (uint32_t)i) * PART_BYTES + (uint32_t)v * 1024u);
+                    }
+#pragma unroll
+                for (int i = 0; i < 3; ++i)
+                    if ((uint32_t)i < n) {
+#pragma unroll
+                        for (int v = 0; v < 16; ++v) acc[0][v] += part[i][v];
+                    }
+                __syncthreads();                       // everybody has read the parts before their flags are cleared
+                if ((uint32_t)t < n) __hip_atomic_store(sp.flags + j + (uint32_t)t, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
             }
         }
         if (s_fail) return;
