@@ -109,3 +109,16 @@ def test_dense_activation_names_one_training_step():
         np.testing.assert_allclose(g.reshape(w.shape) if g.size == w.size else g, w.reshape(g.shape), rtol=1e-9, atol=1e-12)
     assert get_activator('no-such-activation') is None and get_activator(None) is None
     assert Dense(3, activation='no-such-activation')._act_layer is None
+
+
+def test_bench_reads_its_traffic_figure_from_the_committed_profile():
+    """bench.py's roofline.traffic is the figure kept beside its measurement in profiles/, not a number typed into
+    the benchmark: the line is there and parses to a plausible byte count (algorithmic bytes of the launch: 51.5 MB)."""
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("bench_for_test", os.path.join(root, "bench.py"))
+    bench = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(bench)
+    traffic = bench.tap_sk_traffic_bytes()
+    assert traffic is not None and 51.5e6 <= traffic <= 200e6
