@@ -250,7 +250,6 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
                     }
                 }
             }
-            xsmi::wait_lgkmcnt0();
             asm volatile("" ::: "memory");
         }
     };
@@ -446,13 +445,20 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         };
         auto body = [&](auto buf_) {
             constexpr int cur = decltype(buf_)::value, nxt = cur ^ 1;
+            if constexpr (VEC == 4) {
+                // the border columns of the chunk that has just landed are cleared first and the LDS writes complete
+                // behind the chunk's first four MFMAs, not between the wait for the loads and the barrier
+                xsmi::wait_vmcnt<0>();
+                fix_borders(nxt * STAGE_FLOATS, ld_fix);   // the chunk that has just landed is the one issued last
+                XSMI_PIN();
+            }
             XSMI_MFMA(acc[0], fa[cur][0].x, fb[cur][0]);
             XSMI_MFMA(acc[1], fa[cur][0].y, fb[cur][1]);
             XSMI_MFMA(acc[0], fa[cur][0].z, fb[cur][2]);
             XSMI_MFMA(acc[1], fa[cur][0].w, fb[cur][3]);
             XSMI_PIN();
-            xsmi::wait_vmcnt<0>();
-            fix_borders(nxt * STAGE_FLOATS, ld_fix);   // the chunk that has just landed is the one issued last
+            if constexpr (VEC == 4) xsmi::wait_lgkmcnt0();
+            else xsmi::wait_vmcnt<0>();
             xsmi::block_barrier();
             XSMI_PIN();
             const float *base = &smem[0][0] + nxt * STAGE_FLOATS;
@@ -495,6 +501,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         compute_segment();
         xsmi::wait_vmcnt<0>();
         fix_borders(0, ld_fix);
+        xsmi::wait_lgkmcnt0();
         xsmi::block_barrier();
         read_chunk(IC<0>{});
         issue_all_at(IC<1>{});
