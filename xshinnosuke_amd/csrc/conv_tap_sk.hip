@@ -112,7 +112,9 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     constexpr int RT = ROWS / 64, PT = PIX / 64;     // 64-row / 64-pixel blocks of the tile (units of one wave-load)
     constexpr int QUADS = KC / 4;                    // 16-byte channel groups of a chunk
     constexpr int GROUPS = KC / 8;
-    constexpr int A_FLOATS = ROWS * KC, B_FLOATS = PIX * KC, STAGE_FLOATS = A_FLOATS + B_FLOATS;
+    // VEC = 4: a stage ends with two rows of 256 slots that take the zero writes of lanes whose run has no border column
+    constexpr int SPARE_FLOATS = VEC == 4 ? 512 : 0;
+    constexpr int A_FLOATS = ROWS * KC, B_FLOATS = PIX * KC, STAGE_FLOATS = A_FLOATS + B_FLOATS + SPARE_FLOATS;
     constexpr int NA = QUADS * RT / 4;               // A wave-loads (64 rows x 16 bytes) per wave and chunk
     constexpr int NB = KC * PT / 4;                  // B wave-loads (64 pixels of one channel) per wave and chunk
     constexpr int NBW = NB / VEC;                    // ... as VEC-wide loads
@@ -150,7 +152,8 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     uint32_t prep_stale = 1;                           // the pixel offset must be formed again (new segment); the uniform
                                                        // flags are integers so that they live in one scalar register each
     uint32_t ld_asoff = 0, ld_voff = 0, ld_soff = 0;
-    int ld_fix = 0;                                    // VEC = 4: what the lane does to its run once it has landed (issue_prep)
+    int ld_fix = 0;                                    // VEC = 4: the slot the lane clears once its run has landed (issue_prep)
+    uint32_t ld_rare = 0;                              // VEC = 4, uniform: a lane of this wave has a run to move (see issue_prep)
     const int csub = VEC == 4 ? lane >> 4 : 0;         // VEC = 4: which of the wave-load's four channels the lane fetches
     const uint32_t a_lane = (uint32_t)lane * 16u;
 
@@ -195,16 +198,20 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if constexpr (VEC == 4) {
             // The lane's run is columns ix .. ix + 3 of one input row; ix = -1 and ix + 3 = IW (one column past either
             // end) are the cases the host admits.  The run is fetched as it lies and the border column's slot is
-            // cleared once it has landed (fix 1: first slot, 2: last slot), except where the run would leave the tensor
-            // at its very beginning or end: there the four columns inside the row are fetched and moved by one place
-            // afterwards (fix 3 / 4: a handful of lanes of the whole launch).
+            // cleared once it has landed: EVERY lane clears one slot per load then, without a test, the lanes without
+            // a border column a spare slot of their own behind the stage's data.  At the very end of the tensor the
+            // buffer's range check has already returned zero for the dword past it.  At its very beginning the whole
+            // run would count as out of range: there the four columns inside the row are fetched and moved by one
+            // place afterwards (the wave concerned takes a slower path for that tap: ld_rare).
             int off = nbase + iy * i_IW + ix;
-            int fix = ix < 0 ? 1 : (ix + 4 > i_IW ? 2 : 0);
-            if (fix == 1 && off < 0) { off += 1; fix = 3; }
-            if (fix == 2 && (uint32_t)(off + 4) * 4u > sp.in_bytes) { off -= 1; fix = 4; }
+            const int fix = ix < 0 ? 1 : (ix + 4 > i_IW ? 2 : 0);
             const bool ok = live && (unsigned)iy < (unsigned)i_IH;
+            const bool moved = ok && fix == 1 && off < 0;
+            if (moved) off += 1;
             ld_voff = ok ? (uint32_t)(off * 4) : 0x80000000u;
-            ld_fix = ok ? fix : 0;
+            const int run = A_FLOATS + chan0 * PIX + lane * 4;
+            ld_fix = !ok || fix == 0 ? A_FLOATS + B_FLOATS + t : moved ? (run | 0x40000000) : run + (fix == 1 ? 0 : 3);
+            ld_rare = (uint32_t)__builtin_amdgcn_readfirstlane(__builtin_amdgcn_ballot_w64(moved) != 0ull ? 1 : 0);
         } else {
             bool ok = live && (unsigned)iy < (unsigned)i_IH && (unsigned)ix < (unsigned)i_IW;
             ld_voff = ok ? (uint32_t)((nbase + iy * i_IW + ix) * 4) : 0x80000000u;
@@ -235,20 +242,20 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     auto fix_borders = [&](int stage_floats, int fix) {
         if constexpr (VEC == 4) {
             asm volatile("" ::: "memory");
-            if (fix != 0) {
-                float *run = &smem[0][0] + stage_floats + A_FLOATS + chan0 * PIX + lane * 4;    // wave-load e: + 4 e PIX
-                if (fix <= 2) {
-                    float *z = run + (fix == 1 ? 0 : 3);
+            float *stage = &smem[0][0] + stage_floats;
+            if (!ld_rare) {                            // uniform
 #pragma unroll
-                    for (int e = 0; e < NBW; ++e) z[4 * e * PIX] = 0.f;
-                } else {
+                for (int e = 0; e < NBW; ++e) stage[fix + 4 * e * PIX] = 0.f;
+            } else if (fix & 0x40000000) {
 #pragma unroll
-                    for (int e = 0; e < NBW; ++e) {
-                        float4 *q4 = reinterpret_cast<float4 *>(run + 4 * e * PIX);
-                        const float4 v = *q4;
-                        *q4 = fix == 3 ? make_float4(0.f, v.x, v.y, v.z) : make_float4(v.y, v.z, v.w, 0.f);
-                    }
+                for (int e = 0; e < NBW; ++e) {
+                    float4 *q4 = reinterpret_cast<float4 *>(stage + (fix & 0xffff) + 4 * e * PIX);
+                    const float4 v = *q4;
+                    *q4 = make_float4(0.f, v.x, v.y, v.z);
                 }
+            } else {
+#pragma unroll
+                for (int e = 0; e < NBW; ++e) stage[fix + 4 * e * PIX] = 0.f;
             }
             asm volatile("" ::: "memory");
         }
