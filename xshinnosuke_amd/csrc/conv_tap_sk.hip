@@ -69,6 +69,10 @@ struct SkParams {
     xsmi::FastDiv dG;
     uint32_t spin_limit;   // polls of a flag before giving up; 0: every wait counts as run out (error-path tests)
     int ncls, rowtiles, accumulate, relu;
+    // staged rows (one class; a unit is a filter row x 16 channels, the filter laid out per unit as three taps)
+    int staged_rows;
+    int out_rows;          // output rows of all images
+    xsmi::FastDiv dPitch;  // by (output row length + 4)
 };
 
 template <int N>
@@ -104,22 +108,34 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t vof
 // one-dword form.  A run that reaches one column past a row end is fetched as it lies, so the slot of the border
 // column holds the neighbouring row's last or first value; the lane overwrites that slot with zero once the load has
 // landed, between the wait for the loads and the workgroup barrier.
+//
+// VEC = 3 (launches of one class; 3 x 3 taps that shift the input by -1, 0, +1 columns over rows as wide as the
+// output's, a multiple of four pixels and at least 20): the unit of work is one filter ROW x 16 channels.  The
+// tile's input pixels of that row are staged once for the row's three taps, as one run per channel in which every
+// image row is followed by four slots of zeros: a tap is then a shift of the fragment read by one slot, and the slot
+// past either end of a row is a zero that the loads themselves wrote (the lanes of those slots fetch out of range).
+// 16-byte loads, nothing to clear, a third of the activation traffic, one barrier per 24 MFMAs.
 template <int VEC>
 __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
-    static_assert(VEC == 1 || VEC == 4, "B loads of one or four dwords per lane");
-    constexpr int ROWS = SK_ROWS, PIX = SK_PIX, KC = SK_KC;
+    static_assert(VEC == 1 || VEC == 4 || VEC == 3, "B loads of one or four dwords per lane, or staged rows");
+    constexpr bool ROW = VEC == 3;
+    constexpr int ROWS = SK_ROWS, PIX = SK_PIX, KC = ROW ? 16 : SK_KC;
+    constexpr int UTAPS = ROW ? 3 : 1;               // taps per unit of work
+    constexpr int BPITCH = 128;                      // ROW: floats from one channel's run to the next (a run has 84)
     constexpr int WCn = PIX / 32;                    // waves along pixels (2 x 2 waves of 32 x 32)
     constexpr int RT = ROWS / 64, PT = PIX / 64;     // 64-row / 64-pixel blocks of the tile (units of one wave-load)
     constexpr int QUADS = KC / 4;                    // 16-byte channel groups of a chunk
     constexpr int GROUPS = KC / 8;
     // VEC = 4: a stage ends with two rows of 256 slots that take the zero writes of lanes whose run has no border column
     constexpr int SPARE_FLOATS = VEC == 4 ? 512 : 0;
-    constexpr int A_FLOATS = ROWS * KC, B_FLOATS = PIX * KC, STAGE_FLOATS = A_FLOATS + B_FLOATS + SPARE_FLOATS;
-    constexpr int NA = QUADS * RT / 4;               // A wave-loads (64 rows x 16 bytes) per wave and chunk
+    constexpr int A_FLOATS = ROWS * KC * UTAPS, B_FLOATS = ROW ? KC * BPITCH : PIX * KC;
+    constexpr int STAGE_FLOATS = A_FLOATS + B_FLOATS + SPARE_FLOATS;
+    constexpr int NA = UTAPS * QUADS * RT / 4;       // A wave-loads (64 rows x 16 bytes) per wave and chunk
     constexpr int NB = KC * PT / 4;                  // B wave-loads (64 pixels of one channel) per wave and chunk
-    constexpr int NBW = NB / VEC;                    // ... as VEC-wide loads
+    constexpr int NBW = ROW ? 2 : NB / VEC;          // ... as VEC-wide loads; ROW: two channels' runs per wave-load
     constexpr int NI = NBW + NA + 2;                 // issue items per chunk: prepare, B loads, A loads, advance
-    static_assert(NB == 8 && NA == 2 && NI <= 12, "64 x 64 tile, 32-channel chunks: the issue items fit the slots of one chunk");
+    static_assert(ROW ? (NA == 3 && NI == 7) : (NB == 8 && NA == 2 && NI <= 12),
+                  "64 x 64 tile: the issue items fit the slots of one chunk");
     __shared__ __attribute__((aligned(16))) float smem[2][STAGE_FLOATS];
     __shared__ __attribute__((aligned(16))) float s_bias[2][ROWS];
     __shared__ uint32_t s_fail;                        // a wait of this workgroup ran out: its tiles are not stored
@@ -171,15 +187,36 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if (n_seg > u1 - iu) n_seg = u1 - iu;
         i_left = n_seg;
         prep_stale = 1;
-        i_nch = c.nch; i_TS = c.TS; i_dstep = c.dstep; i_IH = c.IH; i_IW = c.IW; i_plane = c.plane_bytes;
-        const uint32_t tap = ch / (uint32_t)c.nch;
+        i_nch = c.nch; i_TS = ROW ? 1 : c.TS; i_dstep = c.dstep; i_IH = c.IH; i_IW = c.IW; i_plane = c.plane_bytes;
+        const uint32_t tap = ch / (uint32_t)c.nch;    // ROW: the filter row
         cc = (int)(ch - tap * (uint32_t)c.nch);
-        r = (int)(tap / (uint32_t)c.TS);
-        s = (int)(tap - (uint32_t)r * (uint32_t)c.TS);
-        ld_asoff = c.apk_off + (rt * c.iters + ch) * (uint32_t)(ROWS * KC * 4);
+        r = ROW ? (int)tap : (int)(tap / (uint32_t)c.TS);
+        s = ROW ? 0 : (int)(tap - (uint32_t)r * (uint32_t)c.TS);
+        ld_asoff = c.apk_off + (rt * c.iters + ch) * (uint32_t)(A_FLOATS * 4);
+        iyb = 0; ixb = 0; nbase = 0;
+        if constexpr (ROW) {
+            // The lane's piece is piece `lane & 31` of a channel's run: four slots of the run, which starts four slots
+            // before the tile's first pixel.  In run coordinates an image row is OX + 4 slots long; a piece is either
+            // four pixels of one output row (then it is fetched from the input row the tap row reaches from there, same
+            // columns) or a row's trailing zeros (then the lane fetches out of range, like a row outside the image).
+            const int piece = lane & 31;
+            const int m0 = (int)mt * PIX;
+            const uint32_t ry0 = xsmi::fdiv((uint32_t)m0, c.dOX);
+            const int pitch = c.OX + 4;
+            const int X = m0 - (int)ry0 * c.OX - 4 + 4 * piece + pitch;        // >= 0: counted from the row before
+            const uint32_t d = xsmi::fdiv((uint32_t)X, sp.dPitch);
+            const int xx = X - (int)d * pitch;
+            const int row = (int)ry0 + (int)d - 1;
+            live = piece < 21 && xx < c.OX && (unsigned)row < (unsigned)sp.out_rows;
+            if (live) {
+                const uint32_t n = xsmi::fdiv((uint32_t)row, c.dOY);
+                iyb = (row - (int)n * c.OY) + c.dy0;
+                nbase = (int)n * c.in_n_stride + (lane >> 5) * (int)(c.plane_bytes >> 2) + xx;
+            }
+            return;
+        }
         const int m = VEC == 4 ? (int)mt * PIX + 4 * (lane & 15) : (int)mt * PIX + pb * 64 + lane;
         live = m < c.M;
-        iyb = 0; ixb = 0; nbase = 0;
         if (live) {
             uint32_t q = xsmi::fdiv((uint32_t)m, c.dOX);
             int x = m - (int)q * c.OX;
@@ -195,7 +232,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if (cc != 0 && !prep_stale) return;            // same tap as the previous chunk: same pixel offset
         prep_stale = 0;
         const int iy = iyb + r * i_dstep, ix = ixb + s * i_dstep;
-        if constexpr (VEC == 4) {
+        if constexpr (ROW) {
+            const bool ok = live && (unsigned)iy < (unsigned)i_IH;
+            ld_voff = ok ? (uint32_t)((nbase + iy * i_IW) * 4) : 0x80000000u;
+        } else if constexpr (VEC == 4) {
             // The lane's run is columns ix .. ix + 3 of one input row; ix = -1 and ix + 3 = IW (one column past either
             // end) are the cases the host admits.  The run is fetched as it lies and the border column's slot is
             // cleared once it has landed: EVERY lane clears one slot per load then, without a test, the lanes without
@@ -220,12 +260,15 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     // The LDS place of a load is a wave-uniform base (which of the chunk's channels / filter rows this wave fetches)
     // plus a constant of the unrolled loop body (stage, which of the wave's loads): the constant rides in the load
     // statement itself.
-    const uint32_t lds_b = lds0 + (uint32_t)((VEC == 4 ? chan0 * PIX : chan0 * PIX + pb * 64) * 4);
+    const uint32_t lds_b = lds0 + (uint32_t)((ROW ? chan0 * BPITCH : VEC == 4 ? chan0 * PIX : chan0 * PIX + pb * 64) * 4);
     const uint32_t lds_a = lds0 + (uint32_t)(wave * NA * (ROWS / RT) * 16);
     static_assert(RT == 1, "A wave-load f of a chunk is quad f");
     auto issue_b = [&](auto e_, auto st_) {
         constexpr int e = decltype(e_)::value, st = decltype(st_)::value;
-        if constexpr (VEC == 4)                        // channels chan0 + 4 e .. + 3, the tile's 64 pixels
+        if constexpr (ROW)                             // channels chan0 + 2 e and + 2 e + 1: 32 pieces each, 21 in use
+            xsmi::load_lds_b128_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + 2 * e * BPITCH) * 4)>(rin, lds_b, ld_voff,
+                                                                                                   ld_soff + (uint32_t)(2 * e) * i_plane);
+        else if constexpr (VEC == 4)                   // channels chan0 + 4 e .. + 3, the tile's 64 pixels
             xsmi::load_lds_b128_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + 4 * e * PIX) * 4)>(rin, lds_b, ld_voff,
                                                                                                   ld_soff + (uint32_t)(4 * e) * i_plane);
         else                                           // channel chan0 + e of the chunk, this wave's 64 pixels
@@ -263,7 +306,7 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     auto issue_advance = [&]() {
         if (i_left == 0) return;                       // past the end of the range: dummy chunks, nothing to advance
         ++iu;
-        ld_asoff += (uint32_t)(ROWS * KC * 4);
+        ld_asoff += (uint32_t)(A_FLOATS * 4);
         if (++cc == i_nch) {
             cc = 0;
             if (++s == i_TS) { s = 0; ++r; }
@@ -304,10 +347,14 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     const int wr = wave / WCn, wc = wave % WCn;
     // lane half h takes channels (KC/2) h .. of a chunk: quad (KC/8) h + group, channel (KC/2) h + 4 group + step
     const int a_rd = ((GROUPS * h) * ROWS + wr * 32 + l31) * 4;
-    const int b_rd = A_FLOATS + (KC / 2) * h * PIX + wc * 32 + l31;
+    const int b_rd = A_FLOATS + (KC / 2) * h * (ROW ? BPITCH : PIX) + wc * 32 + l31;
+    // ROW: where the lane's pixel lies in a channel's run depends on the tile (the run has four slots of zeros behind
+    // every image row): float index of the slot one to the LEFT of the pixel, for the segment being multiplied and
+    // for the tile after it (the first fragments of a unit are read while the unit before it is multiplied)
+    int b_run = 0, b_run_next = 0;
     // fragments of a whole chunk, two buffers
-    float4 fa[2][4];                                   // [buffer][quad]
-    float fb[2][16];                                   // [buffer][channel]
+    float4 fa[2][KC / 8];                              // [buffer][quad]
+    float fb[2][KC / 2];                               // [buffer][channel]
 
     // compute-side cursor
     uint32_t cu = u0;
@@ -334,6 +381,15 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         c_head = ch == 0 ? 1u : 0u;
         c_complete = ch + n_seg == c.iters ? 1u : 0u;
         c_tile_end = cu + (c.iters - ch);
+        if constexpr (ROW) {
+            auto run_slot = [&](int m0) {              // pixel m0 + (wc * 32 + l31): slot 4 + p + 4 * (row ends before it)
+                const uint32_t ry0 = xsmi::fdiv((uint32_t)m0, c.dOX);
+                const int xp = m0 - (int)ry0 * c.OX + wc * 32 + l31;
+                return b_rd + 3 + 4 * (int)xsmi::fdiv((uint32_t)xp, c.dOX);
+            };
+            b_run = run_slot(c_m0);
+            b_run_next = run_slot(c_rt + 1 == rowtiles ? c_m0 + PIX : c_m0);
+        }
         // the tile's bias goes through the LDS (one coalesced load); the chunk loop's barriers publish it
         bias_buf ^= 1;
         if (sp.bias && c_head && t < ROWS) s_bias[bias_buf][t] = c_rt * ROWS + t < c.rows ? sp.bias[c_rt * ROWS + t] : 0.f;
@@ -502,6 +558,93 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
             XSMI_SLOT(1, fa[cur][3].w, 15)
 #undef XSMI_SLOT
         };
+        // ROW: a unit is three taps of eight MFMAs each on one stage; the fragments of one TAP live in a register set,
+        // tap t of a unit in stage c in set (c + t) & 1.  While a tap multiplies, the next tap's fragments are read:
+        // from the same stage, and for the unit's last tap (after its first two MFMAs the next unit has landed and the
+        // barrier is crossed: from then on nobody reads this stage) from the next stage, whose unit may belong to the
+        // next tile (b_run_next).  The loads of the unit after next go out behind the same MFMAs.
+        auto read_tap = [&](auto st_, auto tap_, auto set_, int run) {
+            constexpr int st = decltype(st_)::value, tap = decltype(tap_)::value, set = decltype(set_)::value;
+            const float *base = &smem[0][0] + st * STAGE_FLOATS;
+#pragma unroll
+            for (int i = 0; i < KC / 8; ++i)
+                fa[set][i] = *reinterpret_cast<const float4 *>(base + a_rd + (tap * QUADS + i) * ROWS * 4);
+#pragma unroll
+            for (int k = 0; k < KC / 2; ++k) fb[set][k] = base[run + tap + k * BPITCH];
+        };
+        auto body_row = [&](auto buf_) {
+            constexpr int cur = decltype(buf_)::value, nxt = cur ^ 1;
+            constexpr int s0 = cur, s1 = cur ^ 1;      // register sets of taps 0 and 2 / of tap 1
+            const float *base = &smem[0][0] + cur * STAGE_FLOATS;
+            // a tap's eight MFMAs with the next tap's reads from the same stage behind the first six
+#define XSMI_TAP(SA, SB, TAP)                                                                                    \
+            XSMI_MFMA(acc[0], fa[SA][0].x, fb[SA][0]);                                                           \
+            fa[SB][0] = *reinterpret_cast<const float4 *>(base + a_rd + ((TAP) * QUADS) * ROWS * 4);             \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[1], fa[SA][0].y, fb[SA][1]);                                                           \
+            fa[SB][1] = *reinterpret_cast<const float4 *>(base + a_rd + ((TAP) * QUADS + 1) * ROWS * 4);         \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[0], fa[SA][0].z, fb[SA][2]);                                                           \
+            fb[SB][0] = base[b_run + (TAP)];                                                                     \
+            fb[SB][1] = base[b_run + (TAP) + BPITCH];                                                            \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[1], fa[SA][0].w, fb[SA][3]);                                                           \
+            fb[SB][2] = base[b_run + (TAP) + 2 * BPITCH];                                                        \
+            fb[SB][3] = base[b_run + (TAP) + 3 * BPITCH];                                                        \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[0], fa[SA][1].x, fb[SA][4]);                                                           \
+            fb[SB][4] = base[b_run + (TAP) + 4 * BPITCH];                                                        \
+            fb[SB][5] = base[b_run + (TAP) + 5 * BPITCH];                                                        \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[1], fa[SA][1].y, fb[SA][5]);                                                           \
+            fb[SB][6] = base[b_run + (TAP) + 6 * BPITCH];                                                        \
+            fb[SB][7] = base[b_run + (TAP) + 7 * BPITCH];                                                        \
+            XSMI_PIN();                                                                                          \
+            XSMI_MFMA(acc[0], fa[SA][1].z, fb[SA][6]);                                                           \
+            XSMI_MFMA(acc[1], fa[SA][1].w, fb[SA][7]);                                                           \
+            XSMI_PIN();
+            XSMI_TAP(s0, s1, 1)
+            XSMI_TAP(s1, s0, 2)
+#undef XSMI_TAP
+            XSMI_MFMA(acc[0], fa[s0][0].x, fb[s0][0]);
+            XSMI_MFMA(acc[1], fa[s0][0].y, fb[s0][1]);
+            XSMI_PIN();
+            xsmi::wait_vmcnt<0>();
+            xsmi::wait_lgkmcnt0();
+            xsmi::block_barrier();
+            XSMI_PIN();
+            const float *nbase_ = &smem[0][0] + nxt * STAGE_FLOATS;
+            const int run = c_left == 1 ? b_run_next : b_run;
+            XSMI_MFMA(acc[0], fa[s0][0].z, fb[s0][2]);
+            fa[s1][0] = *reinterpret_cast<const float4 *>(nbase_ + a_rd);
+            fb[s1][0] = nbase_[run];
+            fb[s1][1] = nbase_[run + BPITCH];
+            issue_item_at(IC<0>{}, buf_);
+            XSMI_PIN();
+            XSMI_MFMA(acc[1], fa[s0][0].w, fb[s0][3]);
+            fa[s1][1] = *reinterpret_cast<const float4 *>(nbase_ + a_rd + ROWS * 4);
+            fb[s1][2] = nbase_[run + 2 * BPITCH];
+            fb[s1][3] = nbase_[run + 3 * BPITCH];
+            issue_item_at(IC<1>{}, buf_);
+            XSMI_PIN();
+            XSMI_MFMA(acc[0], fa[s0][1].x, fb[s0][4]);
+            fb[s1][4] = nbase_[run + 4 * BPITCH];
+            fb[s1][5] = nbase_[run + 5 * BPITCH];
+            fb[s1][6] = nbase_[run + 6 * BPITCH];
+            fb[s1][7] = nbase_[run + 7 * BPITCH];
+            issue_item_at(IC<2>{}, buf_);
+            XSMI_PIN();
+            XSMI_MFMA(acc[1], fa[s0][1].y, fb[s0][5]);
+            issue_item_at(IC<3>{}, buf_);
+            XSMI_PIN();
+            XSMI_MFMA(acc[0], fa[s0][1].z, fb[s0][6]);
+            issue_item_at(IC<4>{}, buf_);
+            XSMI_PIN();
+            XSMI_MFMA(acc[1], fa[s0][1].w, fb[s0][7]);
+            issue_item_at(IC<5>{}, buf_);
+            issue_item_at(IC<6>{}, buf_);
+            XSMI_PIN();
+        };
         // prologue: chunk 0 landed and in registers, chunk 1 in flight
         issue_segment();
         issue_all_at(IC<0>{});
@@ -510,13 +653,16 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         fix_borders(0, ld_fix);
         xsmi::wait_lgkmcnt0();
         xsmi::block_barrier();
-        read_chunk(IC<0>{});
+        if constexpr (ROW) read_tap(IC<0>{}, IC<0>{}, IC<0>{}, b_run);
+        else read_chunk(IC<0>{});
         issue_all_at(IC<1>{});
         for (uint32_t k = 0; k < total; k += 2) {
-            body(IC<0>{});
+            if constexpr (ROW) body_row(IC<0>{});
+            else body(IC<0>{});
             chunk_done();
             if (k + 1 < total) {
-                body(IC<1>{});
+                if constexpr (ROW) body_row(IC<1>{});
+                else body(IC<1>{});
                 chunk_done();
             }
         }
@@ -576,8 +722,11 @@ __global__ void __launch_bounds__(256) sk_pack_kernel(const float *__restrict__ 
 // 36 floats of w (mode 0: one contiguous run, read as nine float4; mode 1: four runs of nine), and stores one float4 per
 // tap; the lanes of a wavefront are consecutive rows, so a store instruction writes 1 KB of one tap's block and every
 // byte of w is requested once.
+// units != 0: the layout of the staged-row form, [rowtile][filter row][chunk][tap slot][quad][row][4 channels], where
+// slot j holds the tap that shifts the input by j - 1 columns: filter column j (units 1: forward), 2 - j (units 2:
+// backward-data, whose taps walk the other way).
 __global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restrict__ w, float *__restrict__ apk, int mode,
-                                                           int rows, int CH, int rowtiles, int ROWS, int KC) {
+                                                           int rows, int CH, int rowtiles, int ROWS, int KC, int units) {
     const int nch = CH / KC, quads = KC / 4;
     const uint32_t total = (uint32_t)rowtiles * (uint32_t)nch * (uint32_t)quads * (uint32_t)ROWS;
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
@@ -614,6 +763,16 @@ __global__ void __launch_bounds__(256) sk_pack_3x3_kernel(const float *__restric
             for (int t = 0; t < 9; ++t) v[e][t] = 0.f;
     }
     // float4 index ((rt * iters + tap * nch + cc) * quads + q) * ROWS + rr with iters = 9 * nch
+    if (units) {
+#pragma unroll
+        for (int t = 0; t < 9; ++t) {
+            const int tr = t / 3, ts = t % 3, slot = units == 1 ? ts : 2 - ts;
+            float4 *dst = reinterpret_cast<float4 *>(apk) +
+                          (((((size_t)rt * 3 + tr) * nch + cc) * 3 + slot) * quads + q) * ROWS + rr;
+            *dst = make_float4(v[0][t], v[1][t], v[2][t], v[3][t]);
+        }
+        return;
+    }
     float4 *dst = reinterpret_cast<float4 *>(apk) + (((size_t)rt * 9 * nch + cc) * quads + q) * ROWS + rr;
 #pragma unroll
     for (int t = 0; t < 9; ++t) dst[(size_t)t * nch * quads * ROWS] = make_float4(v[0][t], v[1][t], v[2][t], v[3][t]);
@@ -659,11 +818,29 @@ bool sk_wide_loads_ok(const SkParams &p) {
     return true;
 }
 
+// Staged rows (the filter must have been laid out for them): 3 x 3, stride 1, one column and one row of padding, rows
+// as wide as the output's, a multiple of four pixels and at least 20 (a tile of 64 pixels then crosses at most three
+// row ends: 21 pieces per run), channels in chunks of 16.
+bool sk_rows_staged(int R, int S, int sh, int sw, int pad, int in_w, int out_w, int channels) {
+    return xsmi::option(xsmi::OPT_SK_WIDE) >= 2 && R == 3 && S == 3 && sh == 1 && sw == 1 && pad == 1 && in_w == out_w &&
+           out_w % 4 == 0 && out_w >= 20 && channels % 16 == 0;
+}
+
 int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
-    static int res_narrow = 0, res_wide = 0;
-    const bool wide = sk_wide_loads_ok(p);
-    uint32_t gsz = (uint32_t)(wide ? sk_resident(tap_sk_f32_kernel<4>, &res_wide, SK_MAX_GRID)
-                                   : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
+    static int res_narrow = 0, res_wide = 0, res_rows = 0;
+    const bool rows = p.staged_rows != 0;
+    const bool wide = !rows && sk_wide_loads_ok(p);
+    if (rows) {
+        const SkClass &c = p.cls[0];
+        if (p.ncls != 1 || c.sx != 1 || c.sy != 1 || c.TS != 3 || c.dx0 + c.dstep != 0 || c.IW != c.OX || c.OX % 4 != 0 ||
+            c.OX < 20 || (((uintptr_t)p.in) & 3) != 0)
+            return xsmi::set_error("even-split convolution: geometry not served by the staged-row form"), XSMI_ERR_INVALID;
+        p.out_rows = c.M / c.OX;
+        p.dPitch = xsmi::make_fastdiv(c.OX + 4);
+    }
+    uint32_t gsz = (uint32_t)(rows   ? sk_resident(tap_sk_f32_kernel<3>, &res_rows, SK_MAX_GRID)
+                              : wide ? sk_resident(tap_sk_f32_kernel<4>, &res_wide, SK_MAX_GRID)
+                                     : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
     if (gsz > p.units) gsz = p.units;                  // every workgroup gets at least one chunk
     if (gsz == 0) return XSMI_OK;
     p.upg = p.units / gsz; p.urem = p.units % gsz; p.dG = xsmi::make_fastdiv(gsz);
@@ -676,7 +853,8 @@ int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
     p.part_bytes = (uint32_t)xsmi::SK_SCRATCH_PART_BYTES;
     const long spin = xsmi::option(xsmi::OPT_SK_SPIN_LIMIT);
     p.spin_limit = spin < 0 ? 0u : spin > 0x7fffffffL ? 0x7fffffffu : (uint32_t)spin;
-    if (wide) hipLaunchKernelGGL(tap_sk_f32_kernel<4>, dim3(gsz), dim3(256), 0, st, p);
+    if (rows) hipLaunchKernelGGL(tap_sk_f32_kernel<3>, dim3(gsz), dim3(256), 0, st, p);
+    else if (wide) hipLaunchKernelGGL(tap_sk_f32_kernel<4>, dim3(gsz), dim3(256), 0, st, p);
     else hipLaunchKernelGGL(tap_sk_f32_kernel<1>, dim3(gsz), dim3(256), 0, st, p);
     XSMI_LAUNCH_CHECK("tap_sk_f32_kernel");
     return XSMI_OK;
@@ -735,10 +913,12 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     const int rowtiles = ceil_div(K, shp.rows_tile);
     const size_t pack = sk_pack_bytes(K, C, R * S, shp);
     float *apk = (float *)workspace;
+    const bool staged = sk_rows_staged(R, S, sh, sw, pad, W, OW, C) && (((uintptr_t)w) & 15) == 0 && (((uintptr_t)x) & 3) == 0;
+    const int kc = staged ? 16 : shp.kc;
     if (!(opts & 2) && R == 3 && S == 3 && (((uintptr_t)w) & 15) == 0) {
-        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(C / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
+        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(C / kc) * (uint32_t)(kc / 4) * (uint32_t)shp.rows_tile;
         hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, apk, 0, K, C, rowtiles,
-                           shp.rows_tile, shp.kc);
+                           shp.rows_tile, kc, staged ? 1 : 0);
         XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
     } else if (!(opts & 2)) {
         SkPackMulti pm;
@@ -758,13 +938,17 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     memset(&p, 0, sizeof(p));
     SkClass &c = p.cls[0];
     c.apk_off = 0;
-    c.M = N * OH * OW; c.rows = K; c.nch = C / shp.kc; c.TR = R; c.TS = S;
+    c.M = N * OH * OW; c.rows = K; c.nch = C / kc; c.TR = R; c.TS = S;
     c.dy0 = -pad; c.dx0 = -pad; c.dstep = 1;
     c.IH = H; c.IW = W; c.sy = sh; c.sx = sw;
     c.in_n_stride = C * H * W; c.plane_bytes = (uint32_t)(H * W * 4);
     c.OY = OH; c.OX = OW; c.dOX = make_fastdiv(OW); c.dOY = make_fastdiv(OH);
     c.os_n = (long long)K * OH * OW; c.os_k = (long long)OH * OW; c.o_base = 0; c.os_y = OW; c.os_x = 1;
     sk_fill_class(c, shp, rowtiles);
+    if (staged) {                                      // a unit is a filter row x 16 channels
+        c.iters = (uint32_t)(c.TR * c.nch);
+        c.dIT = make_fastdiv(c.iters);
+    }
     c.first_unit = 0;
     const uint32_t tiles = (uint32_t)ceil_div(c.M, shp.pix_tile) * (uint32_t)rowtiles;
     p.units = tiles * c.iters;
@@ -774,6 +958,7 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     p.out_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = 1; p.rowtiles = rowtiles; p.accumulate = 0; p.relu = relu;
+    p.staged_rows = staged ? 1 : 0;
     prof_begin();
     int rc = sk_launch(st, p, shp);
     prof_end();
@@ -818,10 +1003,18 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
         }
     }
     const size_t pack = off;
+    // the pass reads dy (rows of OW pixels) and writes dx (rows of W pixels)
+    const bool staged = nplans == 1 && sk_rows_staged(R, S, sh, sw, pad, OW, W, K) && (((uintptr_t)dy) & 3) == 0;
+    const int kc = staged ? 16 : shp.kc;
+    if (staged) {                                      // a unit is a filter row x 16 channels
+        plans[0].nch = K / kc;
+        plans[0].iters = (uint32_t)(plans[0].TR * plans[0].nch);
+        plans[0].dIT = make_fastdiv(plans[0].iters);
+    }
     if (!(opts & 2) && R == 3 && S == 3 && sh == 1 && sw == 1 && nplans == 1) {
-        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(K / shp.kc) * (uint32_t)(shp.kc / 4) * (uint32_t)shp.rows_tile;
+        const uint32_t total = (uint32_t)rowtiles * (uint32_t)(K / kc) * (uint32_t)(kc / 4) * (uint32_t)shp.rows_tile;
         hipLaunchKernelGGL(sk_pack_3x3_kernel, dim3((total + 255) / 256), dim3(256), 0, st, w, jobs[0].apk, 1, C, K, rowtiles,
-                           shp.rows_tile, shp.kc);
+                           shp.rows_tile, kc, staged ? 2 : 0);
         XSMI_LAUNCH_CHECK("sk_pack_3x3_kernel");
     } else if (!(opts & 2)) {
         SkPackMulti pm;
@@ -864,6 +1057,7 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
     p.out_bytes = (uint32_t)((size_t)N * C * H * W * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = ncls; p.rowtiles = rowtiles; p.accumulate = accumulate; p.relu = 0;
+    p.staged_rows = staged ? 1 : 0;
     prof_begin();
     int rc = sk_launch(st, p, shp);
     prof_end();

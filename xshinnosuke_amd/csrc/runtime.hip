@@ -37,7 +37,7 @@ OptionRow g_options[xsmi::OPT_COUNT] = {
     {"tap_persist", "XSMI_TAP_PERSIST", 1, false},
     {"cl_halo", "XSMI_CL_HALO", 1, false},
     {"cl_stem", "XSMI_CL_STEM", 1, false},
-    {"sk_wide", "XSMI_SK_WIDE", 1, false},
+    {"sk_wide", "XSMI_SK_WIDE", 2, false},
     {"pool_bwd", "XSMI_POOL_BWD", 2, false},
     {"pack_lanes", "XSMI_PACK_LANES", 2, false},
 };
