@@ -734,7 +734,7 @@ def main():
         "frac_fp32_mfma_peak": value / FP32_MFMA_PEAK_TFLOPS,
         "roofline": {"bound": "mfma", "achieved": achieved, "peak": FP32_MFMA_PEAK_TFLOPS, "unit": "TFLOP/s",
                      "frac": achieved / FP32_MFMA_PEAK_TFLOPS, "traffic": tap_sk_traffic_bytes(),
-                     "kernel": "tap_sk_f32_kernel<4>", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
+                     "kernel": "tap_sk_f32_kernel<3>", "flop_per_launch": flops_pass, "avg_launch_ms": igemm_ms},
         "ops_ms": {"conv_fwd": per["fwd"], "conv_bwd_data": per["bwd_data"], "conv_bwd_weight": per["bwd_weight"]},
         "kernels_ms": {"tap_sk_fwd": per["fwd_kernel"], "tap_sk_bwd_data": per["bwd_data_kernel"]},
         "ops_tflops": {k: flops_pass / (per[k] * 1e-3) / 1e12 for k in ("fwd", "bwd_data", "bwd_weight")},

@@ -102,8 +102,9 @@ int xsmi_sync(void);
 /* Tuning switches of the kernel selection, by name: "tap_sk" (0: one tile per workgroup only, 1: even split of
  * the chunks where it pays, 3: even split wherever it applies), "sk_spin_limit" (polls before an even-split
  * workgroup gives up waiting for a partial tile; the calls that wait for the device then fail with
- * XSMI_ERR_RUNTIME), "sk_wide" (0: one-dword loads of the activations in the even-split kernel also where 16-byte
- * loads apply), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
+ * XSMI_ERR_RUNTIME), "sk_wide" (the even-split kernel's activation loads: 2: input rows staged once for the three taps of
+ * a filter row where that form applies, 16-byte loads tap by tap where only those apply; 1: 16-byte loads tap by tap;
+ * 0: one-dword loads everywhere), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
  * several pieces; 0: one piece per workgroup), "pack_lanes" (1 to 4: streams over which xsmi_conv2d_pack deals its
  * layout launches), "tap_stages", "tap_persist", "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
  * A caller that changes one must drop every workspace content it counted on (XSMI_CONV_WS_PACKED) and ask for
