@@ -366,6 +366,14 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
  * reference performs after the forward (xs/nn/functional.py:700-707), done by the normalisation kernel.
  * neg_mask (or NULL) fuses the ReLU that follows the normalisation in a residual block
  * (xs/layers/activators.py:37-50): neg_mask[i] = pre-activation < 0, y = max(pre-activation, 0). */
+/* The end of a residual block as one pass: y = max(0, gamma * xhat + beta + residual), neg_mask[i] = that sum < 0, with
+ * the batch statistics of x as in xsmi_bn_fwd (same outputs, same moving-statistics update, xhat never stored).  It
+ * stands for xsmi_bn_fwd, xsmi_add and xsmi_relu_fwd_mask in a row (xs/nn/functional.py:676-707, xs/layers/ops.py:40-72,
+ * xs/layers/activators.py:37-50) without writing and reading the normalised tensor in between; the backward is
+ * xsmi_relu_mask_bwd on the sum's gradient, which then goes to xsmi_bn_bwd and to the residual branch unchanged. */
+int xsmi_bn_add_relu_fwd(const float *x, const float *gamma, const float *beta, const float *residual, float *y,
+                         float *sqrtvar, float *mean, float *var, float *moving_mean, float *moving_var, float momentum,
+                         uint8_t *neg_mask, int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
 /* Inference form with given statistics (xs/nn/functional.py:708-725); relu != 0 clips at zero. */
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
                   int N, int C, int HW, float eps, int relu);

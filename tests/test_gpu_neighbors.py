@@ -74,6 +74,61 @@ def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     np.testing.assert_array_equal(yir.numpy(), np.maximum(yi.numpy(), 0))
 
 
+# two-kernel float4 form, two-kernel scalar form (planes not a multiple of four), single-kernel forms (256 / 1024 threads)
+@pytest.mark.parametrize("shape", [(8, 16, 40, 40), (6, 5, 37, 41), (32, 64, 14, 14), (4, 8, 6, 6), (64, 16)])
+def test_batch_norm_add_relu_as_one_pass(gpu, shape):
+    """The end of a residual block: a held-back normalisation, the held-back add of its result and a shortcut, and the
+    in-place ReLU of the sum run as one normalisation whose second pass adds and clips.  Same float operations as
+    the three passes, hence the same bits; the normalisation's own result is never stored and says so when read; any
+    other call in between makes the plain passes run."""
+    K = gpu.kernels
+    rng = np.random.default_rng(sum(shape) + 1)
+    c = shape[1]
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    r = rng.standard_normal(shape).astype(np.float32)
+    gamma = rng.uniform(0.5, 1.5, c).astype(np.float32); beta = rng.standard_normal(c).astype(np.float32)
+    mm0 = rng.standard_normal(c).astype(np.float32); mv0 = rng.uniform(0.5, 2.0, c).astype(np.float32)
+    eps = 1e-5
+    xd, rd, gd, bd = gpu.to_device(x), gpu.to_device(r), gpu.to_device(gamma), gpu.to_device(beta)
+
+    def three_passes():
+        mm, mv = gpu.to_device(mm0), gpu.to_device(mv0)
+        y, _, sq, mean, var = K.bn_fwd(xd, gd, bd, eps, moving=(mm, mv), momentum=0.9, want_xhat=False)
+        s = K.add(y, rd)
+        out, mask = K.relu_fwd_mask(s, s)
+        return [a.numpy() for a in (out, mask, sq, mean, var, mm, mv)], y.numpy()
+
+    ref, y_plain = three_passes()
+    assert (ref[0] > 0).any() and (ref[1] == 1).any()
+    for first in (True, False):                      # the normalisation's result as the add's first or second operand
+        mm, mv = gpu.to_device(mm0), gpu.to_device(mv0)
+        y, _, sq, mean, var = K.bn_fwd(xd, gd, bd, eps, moving=(mm, mv), momentum=0.9, want_xhat=False, defer=True)
+        s = K.add(y, rd, defer=True) if first else K.add(rd, y, defer=True)
+        out, mask = K.relu_fwd_mask(s, s)
+        assert out is s
+        got = [a.numpy() for a in (out, mask, sq, mean, var, mm, mv)]
+        for g, e in zip(got, ref):
+            np.testing.assert_array_equal(g, e)
+        with pytest.raises(gpu.XsmiError, match="not stored"):
+            y.numpy()
+        # the same array as the output of the next normalisation is simply written again
+        y2, _, _, _, _ = K.bn_fwd(xd, gd, bd, eps, y=y, want_xhat=False)
+        assert y2 is y
+        np.testing.assert_array_equal(y.numpy(), y_plain)
+    # a read of the normalisation's result before the add, and a read of the sum before the ReLU: plain passes
+    y, _, sq, mean, var = K.bn_fwd(xd, gd, bd, eps, want_xhat=False, defer=True)
+    np.testing.assert_array_equal(y.numpy(), y_plain)
+    s = K.add(y, rd, defer=True)
+    np.testing.assert_array_equal(K.relu_fwd_mask(s, s)[0].numpy(), ref[0])
+    y, _, sq, mean, var = K.bn_fwd(xd, gd, bd, eps, want_xhat=False, defer=True)
+    s = K.add(y, rd, defer=True)
+    np.testing.assert_array_equal(s.numpy(), y_plain + r)
+    np.testing.assert_array_equal(y.numpy(), y_plain)
+    np.testing.assert_array_equal(K.relu_fwd_mask(s, s)[0].numpy(), ref[0])
+    np.testing.assert_array_equal(sq.numpy(), ref[2])
+
+
+
 def test_multi_tensor_axpy_is_one_sgd_step(gpu):
     """xs/optim/sgd.py:4-9 over many parameters of ragged sizes, more than one launch group."""
     K = gpu.kernels
@@ -140,7 +195,7 @@ def test_held_back_add_joins_the_in_place_relu(gpu):
     b = rng.standard_normal((3, 5, 7, 9)).astype(np.float32)
     da, db = gpu.to_device(a), gpu.to_device(b)
     c = K.add(da, db, defer=True)
-    assert capi._deferred and capi._deferred[0][2] is c
+    assert capi._deferred and capi._deferred[0][-1] is c
     r = K.relu_fwd(c, out=c)
     assert r is c and not capi._deferred
     np.testing.assert_array_equal(c.numpy(), np.maximum(a + b, 0.0))

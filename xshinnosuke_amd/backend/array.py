@@ -43,12 +43,13 @@ class _Block:
     runs in order on one stream, so reuse needs no synchronisation and avoids hipMalloc/hipFree
     (which serialise with the device) in the steady state."""
 
-    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl", "owner", "__weakref__")
+    __slots__ = ("ptr", "nbytes", "logical", "lazy_zero", "version", "cl", "owner", "unwritten", "__weakref__")
 
     def __init__(self, nbytes):
         ensure_init()
         self.logical = int(nbytes)
         self.lazy_zero = False
+        self.unwritten = None                # why the contents were never produced (a message), see never_written()
         self.cl = None                       # ChannelsLast form of the array that fills this block, if it has one
         self.version = 0                     # counts every hand-out of the address and every pending clear
         size = _round_size(nbytes)
@@ -154,6 +155,8 @@ class DeviceArray:
     @property
     def ptr(self):
         blk = self._block
+        if blk.unwritten is not None:
+            raise XsmiError(blk.unwritten)
         blk.version += 1                     # whoever takes the address may write through it
         graph = _CAPTURE[0]
         if graph is not None and blk.owner is not graph:
@@ -214,11 +217,23 @@ class DeviceArray:
         blk = self._block
         return blk.lazy_zero and self._offset == 0 and self.nbytes >= blk.logical
 
+    def is_whole(self):
+        """True if the array fills its allocation (not a part of a larger buffer)."""
+        return self._offset == 0 and self.nbytes >= self._block.logical
+
+    def never_written(self, why):
+        """Declare that the operation that was to produce this array (a whole allocation) ran fused into its consumer
+        and stored nothing here: handing out the address raises ``why`` until the array is overwritten as a whole."""
+        self._block.unwritten = str(why)
+        self._block.version += 1
+
     def take_fresh(self):
         """True if this array is a pending all-zero buffer that the caller will now overwrite completely
         (the pending clear is dropped).  An array that covers only part of its allocation is cleared
         for real instead and reports False."""
         blk = self._block
+        if self._offset == 0 and self.nbytes >= blk.logical:
+            blk.unwritten = None
         if not blk.lazy_zero:
             return False
         if self._offset == 0 and self.nbytes >= blk.logical:

@@ -96,6 +96,7 @@ SIGNATURES = {
     "xsmi_lerp": (_i, [_vp, _vp, _f, _sz]),
     "xsmi_bn_workspace_bytes": (_sz, [_i]),
     "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
+    "xsmi_bn_add_relu_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f, _i]),
     "xsmi_bn_fold": (_i, [_vp] * 8 + [_i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 9 + [_i, _i, _i, _vp, _sz]),
@@ -212,30 +213,74 @@ def layouts_enqueued(*held):
     _layouts_hold.extend(held)
 
 
-# One element-wise add may be held back until the next call into the library: if that call is the in-place ReLU
-# of its result, both run as one pass (kernels.add / kernels.relu_fwd).  Every other call enqueues the add first,
-# so nothing can read or change the operands or the result between the add and the point where it was asked for.
-_deferred = []          # at most one (a, b, out) triple of device arrays
+# One operation may be held back until the next call into the library, so that the end of a residual block runs as
+# few passes as it needs (kernels.bn_fwd / kernels.add / kernels.relu_fwd):
+#   ("add", a, b, out)            an element-wise add into a new array; if the next call is the in-place ReLU of its
+#                                 result, both run as one pass;
+#   ("bn", entry)                 a training batch normalisation (kernels.BnEntry: operands, outputs, launch); if the
+#                                 next call is a held-back add with its result as one operand, it becomes
+#   ("bn_add", entry, a, b, out)  and if the call after that is the in-place ReLU (with mask) of the sum, the three run
+#                                 as one normalisation whose second pass adds the other operand and clips.
+# Every other call enqueues what is held back first, in order, so nothing can read or change the operands or the
+# results between an operation and the point where it was asked for.
+_deferred = []          # at most one entry
 
 
 def _flush_deferred():
-    a, b, out = _deferred.pop()
-    lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
+    op = _deferred.pop()
+    if op[0] == "add":
+        _, a, b, out = op
+        lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
+    elif op[0] == "bn":
+        op[1].launch()
+    else:
+        _, entry, a, b, out = op
+        entry.launch()
+        lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
 
 
 def defer_add(a, b, out):
     if _deferred:
         _flush_deferred()
-    _deferred.append((a, b, out))
+    _deferred.append(("add", a, b, out))
 
 
-def take_deferred_add(out):
-    """The operands of the held-back add whose result is ``out``, or None (a different pending add is enqueued)."""
+def defer_bn(entry):
+    if _deferred:
+        _flush_deferred()
+    _deferred.append(("bn", entry))
+
+
+def take_deferred_bn(a, b):
+    """The held-back normalisation whose result is ``a`` or ``b`` (it is no longer pending: the caller launches it or
+    holds it back again), or None (anything else that was pending is enqueued)."""
     if not _deferred:
         return None
-    if _deferred[0][2] is out:
-        a, b, _ = _deferred.pop()
-        return a, b
+    if _deferred[0][0] == "bn" and (_deferred[0][1].y is a or _deferred[0][1].y is b):
+        return _deferred.pop()[1]
+    _flush_deferred()
+    return None
+
+
+def defer_bn_add(entry, a, b, out):
+    if _deferred:
+        _flush_deferred()
+    _deferred.append(("bn_add", entry, a, b, out))
+
+
+def take_deferred_add(out, with_bn=False):
+    """The operands ``(a, b)`` of the held-back add whose result is ``out``, or None (a different pending operation is
+    enqueued).  ``with_bn``: a held-back normalisation + add is handed over too, as ``(a, b, entry)``; without it that
+    pair is enqueued as two launches and reported as None."""
+    if not _deferred:
+        return None
+    op = _deferred[0]
+    if op[0] == "add" and op[3] is out:
+        _deferred.pop()
+        return op[1], op[2]
+    if op[0] == "bn_add" and op[4] is out and with_bn:
+        _deferred.pop()
+        return op[2], op[3], op[1]
     _flush_deferred()
     return None
 

@@ -447,7 +447,13 @@ def add(a, b, out=None, defer=False):
     an in-place ReLU of the result can run in the same pass; any other call enqueues the add first."""
     _f32(a, "a"); _f32(b, "b")
     if defer and out is None and a.size == b.size:
+        entry = capi.take_deferred_bn(a, b) if a is not b else None
         out = empty(a.shape)
+        if entry is not None:
+            # one operand is a normalisation that has not been launched yet: both wait for the call after this one
+            (b if entry.y is a else a).ptr            # the other operand: a pending clear is carried out now
+            capi.defer_bn_add(entry, a, b, out)
+            return out
         acl, bcl = a.channels_last(), b.channels_last()
         if acl is None or bcl is None or not acl.same_layout(bcl):
             a.ptr; b.ptr                              # operands with a pending clear are cleared now
@@ -491,9 +497,13 @@ def relu_fwd_mask(x, out=None):
     """Returns (max(0, x), uint8 mask of x < 0); ``out`` may be ``x`` itself."""
     _f32(x, "x")
     if out is x:                                      # in place: a held-back add that produced x joins this pass
-        ops = capi.take_deferred_add(x)
+        ops = capi.take_deferred_add(x, with_bn=True)
         if ops is not None:
             mask = empty(x.shape, np.uint8)
+            if len(ops) == 3:                         # ... and the normalisation that produced one of its operands
+                entry = ops[2]
+                entry.launch(residual=ops[1] if entry.y is ops[0] else ops[0], out=x, neg_mask=mask)
+                return x, mask
             lib.call("xsmi_add_relu", ops[0].cptr, ops[1].cptr, x.cptr, mask.cptr, x.size)
             return x, mask
     out = _like(x, out)
@@ -544,11 +554,39 @@ def _nchw3(shape):
     return int(n), int(c), int(hw)
 
 
-def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None, want_xhat=True):
+FUSE_BN_ADD_RELU = os.environ.get("XSMI_FUSE_BN_ADD_RELU", "1") != "0"
+
+
+class BnEntry:
+    """A training batch normalisation that has been asked for and not launched yet (see capi._deferred)."""
+
+    __slots__ = ("x", "gamma", "beta", "eps", "y", "sqrtvar", "mean", "var", "mm", "mv", "momentum", "dims", "ws")
+
+    def launch(self, residual=None, out=None, neg_mask=None):
+        """Plain: y = gamma * xhat + beta.  With ``residual``: out = max(0, y + residual) and its sign mask in one
+        pass; y itself is then never written, and reading it raises."""
+        n, c, hw = self.dims
+        ws, ws_bytes = self.ws
+        mm, mv = self.mm, self.mv
+        stats = (self.sqrtvar.cptr, self.mean.cptr, self.var.cptr, mm.cptr if mm is not None else None,
+                 mv.cptr if mv is not None else None, float(self.momentum))
+        if residual is None:
+            lib.call("xsmi_bn_fwd", self.x.cptr, self.gamma.cptr, self.beta.cptr, self.y.cptr, None, *stats, None,
+                     n, c, hw, float(self.eps), ws, ws_bytes)
+            return
+        self.y.never_written("this batch normalisation's result was consumed by the add and ReLU that followed it, in "
+                             "one pass, and was not stored (XSMI_FUSE_BN_ADD_RELU=0 keeps the three passes apart)")
+        lib.call("xsmi_bn_add_relu_fwd", self.x.cptr, self.gamma.cptr, self.beta.cptr, residual.cptr, out.cptr, *stats,
+                 neg_mask.cptr, n, c, hw, float(self.eps), ws, ws_bytes)
+
+
+def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None, want_xhat=True, defer=False):
     """``moving=(moving_mean, moving_var)`` device arrays are updated in place: m = momentum*m + (1-momentum)*stat.
     A uint8 ``neg_mask`` of x's size fuses a ReLU: it receives pre-activation < 0 and y is clipped at 0.
     ``want_xhat=False`` skips the store of the normalised input (None is returned for it): ``bn_bwd`` forms it
-    again from x and the batch mean."""
+    again from x and the batch mean.  ``defer=True`` (without mask and normalised input) holds the launch back until
+    the next call into the library: an add of y and another tensor followed by the in-place ReLU of the sum then runs
+    inside the normalisation's second pass; any other call enqueues the normalisation first."""
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
     y = _like(x, y); xhat = empty(x.shape) if want_xhat else None
@@ -558,6 +596,15 @@ def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None
     if mm is not None and (mm.size != c or mv.size != c):
         raise ValueError("bn_fwd: moving statistics must have %d elements" % c)
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
+    if defer and FUSE_BN_ADD_RELU and neg_mask is None and not want_xhat and y.is_whole():
+        e = BnEntry()
+        e.x, e.gamma, e.beta, e.eps, e.y = x, gamma, beta, eps, y
+        e.sqrtvar, e.mean, e.var, e.mm, e.mv, e.momentum = sqrtvar, mean, var, mm, mv, momentum
+        e.dims, e.ws = (n, c, hw), (ws, ws_bytes)
+        for a in (x, gamma, beta) + ((mm, mv) if mm is not None else ()):
+            a.ptr                                     # pending clears and channels-last forms are settled now
+        capi.defer_bn(e)
+        return y, None, sqrtvar, mean, var
     lib.call("xsmi_bn_fwd", x.cptr, gamma.cptr, beta.cptr, y.cptr, xhat.cptr if want_xhat else None, sqrtvar.cptr,
              mean.cptr, var.cptr,
              mm.cptr if mm is not None else None, mv.cptr if mv is not None else None, float(momentum),

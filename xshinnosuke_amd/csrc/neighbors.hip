@@ -317,10 +317,12 @@ __device__ __forceinline__ void bn_channel_sums(const double *__restrict__ part,
 // pass 2 of the forward: block (c, sp) turns the channel's partial sums into mean and sqrt(var + eps) (block sp == 0
 // also stores them and updates the moving statistics: m = momentum*m + (1-momentum)*cur, as xsmi_lerp computes it)
 // and normalises its units of the channel, numbered as in bn_partial_kernel.  neg_mask != nullptr fuses a ReLU:
-// mask = pre-activation < 0, y = max(pre-activation, 0).
+// mask = pre-activation < 0, y = max(pre-activation, 0).  residual != nullptr: a tensor of x's shape that is added to
+// the normalised value before the ReLU (the end of a residual block as one pass).
 struct BnFwdOut {
     float *y, *xhat, *sqrtvar, *mean, *var, *moving_mean, *moving_var;
     uint8_t *neg_mask;
+    const float *residual;
 };
 template <bool VEC>
 __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
@@ -347,15 +349,21 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__
     }
     const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
     for (uint32_t e0 = beg + threadIdx.x; e0 < end; e0 += 256 * UNR) {
-        float xv[UNR][W];
+        float xv[UNR][W], rv[UNR][W];
         size_t off[UNR];
 #pragma unroll
         for (int k = 0; k < UNR; ++k) {
             const uint32_t e = e0 + 256u * k;
             const uint32_t j = xsmi::fdiv(e, dU), i = e - j * dU.d;
             off[k] = ((size_t)j * C + c) * (size_t)HW + (size_t)i * W;
+#pragma unroll
+            for (int q = 0; q < W; ++q) rv[k][q] = 0.f;
             if (e < end) {
                 if (VEC) *reinterpret_cast<float4 *>(xv[k]) = *reinterpret_cast<const float4 *>(x + off[k]); else xv[k][0] = x[off[k]];
+                if (o.residual) {
+                    if (VEC) *reinterpret_cast<float4 *>(rv[k]) = *reinterpret_cast<const float4 *>(o.residual + off[k]);
+                    else rv[k][0] = o.residual[off[k]];
+                }
             }
         }
 #pragma unroll
@@ -366,7 +374,8 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__
 #pragma unroll
             for (int q = 0; q < W; ++q) {
                 hv[q] = (xv[k][q] - mu) / rs;
-                const float pre = g * hv[q] + bt;
+                float pre = g * hv[q] + bt;
+                if (o.residual) pre += rv[k][q];
                 mv[q] = pre < 0.f ? 1 : 0;
                 yv[q] = (o.neg_mask && pre < 0.f) ? 0.f : pre;
             }
@@ -508,7 +517,8 @@ __global__ void __launch_bounds__(NT) bn_fwd_small_kernel(const float *__restric
         if (e >= total) break;
         const size_t off = offs[u];
         const float hv = (v[u] - mu) / rs;
-        const float pre = g * hv + bt;
+        float pre = g * hv + bt;
+        if (o.residual) pre += o.residual[off];
         if (o.xhat) o.xhat[off] = hv;
         o.y[off] = (o.neg_mask && pre < 0.f) ? 0.f : pre;
         if (o.neg_mask) o.neg_mask[off] = pre < 0.f ? 1 : 0;
@@ -908,9 +918,28 @@ int xsmi_lerp(float *m, const float *cur, float momentum, size_t n) {
 
 size_t xsmi_bn_workspace_bytes(int C) { return C > 0 ? (size_t)C * BN_SPLIT * 2 * sizeof(double) : 0; }
 
+static int bn_fwd_impl(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
+                       float *mean, float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask,
+                       const float *residual, int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
+
 int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar, float *mean,
                 float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask, int N, int C, int HW,
                 float eps, void *ws, size_t ws_bytes) {
+    return bn_fwd_impl(x, gamma, beta, y, xhat, sqrtvar, mean, var, moving_mean, moving_var, momentum, neg_mask, nullptr, N,
+                       C, HW, eps, ws, ws_bytes);
+}
+
+int xsmi_bn_add_relu_fwd(const float *x, const float *gamma, const float *beta, const float *residual, float *y,
+                         float *sqrtvar, float *mean, float *var, float *moving_mean, float *moving_var, float momentum,
+                         uint8_t *neg_mask, int N, int C, int HW, float eps, void *ws, size_t ws_bytes) {
+    XSMI_CHECK_ARG(residual && neg_mask, "xsmi_bn_add_relu_fwd: null pointer");
+    return bn_fwd_impl(x, gamma, beta, y, nullptr, sqrtvar, mean, var, moving_mean, moving_var, momentum, neg_mask, residual,
+                       N, C, HW, eps, ws, ws_bytes);
+}
+
+static int bn_fwd_impl(const float *x, const float *gamma, const float *beta, float *y, float *xhat, float *sqrtvar,
+                       float *mean, float *var, float *moving_mean, float *moving_var, float momentum, uint8_t *neg_mask,
+                       const float *residual, int N, int C, int HW, float eps, void *ws, size_t ws_bytes) {
     XSMI_REQUIRE_INIT();
     XSMI_CHECK_ARG(N > 0 && C > 0 && HW > 0, "xsmi_bn_fwd: empty tensor");
     XSMI_CHECK_ARG((double)N * C * HW < 536870912.0, "xsmi_bn_fwd: tensors of 2^29 elements or more are not supported");
@@ -919,7 +948,7 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_fwd: workspace too small");
     hipStream_t st = xsmi::stream();
     if ((size_t)N * HW <= (size_t)BN_SMALL_MAX) {
-        const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask};
+        const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask, residual};
         const uint32_t total = (uint32_t)(N * HW);
         const xsmi::FastDiv dHW = xsmi::make_fastdiv(HW);
         if (total <= 256u * BN_SMALL_PER) hipLaunchKernelGGL(bn_fwd_small_kernel<256>, dim3(C), dim3(256), 0, st, x, gamma, beta, (double)N * HW, eps, momentum, o, C, HW, dHW, total);
@@ -933,8 +962,8 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
     launch_bn_partial(st, x, nullptr, nullptr, part, C, HW, split, nullptr, nullptr);
     XSMI_LAUNCH_CHECK("bn_partial_kernel");
     const BnSplit ap = bn_split(N, HW, (HW & 3) == 0 && aligned16(x) && aligned16(y) && (!xhat || aligned16(xhat)) &&
-                                           (!neg_mask || ((uintptr_t)neg_mask & 3) == 0));
-    const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask};
+                                           (!neg_mask || ((uintptr_t)neg_mask & 3) == 0) && (!residual || aligned16(residual)));
+    const BnFwdOut o{y, xhat, sqrtvar, mean, var, moving_mean, moving_var, neg_mask, residual};
     if (ap.vec)
         hipLaunchKernelGGL(bn_apply_kernel<true>, dim3(C, ap.nsplit), dim3(256), 0, st, x, gamma, beta, part, nsplit,
                            (double)N * HW, eps, momentum, o, C, HW, ap.dU, ap.total, ap.per);

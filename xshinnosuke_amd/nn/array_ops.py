@@ -150,15 +150,15 @@ def fill_like(a, value):
     return np.full(a.shape, value, dtype=a.dtype)
 
 
-def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0, neg_mask=None, want_xhat=True):
+def batch_norm_train(x, gamma, beta, eps, out=None, moving=None, momentum=0.0, neg_mask=None, want_xhat=True, defer=False):
     """Per-channel batch statistics over (N, H, W) or (N,).  Returns y, xhat, sqrtvar, mean, var.  A device
     ``out`` of the right size receives y directly; device ``moving`` statistics are updated by the same call
     (host ones are left to the caller).  On the device ``want_xhat=False`` returns None for xhat: the backward
-    then takes x and the mean."""
+    then takes x and the mean; ``defer``: see kernels.bn_fwd."""
     if is_device(x):
         y = out if (out is not None and is_device(out) and out.size == x.size) else None
         return K.bn_fwd(x, same_place(x, gamma), same_place(x, beta), eps, y=y, moving=moving, momentum=momentum,
-                        neg_mask=neg_mask, want_xhat=want_xhat)
+                        neg_mask=neg_mask, want_xhat=want_xhat, defer=defer)
     axes = tuple(i for i in range(x.ndim) if i != 1)
     mean = x.mean(axis=axes, keepdims=True)
     var = x.var(axis=axes, keepdims=True)
