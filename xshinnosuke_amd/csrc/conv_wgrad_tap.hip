@@ -55,6 +55,11 @@ struct WgradTapParams {
     xsmi::FastDiv dOW, dCT, dS;
 };
 
+// DIRECT: chunks run over the pixels of the whole batch (p.flat) and dy is read where it lies, [N][K][OHW] with OHW a
+// multiple of 4 and at least MC: a lane's 16-byte piece of a filter's row never straddles two images, and its address
+// is walked from chunk to chunk (MC pixels on, with a jump to the same filter's plane in the next image when the
+// piece leaves its image).
+template <bool DIRECT>
 __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p) {
     __shared__ __attribute__((aligned(16))) float smem[STAGES][STAGE_FLOATS];
     constexpr int D = STAGES - 1;
@@ -104,6 +109,15 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
     }
     uint32_t ld_vb = 0, ld_sa = 0, ld_sb = 0;
     int ld_ml0 = 0;
+    // DIRECT: pixel-in-image, byte offset (row a_row0) and pixels left in the batch of this lane's piece of the next chunk
+    int d_pl = 0, d_addr = 0, d_left = 0;
+    if constexpr (DIRECT) {
+        const int m = chunk_begin * MC + 4 * a_q;
+        const int img = (int)xsmi::fdiv((uint32_t)m, p.dOHW);
+        d_pl = m - img * p.OHW;
+        d_addr = (((img * p.K + k0 + a_row0) * p.OHW) + d_pl) * 4;
+        d_left = p.Mtot - m;
+    }
     int ld_tail = 0;                                                 // the chunk to load runs past the end of its image
     // The input position of this lane's pixel is walked from chunk to chunk instead of being formed by two divisions per
     // chunk (every vector instruction beside the MFMAs takes matrix-pipe time): the pixel advances by MC = q32 rows and
@@ -154,6 +168,11 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
         ld_vb = ok ? (uint32_t)w_addr : 0x80000000u;
     };
     auto issue_a = [&](int j, uint32_t stage) {
+        if constexpr (DIRECT) {                       // row a_row0 + 32 j: 32 planes further in the same image
+            xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), d_left > 0 ? (uint32_t)d_addr : 0x80000000u,
+                                (uint32_t)j * 32u * p.yplane_bytes);
+            return;
+        }
         const uint32_t v = j == 0 ? a_v0 : a_v1;
         // (a load in each branch keeps this a branch: as a select it would cost five vector instructions per chunk)
         if (ld_tail) xsmi::load_lds_b128(ry, stage + (uint32_t)((wave + 4 * j) * 1024), ld_ml0 + 4 * a_q < p.OHWa ? v : 0x80000000u, ld_sa);
@@ -163,6 +182,13 @@ __global__ void __launch_bounds__(256, 4) wgrad_tap_f32_kernel(WgradTapParams p)
         xsmi::load_lds_b32(rx, stage + (uint32_t)(8192 + (wave + 4 * e) * 256), ld_vb, ld_sb + (uint32_t)(8 * e) * p.xplane_bytes);
     };
     auto issue_advance = [&]() {
+        if constexpr (DIRECT) {
+            d_pl += MC;
+            const bool leaves = d_pl >= p.OHW;
+            d_pl -= leaves ? p.OHW : 0;
+            d_addr += MC * 4 + (leaves ? (p.K - 1) * (int)p.yplane_bytes : 0);
+            d_left -= MC;
+        }
         if (++ci == p.cpi) {
             ci = 0; ++in_img;
             w_oh = b_m / p.OW;                                       // the lane's pixel in an image's first chunk
@@ -452,7 +478,7 @@ size_t wgrad_tap_ws_bytes(int N, int C, int K, int R, int S, int OH, int OW) {
     plan(N, C, K, R, S, OH * OW, &cpi, &total, &cps, &splits);
     const int OHW = OH * OW, OHWa = (OHW + 3) & ~3;
     size_t padded = OHWa != OHW ? align_up((size_t)N * K * OHWa * sizeof(float), 256) : 0;
-    if (use_flat(OHW)) padded = align_up((size_t)K * ((N * OHW + 3) & ~3) * sizeof(float), 256);
+    if (use_flat(OHW)) padded = OHW % 4 == 0 && OHW >= MC ? 0 : align_up((size_t)K * ((N * OHW + 3) & ~3) * sizeof(float), 256);
     return align_up((size_t)splits * R * S * K * C * sizeof(float), 256) + align_up((size_t)splits * K * sizeof(float), 256) + padded;
 }
 
@@ -470,7 +496,11 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     p.flat = flat ? 1 : 0;
     p.Mtot = N * OHW;
     p.dOHW = make_fastdiv(OHW);
-    if (flat) {
+    // dy as it lies when its planes are whole 16-byte pieces and at least a chunk long
+    const bool direct = flat && OHW % 4 == 0 && OHW >= MC;
+    if (direct) {
+        OHWa = OHW;
+    } else if (flat) {
         float *dyp = (float *)((char *)dbpart + align_up((size_t)splits * K * sizeof(float), 256));
         const int Ma = (p.Mtot + 3) & ~3;
         const uint32_t total = (uint32_t)((size_t)K * Ma);
@@ -492,7 +522,7 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
     }
     p.dbpart = db ? dbpart : nullptr;
     p.x_bytes = (uint32_t)((size_t)N * C * H * W * 4);
-    p.dy_bytes = flat ? (uint32_t)((size_t)K * OHWa * 4) : (uint32_t)((size_t)N * K * OHWa * 4);
+    p.dy_bytes = flat && !direct ? (uint32_t)((size_t)K * OHWa * 4) : (uint32_t)((size_t)N * K * OHWa * 4);
     p.N = N; p.C = C; p.K = K; p.H = H; p.W = W; p.OH = OH; p.OW = OW; p.OHW = OHW; p.OHWa = OHWa; p.R = R; p.S = S;
     p.sh = sh; p.sw = sw; p.pad = pad;
     p.ctiles = C / TC;
@@ -501,7 +531,8 @@ int wgrad_tap(const float *dy, const float *x, float *dw, float *db, int N, int 
 
     dim3 grid(R * S * p.ctiles, K / TK, splits);
     prof_begin();
-    hipLaunchKernelGGL(wgrad_tap_f32_kernel, grid, dim3(256), 0, st, p);
+    if (direct) hipLaunchKernelGGL(wgrad_tap_f32_kernel<true>, grid, dim3(256), 0, st, p);
+    else hipLaunchKernelGGL(wgrad_tap_f32_kernel<false>, grid, dim3(256), 0, st, p);
     prof_end();
     XSMI_LAUNCH_CHECK("wgrad_tap_f32_kernel");
     if (R * S == 9 && (size_t)K * C >= 65536 && splits <= 16) {
