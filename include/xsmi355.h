@@ -103,8 +103,8 @@ int xsmi_sync(void);
  * the chunks where it pays, 3: even split wherever it applies), "sk_spin_limit" (polls before an even-split
  * workgroup gives up waiting for a partial tile; the calls that wait for the device then fail with
  * XSMI_ERR_RUNTIME), "sk_wide" (the even-split kernel's activation loads: 2: input rows staged once for the three taps of
- * a filter row where that form applies, 16-byte loads tap by tap where only those apply; 1: 16-byte loads tap by tap;
- * 0: one-dword loads everywhere), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
+ * a filter row where that form pays, 16-byte loads tap by tap where only those apply; 3: staged rows wherever they
+ * apply; 1: 16-byte loads tap by tap; 0: one-dword loads everywhere), "pool_bwd" (workgroups per compute unit of the 3x3/2 max-pool gradient kernel whose workgroups walk
  * several pieces; 0: one piece per workgroup), "pack_lanes" (1 to 4: streams over which xsmi_conv2d_pack deals its
  * layout launches), "tap_stages", "tap_persist", "cl_halo", "cl_stem".  Each starts from the environment variable XSMI_<NAME IN CAPITALS> when that is set.
  * A caller that changes one must drop every workspace content it counted on (XSMI_CONV_WS_PACKED) and ask for

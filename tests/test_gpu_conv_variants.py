@@ -60,15 +60,17 @@ GEOMETRIES = [   # n c h w k r s sh sw pad
     (2, 64, 16, 16, 64, 1, 1, 1, 1, 0),      # 1 x 1
     (2, 32, 6, 112, 32, 3, 3, 1, 1, 1),      # rows longer than a tile of 64 pixels
     (3, 32, 7, 24, 96, 3, 3, 1, 1, 1),       # short images: tiles that span two images, 16-channel units in twos
+    (2, 32, 9, 3, 64, 3, 3, 1, 1, 1),        # rows of three pixels: one-dword pieces, 21 row ends inside a tile
+    (5, 32, 3, 2, 64, 3, 3, 1, 1, 1),        # rows of two pixels, images of six: a tile spans eleven images
 ]
 
 
-@pytest.mark.parametrize("tap_sk,sk_wide", [(3, 2), (3, 1), (3, 0), (1, 2), (0, 2)])
+@pytest.mark.parametrize("tap_sk,sk_wide", [(3, 3), (3, 2), (3, 1), (3, 0), (1, 2), (0, 2)])
 @pytest.mark.parametrize("geom", GEOMETRIES)
 def test_even_split_and_whole_tile_kernels(gpu, geom, tap_sk, sk_wide):
     """tap_sk 3: the even-split kernel wherever it applies (sk_wide 2: input rows staged once for a filter row's three
-    taps where that form applies; 1: 16-byte activation loads tap by tap; 0: one-dword loads); 1: where the library
-    finds it pays; 0: whole tiles per workgroup only."""
+    taps where that form pays, 3: wherever it applies; 1: 16-byte activation loads tap by tap; 0: one-dword loads);
+    1: where the library finds it pays; 0: whole tiles per workgroup only."""
     with options(gpu, tap_sk=tap_sk, sk_wide=sk_wide):
         _run(gpu, *geom)
 

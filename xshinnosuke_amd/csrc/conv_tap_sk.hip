@@ -72,7 +72,8 @@ struct SkParams {
     // staged rows (one class; a unit is a filter row x 16 channels, the filter laid out per unit as three taps)
     int staged_rows;
     int out_rows;          // output rows of all images
-    xsmi::FastDiv dPitch;  // by (output row length + 4)
+    int run_slots;         // one-dword pieces: slots of a channel's run that a tile can need
+    xsmi::FastDiv dPitch;  // by (output row length + zeros behind a row: 4, one-dword pieces: 1)
 };
 
 template <int N>
@@ -115,10 +116,16 @@ __device__ __forceinline__ float buf_load(__amdgpu_buffer_rsrc_t r, uint32_t vof
 // image row is followed by four slots of zeros: a tap is then a shift of the fragment read by one slot, and the slot
 // past either end of a row is a zero that the loads themselves wrote (the lanes of those slots fetch out of range).
 // 16-byte loads, nothing to clear, a third of the activation traffic, one barrier per 24 MFMAs.
+//
+// VEC = 2: the same for rows of any width from two pixels on (14 x 14 and 7 x 7 feature maps), with one-dword pieces: a
+// lane owns one slot of a run, every image row is followed by ONE slot of zeros, and a channel's run (at most 66
+// slots plus one per row end inside the tile) takes two wave-loads, the second one mostly idle.
 template <int VEC>
 __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
-    static_assert(VEC == 1 || VEC == 4 || VEC == 3, "B loads of one or four dwords per lane, or staged rows");
-    constexpr bool ROW = VEC == 3;
+    static_assert(VEC == 1 || VEC == 4 || VEC == 3 || VEC == 2, "B loads of one or four dwords per lane, or staged rows");
+    constexpr bool ROW = VEC == 3 || VEC == 2;       // staged rows
+    constexpr bool ROWD = VEC == 2;                  // ... with one-dword pieces
+    constexpr int RPAD = ROWD ? 1 : 4;               // slots of zeros behind an image row = slots of a piece
     constexpr int ROWS = SK_ROWS, PIX = SK_PIX, KC = ROW ? 16 : SK_KC;
     constexpr int UTAPS = ROW ? 3 : 1;               // taps per unit of work
     constexpr int BPITCH = 128;                      // ROW: floats from one channel's run to the next (a run has 84)
@@ -132,9 +139,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     constexpr int STAGE_FLOATS = A_FLOATS + B_FLOATS + SPARE_FLOATS;
     constexpr int NA = UTAPS * QUADS * RT / 4;       // A wave-loads (64 rows x 16 bytes) per wave and chunk
     constexpr int NB = KC * PT / 4;                  // B wave-loads (64 pixels of one channel) per wave and chunk
-    constexpr int NBW = ROW ? 2 : NB / VEC;          // ... as VEC-wide loads; ROW: two channels' runs per wave-load
+    constexpr int NBW = ROWD ? 8 : ROW ? 2 : NB / VEC;   // ... as VEC-wide loads; ROW: two channels' runs per wave-load
+                                                     // (one-dword pieces: half a channel's run)
     constexpr int NI = NBW + NA + 2;                 // issue items per chunk: prepare, B loads, A loads, advance
-    static_assert(ROW ? (NA == 3 && NI == 7) : (NB == 8 && NA == 2 && NI <= 12),
+    static_assert(ROWD ? (NA == 3 && NI == 13) : ROW ? (NA == 3 && NI == 7) : (NB == 8 && NA == 2 && NI <= 12),
                   "64 x 64 tile: the issue items fit the slots of one chunk");
     __shared__ __attribute__((aligned(16))) float smem[2][STAGE_FLOATS];
     __shared__ __attribute__((aligned(16))) float s_bias[2][ROWS];
@@ -168,6 +176,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     uint32_t prep_stale = 1;                           // the pixel offset must be formed again (new segment); the uniform
                                                        // flags are integers so that they live in one scalar register each
     uint32_t ld_asoff = 0, ld_voff = 0, ld_soff = 0;
+    // one-dword staged rows: the lane's second slot (lane + 64) of a run
+    int iyb2 = 0, nbase2 = 0;
+    bool live2 = false;
+    uint32_t ld_voff2 = 0x80000000u;
     int ld_fix = 0;                                    // VEC = 4: the slot the lane clears once its run has landed (issue_prep)
     uint32_t ld_rare = 0;                              // VEC = 4, uniform: a lane of this wave has a run to move (see issue_prep)
     const int csub = VEC == 4 ? lane >> 4 : 0;         // VEC = 4: which of the wave-load's four channels the lane fetches
@@ -194,6 +206,29 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         s = ROW ? 0 : (int)(tap - (uint32_t)r * (uint32_t)c.TS);
         ld_asoff = c.apk_off + (rt * c.iters + ch) * (uint32_t)(A_FLOATS * 4);
         iyb = 0; ixb = 0; nbase = 0;
+        if constexpr (ROWD) {
+            // The lane's slots are slots `lane` and `lane + 64` of a channel's run, which starts one slot before the
+            // tile's first pixel; in run coordinates an image row is OX + 1 slots long, the last one a zero.
+            const int m0 = (int)mt * PIX;
+            const uint32_t ry0 = xsmi::fdiv((uint32_t)m0, c.dOX);
+            const int pitch = c.OX + 1;
+            auto place = [&](int slot, bool &lv, int &yb, int &nb) {
+                const int X = m0 - (int)ry0 * c.OX - 1 + slot + pitch;          // >= 0: counted from the row before
+                const uint32_t d = xsmi::fdiv((uint32_t)X, sp.dPitch);
+                const int xx = X - (int)d * pitch;
+                const int row = (int)ry0 + (int)d - 1;
+                lv = slot < sp.run_slots && xx < c.OX && (unsigned)row < (unsigned)sp.out_rows;
+                yb = 0; nb = 0;
+                if (lv) {
+                    const uint32_t n = xsmi::fdiv((uint32_t)row, c.dOY);
+                    yb = (row - (int)n * c.OY) + c.dy0;
+                    nb = (int)n * c.in_n_stride + xx;
+                }
+            };
+            place(lane, live, iyb, nbase);
+            place(lane + 64, live2, iyb2, nbase2);
+            return;
+        }
         if constexpr (ROW) {
             // The lane's piece is piece `lane & 31` of a channel's run: four slots of the run, which starts four slots
             // before the tile's first pixel.  In run coordinates an image row is OX + 4 slots long; a piece is either
@@ -235,6 +270,11 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         if constexpr (ROW) {
             const bool ok = live && (unsigned)iy < (unsigned)i_IH;
             ld_voff = ok ? (uint32_t)((nbase + iy * i_IW) * 4) : 0x80000000u;
+            if constexpr (ROWD) {
+                const int iy2 = iyb2 + r * i_dstep;
+                const bool ok2 = live2 && (unsigned)iy2 < (unsigned)i_IH;
+                ld_voff2 = ok2 ? (uint32_t)((nbase2 + iy2 * i_IW) * 4) : 0x80000000u;
+            }
         } else if constexpr (VEC == 4) {
             // The lane's run is columns ix .. ix + 3 of one input row; ix = -1 and ix + 3 = IW (one column past either
             // end) are the cases the host admits.  The run is fetched as it lies and the border column's slot is
@@ -265,7 +305,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
     static_assert(RT == 1, "A wave-load f of a chunk is quad f");
     auto issue_b = [&](auto e_, auto st_) {
         constexpr int e = decltype(e_)::value, st = decltype(st_)::value;
-        if constexpr (ROW)                             // channels chan0 + 2 e and + 2 e + 1: 32 pieces each, 21 in use
+        if constexpr (ROWD)                            // channel chan0 + e / 2, slots 64 (e % 2) .. + 63 of its run
+            xsmi::load_lds_b32_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + (e / 2) * BPITCH + (e % 2) * 64) * 4)>(
+                rin, lds_b, e % 2 ? ld_voff2 : ld_voff, ld_soff + (uint32_t)(e / 2) * i_plane);
+        else if constexpr (ROW)                        // channels chan0 + 2 e and + 2 e + 1: 32 pieces each, 21 in use
             xsmi::load_lds_b128_at<(uint32_t)((st * STAGE_FLOATS + A_FLOATS + 2 * e * BPITCH) * 4)>(rin, lds_b, ld_voff,
                                                                                                    ld_soff + (uint32_t)(2 * e) * i_plane);
         else if constexpr (VEC == 4)                   // channels chan0 + 4 e .. + 3, the tile's 64 pixels
@@ -382,10 +425,10 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
         c_complete = ch + n_seg == c.iters ? 1u : 0u;
         c_tile_end = cu + (c.iters - ch);
         if constexpr (ROW) {
-            auto run_slot = [&](int m0) {              // pixel m0 + (wc * 32 + l31): slot 4 + p + 4 * (row ends before it)
+            auto run_slot = [&](int m0) {              // pixel m0 + (wc * 32 + l31): slot RPAD + p + RPAD * (row ends before it)
                 const uint32_t ry0 = xsmi::fdiv((uint32_t)m0, c.dOX);
                 const int xp = m0 - (int)ry0 * c.OX + wc * 32 + l31;
-                return b_rd + 3 + 4 * (int)xsmi::fdiv((uint32_t)xp, c.dOX);
+                return b_rd + (RPAD - 1) + RPAD * (int)xsmi::fdiv((uint32_t)xp, c.dOX);
             };
             b_run = run_slot(c_m0);
             b_run_next = run_slot(c_rt + 1 == rowtiles ? c_m0 + PIX : c_m0);
@@ -572,6 +615,13 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
 #pragma unroll
             for (int k = 0; k < KC / 2; ++k) fb[set][k] = base[run + tap + k * BPITCH];
         };
+        // the issue items of a unit over the six MFMAs behind the barrier: one per MFMA (one-dword pieces: two), the
+        // rest with the last
+        auto issue_slot = [&](auto q_, auto buf_) {
+            constexpr int q = decltype(q_)::value, per = ROWD ? 2 : 1;
+            static_for<per>([&](auto i) { issue_item_at(IC<q * per + decltype(i)::value>{}, buf_); });
+            if constexpr (q == 5) static_for<NI - 6 * per>([&](auto i) { issue_item_at(IC<6 * per + decltype(i)::value>{}, buf_); });
+        };
         auto body_row = [&](auto buf_) {
             constexpr int cur = decltype(buf_)::value, nxt = cur ^ 1;
             constexpr int s0 = cur, s1 = cur ^ 1;      // register sets of taps 0 and 2 / of tap 1
@@ -619,30 +669,29 @@ __global__ void __launch_bounds__(256, 3) tap_sk_f32_kernel(SkParams sp) {
             fa[s1][0] = *reinterpret_cast<const float4 *>(nbase_ + a_rd);
             fb[s1][0] = nbase_[run];
             fb[s1][1] = nbase_[run + BPITCH];
-            issue_item_at(IC<0>{}, buf_);
+            issue_slot(IC<0>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[1], fa[s0][0].w, fb[s0][3]);
             fa[s1][1] = *reinterpret_cast<const float4 *>(nbase_ + a_rd + ROWS * 4);
             fb[s1][2] = nbase_[run + 2 * BPITCH];
             fb[s1][3] = nbase_[run + 3 * BPITCH];
-            issue_item_at(IC<1>{}, buf_);
+            issue_slot(IC<1>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[0], fa[s0][1].x, fb[s0][4]);
             fb[s1][4] = nbase_[run + 4 * BPITCH];
             fb[s1][5] = nbase_[run + 5 * BPITCH];
             fb[s1][6] = nbase_[run + 6 * BPITCH];
             fb[s1][7] = nbase_[run + 7 * BPITCH];
-            issue_item_at(IC<2>{}, buf_);
+            issue_slot(IC<2>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[1], fa[s0][1].y, fb[s0][5]);
-            issue_item_at(IC<3>{}, buf_);
+            issue_slot(IC<3>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[0], fa[s0][1].z, fb[s0][6]);
-            issue_item_at(IC<4>{}, buf_);
+            issue_slot(IC<4>{}, buf_);
             XSMI_PIN();
             XSMI_MFMA(acc[1], fa[s0][1].w, fb[s0][7]);
-            issue_item_at(IC<5>{}, buf_);
-            issue_item_at(IC<6>{}, buf_);
+            issue_slot(IC<5>{}, buf_);
             XSMI_PIN();
         };
         // prologue: chunk 0 landed and in registers, chunk 1 in flight
@@ -819,28 +868,37 @@ bool sk_wide_loads_ok(const SkParams &p) {
 }
 
 // Staged rows (the filter must have been laid out for them): 3 x 3, stride 1, one column and one row of padding, rows
-// as wide as the output's, a multiple of four pixels and at least 20 (a tile of 64 pixels then crosses at most three
-// row ends: 21 pieces per run), channels in chunks of 16.
-bool sk_rows_staged(int R, int S, int sh, int sw, int pad, int in_w, int out_w, int channels) {
-    return xsmi::option(xsmi::OPT_SK_WIDE) >= 2 && R == 3 && S == 3 && sh == 1 && sw == 1 && pad == 1 && in_w == out_w &&
-           out_w % 4 == 0 && out_w >= 20 && channels % 16 == 0;
+// as wide as the output's, channels in chunks of 16.  1: 16-byte pieces, for rows a multiple of four pixels and at
+// least 20 wide (a tile of 64 pixels then crosses at most three row ends: 21 pieces per run); 2: one-dword pieces, for
+// rows of two to eleven pixels (66 slots plus one per row end inside a tile: at most 98 of a run's 128).  The kernel
+// serves wider rows in that form as well, but from 14 pixels on it is no faster than tap by tap (measured at N=32:
+// 512 -> 512 at 7 x 7 65.9 -> 64.7 us, 256 -> 256 at 14 x 14 63.2 -> 63.6 us); sk_wide = 3 takes it wherever it applies.
+int sk_rows_staged(int R, int S, int sh, int sw, int pad, int in_w, int out_w, int channels) {
+    const long opt = xsmi::option(xsmi::OPT_SK_WIDE);
+    if (opt < 2 || R != 3 || S != 3 || sh != 1 || sw != 1 || pad != 1 || in_w != out_w || channels % 16 != 0 || out_w < 2)
+        return 0;
+    if (out_w % 4 == 0 && out_w >= 20) return 1;
+    return out_w < 12 || opt >= 3 ? 2 : 0;
 }
 
 int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
     static int res_narrow = 0, res_wide = 0, res_rows = 0;
-    const bool rows = p.staged_rows != 0;
+    static int res_rows1 = 0;
+    const int rows = p.staged_rows;
     const bool wide = !rows && sk_wide_loads_ok(p);
     if (rows) {
         const SkClass &c = p.cls[0];
-        if (p.ncls != 1 || c.sx != 1 || c.sy != 1 || c.TS != 3 || c.dx0 + c.dstep != 0 || c.IW != c.OX || c.OX % 4 != 0 ||
-            c.OX < 20 || (((uintptr_t)p.in) & 3) != 0)
+        if (p.ncls != 1 || c.sx != 1 || c.sy != 1 || c.TS != 3 || c.dx0 + c.dstep != 0 || c.IW != c.OX || c.OX < 2 ||
+            (rows == 1 && (c.OX % 4 != 0 || c.OX < 20)) || (((uintptr_t)p.in) & 3) != 0)
             return xsmi::set_error("even-split convolution: geometry not served by the staged-row form"), XSMI_ERR_INVALID;
         p.out_rows = c.M / c.OX;
-        p.dPitch = xsmi::make_fastdiv(c.OX + 4);
+        p.dPitch = xsmi::make_fastdiv(c.OX + (rows == 1 ? 4 : 1));
+        p.run_slots = 66 + (c.OX - 1 + 63) / c.OX;
     }
-    uint32_t gsz = (uint32_t)(rows   ? sk_resident(tap_sk_f32_kernel<3>, &res_rows, SK_MAX_GRID)
-                              : wide ? sk_resident(tap_sk_f32_kernel<4>, &res_wide, SK_MAX_GRID)
-                                     : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
+    uint32_t gsz = (uint32_t)(rows == 1 ? sk_resident(tap_sk_f32_kernel<3>, &res_rows, SK_MAX_GRID)
+                              : rows    ? sk_resident(tap_sk_f32_kernel<2>, &res_rows1, SK_MAX_GRID)
+                              : wide    ? sk_resident(tap_sk_f32_kernel<4>, &res_wide, SK_MAX_GRID)
+                                        : sk_resident(tap_sk_f32_kernel<1>, &res_narrow, SK_MAX_GRID));
     if (gsz > p.units) gsz = p.units;                  // every workgroup gets at least one chunk
     if (gsz == 0) return XSMI_OK;
     p.upg = p.units / gsz; p.urem = p.units % gsz; p.dG = xsmi::make_fastdiv(gsz);
@@ -853,7 +911,8 @@ int sk_launch(hipStream_t st, SkParams &p, const SkShape &) {
     p.part_bytes = (uint32_t)xsmi::SK_SCRATCH_PART_BYTES;
     const long spin = xsmi::option(xsmi::OPT_SK_SPIN_LIMIT);
     p.spin_limit = spin < 0 ? 0u : spin > 0x7fffffffL ? 0x7fffffffu : (uint32_t)spin;
-    if (rows) hipLaunchKernelGGL(tap_sk_f32_kernel<3>, dim3(gsz), dim3(256), 0, st, p);
+    if (rows == 1) hipLaunchKernelGGL(tap_sk_f32_kernel<3>, dim3(gsz), dim3(256), 0, st, p);
+    else if (rows) hipLaunchKernelGGL(tap_sk_f32_kernel<2>, dim3(gsz), dim3(256), 0, st, p);
     else if (wide) hipLaunchKernelGGL(tap_sk_f32_kernel<4>, dim3(gsz), dim3(256), 0, st, p);
     else hipLaunchKernelGGL(tap_sk_f32_kernel<1>, dim3(gsz), dim3(256), 0, st, p);
     XSMI_LAUNCH_CHECK("tap_sk_f32_kernel");
@@ -913,7 +972,7 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     const int rowtiles = ceil_div(K, shp.rows_tile);
     const size_t pack = sk_pack_bytes(K, C, R * S, shp);
     float *apk = (float *)workspace;
-    const bool staged = sk_rows_staged(R, S, sh, sw, pad, W, OW, C) && (((uintptr_t)w) & 15) == 0 && (((uintptr_t)x) & 3) == 0;
+    const int staged = (((uintptr_t)w) & 15) == 0 && (((uintptr_t)x) & 3) == 0 ? sk_rows_staged(R, S, sh, sw, pad, W, OW, C) : 0;
     const int kc = staged ? 16 : shp.kc;
     if (!(opts & 2) && R == 3 && S == 3 && (((uintptr_t)w) & 15) == 0) {
         const uint32_t total = (uint32_t)rowtiles * (uint32_t)(C / kc) * (uint32_t)(kc / 4) * (uint32_t)shp.rows_tile;
@@ -958,7 +1017,7 @@ int sk_conv_fwd(const float *x, const float *w, const float *bias, float *y, uin
     p.out_bytes = (uint32_t)((size_t)N * K * OH * OW * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = 1; p.rowtiles = rowtiles; p.accumulate = 0; p.relu = relu;
-    p.staged_rows = staged ? 1 : 0;
+    p.staged_rows = staged;
     prof_begin();
     int rc = sk_launch(st, p, shp);
     prof_end();
@@ -1004,7 +1063,7 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
     }
     const size_t pack = off;
     // the pass reads dy (rows of OW pixels) and writes dx (rows of W pixels)
-    const bool staged = nplans == 1 && sk_rows_staged(R, S, sh, sw, pad, OW, W, K) && (((uintptr_t)dy) & 3) == 0;
+    const int staged = nplans == 1 && (((uintptr_t)dy) & 3) == 0 ? sk_rows_staged(R, S, sh, sw, pad, OW, W, K) : 0;
     const int kc = staged ? 16 : shp.kc;
     if (staged) {                                      // a unit is a filter row x 16 channels
         plans[0].nch = K / kc;
@@ -1057,7 +1116,7 @@ int sk_conv_bwd_data(const float *dy, const float *w, float *dx, int N, int C, i
     p.out_bytes = (uint32_t)((size_t)N * C * H * W * 4);
     p.apk_bytes = (uint32_t)pack;
     p.ncls = ncls; p.rowtiles = rowtiles; p.accumulate = accumulate; p.relu = 0;
-    p.staged_rows = staged ? 1 : 0;
+    p.staged_rows = staged;
     prof_begin();
     int rc = sk_launch(st, p, shp);
     prof_end();
