@@ -1,9 +1,9 @@
 // Tap-major implicit-GEMM convolution (forward and backward-data), fp32 MFMA, with an even split of the launch's
 // work over the resident workgroups.
 //
-// Same reduction order and data path as conv_tap.hip (reduction index = (tap, channel); global -> LDS directly; zero
-// border through the buffer range check; 64 x 64 outputs per workgroup, 32 x 32 per wave, 32-channel chunks), but
-// work is counted in chunks (one tap x 32 channels of one tile): the launch has exactly as many workgroups as fit on
+// Same data path as conv_tap.hip (reduction index = (tap, channel); global -> LDS directly; zero border through the
+// buffer range check; 64 x 64 outputs per workgroup, 32 x 32 per wave), but work is counted in chunks (one tap x 32
+// channels of one tile; in the staged-row forms below one filter row x 16 channels): the launch has exactly as many workgroups as fit on
 // the chip at once and workgroup g takes the contiguous range [g * U / G, (g + 1) * U / G) of the U chunks of all
 // tiles, walking it as one software-pipelined stream.  Every compute unit therefore gets the same amount of matrix
 // work whatever the tile count is (ResNet-18 at N=32 has 1.5 to 6.1 tiles per CU: up to a quarter of the machine
