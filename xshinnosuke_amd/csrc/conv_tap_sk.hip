@@ -934,11 +934,15 @@ bool sk_path_ok(int reduce_channels, int rows) {
 // tiles): every stride-1 pass with at least four taps (+1 to +17 %: no idle compute units when there are fewer tiles
 // than CUs, no mostly empty last round of tiles otherwise), and every strided backward-data pass, whose four residue
 // classes of different lengths then share one balanced launch (+20 to +26 %).  Strided forwards (mixed: -13 to +5 %)
-// and 1 x 1 filters (a handful of chunks per tile) stay on whole tiles.
+// and 1 x 1 filters (a handful of chunks per tile) stay on whole tiles, except strided forwards with fewer tiles than CUs.
 bool sk_fwd_pays(int M, int rows, int R, int S, int sh, int sw) {
-    (void)M; (void)rows;
     if (sk_env() >= 3) return true;                    // forced, for tests and measurements
-    return sh == 1 && sw == 1 && R * S >= 4;
+    if (R * S < 4) return false;
+    if (sh == 1 && sw == 1) return true;
+    // a strided forward with fewer tiles than compute units: whole tiles leave CUs idle from the start
+    // (256 -> 512, 3 x 3 / 2 at 14 x 14, N=32: 200 tiles, 53.6 -> 49.6 us)
+    return (long)ceil_div(M, SK_PIX) * ceil_div(rows, SK_ROWS) <= 256;        // the MI355X's CU count, as a constant: the
+                                                                               // choice must not depend on whether a device is open
 }
 bool sk_bwd_data_pays(int M, int rows, int R, int S, int sh, int sw) {
     if (sk_env() >= 3) return true;
