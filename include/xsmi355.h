@@ -374,6 +374,15 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
 int xsmi_bn_add_relu_fwd(const float *x, const float *gamma, const float *beta, const float *residual, float *y,
                          float *sqrtvar, float *mean, float *var, float *moving_mean, float *moving_var, float momentum,
                          uint8_t *neg_mask, int N, int C, int HW, float eps, void *ws, size_t ws_bytes);
+/* The head of a ResNet as two passes over the convolution's output instead of four: batch statistics, then
+ * normalisation, ReLU and the 3 x 3 / stride 2 / pad 1 max-pool in one kernel.  pooled (N, C, H/2, W/2) and idx are what
+ * xsmi_maxpool2d_fwd would give on the output of xsmi_bn_fwd with neg_mask (same comparisons on the same float values,
+ * hence the same bits), neg_mask (N*C*H*W) and the statistics are xsmi_bn_fwd's; the normalised tensor is not stored.
+ * H even, W a multiple of 4.  Stands for xs/nn/functional.py:676-707, xs/layers/activators.py:37-50 and
+ * xs/nn/functional.py:445-491 in a row; the backward is xsmi_maxpool2d_bwd followed by xsmi_bn_bwd with the mask. */
+int xsmi_bn_relu_maxpool_fwd(const float *x, const float *gamma, const float *beta, float *pooled, uint8_t *idx,
+                             uint8_t *neg_mask, float *sqrtvar, float *mean, float *var, float *moving_mean, float *moving_var,
+                             float momentum, int N, int C, int H, int W, float eps, void *ws, size_t ws_bytes);
 /* Inference form with given statistics (xs/nn/functional.py:708-725); relu != 0 clips at zero. */
 int xsmi_bn_infer(const float *x, const float *gamma, const float *beta, const float *mean, const float *var, float *y,
                   int N, int C, int HW, float eps, int relu);

@@ -74,6 +74,51 @@ def test_batch_norm_forward_backward_and_moving_statistics(gpu, shape):
     np.testing.assert_array_equal(yir.numpy(), np.maximum(yi.numpy(), 0))
 
 
+@pytest.mark.parametrize("shape", [(4, 8, 56, 56), (2, 3, 112, 112), (33, 5, 16, 20), (2, 4, 8, 12)])
+def test_batch_norm_relu_max_pool_as_one_pass(gpu, shape):
+    """The head of a ResNet: a held-back normalisation with its own ReLU followed by the 3x3 / stride 2 / pad 1 max-pool
+    of its result runs as one normalisation whose second pass pools.  Pooled values, window indices, sign mask and
+    statistics equal those of the separate passes bit for bit (same operations on the same values; the last shape is
+    small enough for the separate normalisation to take its single-kernel form, whose sums are added in another order:
+    compared to float32 accuracy there); the normalisation's own result is not stored and says so when read."""
+    K = gpu.kernels
+    rng = np.random.default_rng(sum(shape) + 2)
+    n, c, h, w = shape
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    x[0, 0, :2, :4] = x[0, 0, 0, 0]                  # ties inside a window: the first maximum in window order wins
+    gamma = rng.uniform(0.5, 1.5, c).astype(np.float32); beta = rng.standard_normal(c).astype(np.float32)
+    mm0 = rng.standard_normal(c).astype(np.float32); mv0 = rng.uniform(0.5, 2.0, c).astype(np.float32)
+    eps = 1e-5
+    xd, gd, bd = gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta)
+    mm, mv = gpu.to_device(mm0), gpu.to_device(mv0)
+    mask = gpu.empty(shape, np.uint8)
+    y, _, sq, mean, var = K.bn_fwd(xd, gd, bd, eps, moving=(mm, mv), momentum=0.9, neg_mask=mask, want_xhat=False)
+    p, i = K.maxpool2d_fwd(y, 3, (2, 2), 1)
+    ref = [a.numpy() for a in (p, i, mask, sq, mean, var, mm, mv)]
+    mm, mv = gpu.to_device(mm0), gpu.to_device(mv0)
+    mask2 = gpu.empty(shape, np.uint8)
+    y2, _, sq2, mean2, var2 = K.bn_fwd(xd, gd, bd, eps, moving=(mm, mv), momentum=0.9, neg_mask=mask2, want_xhat=False,
+                                       defer=True)
+    p2, i2 = K.maxpool2d_fwd(y2, 3, (2, 2), 1)
+    got = [a.numpy() for a in (p2, i2, mask2, sq2, mean2, var2, mm, mv)]
+    exact = n * h * w > 8192
+    for g, e in zip(got, ref):
+        if exact or g.dtype == np.uint8:
+            np.testing.assert_array_equal(g, e)
+        else:
+            np.testing.assert_allclose(g, e, rtol=2e-6, atol=1e-6)
+    with pytest.raises(gpu.XsmiError, match="not stored"):
+        y2.numpy()
+    # any other pool geometry, and any other call in between: the separate passes
+    y3, _, _, _, _ = K.bn_fwd(xd, gd, bd, eps, neg_mask=mask2, want_xhat=False, defer=True)
+    p3, _ = K.maxpool2d_fwd(y3, 2, (2, 2), 0)
+    np.testing.assert_array_equal(y3.numpy(), y.numpy())
+    np.testing.assert_array_equal(p3.numpy(), K.maxpool2d_fwd(y, 2, (2, 2), 0)[0].numpy())
+    y4, _, _, _, _ = K.bn_fwd(xd, gd, bd, eps, neg_mask=mask2, want_xhat=False, defer=True)
+    np.testing.assert_array_equal(y4.numpy(), y.numpy())
+    np.testing.assert_array_equal(K.maxpool2d_fwd(y4, 3, (2, 2), 1)[0].numpy(), ref[0])
+
+
 # two-kernel float4 form, two-kernel scalar form (planes not a multiple of four), single-kernel forms (256 / 1024 threads)
 @pytest.mark.parametrize("shape", [(8, 16, 40, 40), (6, 5, 37, 41), (32, 64, 14, 14), (4, 8, 6, 6), (64, 16)])
 def test_batch_norm_add_relu_as_one_pass(gpu, shape):

@@ -97,6 +97,7 @@ SIGNATURES = {
     "xsmi_bn_workspace_bytes": (_sz, [_i]),
     "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_add_relu_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
+    "xsmi_bn_relu_maxpool_fwd": (_i, [_vp] * 11 + [_f, _i, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f, _i]),
     "xsmi_bn_fold": (_i, [_vp] * 8 + [_i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 9 + [_i, _i, _i, _vp, _sz]),
@@ -217,7 +218,9 @@ def layouts_enqueued(*held):
 # few passes as it needs (kernels.bn_fwd / kernels.add / kernels.relu_fwd):
 #   ("add", a, b, out)            an element-wise add into a new array; if the next call is the in-place ReLU of its
 #                                 result, both run as one pass;
-#   ("bn", entry)                 a training batch normalisation (kernels.BnEntry: operands, outputs, launch); if the
+#   ("bn", entry)                 a training batch normalisation (kernels.BnEntry: operands, outputs, launch); with a
+#                                 ReLU of its own, if the next call is the 3x3/2 max-pool of its result, both run as one
+#                                 normalisation whose second pass pools; without one, if the
 #                                 next call is a held-back add with its result as one operand, it becomes
 #   ("bn_add", entry, a, b, out)  and if the call after that is the in-place ReLU (with mask) of the sum, the three run
 #                                 as one normalisation whose second pass adds the other operand and clips.

@@ -345,12 +345,28 @@ def maxpool2d_fwd(x, k, stride, pad=0, out=None, idx=None, want_idx=True):
     oh, ow = pool_out_hw(h, w, k, stride, pad)
     if oh <= 0 or ow <= 0:
         raise ValueError("max_pool2d: window %d does not fit the padded input %dx%d" % (k, h + 2 * pad, w + 2 * pad))
-    if out is None:
-        out = empty((n, c, oh, ow))
-    elif out.shape != (n, c, oh, ow):
-        raise ValueError("max_pool2d: out has shape %s, expected %s" % (out.shape, (n, c, oh, ow)))
-    if idx is None and want_idx:
-        idx = empty((n, c, oh, ow), np.uint8)
+    # a normalisation of x that has not been launched yet is taken out of the queue first (an allocation below may
+    # call into the library, which would launch it)
+    entry = capi.take_deferred_bn(x, None)
+    try:
+        if out is None:
+            out = empty((n, c, oh, ow))
+        elif out.shape != (n, c, oh, ow):
+            raise ValueError("max_pool2d: out has shape %s, expected %s" % (out.shape, (n, c, oh, ow)))
+        if idx is None and want_idx:
+            idx = empty((n, c, oh, ow), np.uint8)
+    except Exception:
+        if entry is not None:
+            entry.launch()                            # what was asked for before this call still happens
+        raise
+    if entry is not None:
+        # the input is a normalisation with a ReLU that has not been launched yet: the head of a ResNet in one pass
+        if (entry.relu_mask is not None and k == 3 and tuple(stride) == (2, 2) and pad == 1 and h % 2 == 0 and w % 4 == 0
+                and out.is_whole()):
+            out.take_fresh()
+            entry.launch(pooled=out, idx=idx)
+            return out, idx
+        entry.launch()
     xcl = x.channels_last() if idx is None else None
     if xcl is not None and xcl.border >= pad:         # no argmax wanted and the input lives in channels-last form
         ycl = out.channels_last_out(1)
@@ -448,7 +464,15 @@ def add(a, b, out=None, defer=False):
     _f32(a, "a"); _f32(b, "b")
     if defer and out is None and a.size == b.size:
         entry = capi.take_deferred_bn(a, b) if a is not b else None
-        out = empty(a.shape)
+        if entry is not None and entry.relu_mask is not None:       # a normalisation with a ReLU of its own: as it is
+            entry.launch()
+            entry = None
+        try:
+            out = empty(a.shape)
+        except Exception:
+            if entry is not None:
+                entry.launch()                        # what was asked for before this call still happens
+            raise
         if entry is not None:
             # one operand is a normalisation that has not been launched yet: both wait for the call after this one
             (b if entry.y is a else a).ptr            # the other operand: a pending clear is carried out now
@@ -560,19 +584,30 @@ FUSE_BN_ADD_RELU = os.environ.get("XSMI_FUSE_BN_ADD_RELU", "1") != "0"
 class BnEntry:
     """A training batch normalisation that has been asked for and not launched yet (see capi._deferred)."""
 
-    __slots__ = ("x", "gamma", "beta", "eps", "y", "sqrtvar", "mean", "var", "mm", "mv", "momentum", "dims", "ws")
+    __slots__ = ("x", "gamma", "beta", "eps", "y", "sqrtvar", "mean", "var", "mm", "mv", "momentum", "dims", "ws",
+                 "relu_mask")
 
-    def launch(self, residual=None, out=None, neg_mask=None):
-        """Plain: y = gamma * xhat + beta.  With ``residual``: out = max(0, y + residual) and its sign mask in one
-        pass; y itself is then never written, and reading it raises."""
+    def launch(self, residual=None, out=None, neg_mask=None, pooled=None, idx=None):
+        """Plain: y = gamma * xhat + beta (clipped at zero, with the sign mask, when the entry has a ReLU of its own).
+        With ``residual``: out = max(0, y + residual) and its sign mask in one pass.  With ``pooled``: the 3x3/2
+        max-pool of the clipped y (and ``idx``) in one pass.  In both fused forms y itself is never written, and
+        reading it raises."""
         n, c, hw = self.dims
         ws, ws_bytes = self.ws
         mm, mv = self.mm, self.mv
         stats = (self.sqrtvar.cptr, self.mean.cptr, self.var.cptr, mm.cptr if mm is not None else None,
                  mv.cptr if mv is not None else None, float(self.momentum))
+        if pooled is not None:
+            _, _, h, w = self.x.shape
+            self.y.never_written("this batch normalisation's result was consumed by the max-pool that followed it, in one "
+                                 "pass, and was not stored (XSMI_FUSE_BN_ADD_RELU=0 keeps the passes apart)")
+            lib.call("xsmi_bn_relu_maxpool_fwd", self.x.cptr, self.gamma.cptr, self.beta.cptr, pooled.cptr,
+                     idx.cptr if idx is not None else None, self.relu_mask.cptr, *stats, n, c, h, w, float(self.eps),
+                     ws, ws_bytes)
+            return
         if residual is None:
-            lib.call("xsmi_bn_fwd", self.x.cptr, self.gamma.cptr, self.beta.cptr, self.y.cptr, None, *stats, None,
-                     n, c, hw, float(self.eps), ws, ws_bytes)
+            lib.call("xsmi_bn_fwd", self.x.cptr, self.gamma.cptr, self.beta.cptr, self.y.cptr, None, *stats,
+                     self.relu_mask.cptr if self.relu_mask is not None else None, n, c, hw, float(self.eps), ws, ws_bytes)
             return
         self.y.never_written("this batch normalisation's result was consumed by the add and ReLU that followed it, in "
                              "one pass, and was not stored (XSMI_FUSE_BN_ADD_RELU=0 keeps the three passes apart)")
@@ -586,7 +621,8 @@ def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None
     ``want_xhat=False`` skips the store of the normalised input (None is returned for it): ``bn_bwd`` forms it
     again from x and the batch mean.  ``defer=True`` (without mask and normalised input) holds the launch back until
     the next call into the library: an add of y and another tensor followed by the in-place ReLU of the sum then runs
-    inside the normalisation's second pass; any other call enqueues the normalisation first."""
+    inside the normalisation's second pass, and so does (with ``neg_mask``, i.e. a ReLU of the normalisation's own) a
+    3x3 / stride 2 / pad 1 max-pool of y; any other call enqueues the normalisation first."""
     _f32(x, "x")
     n, c, hw = _nchw3(x.shape)
     y = _like(x, y); xhat = empty(x.shape) if want_xhat else None
@@ -596,8 +632,9 @@ def bn_fwd(x, gamma, beta, eps, y=None, moving=None, momentum=0.0, neg_mask=None
     if mm is not None and (mm.size != c or mv.size != c):
         raise ValueError("bn_fwd: moving statistics must have %d elements" % c)
     ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
-    if defer and FUSE_BN_ADD_RELU and neg_mask is None and not want_xhat and y.is_whole():
+    if defer and FUSE_BN_ADD_RELU and not want_xhat and y.is_whole():
         e = BnEntry()
+        e.relu_mask = neg_mask
         e.x, e.gamma, e.beta, e.eps, e.y = x, gamma, beta, eps, y
         e.sqrtvar, e.mean, e.var, e.mm, e.mv, e.momentum = sqrtvar, mean, var, mm, mv, momentum
         e.dims, e.ws = (n, c, hw), (ws, ws_bytes)

@@ -391,6 +391,90 @@ __global__ void __launch_bounds__(256) bn_apply_kernel(const float *__restrict__
         }
     }
 }
+// Pass 2 of the forward with the ReLU and the 3 x 3 / stride 2 / pad 1 max-pool that follow it (the head of a ResNet):
+// block (c, sp) forms the channel's statistics like bn_apply_kernel and then produces pooled outputs of that channel,
+// two per thread and step (unit u of the channel = (image, output row, output pair)): the 3 x 5 inputs of the pair are
+// normalised and clipped in registers, exactly as bn_apply_kernel would have stored them, and compared exactly as
+// maxpool_fwd_3x3s2p1 compares them (first maximum in window order wins, the zero border competes).  The normalised
+// tensor itself is never written; the sign mask of the pre-activation is (every input element once, by the thread whose
+// pair has it in window rows 1 and 2 at columns 4j .. 4j + 3).  H even, W a multiple of 4.
+typedef float bn_f2v __attribute__((ext_vector_type(2)));
+__global__ void __launch_bounds__(256) bn_relu_maxpool_kernel(const float *__restrict__ x, const float *__restrict__ gamma,
+                                                               const float *__restrict__ beta, const double *__restrict__ part,
+                                                               int nsplit_part, double m, float eps, float momentum, BnFwdOut o,
+                                                               uint8_t *__restrict__ idx, int C, int H, int W,
+                                                               xsmi::FastDiv dQ, xsmi::FastDiv dOHQ, uint32_t total, uint32_t per) {
+    __shared__ double sm[2];
+    const int c = blockIdx.x, sp = blockIdx.y;
+    double s0, s1;
+    bn_channel_sums(part, c, nsplit_part, sm, s0, s1);
+    const double mu_d = s0 / m;
+    double var = s1 / m - mu_d * mu_d;
+    if (var < 0.0) var = 0.0;
+    const float mu = (float)mu_d, rs = (float)sqrt(var + (double)eps), g = gamma[c], bt = beta[c];
+    if (sp == 0 && threadIdx.x == 0) {
+        o.mean[c] = mu;
+        o.var[c] = (float)var;
+        o.sqrtvar[c] = rs;
+        if (o.moving_mean) {
+            o.moving_mean[c] = momentum * o.moving_mean[c] + (1.f - momentum) * mu;
+            o.moving_var[c] = momentum * o.moving_var[c] + (1.f - momentum) * (float)var;
+        }
+    }
+    const int OH = H >> 1, OW = W >> 1, Q = OW >> 1;
+    const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
+    for (uint32_t u = beg + threadIdx.x; u < end; u += 256) {
+        const uint32_t n = xsmi::fdiv(u, dOHQ), rem = u - n * dOHQ.d;
+        const int oh = (int)xsmi::fdiv(rem, dQ), j = (int)rem - oh * Q;
+        const size_t pl = (size_t)n * C + c;
+        const float *plane = x + pl * (size_t)H * W;
+        float4 v[3];
+        float lf[3];
+        bool have[3];
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const int ih = 2 * oh - 1 + r;
+            have[r] = (unsigned)ih < (unsigned)H;
+            v[r] = make_float4(0.f, 0.f, 0.f, 0.f);
+            lf[r] = 0.f;
+            if (have[r]) {
+                v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * W + 4 * j);
+                if (j > 0) lf[r] = plane[(size_t)ih * W + 4 * j - 1];
+            }
+        }
+        auto act = [&](float xv, unsigned char &neg) {
+            const float pre = g * ((xv - mu) / rs) + bt;
+            neg = pre < 0.f ? 1 : 0;
+            return pre < 0.f ? 0.f : pre;
+        };
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            unsigned char nl, n0, n1, n2, n3;
+            if (have[r]) {                             // a row outside the image is the pool's zero border as it is
+                lf[r] = j > 0 ? act(lf[r], nl) : 0.f;
+                v[r].x = act(v[r].x, n0); v[r].y = act(v[r].y, n1); v[r].z = act(v[r].z, n2); v[r].w = act(v[r].w, n3);
+                if (r > 0)
+                    *reinterpret_cast<uchar4 *>(o.neg_mask + (pl * H + (2 * oh - 1 + r)) * (size_t)W + 4 * j) = make_uchar4(n0, n1, n2, n3);
+            }
+        }
+        float b0 = 0.f, b1 = 0.f;
+        int w0 = 0, w1 = 0;
+#pragma unroll
+        for (int r = 0; r < 3; ++r) {
+            const float left = lf[r];
+            if (r == 0 || left > b0) { b0 = left; w0 = r * 3 + 0; }
+            if (v[r].x > b0) { b0 = v[r].x; w0 = r * 3 + 1; }
+            if (v[r].y > b0) { b0 = v[r].y; w0 = r * 3 + 2; }
+            if (r == 0 || v[r].y > b1) { b1 = v[r].y; w1 = r * 3 + 0; }
+            if (v[r].z > b1) { b1 = v[r].z; w1 = r * 3 + 1; }
+            if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
+        }
+        const size_t ob = (pl * OH + oh) * (size_t)OW + 2 * j;
+        bn_f2v yv; yv.x = b0; yv.y = b1;
+        __builtin_nontemporal_store(yv, reinterpret_cast<bn_f2v *>(o.y + ob));
+        if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + ob));
+    }
+}
 // pass 2 of the backward: block (c, sp) turns the partial sums into dbeta = sum(dy) and dgamma = sum(dy*xhat) (block
 // sp == 0 stores them) and writes dx for its units of the channel.  With `mean`, xhat holds the values before
 // normalisation and (xhat - mean) / sqrtvar is formed here.
@@ -927,6 +1011,38 @@ int xsmi_bn_fwd(const float *x, const float *gamma, const float *beta, float *y,
                 float eps, void *ws, size_t ws_bytes) {
     return bn_fwd_impl(x, gamma, beta, y, xhat, sqrtvar, mean, var, moving_mean, moving_var, momentum, neg_mask, nullptr, N,
                        C, HW, eps, ws, ws_bytes);
+}
+
+int xsmi_bn_relu_maxpool_fwd(const float *x, const float *gamma, const float *beta, float *pooled, uint8_t *idx,
+                             uint8_t *neg_mask, float *sqrtvar, float *mean, float *var, float *moving_mean, float *moving_var,
+                             float momentum, int N, int C, int H, int W, float eps, void *ws, size_t ws_bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0, "xsmi_bn_relu_maxpool_fwd: empty tensor");
+    XSMI_CHECK_ARG(H % 2 == 0 && W % 4 == 0, "xsmi_bn_relu_maxpool_fwd: planes of an even number of rows, a multiple of four wide");
+    XSMI_CHECK_ARG((double)N * C * H * W < 536870912.0, "xsmi_bn_relu_maxpool_fwd: tensors of 2^29 elements or more are not supported");
+    XSMI_CHECK_ARG(x && gamma && beta && pooled && neg_mask && sqrtvar && mean && var, "xsmi_bn_relu_maxpool_fwd: null pointer");
+    XSMI_CHECK_ARG(aligned16(x) && ((uintptr_t)neg_mask & 3) == 0 && ((uintptr_t)pooled & 7) == 0 && (!idx || ((uintptr_t)idx & 1) == 0),
+                   "xsmi_bn_relu_maxpool_fwd: misaligned tensor");
+    XSMI_CHECK_ARG((moving_mean == nullptr) == (moving_var == nullptr), "xsmi_bn_relu_maxpool_fwd: give both moving statistics or neither");
+    XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_relu_maxpool_fwd: workspace too small");
+    hipStream_t st = xsmi::stream();
+    const int HW = H * W;
+    double *part = (double *)ws;
+    const BnSplit split = bn_split(N, HW, true);
+    launch_bn_partial(st, x, nullptr, nullptr, part, C, HW, split, nullptr, nullptr);
+    XSMI_LAUNCH_CHECK("bn_partial_kernel");
+    const int Q = W / 4, OH = H / 2;
+    const uint32_t total = (uint32_t)N * OH * Q;
+    uint32_t sp = total / 2048;
+    if (sp < 1) sp = 1;
+    if (sp > (uint32_t)BN_SPLIT) sp = BN_SPLIT;
+    const uint32_t per = (total + sp - 1) / sp;
+    const int nsp = (int)((total + per - 1) / per);
+    const BnFwdOut o{pooled, nullptr, sqrtvar, mean, var, moving_mean, moving_var, neg_mask, nullptr};
+    hipLaunchKernelGGL(bn_relu_maxpool_kernel, dim3(C, nsp), dim3(256), 0, st, x, gamma, beta, part, split.nsplit, (double)N * HW,
+                       eps, momentum, o, idx, C, H, W, xsmi::make_fastdiv(Q), xsmi::make_fastdiv(OH * Q), total, per);
+    XSMI_LAUNCH_CHECK("bn_relu_maxpool_kernel");
+    return XSMI_OK;
 }
 
 int xsmi_bn_add_relu_fwd(const float *x, const float *gamma, const float *beta, const float *residual, float *y,

@@ -471,13 +471,13 @@ def batch_norm(inputs, gamma, beta, moving_mean, moving_variance, axis=1, traini
         fused = is_device(x) and is_device(mm) and is_device(mv)      # the normalisation kernel updates them
         track = GLOBAL.COMPUTE_GRAD and bool(inputs.requires_grad or gamma.requires_grad or beta.requires_grad)
         neg_mask = dev.empty(x.shape, np.uint8) if relu else None
-        # Without a ReLU of its own the device launch is held back until the next operation: at the end of a residual
-        # block that is the add of the shortcut and then the in-place ReLU, and the three run as one normalisation
-        # (backend/kernels.bn_fwd); anything else sees the plain result.
+        # The device launch is held back until the next operation: at the end of a residual block that is the add of
+        # the shortcut and then the in-place ReLU, behind the first convolution of a ResNet the 3x3/2 max-pool, and
+        # either runs inside the normalisation's second pass (backend/kernels.bn_fwd); anything else sees the plain result.
         y, xhat, sqrtvar, mean_, var_ = A.batch_norm_train(x, gamma.eval, beta.eval, epsilon, dst,
                                                            (mm.reshape(-1), mv.reshape(-1)) if fused else None, momentum,
                                                            neg_mask, want_xhat=False,
-                                                           defer=fused and track and not relu)
+                                                           defer=fused and track)
         if not track:
             neg_mask = None
         if not fused:
