@@ -404,6 +404,16 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
                 const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C, int HW, void *ws,
                 size_t ws_bytes);
 
+/* xsmi_maxpool2d_bwd (3 x 3, stride 2, pad 1, beta 0) followed by xsmi_bn_bwd in its mean != NULL form, without the
+ * pool's input gradient ever being stored: dpooled / idx are the pool's (N, C, H/2, W/2) upstream gradient and window
+ * indices, x / mean / sqrtvar / gamma / neg_mask the normalisation's, as in xsmi_bn_bwd.  The routed gradient is formed
+ * where the two passes need it, with the pool kernel's own arithmetic; dx is within float32 rounding of the two
+ * separate calls (the channel sums are added in another order) and reproducible.  H even, W a multiple of 4.
+ * Stands for xs/nn/grad_fn.py:206-235 followed by xs/nn/grad_fn.py:379-411 (and 146-157 through neg_mask). */
+int xsmi_bn_bwd_maxpool(const float *dpooled, const uint8_t *idx, const float *x, const float *mean, const float *sqrtvar,
+                        const float *gamma, const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C,
+                        int H, int W, void *ws, size_t ws_bytes);
+
 /* Mean over k x k windows at stride (sh, sw) of an NCHW tensor, no padding: y is (N, C, (H-k)/sh+1, (W-k)/sw+1),
  * float64 sum, one rounding; and its gradient, overwritten into dx: every window hands dy / k^2 (a float32 quotient)
  * to its cells, overlapping windows add up in float64 (avg_pool2d, xs/nn/functional.py:539-583,

@@ -119,6 +119,49 @@ def test_batch_norm_relu_max_pool_as_one_pass(gpu, shape):
     np.testing.assert_array_equal(K.maxpool2d_fwd(y4, 3, (2, 2), 1)[0].numpy(), ref[0])
 
 
+@pytest.mark.parametrize("shape", [(4, 8, 56, 56), (2, 3, 112, 112), (33, 5, 16, 20), (2, 4, 8, 12)])
+def test_max_pool_gradient_inside_the_batch_norm_backward(gpu, shape):
+    """The backward of the same chain: a held-back 3x3 / stride 2 / pad 1 max-pool gradient followed by the backward of
+    the normalisation that fed the pool runs as that backward's two passes, which form the routed gradient themselves.
+    The routed values are the pool kernel's own; the channel sums are added in another order, so dx, dgamma and dbeta
+    agree with the separate passes to float32 rounding; the pool's gradient tensor is not stored and says so."""
+    K = gpu.kernels
+    rng = np.random.default_rng(sum(shape) + 3)
+    n, c, h, w = shape
+    x = (rng.standard_normal(shape) * 2 + 0.5).astype(np.float32)
+    x[0, 0, :2, :4] = x[0, 0, 0, 0]
+    gamma = rng.uniform(0.5, 1.5, c).astype(np.float32); beta = rng.standard_normal(c).astype(np.float32)
+    xd, gd, bd = gpu.to_device(x), gpu.to_device(gamma), gpu.to_device(beta)
+    mask = gpu.empty(shape, np.uint8)
+    y, _, sq, mean, _ = K.bn_fwd(xd, gd, bd, 1e-5, neg_mask=mask, want_xhat=False)
+    p, idx = K.maxpool2d_fwd(y, 3, (2, 2), 1)
+    dp = gpu.to_device(rng.standard_normal(p.shape).astype(np.float32))
+    g_sep = K.maxpool2d_bwd(dp, idx, shape, 3, (2, 2), 1)
+    g_np = g_sep.numpy()                              # a read in between: the pool gradient is launched by itself
+    dx_s, dg_s, db_s = K.bn_bwd(g_sep, xd, sq, gd, neg_mask=mask, mean=mean)
+    g_fused = K.maxpool2d_bwd(dp, idx, shape, 3, (2, 2), 1)
+    dx_f, dg_f, db_f = K.bn_bwd(g_fused, xd, sq, gd, neg_mask=mask, mean=mean)
+    assert rel_l2(dx_f.numpy(), dx_s.numpy()) <= 1e-6
+    np.testing.assert_allclose(dg_f.numpy(), dg_s.numpy(), rtol=2e-6, atol=1e-5)
+    np.testing.assert_allclose(db_f.numpy(), db_s.numpy(), rtol=2e-6, atol=1e-5)
+    with pytest.raises(gpu.XsmiError, match="not stored"):
+        g_fused.numpy()
+    # against float64 formulas on the routed gradient
+    m = x.size // c
+    b = [1, -1, 1, 1]
+    d = np.where(mask.numpy() != 0, 0.0, g_np.astype(np.float64))
+    xh = (x.astype(np.float64) - mean.numpy().astype(np.float64).reshape(b)) / sq.numpy().astype(np.float64).reshape(b)
+    dxh = d * gamma.reshape(b)
+    ref = (dxh * m - dxh.sum(axis=(0, 2, 3)).reshape(b) - xh * (dxh * xh).sum(axis=(0, 2, 3)).reshape(b)) / (m * sq.numpy().reshape(b))
+    assert rel_l2(dx_f.numpy(), ref) <= 2e-5
+    # the normalisation without the batch mean (stored normalised input) and a pool gradient that accumulates: separate
+    g2 = K.maxpool2d_bwd(dp, idx, shape, 3, (2, 2), 1)
+    xh32 = gpu.to_device(xh.astype(np.float32))
+    dx2, _, _ = K.bn_bwd(g2, xh32, sq, gd, neg_mask=mask)
+    np.testing.assert_array_equal(g2.numpy(), g_np)
+    assert rel_l2(dx2.numpy(), ref) <= 2e-5
+
+
 # two-kernel float4 form, two-kernel scalar form (planes not a multiple of four), single-kernel forms (256 / 1024 threads)
 @pytest.mark.parametrize("shape", [(8, 16, 40, 40), (6, 5, 37, 41), (32, 64, 14, 14), (4, 8, 6, 6), (64, 16)])
 def test_batch_norm_add_relu_as_one_pass(gpu, shape):

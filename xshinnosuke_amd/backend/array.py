@@ -5,7 +5,7 @@ import weakref
 
 import numpy as np
 
-from .capi import lib, ensure_init, XsmiError
+from .capi import lib, ensure_init, XsmiError, flush_deferred
 
 
 _DTYPE_CLASS = np.dtype(np.float32).__class__
@@ -207,9 +207,13 @@ class DeviceArray:
         return cl
 
     def _overwritten(self):
-        """Called before the whole array is overwritten: a channels-last form need not be converted back."""
+        """Called before the whole array is overwritten: a channels-last form need not be converted back, and contents
+        that were never produced (never_written) no longer matter."""
+        whole = self._offset == 0 and self.nbytes >= self._block.logical
+        if whole:
+            self._block.unwritten = None
         cl = self._block.cl
-        if cl is not None and cl.valid and self._offset == 0 and self.nbytes >= self._block.logical:
+        if cl is not None and cl.valid and whole:
             cl.valid = False
 
     def is_fresh(self):
@@ -309,6 +313,7 @@ class DeviceArray:
         """Clear the array.  ``lazy=True`` only marks a whole allocation as zero: the memset happens on
         the first ordinary use, and not at all if the first use overwrites everything (take_fresh)."""
         blk = self._block
+        flush_deferred(blk)                   # a held-back operation that uses this allocation comes first
         self._overwritten()
         if lazy and self._offset == 0 and self.nbytes >= blk.logical:
             blk.lazy_zero = True

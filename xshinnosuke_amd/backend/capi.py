@@ -98,6 +98,7 @@ SIGNATURES = {
     "xsmi_bn_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_add_relu_fwd": (_i, [_vp] * 10 + [_f, _vp, _i, _i, _i, _f, _vp, _sz]),
     "xsmi_bn_relu_maxpool_fwd": (_i, [_vp] * 11 + [_f, _i, _i, _i, _i, _f, _vp, _sz]),
+    "xsmi_bn_bwd_maxpool": (_i, [_vp] * 10 + [_i, _i, _i, _i, _vp, _sz]),
     "xsmi_bn_infer": (_i, [_vp] * 6 + [_i, _i, _i, _f, _i]),
     "xsmi_bn_fold": (_i, [_vp] * 8 + [_i, _i, _f]),
     "xsmi_bn_bwd": (_i, [_vp] * 9 + [_i, _i, _i, _vp, _sz]),
@@ -224,6 +225,9 @@ def layouts_enqueued(*held):
 #                                 next call is a held-back add with its result as one operand, it becomes
 #   ("bn_add", entry, a, b, out)  and if the call after that is the in-place ReLU (with mask) of the sum, the three run
 #                                 as one normalisation whose second pass adds the other operand and clips.
+#   ("pool_bwd", entry)           the gradient of a 3x3/2 max-pool into a fresh buffer (kernels.PoolBwdEntry); if the
+#                                 next call is the backward of the normalisation that fed the pool, the routed gradient
+#                                 is formed inside that backward's two passes instead of being stored.
 # Every other call enqueues what is held back first, in order, so nothing can read or change the operands or the
 # results between an operation and the point where it was asked for.
 _deferred = []          # at most one entry
@@ -234,12 +238,30 @@ def _flush_deferred():
     if op[0] == "add":
         _, a, b, out = op
         lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
-    elif op[0] == "bn":
+    elif op[0] in ("bn", "pool_bwd"):
         op[1].launch()
     else:
         _, entry, a, b, out = op
         entry.launch()
         lib.call("xsmi_add", a.cptr, b.cptr, out.cptr, a.size)
+
+
+def _deferred_arrays():
+    op = _deferred[0]
+    if op[0] == "add":
+        return op[1:]
+    arrays = list(op[1].arrays())
+    if op[0] == "bn_add":
+        arrays.extend(op[2:])
+    return arrays
+
+
+def flush_deferred(block=None):
+    """Enqueue what is held back, if anything (with ``block``: only if it uses that allocation).  For changes of an
+    array's state that make no call into the library (a clear that is only noted): a held-back operation may still
+    have to read the array as it was, or to write it first."""
+    if _deferred and (block is None or any(a is not None and a._block is block for a in _deferred_arrays())):
+        _flush_deferred()
 
 
 def defer_add(a, b, out):
@@ -260,6 +282,23 @@ def take_deferred_bn(a, b):
     if not _deferred:
         return None
     if _deferred[0][0] == "bn" and (_deferred[0][1].y is a or _deferred[0][1].y is b):
+        return _deferred.pop()[1]
+    _flush_deferred()
+    return None
+
+
+def defer_pool_bwd(entry):
+    if _deferred:
+        _flush_deferred()
+    _deferred.append(("pool_bwd", entry))
+
+
+def take_deferred_pool_bwd(dx):
+    """The held-back max-pool gradient whose result is ``dx`` (no longer pending), or None (anything else that was
+    pending is enqueued)."""
+    if not _deferred:
+        return None
+    if _deferred[0][0] == "pool_bwd" and _deferred[0][1].dx is dx:
         return _deferred.pop()[1]
     _flush_deferred()
     return None

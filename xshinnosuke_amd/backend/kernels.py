@@ -391,9 +391,32 @@ def maxpool2d_bwd(dy, idx, x_shape, k, stride, pad=0, dx=None, accumulate=False)
     elif dx.shape != tuple(x_shape):
         raise ValueError("max_pool2d backward: dx has shape %s, expected %s" % (dx.shape, tuple(x_shape)))
     beta = _beta(accumulate, dx)
+    if (FUSE_BN_ADD_RELU and beta == 0.0 and k == 3 and tuple(stride) == (2, 2) and pad == 1 and h % 2 == 0 and w % 4 == 0
+            and dx.is_whole()):
+        # held back: if the next call is the backward of the normalisation that fed the pool, the routed gradient is
+        # formed inside that backward (bn_bwd) and never stored
+        e = PoolBwdEntry()
+        e.dy, e.idx, e.dx, e.dims = dy, idx, dx, (n, c, h, w)
+        dy.ptr; idx.ptr                               # pending clears are settled now
+        capi.defer_pool_bwd(e)
+        return dx
     lib.call("xsmi_maxpool2d_bwd", dy.cptr, idx.cptr, dx.cptr, n, c, h, w, int(k), int(stride[0]), int(stride[1]),
              int(pad), beta)
     return dx
+
+
+class PoolBwdEntry:
+    """The gradient of a 3x3 / stride 2 / pad 1 max-pool into a buffer that is overwritten, asked for and not launched
+    yet (see capi._deferred)."""
+
+    __slots__ = ("dy", "idx", "dx", "dims")
+
+    def arrays(self):
+        return (self.dy, self.idx, self.dx)
+
+    def launch(self):
+        n, c, h, w = self.dims
+        lib.call("xsmi_maxpool2d_bwd", self.dy.cptr, self.idx.cptr, self.dx.cptr, n, c, h, w, 3, 2, 2, 1, 0.0)
 
 
 def relu_mask_bwd(dy, neg_mask, dx=None, accumulate=False):
@@ -587,6 +610,9 @@ class BnEntry:
     __slots__ = ("x", "gamma", "beta", "eps", "y", "sqrtvar", "mean", "var", "mm", "mv", "momentum", "dims", "ws",
                  "relu_mask")
 
+    def arrays(self):
+        return (self.x, self.gamma, self.beta, self.y, self.sqrtvar, self.mean, self.var, self.mm, self.mv, self.relu_mask)
+
     def launch(self, residual=None, out=None, neg_mask=None, pooled=None, idx=None):
         """Plain: y = gamma * xhat + beta (clipped at zero, with the sign mask, when the entry has a ReLU of its own).
         With ``residual``: out = max(0, y + residual) and its sign mask in one pass.  With ``pooled``: the 3x3/2
@@ -680,14 +706,33 @@ def bn_bwd(dy, xhat, sqrtvar, gamma, dx=None, dgamma=None, dbeta=None, neg_mask=
     if xhat.size != dy.size or (mean is not None and mean.size != dy.shape[1]):
         raise ValueError("bn_bwd: operands do not match %s" % (dy.shape,))
     n, c, hw = _nchw3(dy.shape)
-    dx = empty(dy.shape) if dx is None else dx
-    dgamma = empty((c,)) if dgamma is None else dgamma
-    dbeta = empty((c,)) if dbeta is None else dbeta
-    if dx.size != dy.size or dgamma.size != c or dbeta.size != c:
-        raise ValueError("bn_bwd: output buffers do not match %s" % (dy.shape,))
-    for o in (dx, dgamma, dbeta):
-        o.take_fresh()
-    ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
+    # dy may be the gradient of a max-pool that has not been launched yet: it is taken out of the queue first (an
+    # allocation below may call into the library, which would launch it)
+    pool = capi.take_deferred_pool_bwd(dy)
+    try:
+        dx = empty(dy.shape) if dx is None else dx
+        dgamma = empty((c,)) if dgamma is None else dgamma
+        dbeta = empty((c,)) if dbeta is None else dbeta
+        if dx.size != dy.size or dgamma.size != c or dbeta.size != c:
+            raise ValueError("bn_bwd: output buffers do not match %s" % (dy.shape,))
+        for o in (dx, dgamma, dbeta):
+            o.take_fresh()
+        ws, ws_bytes = _ws.get(lib.raw("xsmi_bn_workspace_bytes")(c))
+    except Exception:
+        if pool is not None:
+            pool.launch()                             # what was asked for before this call still happens
+        raise
+    if pool is not None:
+        if mean is not None and len(dy.shape) == 4 and dx is not dy and dx.is_whole():
+            # pool gradient and normalisation gradient as two passes over (pooled gradient, indices, x, mask)
+            pn, pc, ph, pw = pool.dims
+            dy.never_written("this max-pool gradient was consumed by the batch-norm backward that followed it and was not "
+                             "stored (XSMI_FUSE_BN_ADD_RELU=0 keeps the passes apart)")
+            lib.call("xsmi_bn_bwd_maxpool", pool.dy.cptr, pool.idx.cptr, xhat.cptr, mean.cptr, sqrtvar.cptr, gamma.cptr,
+                     neg_mask.cptr if neg_mask is not None else None, dx.cptr, dgamma.cptr, dbeta.cptr, pn, pc, ph, pw,
+                     ws, ws_bytes)
+            return dx, dgamma, dbeta
+        pool.launch()
     lib.call("xsmi_bn_bwd", dy.cptr, xhat.cptr, mean.cptr if mean is not None else None, sqrtvar.cptr, gamma.cptr,
              neg_mask.cptr if neg_mask is not None else None, dx.cptr, dgamma.cptr, dbeta.cptr, n, c, hw, ws, ws_bytes)
     return dx, dgamma, dbeta

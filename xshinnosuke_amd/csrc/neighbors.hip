@@ -423,56 +423,74 @@ __global__ void __launch_bounds__(256) bn_relu_maxpool_kernel(const float *__res
     }
     const int OH = H >> 1, OW = W >> 1, Q = OW >> 1;
     const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
-    for (uint32_t u = beg + threadIdx.x; u < end; u += 256) {
-        const uint32_t n = xsmi::fdiv(u, dOHQ), rem = u - n * dOHQ.d;
-        const int oh = (int)xsmi::fdiv(rem, dQ), j = (int)rem - oh * Q;
-        const size_t pl = (size_t)n * C + c;
-        const float *plane = x + pl * (size_t)H * W;
-        float4 v[3];
-        float lf[3];
-        bool have[3];
+    auto act = [&](float xv, unsigned char &neg) {
+        const float pre = g * ((xv - mu) / rs) + bt;
+        neg = pre < 0.f ? 1 : 0;
+        return pre < 0.f ? 0.f : pre;
+    };
+    // two units per thread and step, the loads of both before the first use (a unit past the end repeats the first
+    // one's loads and stores nothing)
+    for (uint32_t u0 = beg + threadIdx.x; u0 < end; u0 += 512) {
+        constexpr int UNR = 2;
+        bool ok[UNR], have[UNR][3];
+        int oh[UNR], jj[UNR];
+        size_t pl[UNR];
+        float4 v[UNR][3];
+        float lf[UNR][3];
 #pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const int ih = 2 * oh - 1 + r;
-            have[r] = (unsigned)ih < (unsigned)H;
-            v[r] = make_float4(0.f, 0.f, 0.f, 0.f);
-            lf[r] = 0.f;
-            if (have[r]) {
-                v[r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * W + 4 * j);
-                if (j > 0) lf[r] = plane[(size_t)ih * W + 4 * j - 1];
+        for (int k = 0; k < UNR; ++k) {
+            ok[k] = u0 + 256u * k < end;
+            const uint32_t u = ok[k] ? u0 + 256u * k : u0;
+            const uint32_t n = xsmi::fdiv(u, dOHQ), rem = u - n * dOHQ.d;
+            oh[k] = (int)xsmi::fdiv(rem, dQ);
+            jj[k] = (int)rem - oh[k] * Q;
+            pl[k] = (size_t)n * C + c;
+            const float *plane = x + pl[k] * (size_t)H * W;
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                const int ih = 2 * oh[k] - 1 + r;
+                have[k][r] = (unsigned)ih < (unsigned)H;
+                v[k][r] = make_float4(0.f, 0.f, 0.f, 0.f);
+                lf[k][r] = 0.f;
+                if (have[k][r]) {
+                    v[k][r] = *reinterpret_cast<const float4 *>(plane + (size_t)ih * W + 4 * jj[k]);
+                    if (jj[k] > 0) lf[k][r] = plane[(size_t)ih * W + 4 * jj[k] - 1];
+                }
             }
         }
-        auto act = [&](float xv, unsigned char &neg) {
-            const float pre = g * ((xv - mu) / rs) + bt;
-            neg = pre < 0.f ? 1 : 0;
-            return pre < 0.f ? 0.f : pre;
-        };
 #pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            unsigned char nl, n0, n1, n2, n3;
-            if (have[r]) {                             // a row outside the image is the pool's zero border as it is
-                lf[r] = j > 0 ? act(lf[r], nl) : 0.f;
-                v[r].x = act(v[r].x, n0); v[r].y = act(v[r].y, n1); v[r].z = act(v[r].z, n2); v[r].w = act(v[r].w, n3);
-                if (r > 0)
-                    *reinterpret_cast<uchar4 *>(o.neg_mask + (pl * H + (2 * oh - 1 + r)) * (size_t)W + 4 * j) = make_uchar4(n0, n1, n2, n3);
+        for (int k = 0; k < UNR; ++k) {
+            if (!ok[k]) break;
+            const int j = jj[k];
+#pragma unroll
+            for (int r = 0; r < 3; ++r) {
+                unsigned char nl, n0, n1, n2, n3;
+                if (have[k][r]) {                      // a row outside the image is the pool's zero border as it is
+                    lf[k][r] = j > 0 ? act(lf[k][r], nl) : 0.f;
+                    v[k][r].x = act(v[k][r].x, n0); v[k][r].y = act(v[k][r].y, n1);
+                    v[k][r].z = act(v[k][r].z, n2); v[k][r].w = act(v[k][r].w, n3);
+                    if (r > 0)
+                        *reinterpret_cast<uchar4 *>(o.neg_mask + (pl[k] * H + (2 * oh[k] - 1 + r)) * (size_t)W + 4 * j) =
+                            make_uchar4(n0, n1, n2, n3);
+                }
             }
-        }
-        float b0 = 0.f, b1 = 0.f;
-        int w0 = 0, w1 = 0;
+            float b0 = 0.f, b1 = 0.f;
+            int w0 = 0, w1 = 0;
 #pragma unroll
-        for (int r = 0; r < 3; ++r) {
-            const float left = lf[r];
-            if (r == 0 || left > b0) { b0 = left; w0 = r * 3 + 0; }
-            if (v[r].x > b0) { b0 = v[r].x; w0 = r * 3 + 1; }
-            if (v[r].y > b0) { b0 = v[r].y; w0 = r * 3 + 2; }
-            if (r == 0 || v[r].y > b1) { b1 = v[r].y; w1 = r * 3 + 0; }
-            if (v[r].z > b1) { b1 = v[r].z; w1 = r * 3 + 1; }
-            if (v[r].w > b1) { b1 = v[r].w; w1 = r * 3 + 2; }
+            for (int r = 0; r < 3; ++r) {
+                const float left = lf[k][r];
+                if (r == 0 || left > b0) { b0 = left; w0 = r * 3 + 0; }
+                if (v[k][r].x > b0) { b0 = v[k][r].x; w0 = r * 3 + 1; }
+                if (v[k][r].y > b0) { b0 = v[k][r].y; w0 = r * 3 + 2; }
+                if (r == 0 || v[k][r].y > b1) { b1 = v[k][r].y; w1 = r * 3 + 0; }
+                if (v[k][r].z > b1) { b1 = v[k][r].z; w1 = r * 3 + 1; }
+                if (v[k][r].w > b1) { b1 = v[k][r].w; w1 = r * 3 + 2; }
+            }
+            const size_t ob = (pl[k] * OH + oh[k]) * (size_t)OW + 2 * j;
+            bn_f2v yv; yv.x = b0; yv.y = b1;
+            __builtin_nontemporal_store(yv, reinterpret_cast<bn_f2v *>(o.y + ob));
+            if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + ob));
         }
-        const size_t ob = (pl * OH + oh) * (size_t)OW + 2 * j;
-        bn_f2v yv; yv.x = b0; yv.y = b1;
-        __builtin_nontemporal_store(yv, reinterpret_cast<bn_f2v *>(o.y + ob));
-        if (idx) __builtin_nontemporal_store((unsigned short)(w0 | (w1 << 8)), reinterpret_cast<unsigned short *>(idx + ob));
     }
 }
 // pass 2 of the backward: block (c, sp) turns the partial sums into dbeta = sum(dy) and dgamma = sum(dy*xhat) (block
@@ -531,6 +549,138 @@ __global__ void __launch_bounds__(256) bn_bwd_apply_kernel(const float *__restri
                 ov[q] = g * (m * d - db - h * dg) / den;
             }
             if (VEC) *reinterpret_cast<float4 *>(dx + off[k]) = *reinterpret_cast<float4 *>(ov); else dx[off[k]] = ov[0];
+        }
+    }
+}
+
+// The backward of bn_relu_maxpool_kernel's chain: the gradient of the 3 x 3 / stride 2 / pad 1 max-pool is not stored
+// as a tensor of the input's size and read twice, it is formed where the normalisation's two backward passes need it.
+// A unit is columns 4j .. 4j + 3 of the input rows 2a and 2a + 1 of one plane: their routed gradients come from the
+// pooled rows a and a + 1, columns 2j .. 2j + 2 (gradient and window index), as in maxpool_bwd_3x3s2p1: one, two, two
+// and four contributors per cell, the four-term cells added in float64 (the reference's order), -0 turned into +0.
+struct PoolRouted { float e[4], o[4]; };
+__device__ __forceinline__ PoolRouted pool_routed_3x3s2p1(const float *__restrict__ dp, const uint8_t *__restrict__ idx,
+                                                          size_t obase, int OH, int OW, int a, int j) {
+    float gv[2][3];
+    int iv[2][3];
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        const int oh = a + q;                          // a + 1 == OH: below the last output row
+        float2 gg = make_float2(0.f, 0.f);
+        int i0 = -1, i1 = -1, in = -1;
+        float gn = 0.f;
+        const size_t ro = obase + (size_t)oh * OW + 2 * j;
+        if (oh < OH) {
+            gg = *reinterpret_cast<const float2 *>(dp + ro);
+            const uchar2 ii = *reinterpret_cast<const uchar2 *>(idx + ro);
+            i0 = ii.x; i1 = ii.y;
+            if (2 * j + 2 < OW) { gn = dp[ro + 2]; in = idx[ro + 2]; }
+        }
+        gv[q][0] = gg.x + 0.f; gv[q][1] = gg.y + 0.f; gv[q][2] = gn + 0.f;
+        iv[q][0] = i0; iv[q][1] = i1; iv[q][2] = in;
+    }
+    auto pick = [&](int q, int m, int tap) { return iv[q][m] == tap ? gv[q][m] : 0.f; };
+    PoolRouted r;
+#pragma unroll
+    for (int m = 0; m < 2; ++m) {
+        r.e[2 * m] = pick(0, m, 4);
+        r.e[2 * m + 1] = pick(0, m + 1, 3) + pick(0, m, 5);
+        r.o[2 * m] = pick(1, m, 1) + pick(0, m, 7);
+        r.o[2 * m + 1] = (float)((((double)pick(1, m + 1, 0) + (double)pick(1, m, 2)) + (double)pick(0, m + 1, 6)) +
+                                 (double)pick(0, m, 8));
+    }
+    return r;
+}
+// APPLY false: pass 1, per (channel, split) partial sums of dy and dy * xhat; true: pass 2, dx.  Units of a channel are
+// numbered (image, row pair, column quad); split sp owns units [sp * per, (sp + 1) * per).
+template <bool APPLY>
+__global__ void __launch_bounds__(256) bn_bwd_maxpool_kernel(const float *__restrict__ dp, const uint8_t *__restrict__ idx,
+                                                              const float *__restrict__ x, const float *__restrict__ mean,
+                                                              const float *__restrict__ sqrtvar, const float *__restrict__ gamma,
+                                                              const uint8_t *__restrict__ zero, double *__restrict__ part,
+                                                              int nsplit_part, float *__restrict__ dgamma, float *__restrict__ dbeta,
+                                                              float *__restrict__ dx, float m, int C, int H, int W,
+                                                              xsmi::FastDiv dQ4, xsmi::FastDiv dGQ, uint32_t total, uint32_t per) {
+    __shared__ double sm[4];
+    const int c = blockIdx.x, sp = blockIdx.y;
+    const int OH = H >> 1, OW = W >> 1, Q4 = W >> 2;
+    const float mu = mean[c], rs = sqrtvar[c];
+    float db = 0.f, dg = 0.f, g = 0.f, den = 1.f;
+    if (APPLY) {
+        double t0, t1;
+        bn_channel_sums(part, c, nsplit_part, sm, t0, t1);
+        db = (float)t0; dg = (float)t1;
+        if (sp == 0 && threadIdx.x == 0) {
+            dbeta[c] = db;
+            dgamma[c] = dg;
+        }
+        g = gamma[c];
+        den = m * rs;
+    }
+    const uint32_t beg = (uint32_t)sp * per, end = min(total, beg + per);
+    double s0 = 0.0, s1 = 0.0;
+    // two units per thread and step, all loads of both before the first use (a unit past the end repeats the first
+    // one's loads and contributes nothing): one unit at a time left the kernel waiting on memory latency
+    for (uint32_t u0 = beg + threadIdx.x; u0 < end; u0 += 512) {
+        constexpr int UNR = 2;
+        size_t off[UNR];
+        bool ok[UNR];
+        float4 xe[UNR], xo[UNR];
+        uchar4 ze[UNR], zo[UNR];
+        PoolRouted r[UNR];
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            ok[k] = u0 + 256u * k < end;
+            const uint32_t u = ok[k] ? u0 + 256u * k : u0;
+            const uint32_t n = xsmi::fdiv(u, dGQ), rem = u - n * dGQ.d;
+            const int a = (int)xsmi::fdiv(rem, dQ4), j = (int)rem - a * Q4;
+            const size_t pl = (size_t)n * C + c;
+            off[k] = (pl * H + 2 * a) * (size_t)W + 4 * j;
+            xe[k] = *reinterpret_cast<const float4 *>(x + off[k]);
+            xo[k] = *reinterpret_cast<const float4 *>(x + off[k] + W);
+            ze[k] = make_uchar4(0, 0, 0, 0); zo[k] = ze[k];
+            if (zero) {
+                ze[k] = *reinterpret_cast<const uchar4 *>(zero + off[k]);
+                zo[k] = *reinterpret_cast<const uchar4 *>(zero + off[k] + W);
+            }
+            r[k] = pool_routed_3x3s2p1(dp, idx, pl * OH * (size_t)OW, OH, OW, a, j);
+        }
+#pragma unroll
+        for (int k = 0; k < UNR; ++k) {
+            const float xv[2][4] = {{xe[k].x, xe[k].y, xe[k].z, xe[k].w}, {xo[k].x, xo[k].y, xo[k].z, xo[k].w}};
+            const unsigned char zv[2][4] = {{ze[k].x, ze[k].y, ze[k].z, ze[k].w}, {zo[k].x, zo[k].y, zo[k].z, zo[k].w}};
+            float ov[2][4];
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                double t0 = 0.0, t1 = 0.0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    const float d = zv[q][i] ? 0.f : (q ? r[k].o[i] : r[k].e[i]);
+                    const float h = (xv[q][i] - mu) / rs;
+                    if (APPLY) {
+                        ov[q][i] = g * (m * d - db - h * dg) / den;
+                    } else {
+                        t0 += (double)d;
+                        t1 += (double)d * (double)h;
+                    }
+                }
+                if (ok[k]) {
+                    s0 += t0;
+                    s1 += t1;
+                }
+            }
+            if (APPLY && ok[k]) {
+                *reinterpret_cast<float4 *>(dx + off[k]) = make_float4(ov[0][0], ov[0][1], ov[0][2], ov[0][3]);
+                *reinterpret_cast<float4 *>(dx + off[k] + W) = make_float4(ov[1][0], ov[1][1], ov[1][2], ov[1][3]);
+            }
+        }
+    }
+    if (!APPLY) {
+        s0 = block_sum(s0, sm);
+        s1 = block_sum(s1, sm);
+        if (threadIdx.x == 0) {
+            part[((size_t)c * BN_SPLIT + sp) * 2 + 0] = s0;
+            part[((size_t)c * BN_SPLIT + sp) * 2 + 1] = s1;
         }
     }
 }
@@ -1151,6 +1301,37 @@ int xsmi_bn_bwd(const float *dy, const float *xhat, const float *mean, const flo
         hipLaunchKernelGGL(bn_bwd_apply_kernel<false>, dim3(C, ap.nsplit), dim3(256), 0, st, dy, xhat, sqrtvar, gamma, part,
                            nsplit, dgamma, dbeta, neg_mask, dx, m, mean, C, HW, ap.dU, ap.total, ap.per);
     XSMI_LAUNCH_CHECK("bn_bwd_apply_kernel");
+    return XSMI_OK;
+}
+
+int xsmi_bn_bwd_maxpool(const float *dpooled, const uint8_t *idx, const float *x, const float *mean, const float *sqrtvar,
+                        const float *gamma, const uint8_t *neg_mask, float *dx, float *dgamma, float *dbeta, int N, int C,
+                        int H, int W, void *ws, size_t ws_bytes) {
+    XSMI_REQUIRE_INIT();
+    XSMI_CHECK_ARG(N > 0 && C > 0 && H > 0 && W > 0, "xsmi_bn_bwd_maxpool: empty tensor");
+    XSMI_CHECK_ARG(H % 2 == 0 && W % 4 == 0, "xsmi_bn_bwd_maxpool: planes of an even number of rows, a multiple of four wide");
+    XSMI_CHECK_ARG((double)N * C * H * W < 536870912.0, "xsmi_bn_bwd_maxpool: tensors of 2^29 elements or more are not supported");
+    XSMI_CHECK_ARG(dpooled && idx && x && mean && sqrtvar && gamma && dx && dgamma && dbeta, "xsmi_bn_bwd_maxpool: null pointer");
+    XSMI_CHECK_ARG(aligned16(x) && aligned16(dx) && ((uintptr_t)dpooled & 7) == 0 && ((uintptr_t)idx & 1) == 0 &&
+                       (!neg_mask || ((uintptr_t)neg_mask & 3) == 0), "xsmi_bn_bwd_maxpool: misaligned tensor");
+    XSMI_CHECK_ARG(ws && ws_bytes >= xsmi_bn_workspace_bytes(C), "xsmi_bn_bwd_maxpool: workspace too small");
+    hipStream_t st = xsmi::stream();
+    double *part = (double *)ws;
+    const int Q4 = W / 4, G = H / 2;
+    const uint32_t total = (uint32_t)N * G * Q4;         // units of eight elements per channel
+    uint32_t sp = total / 1024;
+    if (sp < 1) sp = 1;
+    if (sp > (uint32_t)BN_SPLIT) sp = BN_SPLIT;
+    const uint32_t per = (total + sp - 1) / sp;
+    const int nsp = (int)((total + per - 1) / per);
+    const float m = (float)((double)N * H * W);
+    const xsmi::FastDiv dQ4 = xsmi::make_fastdiv(Q4), dGQ = xsmi::make_fastdiv(G * Q4);
+    hipLaunchKernelGGL(bn_bwd_maxpool_kernel<false>, dim3(C, nsp), dim3(256), 0, st, dpooled, idx, x, mean, sqrtvar, gamma,
+                       neg_mask, part, nsp, dgamma, dbeta, dx, m, C, H, W, dQ4, dGQ, total, per);
+    XSMI_LAUNCH_CHECK("bn_bwd_maxpool_kernel");
+    hipLaunchKernelGGL(bn_bwd_maxpool_kernel<true>, dim3(C, nsp), dim3(256), 0, st, dpooled, idx, x, mean, sqrtvar, gamma,
+                       neg_mask, part, nsp, dgamma, dbeta, dx, m, C, H, W, dQ4, dGQ, total, per);
+    XSMI_LAUNCH_CHECK("bn_bwd_maxpool_kernel");
     return XSMI_OK;
 }
 
