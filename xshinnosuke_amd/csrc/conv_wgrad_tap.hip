@@ -377,9 +377,9 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce9_kernel(const float *__r
         db[k] = (float)s;
         return;
     }
-    const size_t kc = (size_t)blockIdx.x * 256 + threadIdx.x;      // k * C + c
     const size_t KC = (size_t)K * C;
-    if (kc >= KC) return;
+    const bool live = (size_t)blockIdx.x * 256 + threadIdx.x < KC;
+    const size_t kc = live ? (size_t)blockIdx.x * 256 + threadIdx.x : 0;      // k * C + c
     double s[9];
 #pragma unroll
     for (int t = 0; t < 9; ++t) s[t] = 0.0;
@@ -397,9 +397,19 @@ __global__ void __launch_bounds__(256) wgrad_tap_reduce9_kernel(const float *__r
 #pragma unroll
         for (int t = 0; t < 9; ++t) s[t] += (double)src[(size_t)t * KC];
     }
-    float *dst = dw + kc * 9;
+    // A thread's nine values are nine consecutive floats of dw, a workgroup's 2304 one contiguous run: they go through
+    // the LDS so that every store instruction writes 256 consecutive floats (a lane storing its own nine one by one
+    // touches eighteen cache lines per instruction).
+    __shared__ double tile[256 * 9];                   // (float64: with `accumulate` the old value joins before the one rounding)
 #pragma unroll
-    for (int t = 0; t < 9; ++t) dst[t] = (float)(accumulate ? s[t] + (double)dst[t] : s[t]);
+    for (int t = 0; t < 9; ++t) tile[threadIdx.x * 9 + t] = s[t];
+    __syncthreads();
+    const size_t base = (size_t)blockIdx.x * 256 * 9, limit = KC * 9;
+#pragma unroll
+    for (int i = 0; i < 9; ++i) {
+        const size_t o = base + (size_t)i * 256 + threadIdx.x;
+        if (o < limit) dw[o] = (float)(accumulate ? tile[i * 256 + threadIdx.x] + (double)dw[o] : tile[i * 256 + threadIdx.x]);
+    }
 }
 
 // dst[plane][0 .. OHWa) = src[plane][0 .. OHW) followed by zeros
