@@ -212,6 +212,16 @@ inline ChanIdx make_chan(int C, int HW) {
     return ci;
 }
 
+// Stores of results that this kernel does not read again: non-temporal, lanes contiguous.
+typedef float nt_f4 __attribute__((ext_vector_type(4)));
+__device__ __forceinline__ void nt_store4(float *p, float a, float b, float c, float d) {
+    nt_f4 v; v.x = a; v.y = b; v.z = c; v.w = d;
+    __builtin_nontemporal_store(v, reinterpret_cast<nt_f4 *>(p));
+}
+__device__ __forceinline__ void nt_store_mask4(uint8_t *p, unsigned a, unsigned b, unsigned c, unsigned d) {
+    __builtin_nontemporal_store((uint32_t)(a | (b << 8) | (c << 16) | (d << 24)), reinterpret_cast<uint32_t *>(p));
+}
+
 // ---- batch norm --------------------------------------------------------------
 // pass 1: per (channel, split) partial sums of a and a*b over the N*HW elements of the channel
 // `zero` (optional, one byte per element): elements whose byte is set count as a == 0 (the gradient of a fused
@@ -470,8 +480,7 @@ __global__ void __launch_bounds__(256) bn_relu_maxpool_kernel(const float *__res
                     v[k][r].x = act(v[k][r].x, n0); v[k][r].y = act(v[k][r].y, n1);
                     v[k][r].z = act(v[k][r].z, n2); v[k][r].w = act(v[k][r].w, n3);
                     if (r > 0)
-                        *reinterpret_cast<uchar4 *>(o.neg_mask + (pl[k] * H + (2 * oh[k] - 1 + r)) * (size_t)W + 4 * j) =
-                            make_uchar4(n0, n1, n2, n3);
+                        nt_store_mask4(o.neg_mask + (pl[k] * H + (2 * oh[k] - 1 + r)) * (size_t)W + 4 * j, n0, n1, n2, n3);
                 }
             }
             float b0 = 0.f, b1 = 0.f;
@@ -670,8 +679,8 @@ __global__ void __launch_bounds__(256) bn_bwd_maxpool_kernel(const float *__rest
                 }
             }
             if (APPLY && ok[k]) {
-                *reinterpret_cast<float4 *>(dx + off[k]) = make_float4(ov[0][0], ov[0][1], ov[0][2], ov[0][3]);
-                *reinterpret_cast<float4 *>(dx + off[k] + W) = make_float4(ov[1][0], ov[1][1], ov[1][2], ov[1][3]);
+                nt_store4(dx + off[k], ov[0][0], ov[0][1], ov[0][2], ov[0][3]);
+                nt_store4(dx + off[k] + W, ov[1][0], ov[1][1], ov[1][2], ov[1][3]);
             }
         }
     }
